@@ -1,0 +1,62 @@
+// Shared device/host helpers for the gfx950 stage kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+namespace elf {
+
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+#define ELF_LDS __attribute__((address_space(3)))
+
+// Error plumbing: every C-ABI entry point returns 0 on success and a negative
+// code on failure; the message is kept per host thread.
+void set_error(const char* fmt, ...);
+const char* get_error();
+
+#define ELF_CHECK_HIP(expr)                                                             \
+	do {                                                                                \
+		hipError_t _e = (expr);                                                         \
+		if (_e != hipSuccess) {                                                         \
+			elf::set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e),      \
+			               __FILE__, __LINE__);                                         \
+			return -2;                                                                  \
+		}                                                                               \
+	} while (0)
+
+#define ELF_REQUIRE(cond, ...)                \
+	do {                                      \
+		if (!(cond)) {                        \
+			elf::set_error(__VA_ARGS__);      \
+			return -1;                        \
+		}                                     \
+	} while (0)
+
+__device__ __forceinline__ float bf2f(bf16_t v) { return (float)v; }
+__device__ __forceinline__ bf16_t f2bf(float v) { return (bf16_t)v; }
+
+// 64-lane butterfly reductions (wavefront = 64 on CDNA).
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+	for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+	return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+	for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+	return v;
+}
+
+}  // namespace elf

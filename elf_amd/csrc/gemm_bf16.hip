@@ -1,0 +1,330 @@
+// bf16 MFMA GEMM for gfx950 (CDNA4): C[M,N] (+)= sum_k A(m,k) * B(n,k), fp32 accumulation.
+//
+// The three contractions of a linear layer under the split backward map onto one kernel:
+//   forward  Y  = X  . W^T   A = X  [M,K] k-contiguous ("R"), B = W  [N,K] k-contiguous ("R")
+//   dX       dX = dY . W     A = dY [M,K] k-contiguous ("R"), B = W  [K,N] n-contiguous ("T")
+//   dW       dW += dY^T . X  A = dY [K,M] m-contiguous ("T"), B = X  [K,N] n-contiguous ("T")
+// (reference semantics: elf/zb_utils.py:20 forward, :34-37 dX, :235-244 dW accumulate).
+//
+// Tiling: one workgroup owns a BM x BN tile of C and walks K in steps of 64.  Global loads
+// are 16 B per lane into registers, then written to a double-buffered LDS tile, so the loads
+// of step k+1 are in flight while the MFMAs of step k run.  "R" operands are stored [row][k]
+// with 8 elements of padding and read with ds_read_b128; "T" operands are stored [k][row] as
+// they sit in memory and read with ds_read_b64_tr_b16, the LDS transpose read of gfx950, so
+// no operand is ever transposed through HBM.  Each wave owns a (BM/WR) x (BN/WC) sub-tile
+// built from v_mfma_f32_32x32x16_bf16.
+#include "common.h"
+#include "kernels.h"
+
+namespace elf {
+
+constexpr int BK = 64;
+constexpr int PAD_R = 8;    // elements of padding per row of an "R" tile ([row][BK+8])
+constexpr int PAD_T = 16;   // elements of padding per row of a "T" tile ([k][rows+16])
+
+struct GemmArgs {
+	const bf16_t* A;
+	const bf16_t* B;
+	void* C;
+	const bf16_t* R;  // residual (EPI_BF16_RESID)
+	int64_t lda, ldb, ldc, ldr;
+	int M, N, K;
+	int tiles_m, tiles_n;
+	int k_splits;      // >1: split-K with fp32 atomics (EPI_F32_ACC only)
+};
+
+template <int ROWS, bool T>
+struct TileShape {
+	static constexpr int LD = T ? (ROWS + PAD_T) : (BK + PAD_R);
+	static constexpr int ELEMS = T ? BK * LD : ROWS * LD;
+};
+
+// Global -> register staging of one operand tile. NT threads cooperatively fetch ROWS x BK
+// (or BK x ROWS) elements as 16-byte chunks.
+template <int ROWS, bool T, int NT>
+struct TileLoader {
+	static constexpr int CHUNKS = ROWS * BK / 8 / NT;  // 16-byte chunks per thread
+	static constexpr int CPR = T ? ROWS / 8 : BK / 8;  // chunks per stored row
+	static constexpr int RPP = NT / CPR;               // stored rows per pass
+	static_assert(CHUNKS >= 1 && (NT % CPR) == 0, "tile/threads mismatch");
+
+	u32x4 regs[CHUNKS];
+
+	// p points at the tile origin: for R, &A[row0][k0]; for T, &A[k0][row0].
+	__device__ __forceinline__ void load(const bf16_t* __restrict__ p, int64_t ld, int tid) {
+		const int c = tid % CPR, r = tid / CPR;
+#pragma unroll
+		for (int i = 0; i < CHUNKS; i++) {
+			const bf16_t* q = p + (int64_t)(r + i * RPP) * ld + c * 8;
+			regs[i] = *reinterpret_cast<const u32x4*>(q);
+		}
+	}
+	__device__ __forceinline__ void store(bf16_t* lds, int tid) const {
+		constexpr int LD = TileShape<ROWS, T>::LD;
+		const int c = tid % CPR, r = tid / CPR;
+#pragma unroll
+		for (int i = 0; i < CHUNKS; i++) {
+			*reinterpret_cast<u32x4*>(lds + (r + i * RPP) * LD + c * 8) = regs[i];
+		}
+	}
+};
+
+// One MFMA operand fragment (8 consecutive k for row lane%32, k-group lane/32) for the
+// 32-row slab starting at `row`, k-step `ks` (16 wide).
+template <int ROWS, bool T>
+__device__ __forceinline__ bf16x8 read_frag(const bf16_t* lds, int row, int ks, int lane) {
+	constexpr int LD = TileShape<ROWS, T>::LD;
+	if constexpr (!T) {
+		const bf16_t* p = lds + (row + (lane & 31)) * LD + ks * 16 + 8 * (lane >> 5);
+		return *reinterpret_cast<const bf16x8*>(p);
+	} else {
+		// Transposing read: inside each group of 16 lanes, lane j supplies the address of the
+		// 8-byte chunk (k = k0 + j/4, rows 4*(j%4)..+3) and receives rows (j) of k0..k0+3.
+		const int j = lane & 15;
+		const int rbase = row + 16 * ((lane & 31) >> 4) + 4 * (j & 3);
+		const int k0 = ks * 16 + 8 * (lane >> 5) + (j >> 2);
+		const bf16_t* p0 = lds + k0 * LD + rbase;
+		const bf16_t* p1 = p0 + 4 * LD;
+		s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 ELF_LDS*)(p0));
+		s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 ELF_LDS*)(p1));
+		s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+		return __builtin_bit_cast(bf16x8, v);
+	}
+}
+
+template <int BM, int BN, int WR, int WC, bool AT, bool BT, int EPI>
+__global__ __launch_bounds__(WR* WC * 64) void gemm_kernel(GemmArgs g) {
+	constexpr int NT = WR * WC * 64;
+	constexpr int WM = BM / WR, WN = BN / WC;
+	constexpr int TM = WM / 32, TN = WN / 32;
+	constexpr int A_ELEMS = TileShape<BM, AT>::ELEMS;
+	constexpr int B_ELEMS = TileShape<BN, BT>::ELEMS;
+
+	extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+	bf16_t* smem = reinterpret_cast<bf16_t*>(smem_raw);
+	bf16_t* sA[2] = {smem, smem + A_ELEMS + B_ELEMS};
+	bf16_t* sB[2] = {smem + A_ELEMS, smem + 2 * A_ELEMS + B_ELEMS};
+
+	const int tid = threadIdx.x;
+	const int lane = tid & 63;
+	const int wave = tid >> 6;
+	const int wr = wave / WC, wc = wave % WC;
+
+	// Tile assignment. Workgroups are dealt round-robin to the 8 XCDs, each with a private
+	// L2: give every XCD a contiguous run of tile ids, then walk tiles in column-major
+	// groups of GROUP_M tile rows so that a group shares its B panel and A rows in L2.
+	int pid = blockIdx.x;
+	const int ntiles = g.tiles_m * g.tiles_n;
+	int ksplit = 0;
+	if (g.k_splits > 1) {
+		ksplit = pid / ntiles;
+		pid = pid % ntiles;
+	}
+	if ((ntiles & 7) == 0) pid = (pid & 7) * (ntiles >> 3) + (pid >> 3);
+	constexpr int GROUP_M = 8;
+	const int per_group = GROUP_M * g.tiles_n;
+	const int group = pid / per_group;
+	const int first_m = group * GROUP_M;
+	const int gsz = min(g.tiles_m - first_m, GROUP_M);
+	const int tm_idx = first_m + (pid % per_group) % gsz;
+	const int tn_idx = (pid % per_group) / gsz;
+	const int m0 = tm_idx * BM, n0 = tn_idx * BN;
+
+	const int nk_total = g.K / BK;
+	const int nk_per = (nk_total + g.k_splits - 1) / g.k_splits;
+	const int kt_begin = ksplit * nk_per;
+	const int kt_end = min(nk_total, kt_begin + nk_per);
+	if (kt_begin >= kt_end) return;
+
+	const bf16_t* Ap = AT ? g.A + (int64_t)kt_begin * BK * g.lda + m0 : g.A + (int64_t)m0 * g.lda + (int64_t)kt_begin * BK;
+	const bf16_t* Bp = BT ? g.B + (int64_t)kt_begin * BK * g.ldb + n0 : g.B + (int64_t)n0 * g.ldb + (int64_t)kt_begin * BK;
+	const int64_t a_step = AT ? (int64_t)BK * g.lda : BK;
+	const int64_t b_step = BT ? (int64_t)BK * g.ldb : BK;
+
+	TileLoader<BM, AT, NT> la;
+	TileLoader<BN, BT, NT> lb;
+
+	f32x16 acc[TM][TN];
+#pragma unroll
+	for (int i = 0; i < TM; i++)
+#pragma unroll
+		for (int j = 0; j < TN; j++)
+#pragma unroll
+			for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+	la.load(Ap, g.lda, tid);
+	lb.load(Bp, g.ldb, tid);
+	la.store(sA[0], tid);
+	lb.store(sB[0], tid);
+	__syncthreads();
+
+	for (int kt = kt_begin; kt < kt_end; kt++) {
+		const int cur = (kt - kt_begin) & 1;
+		const bool more = (kt + 1) < kt_end;
+		if (more) {
+			Ap += a_step;
+			Bp += b_step;
+			la.load(Ap, g.lda, tid);
+			lb.load(Bp, g.ldb, tid);
+		}
+		const bf16_t* a_s = sA[cur];
+		const bf16_t* b_s = sB[cur];
+#pragma unroll
+		for (int ks = 0; ks < BK / 16; ks++) {
+			bf16x8 af[TM], bfr[TN];
+#pragma unroll
+			for (int i = 0; i < TM; i++) af[i] = read_frag<BM, AT>(a_s, wr * WM + i * 32, ks, lane);
+#pragma unroll
+			for (int j = 0; j < TN; j++) bfr[j] = read_frag<BN, BT>(b_s, wc * WN + j * 32, ks, lane);
+#pragma unroll
+			for (int i = 0; i < TM; i++)
+#pragma unroll
+				for (int j = 0; j < TN; j++)
+					acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+		}
+		if (more) {
+			la.store(sA[cur ^ 1], tid);
+			lb.store(sB[cur ^ 1], tid);
+		}
+		__syncthreads();
+	}
+
+	// Epilogue. Accumulator register r of a 32x32 tile holds row (r/4)*8 + (lane/32)*4 + r%4,
+	// column lane%32: lanes 0..31 cover 32 consecutive columns of one row.
+	const int col_l = lane & 31;
+	const int row_l = (lane >> 5) * 4;
+#pragma unroll
+	for (int i = 0; i < TM; i++) {
+#pragma unroll
+		for (int j = 0; j < TN; j++) {
+			const int col = n0 + wc * WN + j * 32 + col_l;
+#pragma unroll
+			for (int r = 0; r < 16; r++) {
+				const int row = m0 + wr * WM + i * 32 + (r >> 2) * 8 + row_l + (r & 3);
+				const float v = acc[i][j][r];
+				if constexpr (EPI == EPI_BF16) {
+					reinterpret_cast<bf16_t*>(g.C)[(int64_t)row * g.ldc + col] = f2bf(v);
+				} else if constexpr (EPI == EPI_BF16_RESID) {
+					const float res = bf2f(g.R[(int64_t)row * g.ldr + col]);
+					reinterpret_cast<bf16_t*>(g.C)[(int64_t)row * g.ldc + col] = f2bf(v + res);
+				} else if constexpr (EPI == EPI_F32_ACC) {
+					float* c = reinterpret_cast<float*>(g.C) + (int64_t)row * g.ldc + col;
+					if (g.k_splits > 1) {
+						unsafeAtomicAdd(c, v);
+					} else {
+						*c += v;
+					}
+				} else {
+					reinterpret_cast<float*>(g.C)[(int64_t)row * g.ldc + col] = v;
+				}
+			}
+		}
+	}
+}
+
+template <int BM, int BN, int WR, int WC, bool AT, bool BT, int EPI>
+static int launch_cfg(const GemmArgs& g, hipStream_t stream) {
+	constexpr int smem = 2 * (TileShape<BM, AT>::ELEMS + TileShape<BN, BT>::ELEMS) * (int)sizeof(bf16_t);
+	auto kern = gemm_kernel<BM, BN, WR, WC, AT, BT, EPI>;
+	static bool attr_set = false;
+	if (!attr_set) {
+		ELF_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+		                                  hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+		attr_set = true;
+	}
+	GemmArgs a = g;
+	a.tiles_m = g.M / BM;
+	a.tiles_n = g.N / BN;
+	const int grid = a.tiles_m * a.tiles_n * a.k_splits;
+	hipLaunchKernelGGL(kern, dim3(grid), dim3(WR * WC * 64), smem, stream, a);
+	ELF_CHECK_HIP(hipGetLastError());
+	return 0;
+}
+
+template <bool AT, bool BT, int EPI>
+static int launch_layout(GemmArgs& g, int tile_cfg, hipStream_t stream) {
+	const int M = g.M, N = g.N;
+	// Tile choice: the 256x256 tile (8 waves, 128x64 each) has the best MFMA : HBM ratio;
+	// smaller tiles keep all 256 CUs busy when the output is small.
+	int cfg = tile_cfg;
+	if (cfg <= 0) {
+		const int64_t t256 = (M % 256 == 0 && N % 256 == 0) ? (int64_t)(M / 256) * (N / 256) : 0;
+		const int64_t t128 = (M % 128 == 0 && N % 128 == 0) ? (int64_t)(M / 128) * (N / 128) : 0;
+		if (t256 >= 256) cfg = 1;
+		else if (t128 >= 128) cfg = 2;
+		else cfg = 3;
+	}
+	if (EPI == EPI_F32_ACC && g.k_splits <= 0) {
+		// Split K when the weight-gradient tile count cannot fill the chip.
+		int bm = cfg == 1 ? 256 : cfg == 2 ? 128 : 64;
+		int64_t tiles = (int64_t)(M / bm) * (N / bm);
+		int ks = 1;
+		while (tiles * ks < 256 && (g.K / BK) / (ks * 2) >= 8 && ks < 16) ks *= 2;
+		g.k_splits = ks;
+	}
+	if (g.k_splits <= 0 || EPI != EPI_F32_ACC) g.k_splits = 1;
+	switch (cfg) {
+		case 1:
+			ELF_REQUIRE(M % 256 == 0 && N % 256 == 0, "gemm: tile 256 needs M,N multiples of 256 (M=%d N=%d)", M, N);
+			return launch_cfg<256, 256, 2, 4, AT, BT, EPI>(g, stream);
+		case 2:
+			ELF_REQUIRE(M % 128 == 0 && N % 128 == 0, "gemm: tile 128 needs M,N multiples of 128 (M=%d N=%d)", M, N);
+			return launch_cfg<128, 128, 2, 2, AT, BT, EPI>(g, stream);
+		case 3:
+			ELF_REQUIRE(M % 64 == 0 && N % 64 == 0, "gemm: M and N must be multiples of 64 (M=%d N=%d)", M, N);
+			return launch_cfg<64, 64, 2, 2, AT, BT, EPI>(g, stream);
+		case 4:
+			ELF_REQUIRE(M % 256 == 0 && N % 256 == 0, "gemm: tile 256 needs M,N multiples of 256 (M=%d N=%d)", M, N);
+			return launch_cfg<256, 256, 2, 2, AT, BT, EPI>(g, stream);
+		case 5:
+			ELF_REQUIRE(M % 256 == 0 && N % 128 == 0, "gemm: tile 256x128 needs M%%256==0, N%%128==0 (M=%d N=%d)", M, N);
+			return launch_cfg<256, 128, 2, 2, AT, BT, EPI>(g, stream);
+		default:
+			set_error("gemm: unknown tile config %d", cfg);
+			return -1;
+	}
+}
+
+template <bool AT, bool BT>
+static int launch_epi(GemmArgs& g, int epi, int tile_cfg, hipStream_t stream) {
+	switch (epi) {
+		case EPI_BF16: return launch_layout<AT, BT, EPI_BF16>(g, tile_cfg, stream);
+		case EPI_BF16_RESID: return launch_layout<AT, BT, EPI_BF16_RESID>(g, tile_cfg, stream);
+		case EPI_F32_ACC: return launch_layout<AT, BT, EPI_F32_ACC>(g, tile_cfg, stream);
+		case EPI_F32_STORE: return launch_layout<AT, BT, EPI_F32_STORE>(g, tile_cfg, stream);
+		default: set_error("gemm: unknown epilogue %d", epi); return -1;
+	}
+}
+
+int gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda, const void* B, int64_t ldb,
+              void* C, int64_t ldc, int epi, const void* R, int64_t ldr, int tile_cfg, int k_splits,
+              hipStream_t stream) {
+	ELF_REQUIRE(M > 0 && N > 0 && K > 0, "gemm: empty problem M=%d N=%d K=%d", M, N, K);
+	ELF_REQUIRE(K % BK == 0, "gemm: K must be a multiple of %d (K=%d)", BK, K);
+	ELF_REQUIRE(A && B && C, "gemm: null operand");
+	ELF_REQUIRE(lda % 8 == 0 && ldb % 8 == 0, "gemm: leading dimensions must be multiples of 8 elements");
+	ELF_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)B % 16) == 0, "gemm: operands must be 16-byte aligned");
+	ELF_REQUIRE(lda >= (a_t ? M : K) && ldb >= (b_t ? N : K) && ldc >= N, "gemm: leading dimension too small");
+	ELF_REQUIRE(epi != EPI_BF16_RESID || (R != nullptr && ldr >= N), "gemm: residual epilogue needs R");
+	GemmArgs g;
+	g.A = (const bf16_t*)A;
+	g.B = (const bf16_t*)B;
+	g.C = C;
+	g.R = (const bf16_t*)R;
+	g.lda = lda;
+	g.ldb = ldb;
+	g.ldc = ldc;
+	g.ldr = ldr;
+	g.M = M;
+	g.N = N;
+	g.K = K;
+	g.tiles_m = g.tiles_n = 0;
+	g.k_splits = k_splits;
+	if (!a_t && !b_t) return launch_epi<false, false>(g, epi, tile_cfg, stream);
+	if (!a_t && b_t) return launch_epi<false, true>(g, epi, tile_cfg, stream);
+	if (a_t && b_t) return launch_epi<true, true>(g, epi, tile_cfg, stream);
+	set_error("gemm: layout A=T,B=R is not used by any stage contraction");
+	return -1;
+}
+
+}  // namespace elf
