@@ -15,4 +15,49 @@ int elf_gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t 
 	                      (hipStream_t)stream);
 }
 
+#define S_(x) ((hipStream_t)(x))
+int elf_norm_fwd(int kind, const void* x, const void* gamma, const void* beta, void* y, void* stats, int T, int d,
+                 float eps, void* stream) {
+	return elf::norm_fwd(kind, x, gamma, beta, y, stats, T, d, eps, S_(stream));
+}
+int64_t elf_norm_bwd_workspace_floats(int T, int d) { return elf::norm_bwd_workspace_floats(T, d); }
+int elf_norm_bwd(int kind, const void* dy, const void* x, const void* gamma, const void* stats, const void* dres,
+                 void* dx, float* dgamma, float* dbeta, float* workspace, int T, int d, void* stream) {
+	return elf::norm_bwd(kind, dy, x, gamma, stats, dres, dx, dgamma, dbeta, workspace, T, d, S_(stream));
+}
+int elf_gelu_fwd(const void* x, void* y, int64_t n, void* stream) { return elf::gelu_fwd(x, y, n, S_(stream)); }
+int elf_gelu_bwd(const void* dy, const void* x, void* dx, int64_t n, void* stream) {
+	return elf::gelu_bwd(dy, x, dx, n, S_(stream));
+}
+int elf_swiglu_fwd(const void* gu, void* h, int64_t T, int F, void* stream) {
+	return elf::swiglu_fwd(gu, h, T, F, S_(stream));
+}
+int elf_swiglu_bwd(const void* dh, const void* gu, void* dgu, int64_t T, int F, void* stream) {
+	return elf::swiglu_bwd(dh, gu, dgu, T, F, S_(stream));
+}
+int elf_rope_table(void* cs, int S, int D, double theta, void* stream) {
+	return elf::rope_table(cs, S, D, theta, S_(stream));
+}
+int elf_rope_apply(void* buf, const void* cs, int64_t T, int S, int ld, int n_heads, int D, int backward, void* stream) {
+	return elf::rope_apply(buf, cs, T, S, ld, n_heads, D, backward, S_(stream));
+}
+int elf_scale_grads(void* acc_f32, void* out_bf16, int64_t n, float scale, void* stream) {
+	return elf::scale_grads(acc_f32, out_bf16, n, scale, S_(stream));
+}
+int elf_add_bf16(const void* a, const void* b, void* out, int64_t n, void* stream) {
+	return elf::add_bf16(a, b, out, n, S_(stream));
+}
+int elf_attn_fwd(const void* q, const void* k, const void* v, void* o, void* lse, int64_t ldq, int64_t ldk, int64_t ldv,
+                 int64_t ldo, int B, int S, int Hq, int Hkv, int D, int causal, float scale, void* stream) {
+	return elf::attn_fwd(q, k, v, o, lse, ldq, ldk, ldv, ldo, B, S, Hq, Hkv, D, causal, scale, S_(stream));
+}
+int64_t elf_attn_bwd_workspace_bytes(int B, int S, int Hq, int D) { return elf::attn_bwd_workspace_bytes(B, S, Hq, D); }
+int elf_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* dO, const void* lse, void* dq,
+                 void* dk, void* dv, void* workspace, int64_t ldq, int64_t ldk, int64_t ldv, int64_t ldo, int64_t lddo,
+                 int64_t lddq, int64_t lddk, int64_t lddv, int B, int S, int Hq, int Hkv, int D, int causal, float scale,
+                 void* stream) {
+	return elf::attn_bwd(q, k, v, o, dO, lse, dq, dk, dv, workspace, ldq, ldk, ldv, ldo, lddo, lddq, lddk, lddv, B, S, Hq,
+	                     Hkv, D, causal, scale, S_(stream));
+}
+
 }  // extern "C"

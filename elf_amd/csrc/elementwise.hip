@@ -1,0 +1,521 @@
+// Bandwidth-bound kernels of a transformer-block stage on gfx950: RMSNorm / LayerNorm,
+// GELU, SwiGLU, RoPE, gradient scale.  All tensors are bf16 row-major [T, cols]; math is
+// fp32 with one rounding on store.  Every lane moves 16 bytes per access (8 bf16) so that
+// a wavefront reads 1 KiB contiguous; row reductions are wavefront butterflies (one wave
+// per row, the row is held in registers so each input is read from HBM exactly once).
+//
+// These replace the ATen ops the reference stage runs through autograd
+// (benchmarks/models/simple.py:44-52 GELU FFN, :444-445 LayerNorm, :460/:466 residual adds;
+// elf/execution/block.py:518-527 scale_grads).  RMSNorm, RoPE and SwiGLU have no reference
+// module; their definitions are the textbook ones stated next to each kernel.
+#include "common.h"
+#include "kernels.h"
+
+namespace elf {
+
+constexpr int ROWS_PER_BLOCK = 4;  // one wave per row, 4 waves per workgroup
+
+struct Chunk {
+	float v[8];
+};
+
+__device__ __forceinline__ Chunk load8(const bf16_t* p) {
+	bf16x8 r = *reinterpret_cast<const bf16x8*>(p);
+	Chunk c;
+#pragma unroll
+	for (int i = 0; i < 8; i++) c.v[i] = (float)r[i];
+	return c;
+}
+__device__ __forceinline__ void store8(bf16_t* p, const Chunk& c) {
+	bf16x8 r;
+#pragma unroll
+	for (int i = 0; i < 8; i++) r[i] = (bf16_t)c.v[i];
+	*reinterpret_cast<bf16x8*>(p) = r;
+}
+
+// ------------------------------------------------------------------------------------------
+// Norm forward.  RMS:  y = x * rsqrt(mean(x^2) + eps) * gamma
+//                LN :  y = (x - mean) * rsqrt(var + eps) * gamma + beta   (biased variance)
+// stats[row] = {mean (0 for RMS), rstd}.
+// WPR = waves per row: 1 (four rows per workgroup, d <= 2048) or 4 (one row per workgroup).
+template <int WPR>
+__device__ __forceinline__ float row_sum(float v, float* red) {
+	v = wave_sum(v);
+	if constexpr (WPR > 1) {
+		const int wave = threadIdx.x >> 6;
+		__syncthreads();
+		if ((threadIdx.x & 63) == 0) red[wave] = v;
+		__syncthreads();
+		v = red[0] + red[1] + red[2] + red[3];
+	}
+	return v;
+}
+
+template <int NCH, int WPR, bool LN>
+__global__ __launch_bounds__(256) void norm_fwd_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ gamma,
+                                                       const bf16_t* __restrict__ beta, bf16_t* __restrict__ y,
+                                                       float2* __restrict__ stats, int T, int d, float eps) {
+	__shared__ float red[4];
+	const int tr = WPR == 1 ? (threadIdx.x & 63) : threadIdx.x;  // thread index within the row
+	constexpr int TPR = 64 * WPR;
+	const int row = WPR == 1 ? blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6) : blockIdx.x;
+	if (row >= T) return;  // uniform per wave (WPR == 1) or per workgroup (WPR == 4)
+	const int nchunks = d >> 3;
+	const bf16_t* xr = x + (int64_t)row * d;
+	Chunk c[NCH];
+	float s = 0.f, ss = 0.f;
+#pragma unroll
+	for (int i = 0; i < NCH; i++) {
+		const int ch = tr + i * TPR;
+		if (ch < nchunks) {
+			c[i] = load8(xr + ch * 8);
+#pragma unroll
+			for (int j = 0; j < 8; j++) {
+				s += c[i].v[j];
+				ss += c[i].v[j] * c[i].v[j];
+			}
+		}
+	}
+	float mean = 0.f, rstd;
+	if (LN) {
+		mean = row_sum<WPR>(s, red) / d;
+		// second pass over registers for the variance (numerically safer than E[x^2]-mean^2)
+		float var = 0.f;
+#pragma unroll
+		for (int i = 0; i < NCH; i++) {
+			if (tr + i * TPR < nchunks) {
+#pragma unroll
+				for (int j = 0; j < 8; j++) {
+					const float t = c[i].v[j] - mean;
+					var += t * t;
+				}
+			}
+		}
+		rstd = rsqrtf(row_sum<WPR>(var, red) / d + eps);
+	} else {
+		rstd = rsqrtf(row_sum<WPR>(ss, red) / d + eps);
+	}
+	if (tr == 0) stats[row] = make_float2(mean, rstd);
+	bf16_t* yr = y + (int64_t)row * d;
+#pragma unroll
+	for (int i = 0; i < NCH; i++) {
+		const int ch = tr + i * TPR;
+		if (ch < nchunks) {
+			Chunk g = load8(gamma + ch * 8);
+			Chunk o;
+			if (LN) {
+				Chunk b = load8(beta + ch * 8);
+#pragma unroll
+				for (int j = 0; j < 8; j++) o.v[j] = (c[i].v[j] - mean) * rstd * g.v[j] + b.v[j];
+			} else {
+#pragma unroll
+				for (int j = 0; j < 8; j++) o.v[j] = c[i].v[j] * rstd * g.v[j];
+			}
+			store8(yr + ch * 8, o);
+		}
+	}
+}
+
+// Norm backward.  With xhat = (x - mean) * rstd, g = dy * gamma:
+//   RMS: dx = rstd * (g - xhat * mean(g * xhat))
+//   LN : dx = rstd * (g - mean(g) - xhat * mean(g * xhat))
+// dx (+)= dres when a residual gradient bypasses the norm.  Per-workgroup partial sums of
+// dgamma (= sum dy*xhat) and dbeta (= sum dy) go to part[blockIdx][2][d]; a second kernel
+// folds them into the fp32 gradient accumulators.
+template <int NCH, int WPR, bool LN>
+__global__ __launch_bounds__(256) void norm_bwd_kernel(const bf16_t* __restrict__ dy, const bf16_t* __restrict__ x,
+                                                       const bf16_t* __restrict__ gamma,
+                                                       const float2* __restrict__ stats,
+                                                       const bf16_t* __restrict__ dres, bf16_t* __restrict__ dx,
+                                                       float* __restrict__ part, int T, int d) {
+	__shared__ float red[4];
+	__shared__ float fold[WPR == 1 ? ROWS_PER_BLOCK : 1][WPR == 1 ? 64 * 8 : 1];
+	const int lane = threadIdx.x & 63;
+	const int wave = threadIdx.x >> 6;
+	const int tr = WPR == 1 ? lane : threadIdx.x;
+	constexpr int TPR = 64 * WPR;
+	const int nchunks = d >> 3;
+	Chunk g[NCH];
+	float dg[NCH][8], db[NCH][8];
+#pragma unroll
+	for (int i = 0; i < NCH; i++) {
+		const int ch = tr + i * TPR;
+		if (ch < nchunks) g[i] = load8(gamma + ch * 8);
+#pragma unroll
+		for (int j = 0; j < 8; j++) dg[i][j] = db[i][j] = 0.f;
+	}
+	const int row_step = WPR == 1 ? gridDim.x * ROWS_PER_BLOCK : gridDim.x;
+	for (int row = WPR == 1 ? blockIdx.x * ROWS_PER_BLOCK + wave : blockIdx.x; row < T; row += row_step) {
+		const float2 st = stats[row];
+		const float mean = st.x, rstd = st.y;
+		const bf16_t* xr = x + (int64_t)row * d;
+		const bf16_t* dyr = dy + (int64_t)row * d;
+		Chunk xh[NCH], gy[NCH];
+		float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+		for (int i = 0; i < NCH; i++) {
+			const int ch = tr + i * TPR;
+			if (ch < nchunks) {
+				xh[i] = load8(xr + ch * 8);
+				gy[i] = load8(dyr + ch * 8);
+#pragma unroll
+				for (int j = 0; j < 8; j++) {
+					const float xhat = (xh[i].v[j] - mean) * rstd;
+					const float dyv = gy[i].v[j];
+					dg[i][j] += dyv * xhat;
+					if (LN) db[i][j] += dyv;
+					const float gv = dyv * g[i].v[j];
+					xh[i].v[j] = xhat;
+					gy[i].v[j] = gv;
+					s1 += gv;
+					s2 += gv * xhat;
+				}
+			}
+		}
+		const float m2 = row_sum<WPR>(s2, red) / d;
+		const float m1 = LN ? row_sum<WPR>(s1, red) / d : 0.f;
+		bf16_t* dxr = dx + (int64_t)row * d;
+#pragma unroll
+		for (int i = 0; i < NCH; i++) {
+			const int ch = tr + i * TPR;
+			if (ch < nchunks) {
+				Chunk o;
+#pragma unroll
+				for (int j = 0; j < 8; j++) o.v[j] = rstd * (gy[i].v[j] - m1 - xh[i].v[j] * m2);
+				if (dres) {
+					Chunk r = load8(dres + (int64_t)row * d + ch * 8);
+#pragma unroll
+					for (int j = 0; j < 8; j++) o.v[j] += r.v[j];
+				}
+				store8(dxr + ch * 8, o);
+			}
+		}
+	}
+	float* pg = part + (int64_t)blockIdx.x * 2 * d;
+	float* pb = pg + d;
+	if constexpr (WPR > 1) {
+		// every thread owns its columns outright
+#pragma unroll
+		for (int i = 0; i < NCH; i++) {
+			const int ch = tr + i * TPR;
+			if (ch < nchunks) {
+#pragma unroll
+				for (int j = 0; j < 8; j++) {
+					pg[ch * 8 + j] = dg[i][j];
+					if (LN) pb[ch * 8 + j] = db[i][j];
+				}
+			}
+		}
+	} else {
+		// fold the 4 waves (4 different rows, same columns) through LDS, 512 columns at a time
+#pragma unroll
+		for (int i = 0; i < NCH; i++) {
+			for (int which = 0; which < (LN ? 2 : 1); which++) {
+				__syncthreads();
+#pragma unroll
+				for (int j = 0; j < 8; j++) fold[wave][lane * 8 + j] = which ? db[i][j] : dg[i][j];
+				__syncthreads();
+				for (int col = threadIdx.x; col < 512; col += 256) {
+					const int ch = (col >> 3) + i * 64;
+					if (ch < nchunks) {
+						float s = 0.f;
+#pragma unroll
+						for (int w = 0; w < ROWS_PER_BLOCK; w++) s += fold[w][col];
+						(which ? pb : pg)[ch * 8 + (col & 7)] = s;
+					}
+				}
+			}
+		}
+	}
+}
+
+// main_grad[c] += sum_b part[b][which][c]
+__global__ void norm_bwd_finalize_kernel(const float* __restrict__ part, int nparts, int d, float* __restrict__ dgamma,
+                                         float* __restrict__ dbeta) {
+	const int c = blockIdx.x * blockDim.x + threadIdx.x;
+	if (c >= d) return;
+	float sg = 0.f, sb = 0.f;
+	for (int b = 0; b < nparts; b++) {
+		sg += part[(int64_t)b * 2 * d + c];
+		if (dbeta) sb += part[(int64_t)b * 2 * d + d + c];
+	}
+	dgamma[c] += sg;
+	if (dbeta) dbeta[c] += sb;
+}
+
+static inline int norm_bwd_blocks(int T, int d) {
+	const int rows_per_block = d <= 2048 ? ROWS_PER_BLOCK : 1;
+	const int want = (T + rows_per_block - 1) / rows_per_block;
+	return want < 1024 ? want : 1024;
+}
+
+template <bool LN>
+static int norm_fwd_dispatch(const void* x, const void* gamma, const void* beta, void* y, void* stats, int T, int d,
+                             float eps, hipStream_t s) {
+	const dim3 block(256);
+#define ELF_NORM_FWD(N, W)                                                                                          \
+	hipLaunchKernelGGL((norm_fwd_kernel<N, W, LN>), dim3(W == 1 ? (T + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK : T), block, 0, \
+	                   s, (const bf16_t*)x, (const bf16_t*)gamma, (const bf16_t*)beta, (bf16_t*)y, (float2*)stats, T, d, eps)
+	if (d <= 512) ELF_NORM_FWD(1, 1);
+	else if (d <= 1024) ELF_NORM_FWD(2, 1);
+	else if (d <= 2048) ELF_NORM_FWD(4, 1);
+	else if (d <= 4096) ELF_NORM_FWD(2, 4);
+	else ELF_NORM_FWD(4, 4);
+#undef ELF_NORM_FWD
+	ELF_CHECK_HIP(hipGetLastError());
+	return 0;
+}
+
+int norm_fwd(int kind, const void* x, const void* gamma, const void* beta, void* y, void* stats, int T, int d,
+             float eps, hipStream_t s) {
+	ELF_REQUIRE(T > 0 && d > 0 && d % 8 == 0 && d <= 8192, "norm_fwd: d must be a multiple of 8 and <= 8192 (d=%d)", d);
+	ELF_REQUIRE(x && gamma && y && stats, "norm_fwd: null pointer");
+	if (kind == NORM_LAYER) {
+		ELF_REQUIRE(beta != nullptr, "norm_fwd: LayerNorm needs beta");
+		return norm_fwd_dispatch<true>(x, gamma, beta, y, stats, T, d, eps, s);
+	}
+	return norm_fwd_dispatch<false>(x, gamma, beta, y, stats, T, d, eps, s);
+}
+
+int64_t norm_bwd_workspace_floats(int T, int d) { return (int64_t)norm_bwd_blocks(T, d) * 2 * d; }
+
+template <bool LN>
+static int norm_bwd_dispatch(const void* dy, const void* x, const void* gamma, const void* stats, const void* dres,
+                             void* dx, float* part, int T, int d, hipStream_t s) {
+	const dim3 grid(norm_bwd_blocks(T, d)), block(256);
+#define ELF_NORM_BWD(N, W)                                                                                      \
+	hipLaunchKernelGGL((norm_bwd_kernel<N, W, LN>), grid, block, 0, s, (const bf16_t*)dy, (const bf16_t*)x,       \
+	                   (const bf16_t*)gamma, (const float2*)stats, (const bf16_t*)dres, (bf16_t*)dx, part, T, d)
+	if (d <= 512) ELF_NORM_BWD(1, 1);
+	else if (d <= 1024) ELF_NORM_BWD(2, 1);
+	else if (d <= 2048) ELF_NORM_BWD(4, 1);
+	else if (d <= 4096) ELF_NORM_BWD(2, 4);
+	else ELF_NORM_BWD(4, 4);
+#undef ELF_NORM_BWD
+	ELF_CHECK_HIP(hipGetLastError());
+	return 0;
+}
+
+int norm_bwd(int kind, const void* dy, const void* x, const void* gamma, const void* stats, const void* dres,
+             void* dx, float* dgamma, float* dbeta, float* workspace, int T, int d, hipStream_t s) {
+	ELF_REQUIRE(T > 0 && d > 0 && d % 8 == 0 && d <= 8192, "norm_bwd: d must be a multiple of 8 and <= 8192 (d=%d)", d);
+	ELF_REQUIRE(dy && x && gamma && stats && dx && dgamma && workspace, "norm_bwd: null pointer");
+	int rc;
+	if (kind == NORM_LAYER) {
+		ELF_REQUIRE(dbeta != nullptr, "norm_bwd: LayerNorm needs dbeta");
+		rc = norm_bwd_dispatch<true>(dy, x, gamma, stats, dres, dx, workspace, T, d, s);
+	} else {
+		rc = norm_bwd_dispatch<false>(dy, x, gamma, stats, dres, dx, workspace, T, d, s);
+	}
+	if (rc) return rc;
+	hipLaunchKernelGGL(norm_bwd_finalize_kernel, dim3((d + 255) / 256), dim3(256), 0, s, workspace,
+	                   norm_bwd_blocks(T, d), d, dgamma, kind == NORM_LAYER ? dbeta : nullptr);
+	ELF_CHECK_HIP(hipGetLastError());
+	return 0;
+}
+
+// ------------------------------------------------------------------------------------------
+// Activations.  GELU is the exact (erf) form of nn.GELU():  y = 0.5 x (1 + erf(x / sqrt 2)).
+// SwiGLU: h = silu(g) * u with g = gu[:, :F], u = gu[:, F:].
+__device__ __forceinline__ float gelu_f(float x) { return 0.5f * x * (1.f + erff(x * 0.70710678118654752f)); }
+__device__ __forceinline__ float gelu_grad_f(float x) {
+	const float cdf = 0.5f * (1.f + erff(x * 0.70710678118654752f));
+	const float pdf = 0.3989422804014327f * __expf(-0.5f * x * x);
+	return cdf + x * pdf;
+}
+
+__global__ __launch_bounds__(256) void gelu_fwd_kernel(const bf16_t* __restrict__ x, bf16_t* __restrict__ y, int64_t nchunks) {
+	for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < nchunks; i += (int64_t)gridDim.x * blockDim.x) {
+		Chunk c = load8(x + i * 8);
+#pragma unroll
+		for (int j = 0; j < 8; j++) c.v[j] = gelu_f(c.v[j]);
+		store8(y + i * 8, c);
+	}
+}
+__global__ __launch_bounds__(256) void gelu_bwd_kernel(const bf16_t* __restrict__ dy, const bf16_t* __restrict__ x,
+                                                       bf16_t* __restrict__ dx, int64_t nchunks) {
+	for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < nchunks; i += (int64_t)gridDim.x * blockDim.x) {
+		Chunk c = load8(x + i * 8), g = load8(dy + i * 8);
+#pragma unroll
+		for (int j = 0; j < 8; j++) c.v[j] = g.v[j] * gelu_grad_f(c.v[j]);
+		store8(dx + i * 8, c);
+	}
+}
+// gu: [T, 2F]; h: [T, F]
+__global__ __launch_bounds__(256) void swiglu_fwd_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ h, int64_t T, int F) {
+	const int cpr = F >> 3;
+	const int64_t n = T * cpr;
+	for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+		const int64_t row = i / cpr;
+		const int c8 = (int)(i - row * cpr) * 8;
+		Chunk g = load8(gu + row * 2 * F + c8), u = load8(gu + row * 2 * F + F + c8);
+#pragma unroll
+		for (int j = 0; j < 8; j++) {
+			const float sig = 1.f / (1.f + __expf(-g.v[j]));
+			g.v[j] = g.v[j] * sig * u.v[j];
+		}
+		store8(h + row * F + c8, g);
+	}
+}
+// dgu[:, :F] = dh * u * (sig + g sig (1 - sig));  dgu[:, F:] = dh * g * sig
+__global__ __launch_bounds__(256) void swiglu_bwd_kernel(const bf16_t* __restrict__ dh, const bf16_t* __restrict__ gu,
+                                                         bf16_t* __restrict__ dgu, int64_t T, int F) {
+	const int cpr = F >> 3;
+	const int64_t n = T * cpr;
+	for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+		const int64_t row = i / cpr;
+		const int c8 = (int)(i - row * cpr) * 8;
+		Chunk g = load8(gu + row * 2 * F + c8), u = load8(gu + row * 2 * F + F + c8), d = load8(dh + row * F + c8);
+		Chunk dg, du;
+#pragma unroll
+		for (int j = 0; j < 8; j++) {
+			const float sig = 1.f / (1.f + __expf(-g.v[j]));
+			dg.v[j] = d.v[j] * u.v[j] * sig * (1.f + g.v[j] * (1.f - sig));
+			du.v[j] = d.v[j] * g.v[j] * sig;
+		}
+		store8(dgu + row * 2 * F + c8, dg);
+		store8(dgu + row * 2 * F + F + c8, du);
+	}
+}
+
+static inline int ew_grid(int64_t nchunks) {
+	int64_t b = (nchunks + 255) / 256;
+	return (int)(b < 256 * 16 ? (b < 1 ? 1 : b) : 256 * 16);
+}
+
+int gelu_fwd(const void* x, void* y, int64_t n, hipStream_t s) {
+	ELF_REQUIRE(n > 0 && n % 8 == 0 && x && y, "gelu_fwd: n must be a positive multiple of 8");
+	hipLaunchKernelGGL(gelu_fwd_kernel, dim3(ew_grid(n / 8)), dim3(256), 0, s, (const bf16_t*)x, (bf16_t*)y, n / 8);
+	ELF_CHECK_HIP(hipGetLastError());
+	return 0;
+}
+int gelu_bwd(const void* dy, const void* x, void* dx, int64_t n, hipStream_t s) {
+	ELF_REQUIRE(n > 0 && n % 8 == 0 && x && dy && dx, "gelu_bwd: n must be a positive multiple of 8");
+	hipLaunchKernelGGL(gelu_bwd_kernel, dim3(ew_grid(n / 8)), dim3(256), 0, s, (const bf16_t*)dy, (const bf16_t*)x,
+	                   (bf16_t*)dx, n / 8);
+	ELF_CHECK_HIP(hipGetLastError());
+	return 0;
+}
+int swiglu_fwd(const void* gu, void* h, int64_t T, int F, hipStream_t s) {
+	ELF_REQUIRE(T > 0 && F > 0 && F % 8 == 0 && gu && h, "swiglu_fwd: F must be a positive multiple of 8");
+	hipLaunchKernelGGL(swiglu_fwd_kernel, dim3(ew_grid(T * (F / 8))), dim3(256), 0, s, (const bf16_t*)gu, (bf16_t*)h, T, F);
+	ELF_CHECK_HIP(hipGetLastError());
+	return 0;
+}
+int swiglu_bwd(const void* dh, const void* gu, void* dgu, int64_t T, int F, hipStream_t s) {
+	ELF_REQUIRE(T > 0 && F > 0 && F % 8 == 0 && gu && dh && dgu, "swiglu_bwd: F must be a positive multiple of 8");
+	hipLaunchKernelGGL(swiglu_bwd_kernel, dim3(ew_grid(T * (F / 8))), dim3(256), 0, s, (const bf16_t*)dh,
+	                   (const bf16_t*)gu, (bf16_t*)dgu, T, F);
+	ELF_CHECK_HIP(hipGetLastError());
+	return 0;
+}
+
+// ------------------------------------------------------------------------------------------
+// Rotary embedding, half-split ("rotate_half") convention, applied in place to the first
+// n_rot_heads heads of a packed [T, ld] projection buffer (q heads then k heads):
+//   out[i]       = x[i] cos(a_i) - x[i+D/2] sin(a_i)
+//   out[i + D/2] = x[i+D/2] cos(a_i) + x[i] sin(a_i),   a_i = pos * theta^(-2i/D), pos = t mod S.
+// The backward is the same rotation with the sign of sin flipped.  cs is the fp32 table
+// [S, D/2] of (cos, sin) pairs produced by rope_table().
+__global__ void rope_table_kernel(float2* __restrict__ cs, int S, int half, double theta) {
+	const int i = blockIdx.x * blockDim.x + threadIdx.x;
+	if (i >= S * half) return;
+	const int pos = i / half, f = i % half;
+	const double inv = pow(theta, -(double)f / (double)half);
+	const double a = (double)pos * inv;
+	cs[i] = make_float2((float)cos(a), (float)sin(a));
+}
+int rope_table(void* cs, int S, int D, double theta, hipStream_t s) {
+	ELF_REQUIRE(cs && S > 0 && D > 0 && D % 16 == 0, "rope_table: head_dim must be a multiple of 16");
+	const int n = S * (D / 2);
+	hipLaunchKernelGGL(rope_table_kernel, dim3((n + 255) / 256), dim3(256), 0, s, (float2*)cs, S, D / 2, theta);
+	ELF_CHECK_HIP(hipGetLastError());
+	return 0;
+}
+
+__global__ __launch_bounds__(256) void rope_kernel(bf16_t* __restrict__ buf, const float2* __restrict__ cs, int64_t T, int S,
+                                                   int ld, int n_heads, int D, float sign) {
+	const int cph = D >> 4;  // 8-wide chunks per half head
+	const int64_t n = T * n_heads * cph;
+	for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+		const int c = (int)(i % cph);
+		const int64_t th = i / cph;
+		const int h = (int)(th % n_heads);
+		const int64_t t = th / n_heads;
+		const int pos = (int)(t % S);
+		bf16_t* p = buf + t * ld + h * D + c * 8;
+		Chunk a = load8(p), b = load8(p + D / 2);
+		const float2* tab = cs + (int64_t)pos * (D / 2) + c * 8;
+		Chunk oa, ob;
+#pragma unroll
+		for (int j = 0; j < 8; j++) {
+			const float2 t2 = tab[j];
+			const float sn = t2.y * sign;
+			oa.v[j] = a.v[j] * t2.x - b.v[j] * sn;
+			ob.v[j] = b.v[j] * t2.x + a.v[j] * sn;
+		}
+		store8(p, oa);
+		store8(p + D / 2, ob);
+	}
+}
+int rope_apply(void* buf, const void* cs, int64_t T, int S, int ld, int n_heads, int D, int backward, hipStream_t s) {
+	ELF_REQUIRE(buf && cs && T > 0 && S > 0 && T % S == 0, "rope: T must be a multiple of S");
+	ELF_REQUIRE(D % 16 == 0 && ld % 8 == 0 && n_heads * D <= ld, "rope: bad head layout");
+	const int64_t n = T * n_heads * (D / 16);
+	hipLaunchKernelGGL(rope_kernel, dim3(ew_grid(n)), dim3(256), 0, s, (bf16_t*)buf, (const float2*)cs, T, S, ld, n_heads,
+	                   D, backward ? -1.f : 1.f);
+	ELF_CHECK_HIP(hipGetLastError());
+	return 0;
+}
+
+// ------------------------------------------------------------------------------------------
+// Gradient scale: the fp32 accumulator is multiplied by `scale` in place and its bf16
+// rounding is written next to it (the parameter-dtype .grad the reference exposes).
+__global__ __launch_bounds__(256) void scale_grads_kernel(float* __restrict__ acc, bf16_t* __restrict__ out, int64_t n4,
+                                                          int64_t n, float scale) {
+	for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
+		f32x4 v = reinterpret_cast<f32x4*>(acc)[i];
+		v *= scale;
+		reinterpret_cast<f32x4*>(acc)[i] = v;
+		if (out) {
+			bf16x4 o;
+#pragma unroll
+			for (int j = 0; j < 4; j++) o[j] = (bf16_t)v[j];
+			reinterpret_cast<bf16x4*>(out)[i] = o;
+		}
+	}
+	// tail (n not a multiple of 4)
+	if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
+		const int64_t i = n4 * 4 + threadIdx.x;
+		const float v = acc[i] * scale;
+		acc[i] = v;
+		if (out) out[i] = (bf16_t)v;
+	}
+}
+int scale_grads(void* acc_f32, void* out_bf16, int64_t n, float scale, hipStream_t s) {
+	ELF_REQUIRE(acc_f32 && n > 0, "scale_grads: empty");
+	ELF_REQUIRE(((uintptr_t)acc_f32 % 16) == 0 && (!out_bf16 || ((uintptr_t)out_bf16 % 8) == 0), "scale_grads: misaligned");
+	hipLaunchKernelGGL(scale_grads_kernel, dim3(ew_grid(n / 4 + 1)), dim3(256), 0, s, (float*)acc_f32, (bf16_t*)out_bf16,
+	                   n / 4, n, scale);
+	ELF_CHECK_HIP(hipGetLastError());
+	return 0;
+}
+
+// out = a + b (residual add / gradient fan-in, elf/execution/block.py:651-655)
+__global__ __launch_bounds__(256) void add_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ b,
+                                                  bf16_t* __restrict__ o, int64_t nchunks) {
+	for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < nchunks; i += (int64_t)gridDim.x * blockDim.x) {
+		Chunk x = load8(a + i * 8), y = load8(b + i * 8);
+#pragma unroll
+		for (int j = 0; j < 8; j++) x.v[j] += y.v[j];
+		store8(o + i * 8, x);
+	}
+}
+int add_bf16(const void* a, const void* b, void* out, int64_t n, hipStream_t s) {
+	ELF_REQUIRE(n > 0 && n % 8 == 0 && a && b && out, "add: n must be a positive multiple of 8");
+	hipLaunchKernelGGL(add_kernel, dim3(ew_grid(n / 8)), dim3(256), 0, s, (const bf16_t*)a, (const bf16_t*)b, (bf16_t*)out, n / 8);
+	ELF_CHECK_HIP(hipGetLastError());
+	return 0;
+}
+
+}  // namespace elf

@@ -16,4 +16,30 @@ int gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda,
               void* C, int64_t ldc, int epi, const void* R, int64_t ldr, int tile_cfg, int k_splits,
               hipStream_t stream);
 
+enum NormKind { NORM_RMS = 0, NORM_LAYER = 1 };
+
+// stats: float2 per row {mean, rstd}. workspace: norm_bwd_workspace_floats(T, d) floats.
+int norm_fwd(int kind, const void* x, const void* gamma, const void* beta, void* y, void* stats, int T, int d,
+             float eps, hipStream_t s);
+int64_t norm_bwd_workspace_floats(int T, int d);
+int norm_bwd(int kind, const void* dy, const void* x, const void* gamma, const void* stats, const void* dres,
+             void* dx, float* dgamma, float* dbeta, float* workspace, int T, int d, hipStream_t s);
+int gelu_fwd(const void* x, void* y, int64_t n, hipStream_t s);
+int gelu_bwd(const void* dy, const void* x, void* dx, int64_t n, hipStream_t s);
+int swiglu_fwd(const void* gu, void* h, int64_t T, int F, hipStream_t s);
+int swiglu_bwd(const void* dh, const void* gu, void* dgu, int64_t T, int F, hipStream_t s);
+int rope_table(void* cs, int S, int D, double theta, hipStream_t s);
+int rope_apply(void* buf, const void* cs, int64_t T, int S, int ld, int n_heads, int D, int backward, hipStream_t s);
+int scale_grads(void* acc_f32, void* out_bf16, int64_t n, float scale, hipStream_t s);
+int add_bf16(const void* a, const void* b, void* out, int64_t n, hipStream_t s);
+
+// Attention over the packed projection layout; lse is [B, Hq, S] fp32 (natural log).
+int attn_fwd(const void* q, const void* k, const void* v, void* o, void* lse, int64_t ldq, int64_t ldk, int64_t ldv,
+             int64_t ldo, int B, int S, int Hq, int Hkv, int D, int causal, float scale, hipStream_t stream);
+int64_t attn_bwd_workspace_bytes(int B, int S, int Hq, int D);
+int attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* dO, const void* lse, void* dq,
+             void* dk, void* dv, void* workspace, int64_t ldq, int64_t ldk, int64_t ldv, int64_t ldo, int64_t lddo,
+             int64_t lddq, int64_t lddk, int64_t lddv, int B, int S, int Hq, int Hkv, int D, int causal, float scale,
+             hipStream_t stream);
+
 }  // namespace elf

@@ -1,0 +1,145 @@
+"""Thin torch-tensor wrappers over the kernel-level C-ABI entry points.
+
+torch is used for device memory and streams only; every op below is one call into
+libelf_stage.so on ``torch.cuda.current_stream()``.
+"""
+
+import math
+
+import torch
+
+from . import _lib
+
+EPI_BF16, EPI_BF16_RESID, EPI_F32_ACC, EPI_F32_STORE = 0, 1, 2, 3
+NORM_RMS, NORM_LAYER = 0, 1
+
+
+def _stream():
+	return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t):
+	return 0 if t is None else t.data_ptr()
+
+
+def _need(t, dtype, name):
+	if not t.is_cuda:
+		raise _lib.ElfStageError(f"{name}: tensor must live on the GPU (this path has no CPU implementation)")
+	if t.dtype != dtype:
+		raise _lib.ElfStageError(f"{name}: expected {dtype}, got {t.dtype}")
+	if t.dim() >= 2 and t.stride(-1) != 1:
+		raise _lib.ElfStageError(f"{name}: innermost dimension must be contiguous")
+
+
+def gemm(a, b, *, a_t=False, b_t=False, out=None, epilogue=EPI_BF16, residual=None, tile_cfg=0, k_splits=0):
+	"""C[M,N] (+)= sum_k A(m,k) B(n,k).  a: [M,K] (or [K,M] if a_t); b: [N,K] (or [K,N] if b_t)."""
+	_need(a, torch.bfloat16, "gemm.a")
+	_need(b, torch.bfloat16, "gemm.b")
+	K, M = (a.shape[0], a.shape[1]) if a_t else (a.shape[1], a.shape[0])
+	Kb, N = (b.shape[0], b.shape[1]) if b_t else (b.shape[1], b.shape[0])
+	if K != Kb:
+		raise _lib.ElfStageError(f"gemm: reduction sizes differ ({K} vs {Kb})")
+	if out is None:
+		dt = torch.bfloat16 if epilogue in (EPI_BF16, EPI_BF16_RESID) else torch.float32
+		out = (torch.zeros if epilogue == EPI_F32_ACC else torch.empty)((M, N), dtype=dt, device=a.device)
+	lib = _lib.load()
+	rc = lib.elf_gemm_bf16(int(a_t), int(b_t), M, N, K, _ptr(a), a.stride(0), _ptr(b), b.stride(0), _ptr(out), out.stride(0),
+	                       epilogue, _ptr(residual), residual.stride(0) if residual is not None else 0, tile_cfg, k_splits, _stream())
+	_lib.check(rc, "elf_gemm_bf16")
+	return out
+
+
+def norm_fwd(kind, x, gamma, beta=None, eps=1e-5):
+	_need(x, torch.bfloat16, "norm.x")
+	T, d = x.shape
+	y = torch.empty_like(x)
+	stats = torch.empty((T, 2), dtype=torch.float32, device=x.device)
+	rc = _lib.load().elf_norm_fwd(kind, _ptr(x), _ptr(gamma), _ptr(beta), _ptr(y), _ptr(stats), T, d, eps, _stream())
+	_lib.check(rc, "elf_norm_fwd")
+	return y, stats
+
+
+def norm_bwd(kind, dy, x, gamma, stats, dgamma, dbeta=None, dres=None):
+	T, d = x.shape
+	lib = _lib.load()
+	ws = torch.empty(lib.elf_norm_bwd_workspace_floats(T, d), dtype=torch.float32, device=x.device)
+	dx = torch.empty_like(x)
+	rc = lib.elf_norm_bwd(kind, _ptr(dy), _ptr(x), _ptr(gamma), _ptr(stats), _ptr(dres), _ptr(dx), _ptr(dgamma), _ptr(dbeta), _ptr(ws), T, d, _stream())
+	_lib.check(rc, "elf_norm_bwd")
+	return dx
+
+
+def gelu_fwd(x):
+	y = torch.empty_like(x)
+	_lib.check(_lib.load().elf_gelu_fwd(_ptr(x), _ptr(y), x.numel(), _stream()), "elf_gelu_fwd")
+	return y
+
+
+def gelu_bwd(dy, x):
+	dx = torch.empty_like(x)
+	_lib.check(_lib.load().elf_gelu_bwd(_ptr(dy), _ptr(x), _ptr(dx), x.numel(), _stream()), "elf_gelu_bwd")
+	return dx
+
+
+def swiglu_fwd(gu):
+	T, F2 = gu.shape
+	h = torch.empty((T, F2 // 2), dtype=gu.dtype, device=gu.device)
+	_lib.check(_lib.load().elf_swiglu_fwd(_ptr(gu), _ptr(h), T, F2 // 2, _stream()), "elf_swiglu_fwd")
+	return h
+
+
+def swiglu_bwd(dh, gu):
+	T, F2 = gu.shape
+	dgu = torch.empty_like(gu)
+	_lib.check(_lib.load().elf_swiglu_bwd(_ptr(dh), _ptr(gu), _ptr(dgu), T, F2 // 2, _stream()), "elf_swiglu_bwd")
+	return dgu
+
+
+def rope_table(S, D, theta, device="cuda"):
+	cs = torch.empty((S, D // 2, 2), dtype=torch.float32, device=device)
+	_lib.check(_lib.load().elf_rope_table(_ptr(cs), S, D, float(theta), _stream()), "elf_rope_table")
+	return cs
+
+
+def rope_apply_(buf, cs, S, n_heads, D, backward=False):
+	T, ld = buf.shape[0], buf.stride(0)
+	_lib.check(_lib.load().elf_rope_apply(_ptr(buf), _ptr(cs), T, S, ld, n_heads, D, int(backward), _stream()), "elf_rope_apply")
+	return buf
+
+
+def scale_grads_(acc_f32, out_bf16, scale):
+	_lib.check(_lib.load().elf_scale_grads(_ptr(acc_f32), _ptr(out_bf16), acc_f32.numel(), float(scale), _stream()), "elf_scale_grads")
+
+
+def add(a, b):
+	out = torch.empty_like(a)
+	_lib.check(_lib.load().elf_add_bf16(_ptr(a), _ptr(b), _ptr(out), a.numel(), _stream()), "elf_add_bf16")
+	return out
+
+
+def attn_fwd(qkv, B, S, Hq, Hkv, D, causal, scale=None):
+	"""qkv: [B*S, (Hq+2*Hkv)*D] packed projections. Returns (o [B*S, Hq*D], lse [B,Hq,S])."""
+	_need(qkv, torch.bfloat16, "attn.qkv")
+	T, ld = qkv.shape[0], qkv.stride(0)
+	scale = scale if scale is not None else 1.0 / math.sqrt(D)
+	o = torch.empty((T, Hq * D), dtype=torch.bfloat16, device=qkv.device)
+	lse = torch.empty((B, Hq, S), dtype=torch.float32, device=qkv.device)
+	q, k, v = qkv[:, : Hq * D], qkv[:, Hq * D : (Hq + Hkv) * D], qkv[:, (Hq + Hkv) * D :]
+	rc = _lib.load().elf_attn_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), ld, ld, ld, o.stride(0), B, S, Hq, Hkv, D, int(causal), scale, _stream())
+	_lib.check(rc, "elf_attn_fwd")
+	return o, lse
+
+
+def attn_bwd(qkv, o, do, lse, B, S, Hq, Hkv, D, causal, scale=None):
+	"""Returns dqkv packed like qkv."""
+	T, ld = qkv.shape[0], qkv.stride(0)
+	scale = scale if scale is not None else 1.0 / math.sqrt(D)
+	lib = _lib.load()
+	ws = torch.empty(lib.elf_attn_bwd_workspace_bytes(B, S, Hq, D), dtype=torch.uint8, device=qkv.device)
+	dqkv = torch.empty_like(qkv)
+	q, k, v = qkv[:, : Hq * D], qkv[:, Hq * D : (Hq + Hkv) * D], qkv[:, (Hq + Hkv) * D :]
+	dq, dk, dv = dqkv[:, : Hq * D], dqkv[:, Hq * D : (Hq + Hkv) * D], dqkv[:, (Hq + Hkv) * D :]
+	rc = lib.elf_attn_bwd(_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(lse), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ws),
+	                      ld, ld, ld, o.stride(0), do.stride(0), dqkv.stride(0), dqkv.stride(0), dqkv.stride(0), B, S, Hq, Hkv, D, int(causal), scale, _stream())
+	_lib.check(rc, "elf_attn_bwd")
+	return dqkv

@@ -1,0 +1,228 @@
+"""Parity of every HIP kernel (through the C ABI) against a plain PyTorch fp32 evaluation of
+the same op on the same bf16-rounded inputs.  Tolerance: the path's bf16 bar (rel 2e-2 of the
+reference's max magnitude per tensor), plus a much tighter Frobenius-norm bound that catches
+systematic errors (a dropped term, a wrong sign or index)."""
+
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+REL_MAX = 2e-2   # elementwise, relative to max |ref|
+REL_FRO = 6e-3   # Frobenius, bf16 output rounding is ~2^-9 relative
+
+
+def _close(got, ref, rel_max=REL_MAX, rel_fro=REL_FRO, what=""):
+	got = got.float()
+	ref = ref.float()
+	assert got.shape == ref.shape, f"{what}: shape {got.shape} vs {ref.shape}"
+	assert torch.isfinite(got).all(), f"{what}: non-finite output"
+	scale = ref.abs().max().item() + 1e-12
+	err = (got - ref).abs().max().item()
+	fro = ((got - ref).norm() / (ref.norm() + 1e-12)).item()
+	assert err <= rel_max * scale, f"{what}: max err {err:.4g} vs scale {scale:.4g}"
+	assert fro <= rel_fro, f"{what}: relative Frobenius error {fro:.4g}"
+
+
+def _randn(*shape, seed=0, scale=1.0):
+	g = torch.Generator(device="cpu").manual_seed(seed)
+	return (torch.randn(*shape, generator=g) * scale).to(torch.bfloat16).cuda()
+
+
+@pytest.fixture(scope="module")
+def K():
+	from elf_amd import kernels
+
+	return kernels
+
+
+@pytest.mark.parametrize("layout", ["nt", "nn", "tn"])
+@pytest.mark.parametrize("shape", [(256, 256, 64), (512, 768, 256), (1024, 2304, 768), (2048, 1024, 4096)])
+@pytest.mark.parametrize("tile_cfg", [0, 1, 2, 3, 5])
+def test_gemm_layouts(K, layout, shape, tile_cfg):
+	M, N, Kd = shape
+	if tile_cfg in (1, 5) and (M % 256 or N % 256):
+		pytest.skip("tile does not divide")
+	A = _randn(M, Kd, seed=1)
+	B = _randn(N, Kd, seed=2, scale=0.05)
+	ref = A.float() @ B.float().t()
+	if layout == "nt":
+		out = K.gemm(A, B, tile_cfg=tile_cfg)
+	elif layout == "nn":
+		out = K.gemm(A, B.t().contiguous(), b_t=True, tile_cfg=tile_cfg)
+	else:
+		out = K.gemm(A.t().contiguous(), B.t().contiguous(), a_t=True, b_t=True, tile_cfg=tile_cfg)
+	_close(out, ref, what=f"gemm {layout} {shape} cfg{tile_cfg}")
+
+
+def test_gemm_epilogues(K):
+	M, N, Kd = 512, 768, 512
+	A = _randn(M, Kd, seed=3)
+	B = _randn(N, Kd, seed=4, scale=0.05)
+	R = _randn(M, N, seed=5)
+	ref = A.float() @ B.float().t()
+	_close(K.gemm(A, B, epilogue=K.EPI_BF16_RESID, residual=R), ref + R.float(), what="resid")
+	_close(K.gemm(A, B, epilogue=K.EPI_F32_STORE), ref, rel_fro=1e-5, rel_max=1e-5, what="f32 store")
+	# fp32 accumulation across calls (the deferred weight-gradient pattern), with and without split-K
+	for ks in (1, 4):
+		acc = torch.full((M, N), 0.25, dtype=torch.float32, device="cuda")
+		for _ in range(3):
+			K.gemm(A, B, out=acc, epilogue=K.EPI_F32_ACC, k_splits=ks)
+		_close(acc, 3 * ref + 0.25, rel_fro=1e-5, rel_max=1e-5, what=f"f32 acc ks={ks}")
+
+
+def test_gemm_strided_views(K):
+	# operands that are column slices of wider buffers (leading dimension > row length)
+	big = _randn(512, 1024, seed=6)
+	A = big[:, 128:640]                      # [512, 512], ld 1024
+	Bw = _randn(256, 512, seed=7, scale=0.05)
+	out = torch.zeros(512, 512, dtype=torch.bfloat16, device="cuda")
+	K.gemm(A, Bw, out=out[:, 256:])          # writes a column slice
+	_close(out[:, 256:], A.float() @ Bw.float().t(), what="strided")
+	assert out[:, :256].abs().max().item() == 0
+
+
+def test_gemm_rejects_bad_shapes(K):
+	from elf_amd._lib import ElfStageError
+
+	A = _randn(100, 64)
+	B = _randn(64, 64)
+	with pytest.raises(ElfStageError):
+		K.gemm(A, B)
+	with pytest.raises(ElfStageError):
+		K.gemm(_randn(64, 72), _randn(64, 72))  # K not a multiple of 64
+	with pytest.raises(ElfStageError):
+		K.gemm(A.cpu(), B)
+
+
+@pytest.mark.parametrize("d", [256, 768, 1024, 2048, 4096, 8192])
+@pytest.mark.parametrize("kind", ["rms", "ln"])
+def test_norm_fwd_bwd(K, d, kind):
+	T = 515 if d <= 2048 else 130  # ragged row count on purpose
+	x = _randn(T, d, seed=10) * 1.5 + 0.25
+	x = x.to(torch.bfloat16)
+	gamma = (1 + 0.1 * torch.randn(d, generator=torch.Generator().manual_seed(11))).to(torch.bfloat16).cuda()
+	beta = (0.1 * torch.randn(d, generator=torch.Generator().manual_seed(12))).to(torch.bfloat16).cuda()
+	dy = _randn(T, d, seed=13)
+	dres = _randn(T, d, seed=14)
+	eps = 1e-5
+	xr = x.float().requires_grad_(True)
+	gr = gamma.float().requires_grad_(True)
+	br = beta.float().requires_grad_(True)
+	if kind == "rms":
+		yr = xr * torch.rsqrt(xr.pow(2).mean(-1, keepdim=True) + eps) * gr
+	else:
+		yr = torch.nn.functional.layer_norm(xr, (d,), gr, br, eps)
+	yr.backward(dy.float())
+	k = K.NORM_RMS if kind == "rms" else K.NORM_LAYER
+	y, stats = K.norm_fwd(k, x, gamma, beta if kind == "ln" else None, eps)
+	_close(y, yr.detach(), what="norm fwd")
+	dgamma = torch.full((d,), 0.5, dtype=torch.float32, device="cuda")
+	dbeta = torch.full((d,), -0.5, dtype=torch.float32, device="cuda")
+	dx = K.norm_bwd(k, dy, x, gamma, stats, dgamma, dbeta if kind == "ln" else None, dres)
+	_close(dx, xr.grad + dres.float(), what="norm dx")
+	_close(dgamma - 0.5, gr.grad, rel_fro=1e-4, rel_max=1e-3, what="dgamma")
+	if kind == "ln":
+		_close(dbeta + 0.5, br.grad, rel_fro=1e-4, rel_max=1e-3, what="dbeta")
+	dx2 = K.norm_bwd(k, dy, x, gamma, stats, dgamma, dbeta if kind == "ln" else None, None)
+	_close(dx2, xr.grad, what="norm dx no residual")
+
+
+def test_gelu_swiglu(K):
+	x = _randn(300, 1024, seed=20) * 2
+	x = x.to(torch.bfloat16)
+	dy = _randn(300, 1024, seed=21)
+	xr = x.float().requires_grad_(True)
+	yr = torch.nn.functional.gelu(xr)
+	yr.backward(dy.float())
+	_close(K.gelu_fwd(x), yr.detach(), what="gelu")
+	_close(K.gelu_bwd(dy, x), xr.grad, what="gelu bwd")
+	F = 512
+	gu = x  # [300, 2F]
+	dh = _randn(300, F, seed=22)
+	gur = gu.float().requires_grad_(True)
+	hr = torch.nn.functional.silu(gur[:, :F]) * gur[:, F:]
+	hr.backward(dh.float())
+	_close(K.swiglu_fwd(gu), hr.detach(), what="swiglu")
+	_close(K.swiglu_bwd(dh, gu), gur.grad, what="swiglu bwd")
+
+
+def _rope_ref(x, S, D, theta):
+	# x: [T, H, D] fp32; half-split rotation, angles in fp64
+	T = x.shape[0]
+	pos = (torch.arange(T, device=x.device) % S).double()
+	inv = theta ** (-torch.arange(0, D // 2, device=x.device).double() / (D // 2))
+	ang = pos[:, None] * inv[None, :]
+	cos, sin = ang.cos().float()[:, None, :], ang.sin().float()[:, None, :]
+	a, b = x[..., : D // 2], x[..., D // 2 :]
+	return torch.cat([a * cos - b * sin, b * cos + a * sin], dim=-1)
+
+
+def test_rope(K):
+	S, B, Hq, Hkv, D, theta = 256, 2, 4, 2, 128, 5e5
+	T = B * S
+	qkv = _randn(T, (Hq + 2 * Hkv) * D, seed=30)
+	cs = K.rope_table(S, D, theta)
+	ref = qkv.float().clone()
+	nrot = Hq + Hkv
+	ref[:, : nrot * D] = _rope_ref(ref[:, : nrot * D].reshape(T, nrot, D), S, D, theta).reshape(T, -1)
+	out = qkv.clone()
+	K.rope_apply_(out, cs, S, nrot, D)
+	_close(out, ref, what="rope fwd")
+	assert torch.equal(out[:, nrot * D :], qkv[:, nrot * D :]), "v columns must be untouched"
+	# backward = inverse rotation: rotating the forward result back returns the input
+	back = out.clone()
+	K.rope_apply_(back, cs, S, nrot, D, backward=True)
+	_close(back, qkv, what="rope inverse")
+
+
+def test_scale_and_add(K):
+	acc = torch.randn(1000003, device="cuda")
+	ref = acc.clone() * 0.125
+	out = torch.empty(1000003, dtype=torch.bfloat16, device="cuda")
+	K.scale_grads_(acc, out, 0.125)
+	assert torch.equal(acc, ref)
+	assert torch.equal(out, ref.to(torch.bfloat16))
+	a, b = _randn(4096, 64, seed=40), _randn(4096, 64, seed=41)
+	assert torch.equal(K.add(a, b), (a.float() + b.float()).to(torch.bfloat16))
+
+
+def _attn_ref(qkv, B, S, Hq, Hkv, D, causal, do=None):
+	T = B * S
+	x = qkv.float().requires_grad_(True)
+	q = x[:, : Hq * D].reshape(B, S, Hq, D).transpose(1, 2)
+	k = x[:, Hq * D : (Hq + Hkv) * D].reshape(B, S, Hkv, D).transpose(1, 2)
+	v = x[:, (Hq + Hkv) * D :].reshape(B, S, Hkv, D).transpose(1, 2)
+	G = Hq // Hkv
+	k = k.repeat_interleave(G, dim=1)
+	v = v.repeat_interleave(G, dim=1)
+	s = (q @ k.transpose(-1, -2)) / math.sqrt(D)
+	if causal:
+		mask = torch.ones(S, S, dtype=torch.bool, device=x.device).tril()
+		s = s.masked_fill(~mask, float("-inf"))
+	lse = torch.logsumexp(s, dim=-1)
+	o = (torch.softmax(s, dim=-1) @ v).transpose(1, 2).reshape(T, Hq * D)
+	if do is not None:
+		o.backward(do.float())
+		return o.detach(), lse.detach(), x.grad
+	return o.detach(), lse.detach(), None
+
+
+@pytest.mark.parametrize("cfg", [
+	(1, 128, 2, 2, 64, False), (2, 256, 4, 4, 64, False), (2, 256, 4, 2, 128, True),
+	(1, 512, 8, 2, 128, True), (1, 384, 2, 1, 64, True), (2, 128, 4, 4, 128, False),
+])
+def test_attention_fwd_bwd(K, cfg):
+	B, S, Hq, Hkv, D, causal = cfg
+	T = B * S
+	qkv = _randn(T, (Hq + 2 * Hkv) * D, seed=50)
+	do = _randn(T, Hq * D, seed=51)
+	o_ref, lse_ref, dqkv_ref = _attn_ref(qkv, B, S, Hq, Hkv, D, causal, do)
+	o, lse = K.attn_fwd(qkv, B, S, Hq, Hkv, D, causal)
+	_close(o, o_ref, what=f"attn fwd {cfg}")
+	_close(lse, lse_ref, rel_fro=1e-3, rel_max=1e-2, what="lse")
+	dqkv = K.attn_bwd(qkv, o, do, lse, B, S, Hq, Hkv, D, causal)
+	for name, sl in (("dq", slice(0, Hq * D)), ("dk", slice(Hq * D, (Hq + Hkv) * D)), ("dv", slice((Hq + Hkv) * D, None))):
+		_close(dqkv[:, sl], dqkv_ref[:, sl], rel_fro=1.5e-2, what=f"attn {name} {cfg}")
