@@ -1,0 +1,647 @@
+// Stage executor: the per-micro-batch F / B / W / recompute / offload operations of one pipeline
+// stage made of transformer blocks, as a sequence of HIP kernel launches on one stream.
+//
+// What the reference does with nn.Module.__call__ + autograd inside PipelineBlock
+// (elf/execution/block.py:210-391, 624-694) and LinearDX/LinearDW (elf/zb_utils.py:9-256) is done
+// here explicitly:
+//   F  keeps, per block, what B needs (the "activation stash");
+//   B  computes the input gradient and leaves, per linear layer, its input X and its output
+//      gradient dY (the "W stash", the reference's LayerDW.ctx["input"] / ctx["grad_output"]);
+//      norm weight gradients are accumulated here, as autograd does in the reference;
+//   W  accumulates dW += dY^T X in fp32 for the four linear layers of every block and drops the
+//      W stash.
+// Remat and offload variants follow the options of elf/scheduling/scheduling.py:58-86.
+#include <map>
+#include <memory>
+#include <vector>
+
+#include "../../include/elf_stage.h"
+#include "common.h"
+#include "kernels.h"
+#include "pools.h"
+
+namespace elf {
+
+enum BufId {
+	B_X = 0,    // block input (owned by the stage for blocks > 0)
+	B_ST1,      // norm1 statistics
+	B_H1,       // norm1 output = input of the QKV projection
+	B_QKV,      // packed projections (after RoPE for the llama block)
+	B_O,        // attention output = input of the output projection
+	B_LSE,      // attention log-sum-exp
+	B_X2,       // x + attention branch
+	B_ST2,      // norm2 statistics
+	B_H2,       // norm2 output = input of the FFN up projection
+	B_GU,       // FFN pre-activation ([T,2F] gate|up for SwiGLU, [T,F] for GELU)
+	B_A,        // FFN activation = input of the down projection
+	B_DY,       // gradient of the block output = dY of the down projection
+	B_DGU,      // dY of the up projection
+	B_DX2,      // dY of the output projection
+	B_DQKV,     // dY of the QKV projection
+	B_COUNT
+};
+static const unsigned ACT_MASK = (1u << B_X) | (1u << B_ST1) | (1u << B_H1) | (1u << B_QKV) | (1u << B_O) | (1u << B_LSE) |
+                                 (1u << B_X2) | (1u << B_ST2) | (1u << B_H2) | (1u << B_GU) | (1u << B_A);
+static const unsigned WIN_MASK = (1u << B_H1) | (1u << B_O) | (1u << B_H2) | (1u << B_A);
+static const unsigned WGRAD_MASK = (1u << B_DY) | (1u << B_DGU) | (1u << B_DX2) | (1u << B_DQKV);
+
+enum ParamId { P_NORM1_G = 0, P_NORM1_B, P_WQKV, P_WO, P_NORM2_G, P_NORM2_B, P_W1, P_W2, P_COUNT };
+
+struct Buf {
+	void* p = nullptr;
+	size_t bytes = 0;
+	bool owned = false;
+	PinnedPool::Block host;  // valid while offloaded
+	bool offloaded = false;
+};
+
+struct BlockState {
+	Buf b[B_COUNT];
+};
+
+struct MbState {
+	std::vector<BlockState> blk;
+	bool has_acts = false, has_win = false, has_wgrad = false;
+	bool remat_root = false;  // forward kept nothing: B re-runs it
+	bool offloaded = false, prefetched = false;
+	hipEvent_t off_ev = nullptr, pre_ev = nullptr;
+};
+
+struct BlockParams {
+	void* w[P_COUNT] = {};
+	float* g[P_COUNT] = {};
+};
+
+enum FwdMode { SAVE_ALL, SAVE_WIN, SAVE_NONE };
+
+struct Stage {
+	elf_stage_cfg cfg;
+	int T, d, Hq, Hkv, D, F, S, B, nqkv, ffn_in;
+	bool llama;
+	std::vector<BlockParams> params;
+	std::map<int, MbState> mbs;
+	DevicePool pool;
+	std::unique_ptr<PinnedPool> pinned;
+	hipStream_t offload_stream = nullptr, prefetch_stream = nullptr;
+	void* rope_cs = nullptr;
+	float* norm_ws = nullptr;
+	void* attn_ws = nullptr;
+	float* dummy_grad = nullptr;  // sink for norm weight gradients during gradient recompute
+	int64_t d2h_bytes = 0, h2d_bytes = 0;
+
+	size_t buf_bytes(int id) const {
+		switch (id) {
+			case B_X: case B_H1: case B_X2: case B_H2: case B_DY: case B_DX2: return (size_t)T * d * 2;
+			case B_ST1: case B_ST2: return (size_t)T * 2 * 4;
+			case B_QKV: case B_DQKV: return (size_t)T * nqkv * 2;
+			case B_O: return (size_t)T * Hq * D * 2;
+			case B_LSE: return (size_t)B * Hq * S * 4;
+			case B_GU: case B_DGU: return (size_t)T * ffn_in * 2;
+			case B_A: return (size_t)T * F * 2;
+		}
+		return 0;
+	}
+};
+
+#define ELF_TRY(expr)            \
+	do {                         \
+		int _rc = (expr);        \
+		if (_rc) return _rc;     \
+	} while (0)
+
+static int buf_alloc(Stage* s, BlockState& bs, int id) {
+	Buf& b = bs.b[id];
+	if (b.p && b.owned) return 0;
+	b.bytes = s->buf_bytes(id);
+	b.p = s->pool.alloc(b.bytes);
+	if (!b.p) return -3;
+	b.owned = true;
+	return 0;
+}
+static void buf_free(Stage* s, BlockState& bs, int id) {
+	Buf& b = bs.b[id];
+	if (b.p && b.owned) s->pool.free(b.p);  // a pinned copy, if any, stays until release
+	b.p = nullptr;
+	b.owned = false;
+}
+static void free_mask(Stage* s, MbState& m, unsigned mask) {
+	for (auto& bs : m.blk)
+		for (int id = 0; id < B_COUNT; id++)
+			if (mask & (1u << id)) buf_free(s, bs, id);
+}
+
+static MbState& mb_state(Stage* s, int mb) {
+	MbState& m = s->mbs[mb];
+	if (m.blk.empty()) m.blk.resize(s->cfg.n_blocks);
+	return m;
+}
+
+static void destroy_events(MbState& m) {
+	if (m.off_ev) (void)hipEventDestroy(m.off_ev);
+	if (m.pre_ev) (void)hipEventDestroy(m.pre_ev);
+	m.off_ev = m.pre_ev = nullptr;
+}
+
+// ---------------------------------------------------------------------------------------------
+static int run_forward(Stage* s, MbState& m, const void* x, void* y, FwdMode mode, hipStream_t st) {
+	const int nb = s->cfg.n_blocks;
+	const int T = s->T, d = s->d, F = s->F;
+	const int norm_kind = s->llama ? NORM_RMS : NORM_LAYER;
+	const float scale = 1.0f / sqrtf((float)s->D);
+	for (int i = 0; i < nb; i++) {
+		BlockState& bs = m.blk[i];
+		const BlockParams& p = s->params[i];
+		if (i == 0) {
+			bs.b[B_X].p = const_cast<void*>(x);
+			bs.b[B_X].owned = false;
+			bs.b[B_X].bytes = s->buf_bytes(B_X);
+		}
+		const void* xin = bs.b[B_X].p;
+		ELF_TRY(buf_alloc(s, bs, B_ST1));
+		ELF_TRY(buf_alloc(s, bs, B_H1));
+		ELF_TRY(norm_fwd(norm_kind, xin, p.w[P_NORM1_G], p.w[P_NORM1_B], bs.b[B_H1].p, bs.b[B_ST1].p, T, d, s->cfg.eps, st));
+		ELF_TRY(buf_alloc(s, bs, B_QKV));
+		ELF_TRY(gemm_bf16(0, 0, T, s->nqkv, d, bs.b[B_H1].p, d, p.w[P_WQKV], d, bs.b[B_QKV].p, s->nqkv, EPI_BF16, nullptr, 0, 0, 0, st));
+		if (s->llama) ELF_TRY(rope_apply(bs.b[B_QKV].p, s->rope_cs, T, s->S, s->nqkv, s->Hq + s->Hkv, s->D, 0, st));
+		ELF_TRY(buf_alloc(s, bs, B_O));
+		ELF_TRY(buf_alloc(s, bs, B_LSE));
+		{
+			const bf16_t* q = (const bf16_t*)bs.b[B_QKV].p;
+			ELF_TRY(attn_fwd(q, q + s->Hq * s->D, q + (s->Hq + s->Hkv) * s->D, bs.b[B_O].p, bs.b[B_LSE].p, s->nqkv, s->nqkv, s->nqkv,
+			                 s->Hq * s->D, s->B, s->S, s->Hq, s->Hkv, s->D, s->cfg.causal, scale, st));
+		}
+		ELF_TRY(buf_alloc(s, bs, B_X2));
+		ELF_TRY(gemm_bf16(0, 0, T, d, s->Hq * s->D, bs.b[B_O].p, s->Hq * s->D, p.w[P_WO], s->Hq * s->D, bs.b[B_X2].p, d, EPI_BF16_RESID, xin, d, 0, 0, st));
+		ELF_TRY(buf_alloc(s, bs, B_ST2));
+		ELF_TRY(buf_alloc(s, bs, B_H2));
+		ELF_TRY(norm_fwd(norm_kind, bs.b[B_X2].p, p.w[P_NORM2_G], p.w[P_NORM2_B], bs.b[B_H2].p, bs.b[B_ST2].p, T, d, s->cfg.eps, st));
+		ELF_TRY(buf_alloc(s, bs, B_GU));
+		ELF_TRY(gemm_bf16(0, 0, T, s->ffn_in, d, bs.b[B_H2].p, d, p.w[P_W1], d, bs.b[B_GU].p, s->ffn_in, EPI_BF16, nullptr, 0, 0, 0, st));
+		ELF_TRY(buf_alloc(s, bs, B_A));
+		if (s->llama) ELF_TRY(swiglu_fwd(bs.b[B_GU].p, bs.b[B_A].p, T, F, st));
+		else ELF_TRY(gelu_fwd(bs.b[B_GU].p, bs.b[B_A].p, (int64_t)T * F, st));
+		void* yout;
+		if (i == nb - 1) {
+			yout = y;
+		} else {
+			BlockState& nx = m.blk[i + 1];
+			ELF_TRY(buf_alloc(s, nx, B_X));
+			yout = nx.b[B_X].p;
+		}
+		ELF_TRY(gemm_bf16(0, 0, T, d, F, bs.b[B_A].p, F, p.w[P_W2], F, yout, d, EPI_BF16_RESID, bs.b[B_X2].p, d, 0, 0, st));
+		// drop what this mode does not keep (the block input is needed until here)
+		if (mode != SAVE_ALL) {
+			const unsigned keep = mode == SAVE_WIN ? WIN_MASK : 0u;
+			for (int id = 0; id < B_COUNT; id++)
+				if ((ACT_MASK & (1u << id)) && !(keep & (1u << id))) buf_free(s, bs, id);
+		}
+	}
+	m.has_acts = mode == SAVE_ALL;
+	m.has_win = mode != SAVE_NONE;
+	return 0;
+}
+
+// grads_only: recompute of the W stash gradients (RECOMPUTE_BACKWARD_INPUTS): no norm weight
+// gradients, and the chain stops once the first block's QKV output gradient is known
+// (elf/zb_utils.py:584-604, elf/execution/block.py:340-374).
+static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool grads_only, hipStream_t st) {
+	const int nb = s->cfg.n_blocks;
+	const int T = s->T, d = s->d, F = s->F;
+	const int norm_kind = s->llama ? NORM_RMS : NORM_LAYER;
+	const float scale = 1.0f / sqrtf((float)s->D);
+	for (int i = nb - 1; i >= 0; i--) {
+		BlockState& bs = m.blk[i];
+		const BlockParams& p = s->params[i];
+		if (i == nb - 1) {
+			bs.b[B_DY].p = const_cast<void*>(dy);
+			bs.b[B_DY].owned = false;
+			bs.b[B_DY].bytes = s->buf_bytes(B_DY);
+		}
+		const void* dyin = bs.b[B_DY].p;
+		// FFN
+		void* d_a = s->pool.alloc((size_t)T * F * 2);
+		if (!d_a) return -3;
+		ELF_TRY(gemm_bf16(0, 1, T, F, d, dyin, d, p.w[P_W2], F, d_a, F, EPI_BF16, nullptr, 0, 0, 0, st));
+		ELF_TRY(buf_alloc(s, bs, B_DGU));
+		if (s->llama) ELF_TRY(swiglu_bwd(d_a, bs.b[B_GU].p, bs.b[B_DGU].p, T, F, st));
+		else ELF_TRY(gelu_bwd(d_a, bs.b[B_GU].p, bs.b[B_DGU].p, (int64_t)T * F, st));
+		s->pool.free(d_a);
+		void* d_h = s->pool.alloc((size_t)T * d * 2);
+		if (!d_h) return -3;
+		ELF_TRY(gemm_bf16(0, 1, T, d, s->ffn_in, bs.b[B_DGU].p, s->ffn_in, p.w[P_W1], d, d_h, d, EPI_BF16, nullptr, 0, 0, 0, st));
+		ELF_TRY(buf_alloc(s, bs, B_DX2));
+		ELF_TRY(norm_bwd(norm_kind, d_h, bs.b[B_X2].p, p.w[P_NORM2_G], bs.b[B_ST2].p, dyin, bs.b[B_DX2].p,
+		                 grads_only ? s->dummy_grad : p.g[P_NORM2_G], grads_only ? s->dummy_grad + d : p.g[P_NORM2_B], s->norm_ws, T, d, st));
+		// attention
+		void* d_o = s->pool.alloc((size_t)T * s->Hq * s->D * 2);
+		if (!d_o) return -3;
+		ELF_TRY(gemm_bf16(0, 1, T, s->Hq * s->D, d, bs.b[B_DX2].p, d, p.w[P_WO], s->Hq * s->D, d_o, s->Hq * s->D, EPI_BF16, nullptr, 0, 0, 0, st));
+		ELF_TRY(buf_alloc(s, bs, B_DQKV));
+		{
+			const bf16_t* q = (const bf16_t*)bs.b[B_QKV].p;
+			bf16_t* dq = (bf16_t*)bs.b[B_DQKV].p;
+			const int ko = s->Hq * s->D, vo = (s->Hq + s->Hkv) * s->D;
+			ELF_TRY(attn_bwd(q, q + ko, q + vo, bs.b[B_O].p, d_o, bs.b[B_LSE].p, dq, dq + ko, dq + vo, s->attn_ws, s->nqkv, s->nqkv, s->nqkv,
+			                 s->Hq * s->D, s->Hq * s->D, s->nqkv, s->nqkv, s->nqkv, s->B, s->S, s->Hq, s->Hkv, s->D, s->cfg.causal, scale, st));
+		}
+		s->pool.free(d_o);
+		if (s->llama) ELF_TRY(rope_apply(bs.b[B_DQKV].p, s->rope_cs, T, s->S, s->nqkv, s->Hq + s->Hkv, s->D, 1, st));
+		if (!(grads_only && i == 0)) {
+			ELF_TRY(gemm_bf16(0, 1, T, d, s->nqkv, bs.b[B_DQKV].p, s->nqkv, p.w[P_WQKV], d, d_h, d, EPI_BF16, nullptr, 0, 0, 0, st));
+			void* dxout;
+			if (i == 0) {
+				dxout = dx;
+			} else {
+				BlockState& pv = m.blk[i - 1];
+				ELF_TRY(buf_alloc(s, pv, B_DY));
+				dxout = pv.b[B_DY].p;
+			}
+			ELF_TRY(norm_bwd(norm_kind, d_h, bs.b[B_X].p, p.w[P_NORM1_G], bs.b[B_ST1].p, bs.b[B_DX2].p, dxout,
+			                 grads_only ? s->dummy_grad : p.g[P_NORM1_G], grads_only ? s->dummy_grad + d : p.g[P_NORM1_B], s->norm_ws, T, d, st));
+		}
+		s->pool.free(d_h);
+		// B consumed the activation stash; what is left is the W stash
+		for (int id = 0; id < B_COUNT; id++)
+			if ((ACT_MASK & (1u << id)) && !(WIN_MASK & (1u << id))) buf_free(s, bs, id);
+	}
+	m.has_acts = false;
+	m.has_win = true;
+	m.has_wgrad = true;
+	return 0;
+}
+
+static int run_backward_params(Stage* s, MbState& m, hipStream_t st) {
+	const int T = s->T, d = s->d, F = s->F;
+	for (int i = 0; i < s->cfg.n_blocks; i++) {
+		BlockState& bs = m.blk[i];
+		const BlockParams& p = s->params[i];
+		const int hd = s->Hq * s->D;
+		// dW[N_out, K_in] += dY[T, N_out]^T X[T, K_in]
+		ELF_TRY(gemm_bf16(1, 1, d, F, T, bs.b[B_DY].p, d, bs.b[B_A].p, F, p.g[P_W2], F, EPI_F32_ACC, nullptr, 0, 0, 0, st));
+		ELF_TRY(gemm_bf16(1, 1, s->ffn_in, d, T, bs.b[B_DGU].p, s->ffn_in, bs.b[B_H2].p, d, p.g[P_W1], d, EPI_F32_ACC, nullptr, 0, 0, 0, st));
+		ELF_TRY(gemm_bf16(1, 1, d, hd, T, bs.b[B_DX2].p, d, bs.b[B_O].p, hd, p.g[P_WO], hd, EPI_F32_ACC, nullptr, 0, 0, 0, st));
+		ELF_TRY(gemm_bf16(1, 1, s->nqkv, d, T, bs.b[B_DQKV].p, s->nqkv, bs.b[B_H1].p, d, p.g[P_WQKV], d, EPI_F32_ACC, nullptr, 0, 0, 0, st));
+	}
+	free_mask(s, m, WIN_MASK | WGRAD_MASK);
+	m.has_win = m.has_wgrad = false;
+	return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Offload (elf/execution/offload.py:228-268, 330-390): every stage-owned activation buffer of
+// more than 1 MiB goes to the pinned arena on the offload stream; the device copy returns to the
+// pool once that copy has finished.
+static int do_offload(Stage* s, MbState& m, hipStream_t st) {
+	if (!m.has_acts || m.offloaded) return 0;
+	hipEvent_t ready;
+	ELF_CHECK_HIP(hipEventCreateWithFlags(&ready, hipEventDisableTiming));
+	ELF_CHECK_HIP(hipEventRecord(ready, st));
+	ELF_CHECK_HIP(hipStreamWaitEvent(s->offload_stream, ready, 0));
+	ELF_CHECK_HIP(hipEventDestroy(ready));
+	if (!m.off_ev) ELF_CHECK_HIP(hipEventCreateWithFlags(&m.off_ev, hipEventDisableTiming));
+	std::vector<void*> to_free;
+	for (auto& bs : m.blk) {
+		for (int id = 0; id < B_COUNT; id++) {
+			Buf& b = bs.b[id];
+			if (!(ACT_MASK & (1u << id)) || !b.p || !b.owned || b.bytes <= (size_t(1) << 20)) continue;
+			if (!s->pinned->allocate((int64_t)(b.bytes / 2), 2, /*bf16*/ 1, &b.host)) return -3;
+			ELF_CHECK_HIP(hipMemcpyAsync(b.host.ptr, b.p, b.bytes, hipMemcpyDeviceToHost, s->offload_stream));
+			s->d2h_bytes += (int64_t)b.bytes;
+			to_free.push_back(b.p);
+			b.p = nullptr;
+			b.owned = false;
+			b.offloaded = true;
+		}
+	}
+	ELF_CHECK_HIP(hipEventRecord(m.off_ev, s->offload_stream));
+	for (void* p : to_free) s->pool.free_after(p, m.off_ev);
+	m.offloaded = true;
+	m.prefetched = false;
+	return 0;
+}
+
+// Bring offloaded buffers back: on the prefetch stream (async = true, PREFETCH_ACTIVATIONS) or on
+// the compute stream when B finds them still on the host (the reference restores synchronously
+// in that case, offload.py:281-283).
+static int do_restore(Stage* s, MbState& m, bool async, hipStream_t st) {
+	if (!m.offloaded || m.prefetched) return 0;
+	hipStream_t cs = async ? s->prefetch_stream : st;
+	// device buffers are taken from the pool in compute-stream order
+	for (auto& bs : m.blk)
+		for (int id = 0; id < B_COUNT; id++) {
+			Buf& b = bs.b[id];
+			if (!b.offloaded) continue;
+			b.p = s->pool.alloc(b.bytes);
+			if (!b.p) return -3;
+			b.owned = true;
+		}
+	if (async) {
+		hipEvent_t now;
+		ELF_CHECK_HIP(hipEventCreateWithFlags(&now, hipEventDisableTiming));
+		ELF_CHECK_HIP(hipEventRecord(now, st));
+		ELF_CHECK_HIP(hipStreamWaitEvent(cs, now, 0));
+		ELF_CHECK_HIP(hipEventDestroy(now));
+	}
+	ELF_CHECK_HIP(hipStreamWaitEvent(cs, m.off_ev, 0));
+	for (auto& bs : m.blk)
+		for (int id = 0; id < B_COUNT; id++) {
+			Buf& b = bs.b[id];
+			if (!b.offloaded) continue;
+			ELF_CHECK_HIP(hipMemcpyAsync(b.p, b.host.ptr, b.bytes, hipMemcpyHostToDevice, cs));
+			s->h2d_bytes += (int64_t)b.bytes;
+		}
+	if (async) {
+		if (!m.pre_ev) ELF_CHECK_HIP(hipEventCreateWithFlags(&m.pre_ev, hipEventDisableTiming));
+		ELF_CHECK_HIP(hipEventRecord(m.pre_ev, cs));
+	}
+	m.prefetched = true;
+	return 0;
+}
+
+static int do_release(Stage* s, MbState& m) {
+	if (!m.offloaded) return 0;
+	if (m.pre_ev) ELF_CHECK_HIP(hipEventSynchronize(m.pre_ev));
+	else if (m.off_ev && !m.prefetched) ELF_CHECK_HIP(hipEventSynchronize(m.off_ev));
+	for (auto& bs : m.blk)
+		for (int id = 0; id < B_COUNT; id++) {
+			Buf& b = bs.b[id];
+			if (b.offloaded) {
+				s->pinned->free(b.host.ptr);
+				b.offloaded = false;
+			}
+		}
+	m.offloaded = false;
+	m.prefetched = false;
+	return 0;
+}
+
+}  // namespace elf
+
+using namespace elf;
+
+extern "C" {
+
+int elf_stage_create(const elf_stage_cfg* cfg, elf_stage_t** out) {
+	ELF_REQUIRE(cfg && out, "elf_stage_create: null argument");
+	ELF_REQUIRE(cfg->arch == ELF_ARCH_GPT || cfg->arch == ELF_ARCH_LLAMA, "elf_stage_create: unknown arch %d", cfg->arch);
+	ELF_REQUIRE(cfg->n_blocks > 0 && cfg->d_model > 0 && cfg->n_heads > 0 && cfg->n_kv_heads > 0 && cfg->ffn > 0 && cfg->seq > 0 && cfg->mb > 0,
+	            "elf_stage_create: sizes must be positive");
+	ELF_REQUIRE(cfg->n_heads % cfg->n_kv_heads == 0, "elf_stage_create: n_heads must be a multiple of n_kv_heads");
+	ELF_REQUIRE(cfg->head_dim == 64 || cfg->head_dim == 128, "elf_stage_create: head_dim must be 64 or 128");
+	ELF_REQUIRE(cfg->seq % 128 == 0, "elf_stage_create: seq must be a multiple of 128");
+	ELF_REQUIRE(cfg->d_model % 64 == 0 && cfg->ffn % 64 == 0 && cfg->d_model <= 8192, "elf_stage_create: d_model and ffn must be multiples of 64, d_model <= 8192");
+	ELF_REQUIRE(cfg->arch == ELF_ARCH_LLAMA || cfg->n_heads == cfg->n_kv_heads, "elf_stage_create: the GPT block has no grouped-query attention");
+	Stage* s = new Stage();
+	s->cfg = *cfg;
+	s->llama = cfg->arch == ELF_ARCH_LLAMA;
+	s->d = cfg->d_model;
+	s->Hq = cfg->n_heads;
+	s->Hkv = cfg->n_kv_heads;
+	s->D = cfg->head_dim;
+	s->F = cfg->ffn;
+	s->S = cfg->seq;
+	s->B = cfg->mb;
+	s->T = cfg->mb * cfg->seq;
+	s->nqkv = (s->Hq + 2 * s->Hkv) * s->D;
+	s->ffn_in = s->llama ? 2 * s->F : s->F;
+	s->params.resize(cfg->n_blocks);
+	s->pinned.reset(new PinnedPool(false));
+	auto fail = [&](const char* what) {
+		set_error("elf_stage_create: %s failed", what);
+		elf_stage_destroy((elf_stage_t*)s);
+		return -2;
+	};
+	if (hipStreamCreateWithFlags(&s->offload_stream, hipStreamNonBlocking) != hipSuccess) return fail("offload stream");
+	if (hipStreamCreateWithFlags(&s->prefetch_stream, hipStreamNonBlocking) != hipSuccess) return fail("prefetch stream");
+	if (hipMalloc((void**)&s->norm_ws, (size_t)norm_bwd_workspace_floats(s->T, s->d) * 4) != hipSuccess) return fail("norm workspace");
+	if (hipMalloc(&s->attn_ws, (size_t)attn_bwd_workspace_bytes(s->B, s->S, s->Hq, s->D)) != hipSuccess) return fail("attention workspace");
+	if (hipMalloc((void**)&s->dummy_grad, (size_t)2 * s->d * 4) != hipSuccess) return fail("gradient sink");
+	if (hipMemset(s->dummy_grad, 0, (size_t)2 * s->d * 4) != hipSuccess) return fail("gradient sink clear");
+	if (s->llama) {
+		if (hipMalloc(&s->rope_cs, (size_t)s->S * (s->D / 2) * 8) != hipSuccess) return fail("rope table");
+		if (rope_table(s->rope_cs, s->S, s->D, cfg->rope_theta, nullptr) != 0) return fail("rope table fill");
+		if (hipStreamSynchronize(nullptr) != hipSuccess) return fail("rope table sync");
+	}
+	*out = (elf_stage_t*)s;
+	return 0;
+}
+
+void elf_stage_destroy(elf_stage_t* h) {
+	if (!h) return;
+	Stage* s = (Stage*)h;
+	(void)hipDeviceSynchronize();
+	for (auto& kv : s->mbs) {
+		do_release(s, kv.second);
+		free_mask(s, kv.second, ~0u);
+		destroy_events(kv.second);
+	}
+	s->mbs.clear();
+	if (s->offload_stream) (void)hipStreamDestroy(s->offload_stream);
+	if (s->prefetch_stream) (void)hipStreamDestroy(s->prefetch_stream);
+	if (s->norm_ws) (void)hipFree(s->norm_ws);
+	if (s->attn_ws) (void)hipFree(s->attn_ws);
+	if (s->dummy_grad) (void)hipFree(s->dummy_grad);
+	if (s->rope_cs) (void)hipFree(s->rope_cs);
+	delete s;
+}
+
+int elf_stage_bind_param(elf_stage_t* h, int block, int which, void* weight_bf16, void* grad_f32) {
+	Stage* s = (Stage*)h;
+	ELF_REQUIRE(s, "elf_stage_bind_param: null stage");
+	ELF_REQUIRE(block >= 0 && block < s->cfg.n_blocks, "elf_stage_bind_param: block %d out of range", block);
+	ELF_REQUIRE(which >= 0 && which < P_COUNT, "elf_stage_bind_param: parameter id %d out of range", which);
+	ELF_REQUIRE(weight_bf16 && grad_f32, "elf_stage_bind_param: null pointer");
+	ELF_REQUIRE(((uintptr_t)weight_bf16 % 16) == 0 && ((uintptr_t)grad_f32 % 16) == 0, "elf_stage_bind_param: pointers must be 16-byte aligned");
+	s->params[block].w[which] = weight_bf16;
+	s->params[block].g[which] = (float*)grad_f32;
+	return 0;
+}
+
+static int check_bound(Stage* s) {
+	for (int i = 0; i < s->cfg.n_blocks; i++)
+		for (int w = 0; w < P_COUNT; w++) {
+			if (s->llama && (w == P_NORM1_B || w == P_NORM2_B)) continue;
+			ELF_REQUIRE(s->params[i].w[w] != nullptr, "stage: parameter %d of block %d is not bound", w, i);
+		}
+	return 0;
+}
+
+int elf_stage_forward(elf_stage_t* h, int mb, const void* x, void* y, uint32_t flags, void* stream) {
+	Stage* s = (Stage*)h;
+	ELF_REQUIRE(s && x && y && mb >= 0, "elf_stage_forward: bad argument");
+	ELF_TRY(check_bound(s));
+	MbState& m = mb_state(s, mb);
+	ELF_REQUIRE(!m.has_acts && !m.has_win && !m.has_wgrad && !m.remat_root, "elf_stage_forward: micro-batch %d is already in flight", mb);
+	const bool root = flags & ELF_FWD_REMAT_ROOT;
+	ELF_TRY(run_forward(s, m, x, y, root ? SAVE_NONE : SAVE_ALL, (hipStream_t)stream));
+	m.remat_root = root;
+	if (root) m.has_win = false;
+	if ((flags & ELF_FWD_OFFLOAD) && !root) ELF_TRY(do_offload(s, m, (hipStream_t)stream));
+	return 0;
+}
+
+int elf_stage_backward_inputs(elf_stage_t* h, int mb, const void* x, const void* dy, void* dx, uint32_t flags, void* stream) {
+	Stage* s = (Stage*)h;
+	ELF_REQUIRE(s && dy && dx && mb >= 0, "elf_stage_backward_inputs: bad argument");
+	auto it = s->mbs.find(mb);
+	ELF_REQUIRE(it != s->mbs.end(), "elf_stage_backward_inputs: no forward was run for micro-batch %d", mb);
+	MbState& m = it->second;
+	hipStream_t st = (hipStream_t)stream;
+	if (m.remat_root) {
+		// the forward kept only the stage input: re-run it, this time keeping the stash
+		ELF_REQUIRE(x != nullptr, "elf_stage_backward_inputs: micro-batch %d was checkpointed, the stage input is needed", mb);
+		void* ytmp = s->pool.alloc((size_t)s->T * s->d * 2);
+		if (!ytmp) return -3;
+		int rc = run_forward(s, m, x, ytmp, SAVE_ALL, st);
+		s->pool.free(ytmp);
+		if (rc) return rc;
+		m.remat_root = false;
+	}
+	ELF_REQUIRE(m.has_acts, "elf_stage_backward_inputs: micro-batch %d has no saved activations", mb);
+	if (m.offloaded) {
+		if (m.prefetched && m.pre_ev) ELF_CHECK_HIP(hipStreamWaitEvent(st, m.pre_ev, 0));
+		else ELF_TRY(do_restore(s, m, false, st));
+	}
+	if (x) m.blk[0].b[B_X].p = const_cast<void*>(x);
+	ELF_TRY(run_backward(s, m, dy, dx, false, st));
+	if (flags & ELF_BWD_RECOMPUTE_GRADIENTS) free_mask(s, m, WGRAD_MASK), m.has_wgrad = false;
+	if (flags & ELF_BWD_RECOMPUTE_ACTIVATIONS) free_mask(s, m, WIN_MASK), m.has_win = false;
+	return 0;
+}
+
+int elf_stage_backward_params(elf_stage_t* h, int mb, void* stream) {
+	Stage* s = (Stage*)h;
+	ELF_REQUIRE(s && mb >= 0, "elf_stage_backward_params: bad argument");
+	auto it = s->mbs.find(mb);
+	ELF_REQUIRE(it != s->mbs.end() && it->second.has_win && it->second.has_wgrad,
+	            "elf_stage_backward_params: micro-batch %d has no saved inputs / output gradients (run B, or the recompute ops, first)", mb);
+	for (int i = 0; i < s->cfg.n_blocks; i++)
+		for (int w : {P_WQKV, P_WO, P_W1, P_W2}) ELF_REQUIRE(s->params[i].g[w] != nullptr, "elf_stage_backward_params: gradient buffer not bound");
+	ELF_TRY(run_backward_params(s, it->second, (hipStream_t)stream));
+	return 0;
+}
+
+int elf_stage_recompute_forward(elf_stage_t* h, int mb, const void* x, int save, void* stream) {
+	Stage* s = (Stage*)h;
+	ELF_REQUIRE(s && x && mb >= 0, "elf_stage_recompute_forward: bad argument");
+	auto it = s->mbs.find(mb);
+	ELF_REQUIRE(it != s->mbs.end(), "elf_stage_recompute_forward: unknown micro-batch %d", mb);
+	MbState& m = it->second;
+	ELF_REQUIRE(!m.has_acts && !m.has_win, "elf_stage_recompute_forward: micro-batch %d still holds its activations", mb);
+	hipStream_t st = (hipStream_t)stream;
+	void* ytmp = s->pool.alloc((size_t)s->T * s->d * 2);
+	if (!ytmp) return -3;
+	int rc = run_forward(s, m, x, ytmp, save ? SAVE_ALL : SAVE_WIN, st);
+	s->pool.free(ytmp);
+	return rc;
+}
+
+int elf_stage_recompute_backward_inputs(elf_stage_t* h, int mb, const void* dy, void* stream) {
+	Stage* s = (Stage*)h;
+	ELF_REQUIRE(s && dy && mb >= 0, "elf_stage_recompute_backward_inputs: bad argument");
+	auto it = s->mbs.find(mb);
+	ELF_REQUIRE(it != s->mbs.end() && it->second.has_acts,
+	            "elf_stage_recompute_backward_inputs: micro-batch %d has no saved graph (run recompute_forward with save first)", mb);
+	return run_backward(s, it->second, dy, nullptr, true, (hipStream_t)stream);
+}
+
+int elf_stage_offload(elf_stage_t* h, int mb, void* stream) {
+	Stage* s = (Stage*)h;
+	ELF_REQUIRE(s, "elf_stage_offload: null stage");
+	auto it = s->mbs.find(mb);
+	ELF_REQUIRE(it != s->mbs.end(), "elf_stage_offload: unknown micro-batch %d", mb);
+	return do_offload(s, it->second, (hipStream_t)stream);
+}
+
+int elf_stage_prefetch(elf_stage_t* h, int mb, void* stream) {
+	Stage* s = (Stage*)h;
+	ELF_REQUIRE(s, "elf_stage_prefetch: null stage");
+	auto it = s->mbs.find(mb);
+	if (it == s->mbs.end()) return 0;  // nothing offloaded (the offloader of the reference is empty then)
+	return do_restore(s, it->second, true, (hipStream_t)stream);
+}
+
+int elf_stage_release(elf_stage_t* h, int mb) {
+	Stage* s = (Stage*)h;
+	ELF_REQUIRE(s, "elf_stage_release: null stage");
+	auto it = s->mbs.find(mb);
+	if (it == s->mbs.end()) return 0;
+	return do_release(s, it->second);
+}
+
+int elf_stage_clear(elf_stage_t* h) {
+	Stage* s = (Stage*)h;
+	ELF_REQUIRE(s, "elf_stage_clear: null stage");
+	ELF_CHECK_HIP(hipDeviceSynchronize());
+	for (auto& kv : s->mbs) {
+		ELF_TRY(do_release(s, kv.second));
+		free_mask(s, kv.second, ~0u);
+		destroy_events(kv.second);
+	}
+	s->mbs.clear();
+	return 0;
+}
+
+int elf_stage_mem_stats(elf_stage_t* h, elf_mem_stats* out) {
+	Stage* s = (Stage*)h;
+	ELF_REQUIRE(s && out, "elf_stage_mem_stats: null argument");
+	out->live_bytes = (int64_t)s->pool.live_bytes();
+	out->peak_bytes = (int64_t)s->pool.peak_bytes();
+	out->reserved_bytes = (int64_t)s->pool.reserved_bytes();
+	out->pinned_bytes = s->pinned->size_bytes();
+	out->d2h_bytes = s->d2h_bytes;
+	out->h2d_bytes = s->h2d_bytes;
+	return 0;
+}
+
+int elf_stage_reset_peak(elf_stage_t* h) {
+	Stage* s = (Stage*)h;
+	ELF_REQUIRE(s, "elf_stage_reset_peak: null stage");
+	s->pool.reset_peak();
+	return 0;
+}
+
+// Pinned arena exposed on its own so that its placement policy can be checked against the
+// reference's rules without a GPU (host_backing = 1 uses malloc).
+int elf_pinned_pool_create(int host_backing, elf_pinned_pool_t** out) {
+	ELF_REQUIRE(out, "elf_pinned_pool_create: null argument");
+	*out = (elf_pinned_pool_t*)new PinnedPool(host_backing != 0);
+	return 0;
+}
+void elf_pinned_pool_destroy(elf_pinned_pool_t* p) { delete (PinnedPool*)p; }
+int elf_pinned_pool_allocate(elf_pinned_pool_t* p, int64_t elems, int elem_size, int dtype_key, void** ptr, int* parent, int64_t* offset) {
+	ELF_REQUIRE(p && ptr, "elf_pinned_pool_allocate: null argument");
+	ELF_REQUIRE(elem_size > 0, "elf_pinned_pool_allocate: element size must be positive");
+	PinnedPool::Block b;
+	if (!((PinnedPool*)p)->allocate(elems, elem_size, dtype_key, &b)) return -3;
+	*ptr = b.ptr;
+	if (parent) *parent = b.parent;
+	if (offset) *offset = b.offset;
+	return 0;
+}
+int elf_pinned_pool_free(elf_pinned_pool_t* p, void* ptr) {
+	ELF_REQUIRE(p, "elf_pinned_pool_free: null pool");
+	return ((PinnedPool*)p)->free(ptr) ? 0 : 1;  // 1: not a block of this pool (ignored, as in the reference)
+}
+int elf_pinned_pool_reserve(elf_pinned_pool_t* p, int64_t bytes, int elem_size, int dtype_key) {
+	ELF_REQUIRE(p && elem_size > 0 && bytes > 0, "elf_pinned_pool_reserve: bad argument");
+	return ((PinnedPool*)p)->reserve(bytes, elem_size, dtype_key) ? 0 : -3;
+}
+int64_t elf_pinned_pool_size(elf_pinned_pool_t* p) { return p ? ((PinnedPool*)p)->size_bytes() : 0; }
+int elf_pinned_pool_n_parents(elf_pinned_pool_t* p) { return p ? ((PinnedPool*)p)->n_parents() : 0; }
+int elf_pinned_pool_n_free(elf_pinned_pool_t* p, int parent) {
+	PinnedPool* pp = (PinnedPool*)p;
+	if (!pp || parent < 0 || parent >= pp->n_parents()) return -1;
+	return pp->n_free_segments(parent);
+}
+int elf_pinned_pool_free_segment(elf_pinned_pool_t* p, int parent, int i, int64_t* offset, int64_t* length) {
+	PinnedPool* pp = (PinnedPool*)p;
+	ELF_REQUIRE(pp && parent >= 0 && parent < pp->n_parents() && i >= 0 && i < pp->n_free_segments(parent) && offset && length,
+	            "elf_pinned_pool_free_segment: index out of range");
+	auto seg = pp->free_segment(parent, i);
+	*offset = seg.first;
+	*length = seg.second;
+	return 0;
+}
+
+}  // extern "C"

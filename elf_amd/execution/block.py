@@ -1,0 +1,416 @@
+"""Stage executors with the slot semantics of the reference's PipelineBlock.
+
+``Variable`` restates elf/execution/block.py:18-131 (three per-micro-batch slot lists with
+set-once / pop-once rules).  ``HipStageBlock`` is the PipelineBlock duck type (block.py:134-694)
+for a stage made of transformer blocks on an MI355X: every compute op is one call into
+libelf_stage.so; torch only owns the boundary tensors, the weights and the gradient buffers.
+There is no other execution path in this class: without the library, or for a module it does not
+recognise, construction raises.
+"""
+
+import ctypes
+import logging
+
+import torch
+
+from .. import _lib
+from ..models import LlamaBlock, TransformerBlock
+from ..scheduling import OpOptions
+from ..utils import Timer
+
+logger = logging.getLogger("block")
+
+__all__ = ["Variable", "HipStageBlock", "StageConfig", "MemStats"]
+
+
+class Variable:
+	"""One input or output of a block: data received and waiting (``to_process``: (work, tensor)),
+	data kept for the backward (``saved``) and data ready to leave (``to_send``), per micro-batch.
+	A slot can be set once and is emptied when read."""
+
+	def __init__(self, name, peer, group=None):
+		self.name, self.peer, self.group = name, peer, group
+		self.metadata = None
+		self.was_metadata_sent = False
+		self.to_process, self.saved, self.to_send = [], [], []
+
+	def get(self, queue, mb_id, delete=True):
+		if len(queue) <= mb_id:
+			raise Exception(f"Variable {self.name} - Data queue shorter than mb_id {mb_id}")
+		data = queue[mb_id]
+		if data is None:
+			raise Exception(f"Variable {self.name} - Trying to pop data at mb_id {mb_id}, but it's empty")
+		if delete:
+			queue[mb_id] = None
+		return data
+
+	def set(self, queue, mb_id, value):
+		if len(queue) <= mb_id:
+			queue.extend([None] * (mb_id + 1 - len(queue)))
+		if queue[mb_id] is not None:
+			raise Exception(f"Variable {self.name} - Trying to set data at mb_id {mb_id}, but it's already set")
+		queue[mb_id] = value
+
+	def wait_and_pop(self, mb_id):
+		work, tensor = self.get(self.to_process, mb_id)
+		if work is not None:
+			work.wait()
+		return tensor.detach()
+
+	def clear(self):
+		self.to_process.clear()
+		self.saved.clear()
+		self.to_send.clear()
+
+	def _state(self):
+		n = [sum(x is not None for x in q) for q in (self.to_process, self.saved, self.to_send)]
+		return f"{self} - to process: {n[0]}, saved: {n[1]}, to send: {n[2]}"
+
+	def __str__(self):
+		return f"Variable(name={self.name},peer={self.peer},metadata={self.metadata})"
+
+	__repr__ = __str__
+
+
+class StageConfig(ctypes.Structure):
+	"""elf_stage_cfg of include/elf_stage.h."""
+
+	_fields_ = [
+		("arch", ctypes.c_int), ("n_blocks", ctypes.c_int), ("d_model", ctypes.c_int), ("n_heads", ctypes.c_int),
+		("n_kv_heads", ctypes.c_int), ("head_dim", ctypes.c_int), ("ffn", ctypes.c_int), ("seq", ctypes.c_int),
+		("mb", ctypes.c_int), ("causal", ctypes.c_int), ("eps", ctypes.c_float), ("rope_theta", ctypes.c_double),
+	]
+
+
+class MemStats(ctypes.Structure):
+	"""elf_mem_stats of include/elf_stage.h."""
+
+	_fields_ = [(n, ctypes.c_int64) for n in ("live_bytes", "peak_bytes", "reserved_bytes", "pinned_bytes", "d2h_bytes", "h2d_bytes")]
+
+
+_P = ctypes.c_void_p
+_I = ctypes.c_int
+for _name, _ret, _args in [
+	("elf_stage_create", _I, [ctypes.POINTER(StageConfig), ctypes.POINTER(_P)]),
+	("elf_stage_destroy", None, [_P]),
+	("elf_stage_bind_param", _I, [_P, _I, _I, _P, _P]),
+	("elf_stage_forward", _I, [_P, _I, _P, _P, ctypes.c_uint32, _P]),
+	("elf_stage_backward_inputs", _I, [_P, _I, _P, _P, _P, ctypes.c_uint32, _P]),
+	("elf_stage_backward_params", _I, [_P, _I, _P]),
+	("elf_stage_recompute_forward", _I, [_P, _I, _P, _I, _P]),
+	("elf_stage_recompute_backward_inputs", _I, [_P, _I, _P, _P]),
+	("elf_stage_offload", _I, [_P, _I, _P]),
+	("elf_stage_prefetch", _I, [_P, _I, _P]),
+	("elf_stage_release", _I, [_P, _I]),
+	("elf_stage_clear", _I, [_P]),
+	("elf_stage_mem_stats", _I, [_P, ctypes.POINTER(MemStats)]),
+	("elf_stage_reset_peak", _I, [_P]),
+]:
+	_lib.register(_name, _ret, _args)
+
+ARCH_GPT, ARCH_LLAMA = 0, 1
+FWD_REMAT_ROOT, FWD_OFFLOAD = 1, 4
+BWD_RECOMPUTE_ACTIVATIONS, BWD_RECOMPUTE_GRADIENTS = 1, 2
+# parameter ids of elf_stage_bind_param
+P_NORM1_G, P_NORM1_B, P_WQKV, P_WO, P_NORM2_G, P_NORM2_B, P_W1, P_W2 = range(8)
+
+
+def _stream():
+	return torch.cuda.current_stream().cuda_stream
+
+
+class HipStageBlock:
+	"""One pipeline stage (a chain of TransformerBlock or LlamaBlock modules) executed by
+	libelf_stage.so.
+
+	The module's linear weights are re-homed into fused bf16 buffers (q|k|v rows, gate|up rows) of
+	which the original ``nn.Parameter``s become views, so optimizers keep working on the module.
+	Weight gradients accumulate in fp32 (``param.main_grad`` views of fused fp32 buffers) across
+	the W passes of a step; ``scale_grads`` divides by the batch size and writes the bf16
+	``param.grad`` the reference exposes.
+	"""
+
+	def __init__(self, model, id_, placement, signature, pp_group=None, dp_group=None, recv_pgs=None, send_pgs=None, *, mb_size, seq_len=None):
+		if not torch.cuda.is_available():
+			raise _lib.ElfStageError("HipStageBlock needs an MI355X: there is no CPU path for the stage kernels")
+		self.lib = _lib.load()
+		self.id = id_
+		self.placement = placement
+		self.rank = placement[id_]
+		self.is_first = id_ == 0
+		self.is_last = id_ == len(placement) - 1
+		self.signature = signature
+		self.pp_group, self.dp_group = pp_group, dp_group
+		self.recv_pgs, self.send_pgs = recv_pgs, send_pgs
+		self.model = model.cuda()
+		self.device = torch.cuda.current_device()
+		self.input_variables = [Variable(n, s, pp_group) for n, s in zip(signature.inputs, signature.sources)]
+		self.output_variables = [[Variable(n, d, pp_group) for d in dsts] for n, dsts in zip(signature.outputs, signature.targets)]
+		assert len(self.input_variables) == 1 and len(self.output_variables) == 1, "a transformer-block stage has one input and one output"
+		self.compute_time = []
+		self.send_ops = []
+		self._handle = None
+		self._kept = {}  # mb -> external tensors the library still points at (x until B/recompute, dy until W)
+		self._build(mb_size, seq_len)
+
+	# ------------------------------------------------------------------ set-up
+	def _build(self, mb_size, seq_len):
+		blocks = list(self.model.children()) if not isinstance(self.model, (TransformerBlock, LlamaBlock)) else [self.model]
+		if not blocks or not all(isinstance(b, (TransformerBlock, LlamaBlock)) for b in blocks) or len({type(b) for b in blocks}) != 1:
+			raise _lib.ElfStageError("HipStageBlock: the stage must be a chain of TransformerBlock or of LlamaBlock modules")
+		b0 = blocks[0]
+		llama = isinstance(b0, LlamaBlock)
+		seq = seq_len or getattr(self.model, "seq_len", None)
+		if seq is None:
+			raise _lib.ElfStageError("HipStageBlock: seq_len is required (StageModule carries it)")
+		att = b0.attn
+		cfg = StageConfig(
+			ARCH_LLAMA if llama else ARCH_GPT, len(blocks), b0.dim, att.num_heads, att.num_kv_heads, att.head_dim, b0.ffn_dim,
+			seq, mb_size, int(b0.causal), float(b0.eps), float(b0.rope_theta) if llama else 0.0,
+		)
+		self.cfg = cfg
+		self.blocks = blocks
+		dev = torch.device("cuda", self.device)
+		self._fused_w, self._fused_g, self._fused_bf16_grad = [], [], []  # the fused buffers (kept alive here)
+		self._param_loc = {}  # parameter -> (fused buffer index, first row, rows)
+		self.main_grads = {}  # parameter -> fp32 accumulator view
+		handle = ctypes.c_void_p()
+		_lib.check(self.lib.elf_stage_create(ctypes.byref(cfg), ctypes.byref(handle)), "elf_stage_create")
+		self._handle = handle
+
+		def fuse(params):
+			"""Move `params` (row blocks of one matrix) into one bf16 buffer + one fp32 grad buffer."""
+			rows = sum(p.shape[0] for p in params)
+			w = torch.empty((rows,) + tuple(params[0].shape[1:]), dtype=torch.bfloat16, device=dev)
+			g = torch.zeros(w.shape, dtype=torch.float32, device=dev)
+			r = 0
+			for p in params:
+				n = p.shape[0]
+				w[r : r + n].copy_(p.data)
+				p.data = w[r : r + n]
+				p.main_grad = g[r : r + n]
+				self.main_grads[p] = p.main_grad
+				self._param_loc[p] = (len(self._fused_w), r, n)
+				r += n
+			self._fused_w.append(w)
+			self._fused_g.append(g)
+			self._fused_bf16_grad.append(None)
+			return w, g
+
+		for i, b in enumerate(blocks):
+			m = b.mlp
+			groups = {
+				P_NORM1_G: [b.norm1.weight], P_NORM2_G: [b.norm2.weight],
+				P_WQKV: [att_i.weight for att_i in (b.attn.q_proj, b.attn.k_proj, b.attn.v_proj)], P_WO: [b.proj.weight],
+				P_W1: [m.gate_proj.weight, m.up_proj.weight] if llama else [m.fc1.weight],
+				P_W2: [m.down_proj.weight if llama else m.fc2.weight],
+			}
+			if not llama:
+				groups[P_NORM1_B] = [b.norm1.bias]
+				groups[P_NORM2_B] = [b.norm2.bias]
+			for pid, params in groups.items():
+				if any(p.dtype != torch.bfloat16 for p in params):
+					raise _lib.ElfStageError("HipStageBlock: parameters must be bf16")
+				w, g = fuse(params)
+				_lib.check(self.lib.elf_stage_bind_param(self._handle, i, pid, w.data_ptr(), g.data_ptr()), "elf_stage_bind_param")
+		self.T = mb_size * seq
+		self.d = b0.dim
+
+	def __del__(self):
+		try:
+			if self._handle:
+				self.lib.elf_stage_destroy(self._handle)
+				self._handle = None
+		except Exception:
+			pass
+
+	def __str__(self):
+		return f"Rank {self.rank} - Layer {self.id}"
+
+	def _check_io(self, t, what):
+		if t.dtype != torch.bfloat16 or not t.is_cuda or t.numel() != self.T * self.d:
+			raise _lib.ElfStageError(f"{self}: {what} must be a bf16 GPU tensor of {self.T}x{self.d} elements, got {tuple(t.shape)} {t.dtype} {t.device}")
+		return t.contiguous()
+
+	def _timed(self, name):
+		t = Timer(name=name)
+		self.compute_time.append(t)
+		return t
+
+	# ------------------------------------------------------------------ compute ops
+	def forward(self, mb_id, **options):
+		"""F.  Options: ``remat_strategy`` (only a strategy that selects the stage root changes what
+		is kept: whole-stage checkpoint) and ``activation_offload`` (handled by the offloader the
+		engine wraps around this call)."""
+		var = self.input_variables[0]
+		x = self._check_io(var.wait_and_pop(mb_id), "stage input")
+		strategy = options.get(OpOptions.REMAT_STRATEGY)
+		flags = FWD_REMAT_ROOT if (strategy is not None and strategy("", self.model)) else 0
+		y = torch.empty_like(x)
+		with self._timed(f"forward({self.id}:{mb_id})"):
+			_lib.check(self.lib.elf_stage_forward(self._handle, mb_id, x.data_ptr(), y.data_ptr(), flags, _stream()), "elf_stage_forward")
+		self._kept.setdefault(mb_id, {})["x"] = x
+		for dst in self.output_variables[0]:
+			dst.set(dst.to_send, mb_id, y)
+		var.set(var.saved, mb_id, x)
+		out0 = self.output_variables[0][0]
+		out0.set(out0.saved, mb_id, y)
+		if self.is_last:
+			return [out0.get(out0.to_send, mb_id)]
+
+	def backward_inputs(self, mb_id, **options):
+		"""B.  Options ``recompute_activations`` / ``recompute_gradients`` drop the W stash halves."""
+		var = self.input_variables[0]
+		x = var.get(var.saved, mb_id)
+		outs = self.output_variables[0]
+		outs[0].get(outs[0].saved, mb_id)
+		dy = outs[0].wait_and_pop(mb_id)
+		for dst in outs[1:]:
+			dy = dy + dst.wait_and_pop(mb_id)
+		dy = self._check_io(dy, "output gradient")
+		ra = bool(options.get(OpOptions.RECOMPUTE_ACTIVATIONS, False))
+		rg = bool(options.get(OpOptions.RECOMPUTE_GRADIENTS, False))
+		flags = (BWD_RECOMPUTE_ACTIVATIONS if ra else 0) | (BWD_RECOMPUTE_GRADIENTS if rg else 0)
+		dx = torch.empty_like(x)
+		with self._timed(f"backward_inputs({self.id}:{mb_id})"):
+			_lib.check(self.lib.elf_stage_backward_inputs(self._handle, mb_id, x.data_ptr(), dy.data_ptr(), dx.data_ptr(), flags, _stream()), "elf_stage_backward_inputs")
+		kept = self._kept.setdefault(mb_id, {})
+		kept["dy"] = dy  # the last block's dY of the W stash is this tensor
+		if not ra:
+			kept.pop("x", None)
+		var.set(var.to_send, mb_id, dx)
+		if ra:
+			var.set(var.saved, mb_id, x)
+		if rg:
+			outs[0].set(outs[0].to_process, mb_id, dy)
+
+	def backward_params(self, mb_id, **options):
+		"""W: fp32 dW += dY^T X for every linear layer of the stage."""
+		with self._timed(f"backward_params({self.id}:{mb_id})"):
+			_lib.check(self.lib.elf_stage_backward_params(self._handle, mb_id, _stream()), "elf_stage_backward_params")
+		self._kept.pop(mb_id, None)
+
+	def recompute_forward(self, mb_id, **options):
+		var = self.input_variables[0]
+		x = var.get(var.saved, mb_id)
+		save = bool(options.get(OpOptions.SAVE, False))
+		with self._timed(f"recompute_forward({self.id}:{mb_id})"):
+			_lib.check(self.lib.elf_stage_recompute_forward(self._handle, mb_id, x.data_ptr(), int(save), _stream()), "elf_stage_recompute_forward")
+		if save:
+			var.set(var.saved, mb_id, x)
+			out0 = self.output_variables[0][0]
+			out0.set(out0.saved, mb_id, x)  # placeholder: the graph lives inside the library
+
+	def recompute_backward_inputs(self, mb_id, **options):
+		var = self.input_variables[0]
+		var.get(var.saved, mb_id)
+		out0 = self.output_variables[0][0]
+		out0.get(out0.saved, mb_id)
+		dy = out0.get(out0.to_process, mb_id)
+		with self._timed(f"recompute_backward_inputs({self.id}:{mb_id})"):
+			_lib.check(self.lib.elf_stage_recompute_backward_inputs(self._handle, mb_id, dy.data_ptr(), _stream()), "elf_stage_recompute_backward_inputs")
+		self._kept.setdefault(mb_id, {})["dy"] = dy
+
+	# ------------------------------------------------------------------ gradients
+	def scale_grads(self, batch_size):
+		"""main_grad /= batch_size, and param.grad = bf16(main_grad) (block.py:518-527)."""
+		inv = 1.0 / float(batch_size)
+		for i, (w, g) in enumerate(zip(self._fused_w, self._fused_g)):
+			if self._fused_bf16_grad[i] is None:
+				self._fused_bf16_grad[i] = torch.empty_like(w)
+			_lib.check(self.lib.elf_scale_grads(g.data_ptr(), self._fused_bf16_grad[i].data_ptr(), g.numel(), inv, _stream()), "elf_scale_grads")
+		for p, (i, r, n) in self._param_loc.items():
+			p.grad = self._fused_bf16_grad[i][r : r + n]
+
+	def zero_grad(self):
+		for g in self._fused_g:
+			g.zero_()
+		for p in self.main_grads:
+			p.grad = None
+
+	def all_reduce_param_grads(self, **options):
+		if self.dp_group is None:
+			return
+		import torch.distributed as dist
+
+		for g in self._fused_g:
+			dist.all_reduce(g, group=self.dp_group, op=dist.ReduceOp.AVG, async_op=True)
+
+	# ------------------------------------------------------------------ transfers (single GPU: peers are local or absent)
+	def set_boundary(self, inputs=None, grads=None, keep_sent=False):
+		"""Stand-ins for the stage's remote peers: ``inputs(mb)`` / ``grads(mb)`` (callables or
+		sequences of tensors) supply what RECV_FORWARD / RECV_BACKWARD would receive from another
+		rank; what SEND_FORWARD / SEND_BACKWARD would ship is dropped, or collected in
+		``sent_forward`` / ``sent_backward`` when ``keep_sent`` is set."""
+		self._feed_x = (lambda mb: inputs[mb]) if inputs is not None and not callable(inputs) else inputs
+		self._feed_dy = (lambda mb: grads[mb]) if grads is not None and not callable(grads) else grads
+		self._keep_sent = keep_sent
+		self.sent_forward, self.sent_backward = {}, {}
+
+	def _remote(self, peer):
+		return peer is not None and self.placement[peer] != self.rank
+
+	def _need_feed(self, feed, what):
+		if feed is None:
+			raise NotImplementedError(f"{self}: {what} from another rank needs set_boundary(): this build feeds stage boundaries from local buffers")
+		return feed
+
+	def send_forward(self, mb_id, **options):
+		dst = options.get("dst")
+		if self._remote(dst):
+			for target in self.output_variables[0]:
+				if target.peer == dst:
+					y = target.get(target.to_send, mb_id)
+					if getattr(self, "_keep_sent", False):
+						self.sent_forward[mb_id] = y
+
+	def send_backward(self, mb_id, **options):
+		dst = options.get("dst")
+		if self._remote(dst):
+			var = self.input_variables[0]
+			if var.peer == dst:
+				dx = var.get(var.to_send, mb_id)
+				if getattr(self, "_keep_sent", False):
+					self.sent_backward[mb_id] = dx
+
+	def recv_forward(self, mb_id, mb_size, **options):
+		src = options.get("src")
+		if self._remote(src):
+			var = self.input_variables[0]
+			if var.peer == src:
+				x = self._need_feed(getattr(self, "_feed_x", None), "recv_forward")(mb_id)
+				var.set(var.to_process, mb_id, (None, x))
+
+	def recv_backward(self, mb_id, mb_size, **options):
+		src = options.get("src")
+		if self._remote(src):
+			for target in self.output_variables[0]:
+				if target.peer == src:
+					dy = self._need_feed(getattr(self, "_feed_dy", None), "recv_backward")(mb_id)
+					target.set(target.to_process, mb_id, (None, dy))
+
+	def _wait_for_send_ops(self):
+		self.send_ops.clear()
+
+	# ------------------------------------------------------------------ offload hooks used by StageOffloader
+	def offload(self, mb_id):
+		_lib.check(self.lib.elf_stage_offload(self._handle, mb_id, _stream()), "elf_stage_offload")
+
+	def prefetch(self, mb_id):
+		_lib.check(self.lib.elf_stage_prefetch(self._handle, mb_id, _stream()), "elf_stage_prefetch")
+
+	def release(self, mb_id):
+		_lib.check(self.lib.elf_stage_release(self._handle, mb_id), "elf_stage_release")
+
+	def clear(self):
+		"""Drop every micro-batch state held by the library and the tensors pinned for it."""
+		_lib.check(self.lib.elf_stage_clear(self._handle), "elf_stage_clear")
+		self._kept.clear()
+
+	def mem_stats(self):
+		st = MemStats()
+		_lib.check(self.lib.elf_stage_mem_stats(self._handle, ctypes.byref(st)), "elf_stage_mem_stats")
+		return {n: getattr(st, n) for n, _ in MemStats._fields_}
+
+	def reset_peak(self):
+		_lib.check(self.lib.elf_stage_reset_peak(self._handle), "elf_stage_reset_peak")

@@ -1,0 +1,255 @@
+"""Per-rank interpreter of a schedule (the operation stream of the stages this process owns).
+
+Same dispatch, statistics and slot hand-offs as the reference's Engine (elf/execution/engine.py:
+96-371, compute_loss :374-410, same-rank transfers :413-445); the differences are that nothing
+here needs a process group or a GPU to be importable, and that the offload handles come from the
+block when it brings its own (``HipStageBlock`` -> ``StageOffloader``).
+"""
+
+import contextlib
+import logging
+import os
+import time
+from collections import OrderedDict, deque
+
+import torch
+import torch.distributed as dist
+
+from ..scheduling import OperationType, OpOptions
+from ..utils import Timer
+from .offload import StageOffloader
+
+logger = logging.getLogger("engine")
+
+# read once at import, any non-empty value switches them on (as in the reference)
+precise_timings = os.environ.get("ELF_TIMINGS", False)
+precise_memory = os.environ.get("ELF_MEMORY", False)
+
+__all__ = ["Engine", "compute_loss"]
+
+_GPU = torch.cuda.is_available
+
+
+def _fake_p2p(data):
+	"""A (work, tensor) pair with no pending work: how locally produced data enters a slot."""
+	return [None, data.detach()]
+
+
+def _sync():
+	if _GPU():
+		torch.cuda.synchronize()
+
+
+def _mem():
+	return (torch.cuda.memory_allocated(), torch.cuda.max_memory_allocated()) if _GPU() else (0, 0)
+
+
+class Engine:
+	"""Runs a list of operations on the blocks of one rank; feeds the pipeline input to the first
+	block and computes the loss on the last one."""
+
+	def __init__(self, blocks):
+		self.blocks = blocks
+		self.rank = blocks[0].rank if blocks else None
+		for b in blocks:
+			assert b.rank == self.rank, "All blocks in a stage should be on the same rank"
+		self.id_to_block = {b.id: b for b in blocks}
+		self.offload_stream = torch.cuda.Stream() if _GPU() else None
+		self.pool = None  # the pinned arena lives in the stage library
+
+	def _offloader(self, block, mb):
+		if hasattr(block, "offload"):
+			return StageOffloader(block, mb, self.pool)
+		raise NotImplementedError(f"{block}: this block type has no activation offload")
+
+	def train_step(self, batch, target, loss_fn, schedule, mb_sizes, profile=False):
+		"""Execute ``schedule`` (ops of other ranks are skipped).
+
+		Returns (result, losses, stats, detailed_stats): ``result`` = per-micro-batch outputs of the
+		last block, ``stats`` = {total, idle, start_idle, end_idle, bubble} in seconds (meaningful
+		with ELF_TIMINGS), ``detailed_stats`` = {"all_events": {timer name: s}, "memories":
+		{str(op): bytes allocated after it}, "peak_memory": {str(op): peak bytes}}; with a
+		HipStageBlock the byte counts include the library's own stash."""
+		if batch is not None:
+			microbatches = iter(zip(*[t.split(mb_sizes, dim=0) for t in batch]))
+		if target is not None:
+			microtargets = target.split(mb_sizes, dim=0)
+
+		offloaders = {}
+
+		def offloader(block, mb):
+			key = (block.id, mb)
+			if key not in offloaders:
+				offloaders[key] = self._offloader(block, mb)
+			return offloaders[key]
+
+		result, losses, grad_fns = [], [], deque()
+		if precise_timings:
+			if dist.is_available() and dist.is_initialized():
+				dist.barrier()
+			_sync()
+			t_sync = time.time()
+		pipe_start = time.time()
+		warmup_time = None
+		memories, peak_memories = OrderedDict(), OrderedDict()
+		T = OperationType
+
+		for op in schedule:
+			block = self.id_to_block.get(op.block_id)
+			if block is None:
+				continue
+			if profile and _GPU():
+				torch.cuda.nvtx.range_push(f"{block}:{op}")
+			if precise_memory and _GPU():
+				torch.cuda.reset_peak_memory_stats()
+				if hasattr(block, "reset_peak"):
+					block.reset_peak()
+			if warmup_time is None and op.op != T.RECV_FORWARD:
+				warmup_time = 0
+				if precise_timings:
+					_sync()
+					warmup_time = time.time() - t_sync
+
+			kind = op.op
+			if kind == T.FORWARD:
+				ctx = offloader(block, op.mb_id) if op.options.get(OpOptions.ACTIVATION_OFFLOAD) else contextlib.nullcontext()
+				with ctx:
+					y = block.forward(op.mb_id, **op.options)
+				if y is not None:
+					for out in y:
+						result.append(out.detach() if isinstance(out, torch.Tensor) else out)
+			elif kind == T.BACKWARD_INPUTS:
+				block.backward_inputs(op.mb_id, **op.options)
+				if op.options.get(OpOptions.ACTIVATION_OFFLOAD):
+					offloader(block, op.mb_id).release()
+			elif kind == T.BACKWARD_PARAMS:
+				block.backward_params(op.mb_id, **op.options)
+			elif kind == T.SEND_FORWARD:
+				dst = self.id_to_block.get(op.options.get("dst"))
+				if dst is not None:
+					_transfer_forward(block, dst, op.mb_id)
+				block.send_forward(op.mb_id, **op.options)
+			elif kind == T.SEND_BACKWARD:
+				dst = self.id_to_block.get(op.options.get("dst"))
+				if dst is not None:
+					_transfer_backward(block, dst, op.mb_id)
+				block.send_backward(op.mb_id, **op.options)
+			elif kind == T.RECV_FORWARD:
+				if block.is_first:
+					for mb, var in zip(next(microbatches), block.input_variables):
+						var.set(var.to_process, op.mb_id, _fake_p2p(mb))
+				block.recv_forward(op.mb_id, mb_sizes[op.mb_id], **op.options)
+			elif kind == T.RECV_BACKWARD:
+				block.recv_backward(op.mb_id, mb_sizes[op.mb_id], **op.options)
+			elif kind == T.LOSS_FORWARD:
+				if not block.is_last:
+					logger.warning(f"Tried to compute loss on a non-last block {block}")
+					continue
+				assert op.mb_id < len(result), f"Loss forward for mb {op.mb_id} but only {len(result)} results computed"
+				loss, grad_fn = compute_loss(block, result[op.mb_id], microtargets[op.mb_id], loss_fn)
+				losses.append(loss)
+				grad_fns.append(grad_fn)
+			elif kind == T.LOSS_BACKWARD:
+				if not block.is_last:
+					logger.warning(f"Tried to compute loss backward on a non-last block {block}")
+					continue
+				assert op.mb_id < len(losses), f"Loss backward for mb {op.mb_id} but only {len(losses)} losses computed"
+				with Timer(name=f"backward({block.id}:{op.mb_id})") as timer:
+					grads = grad_fns.popleft()()
+				block.compute_time.append(timer)
+				if self.offload_stream is not None:
+					self.offload_stream.wait_stream(torch.cuda.current_stream())
+					with torch.cuda.stream(self.offload_stream), torch.no_grad():
+						result[op.mb_id] = result[op.mb_id].to("cpu", non_blocking=True)
+				for grad, var in zip(grads, block.output_variables):
+					for dst in var:
+						dst.set(dst.to_process, op.mb_id, _fake_p2p(grad))
+			elif kind == T.RECOMPUTE_FORWARD:
+				block.recompute_forward(op.mb_id, **op.options)
+			elif kind == T.RECOMPUTE_BACKWARD_INPUTS:
+				block.recompute_backward_inputs(op.mb_id, **op.options)
+			elif kind == T.PREFETCH_ACTIVATIONS:
+				offloader(block, op.mb_id).prefetch()
+			elif kind == T.ALL_REDUCE_PARAM_GRADS:
+				block.scale_grads(sum(mb_sizes))
+				block.all_reduce_param_grads(**op.options)
+			else:
+				raise Exception(f"Unknown operation : {op}")
+
+			if precise_memory:
+				_sync()
+			alloc, peak = _mem()
+			if hasattr(block, "mem_stats"):
+				st = block.mem_stats()
+				alloc, peak = alloc + st["live_bytes"], peak + st["peak_bytes"]
+			memories[str(op)] = alloc
+			peak_memories[str(op)] = peak
+			if profile and _GPU():
+				torch.cuda.nvtx.range_pop()
+
+		if precise_timings:
+			_sync()
+		cooldown_start = time.time()
+		if precise_timings:
+			_sync()
+		pipe_end = time.time()
+
+		compute_time, all_events = 0, {}
+		if precise_timings:
+			for block in self.blocks:
+				compute_time += sum(t.time() for t in block.compute_time)
+				all_events.update({t.name: t.time() for t in block.compute_time})
+		stats = {
+			"total": pipe_end - pipe_start,
+			"idle": pipe_end - pipe_start - compute_time,
+			"start_idle": warmup_time,
+			"end_idle": pipe_end - cooldown_start,
+		}
+		stats["bubble"] = stats["idle"] - (stats["start_idle"] or 0) - stats["end_idle"]
+		detailed_stats = {"all_events": all_events, "memories": memories, "peak_memory": peak_memories}
+		for block in self.blocks:
+			block.compute_time.clear()
+		if self.offload_stream is not None:
+			torch.cuda.current_stream().wait_stream(self.offload_stream)
+		for off in offloaders.values():
+			off.release()
+		return result, losses, stats, detailed_stats
+
+
+def compute_loss(block, output, target, loss_fn):
+	"""Loss of one micro-batch, summed over its samples and divided by the elements per sample
+	(the division by the batch size happens with the gradient scale at the end of the step), and
+	the closure that back-propagates it to the block output."""
+	if not isinstance(output, torch.Tensor) or not isinstance(target, torch.Tensor):
+		logger.warning("Loss computation with non-tensor output or target")
+	output = output.detach().requires_grad_()
+	with Timer(name="loss_forward") as timer:
+		try:
+			loss = loss_fn(output, target, reduction="sum")
+		except TypeError:
+			loss = loss_fn(output, target)
+	block.compute_time.append(timer)
+	loss = loss / (target.numel() // target.size(0))
+
+	def grad_fn():
+		loss.backward()
+		return (output.grad.data,)
+
+	return loss.detach().requires_grad_(False), grad_fn
+
+
+def _transfer_forward(block, dst_block, mb_id):
+	"""Same-rank hand-off of activations: outputs of ``block`` bound for ``dst_block`` become its
+	pending inputs (matched by position)."""
+	outgoing = [d for var in block.output_variables for d in var if d.peer == dst_block.id]
+	incoming = [v for v in dst_block.input_variables if v.peer == block.id]
+	for src, dst in zip(outgoing, incoming):
+		dst.set(dst.to_process, mb_id, _fake_p2p(src.get(src.to_send, mb_id)))
+
+
+def _transfer_backward(block, dst_block, mb_id):
+	"""Same-rank hand-off of input gradients to the block that produced those inputs."""
+	outgoing = [v for v in block.input_variables if v.peer == dst_block.id]
+	incoming = [s for var in dst_block.output_variables for s in var if s.peer == block.id]
+	for src, dst in zip(outgoing, incoming):
+		dst.set(dst.to_process, mb_id, _fake_p2p(src.get(src.to_send, mb_id)))

@@ -96,6 +96,105 @@ int elf_attn_bwd(const void* q, const void* k, const void* v, const void* o, con
                  int64_t lddv, int B, int S, int Hq, int Hkv, int D, int causal, float scale,
                  void* stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * Stage executor: one pipeline stage = n_blocks transformer blocks on T = mb * seq tokens.
+ * It is what PipelineBlock (elf/execution/block.py:134-694) does through nn.Module.__call__ and
+ * autograd, with the LinearDX / LinearDW split backward (elf/zb_utils.py:9-256) made explicit.
+ * The caller (torch) owns the boundary tensors X, Y, dY, dX, the weights and the fp32 gradient
+ * accumulators; the library owns the per-micro-batch activation stash, the W stash (input X and
+ * output gradient dY of every linear layer), temporaries, the pinned-host arena and the two side
+ * streams of activation offload.  All calls for one stage come from one host thread and use one
+ * stream; the external X of a micro-batch must stay valid until its B (and until its recompute
+ * ops), the external dY until its W. */
+typedef struct elf_stage elf_stage_t;
+
+enum { ELF_ARCH_GPT = 0, ELF_ARCH_LLAMA = 1 };
+/*  GPT block   (benchmarks/models/simple.py:437-468, dropout off): LayerNorm, bias-free q/k/v/o
+ *              projections, multi-head attention, GELU FFN, two residual adds.
+ *  Llama block (no reference module): RMSNorm, RoPE (half-split), grouped-query attention,
+ *              SwiGLU FFN. */
+typedef struct elf_stage_cfg {
+	int arch;        /* ELF_ARCH_* */
+	int n_blocks;
+	int d_model;
+	int n_heads;     /* query heads */
+	int n_kv_heads;  /* == n_heads for ELF_ARCH_GPT */
+	int head_dim;    /* 64 or 128; the attention width n_heads*head_dim may differ from d_model */
+	int ffn;         /* FFN hidden size F */
+	int seq;         /* tokens per sequence, multiple of 128 */
+	int mb;          /* sequences per micro-batch */
+	int causal;
+	float eps;
+	double rope_theta;
+} elf_stage_cfg;
+
+/* Parameter ids for elf_stage_bind_param (weights bf16 row-major [out, in], as nn.Linear):
+ *  0 norm1 gamma [d]   1 norm1 beta [d] (GPT only)   2 Wqkv [(Hq+2Hkv)*D, d] (q rows, k rows, v rows)
+ *  3 Wo [d, Hq*D]      4 norm2 gamma    5 norm2 beta (GPT only)
+ *  6 W1 [F, d] (GPT fc1)  or  [2F, d] (Llama: gate rows then up rows)     7 W2 [d, F] */
+enum { ELF_P_NORM1_G = 0, ELF_P_NORM1_B, ELF_P_WQKV, ELF_P_WO, ELF_P_NORM2_G, ELF_P_NORM2_B, ELF_P_W1, ELF_P_W2, ELF_P_COUNT };
+
+/* Forward flags (FORWARD options, elf/scheduling/scheduling.py:58-86):
+ *  REMAT_ROOT: remat_strategy selects the whole stage (name == ""), i.e. full checkpointing: only
+ *              the stage input is kept and B re-runs the forward (elf/execution/remat.py:26-74);
+ *  OFFLOAD:    activation_offload: the stash goes to pinned host memory on a side stream
+ *              (elf/execution/offload.py:228-268, 330-352). */
+enum { ELF_FWD_REMAT_ROOT = 1u, ELF_FWD_OFFLOAD = 4u };
+/* BACKWARD_INPUTS flags: recompute_activations drops the W-stash inputs after B,
+ * recompute_gradients drops the W-stash output gradients (elf/execution/block.py:659-694). */
+enum { ELF_BWD_RECOMPUTE_ACTIVATIONS = 1u, ELF_BWD_RECOMPUTE_GRADIENTS = 2u };
+
+typedef struct elf_mem_stats {
+	int64_t live_bytes;      /* device bytes held by stashes and temporaries now */
+	int64_t peak_bytes;      /* high-water mark of live_bytes since create / reset_peak */
+	int64_t reserved_bytes;  /* device bytes obtained from the driver (live + cached) */
+	int64_t pinned_bytes;    /* size of the pinned-host arena */
+	int64_t d2h_bytes;       /* total bytes offloaded */
+	int64_t h2d_bytes;       /* total bytes brought back */
+} elf_mem_stats;
+
+int elf_stage_create(const elf_stage_cfg* cfg, elf_stage_t** out);
+void elf_stage_destroy(elf_stage_t* s);
+/* torch keeps ownership; grad_f32 is the fp32 accumulator of the same shape as the weight. */
+int elf_stage_bind_param(elf_stage_t* s, int block, int which, void* weight_bf16, void* grad_f32);
+/* F: PipelineBlock.forward (block.py:210-279). x, y: bf16 [T, d_model]. */
+int elf_stage_forward(elf_stage_t* s, int mb, const void* x, void* y, uint32_t flags, void* stream);
+/* B: PipelineBlock.backward_inputs (block.py:624-694, 281-306). dy, dx: bf16 [T, d_model]; x is the
+ * stage input again (needed when the forward was checkpointed; may be NULL otherwise). */
+int elf_stage_backward_inputs(elf_stage_t* s, int mb, const void* x, const void* dy, void* dx, uint32_t flags, void* stream);
+/* W: PipelineBlock.backward_params + LinearDW.backward (block.py:376-391, zb_utils.py:215-256):
+ * grad_f32 += dY^T X for every linear layer, then the W stash of the micro-batch is dropped. */
+int elf_stage_backward_params(elf_stage_t* s, int mb, void* stream);
+/* RF: PipelineBlock.recompute_forward (block.py:308-338). save = 0 refills only the W-stash inputs,
+ * save != 0 rebuilds the whole activation stash. */
+int elf_stage_recompute_forward(elf_stage_t* s, int mb, const void* x, int save, void* stream);
+/* RB*: PipelineBlock.recompute_backward_inputs + partial_dx_recomputation (block.py:340-374,
+ * zb_utils.py:584-604): refills the W-stash output gradients; no norm gradients, no stage dX. */
+int elf_stage_recompute_backward_inputs(elf_stage_t* s, int mb, const void* dy, void* stream);
+/* Offload life cycle (OffloadToCPU, offload.py:166-411): offload is also implied by
+ * ELF_FWD_OFFLOAD; prefetch = PREFETCH_ACTIVATIONS; release returns the pinned blocks. */
+int elf_stage_offload(elf_stage_t* s, int mb, void* stream);
+int elf_stage_prefetch(elf_stage_t* s, int mb, void* stream);
+int elf_stage_release(elf_stage_t* s, int mb);
+/* Drop every micro-batch state (Pipeline.step clears all slots after a step, pipeline.py:265-275). */
+int elf_stage_clear(elf_stage_t* s);
+int elf_stage_mem_stats(elf_stage_t* s, elf_mem_stats* out);
+int elf_stage_reset_peak(elf_stage_t* s);
+
+/* Pinned-host arena with the placement rules of PinnedHostTensorPool (offload.py:14-158).
+ * host_backing != 0 backs it with malloc so the rules can be exercised without a GPU.
+ * elf_pinned_pool_free returns 1 (and does nothing) for a pointer that is not a live block. */
+typedef struct elf_pinned_pool elf_pinned_pool_t;
+int elf_pinned_pool_create(int host_backing, elf_pinned_pool_t** out);
+void elf_pinned_pool_destroy(elf_pinned_pool_t* p);
+int elf_pinned_pool_allocate(elf_pinned_pool_t* p, int64_t elems, int elem_size, int dtype_key, void** ptr, int* parent, int64_t* offset);
+int elf_pinned_pool_free(elf_pinned_pool_t* p, void* ptr);
+int elf_pinned_pool_reserve(elf_pinned_pool_t* p, int64_t bytes, int elem_size, int dtype_key);
+int64_t elf_pinned_pool_size(elf_pinned_pool_t* p);
+int elf_pinned_pool_n_parents(elf_pinned_pool_t* p);
+int elf_pinned_pool_n_free(elf_pinned_pool_t* p, int parent);
+int elf_pinned_pool_free_segment(elf_pinned_pool_t* p, int parent, int i, int64_t* offset, int64_t* length);
+
 #ifdef __cplusplus
 }
 #endif

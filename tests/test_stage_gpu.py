@@ -1,0 +1,200 @@
+"""F / B / W of a whole stage through the C ABI (HipStageBlock) against the oracle stage
+(oracle/stage_ref.py, fp32 from the same bf16-rounded weights and boundary tensors).
+Tolerance: rel 2e-2 of the tensor's max magnitude (the path's stated bf16 bar), plus a 1e-2
+relative Frobenius bound; weight gradients are accumulated in fp32 over several micro-batches."""
+
+import pytest
+import torch
+
+from tests.helpers import assert_close, cfg_from_stage, oracle_params_from_stage, perturb_norms, product_grads
+
+pytestmark = pytest.mark.gpu
+
+N_MB = 3
+
+
+def _stage(kind):
+	from elf_amd import models
+
+	if kind == "gpt":
+		st = models.gpt_stage(2, 256, 4, 512, 128, causal=False, seed=3)
+	elif kind == "gpt_causal":
+		st = models.gpt_stage(1, 128, 2, 256, 256, causal=True, seed=4)
+	else:
+		st = models.llama_stage(2, 512, 4, 2, 768, 256, head_dim=128, seed=5)
+	perturb_norms(st)
+	return st
+
+
+def _block(stage, mb):
+	from elf_amd.execution import HipStageBlock
+	from elf_amd.partitioners.utils import sequential_signatures
+
+	placement = [0, 1, 2, 3]
+	return HipStageBlock(stage, 1, placement, sequential_signatures(placement)[1], mb_size=mb)
+
+
+def _oracle(stage, mb, **kw):
+	from oracle import stage_ref as R
+
+	cfg = cfg_from_stage(stage, mb)
+	return R, cfg, R.RefStage(cfg, oracle_params_from_stage(stage), device="cuda", **kw)
+
+
+@pytest.mark.parametrize("kind", ["gpt", "gpt_causal", "llama"])
+def test_fbw_matches_oracle(kind):
+	mb = 2
+	stage = _stage(kind)
+	R, cfg, ref = _oracle(stage, mb)
+	blk = _block(stage, mb)
+	xs, dys = R.make_boundary(cfg, N_MB, seed=11)
+	blk.set_boundary(inputs=[x.cuda() for x in xs], grads=[d.cuda() for d in dys], keep_sent=True)
+	# all forwards first, then B, then W (queues hold several micro-batches at once)
+	for m in range(N_MB):
+		blk.recv_forward(m, mb, src=0)
+		blk.forward(m)
+		blk.send_forward(m, dst=2)
+		assert_close(blk.sent_forward[m], ref.forward(m, xs[m]), f"{kind} y[{m}]")
+	for m in range(N_MB):
+		blk.recv_backward(m, mb, src=2)
+		blk.backward_inputs(m)
+		blk.send_backward(m, dst=0)
+		assert_close(blk.sent_backward[m], ref.backward_inputs(m, dys[m]), f"{kind} dx[{m}]")
+	for m in range(N_MB):
+		blk.backward_params(m)
+		ref.backward_params(m)
+	got, want = product_grads(stage), ref.grads()
+	assert set(got) == set(want)
+	for name in sorted(want):
+		assert_close(got[name], want[name], f"{kind} grad {name}")
+	# scale_grads: main_grad /= batch and bf16 .grad appears (block.py:518-527)
+	blk.scale_grads(mb * N_MB)
+	ref.scale_grads(mb * N_MB)
+	got_bf16, got32, want = product_grads(stage, "grad"), product_grads(stage), ref.grads()
+	for name in sorted(want):
+		assert got_bf16[name].dtype == torch.bfloat16
+		assert_close(got32[name], want[name], f"{kind} scaled grad {name}")
+		assert torch.equal(got_bf16[name], got32[name].to(torch.bfloat16))
+	st = blk.mem_stats()
+	assert st["live_bytes"] == 0, "every stash must be gone after W"
+	assert st["peak_bytes"] > 0
+
+
+@pytest.mark.parametrize("kind", ["gpt", "llama"])
+@pytest.mark.parametrize("variant", ["full_fwd", "activations_bwd", "full_bwd", "offload", "offload_no_prefetch"])
+def test_remat_and_offload_variants_equal_plain(kind, variant):
+	"""Every remat / offload variant must give the results of the plain F-B-W sequence (same
+	kernels on the same data; only dQ and split-K accumulate with atomics, hence a tolerance)."""
+	from elf_amd.scheduling import OpOptions
+
+	mb = 16 if variant.startswith("offload") else 2  # only buffers above 1 MiB are offloaded
+	stage = _stage(kind)
+	R, cfg, _ = _oracle(stage, mb)
+	xs, dys = R.make_boundary(cfg, 2, seed=21)
+	xs, dys = [x.cuda() for x in xs], [d.cuda() for d in dys]
+
+	def run(variant):
+		blk = _block(stage, mb)
+		blk.zero_grad()
+		blk.set_boundary(inputs=xs, grads=dys, keep_sent=True)
+		root = lambda name, module: name == ""
+		for m in range(2):
+			blk.recv_forward(m, mb, src=0)
+			if variant == "full_fwd":
+				blk.forward(m, **{OpOptions.REMAT_STRATEGY: root})
+				assert blk.mem_stats()["live_bytes"] == 0, "a checkpointed forward keeps nothing"
+			elif variant.startswith("offload"):
+				blk.forward(m)
+				blk.offload(m)
+			else:
+				blk.forward(m)
+			blk.send_forward(m, dst=2)
+		if variant.startswith("offload"):
+			torch.cuda.synchronize()
+			st = blk.mem_stats()
+			assert st["d2h_bytes"] > 0 and st["pinned_bytes"] >= st["d2h_bytes"]
+		for m in range(2):
+			blk.recv_backward(m, mb, src=2)
+			if variant == "activations_bwd":
+				blk.backward_inputs(m, **{OpOptions.RECOMPUTE_ACTIVATIONS: True})
+				blk.recompute_forward(m)
+			elif variant == "full_bwd":
+				blk.backward_inputs(m, **{OpOptions.RECOMPUTE_ACTIVATIONS: True, OpOptions.RECOMPUTE_GRADIENTS: True})
+				if m == 1:  # no other micro-batch in flight any more
+					assert blk.mem_stats()["live_bytes"] == 0, "full_bwd drops both halves of the W stash"
+				blk.recompute_forward(m, **{OpOptions.SAVE: True})
+				blk.recompute_backward_inputs(m)
+			elif variant == "offload":
+				blk.prefetch(m)
+				blk.backward_inputs(m)
+				blk.release(m)
+			elif variant == "offload_no_prefetch":
+				blk.backward_inputs(m)
+				blk.release(m)
+			else:
+				blk.backward_inputs(m)
+			blk.send_backward(m, dst=0)
+			blk.backward_params(m)
+		torch.cuda.synchronize()
+		assert blk.mem_stats()["live_bytes"] == 0
+		grads = {k: v.clone() for k, v in product_grads(stage).items()}
+		return dict(blk.sent_forward), dict(blk.sent_backward), grads
+
+	y0, dx0, g0 = run("plain")
+	y1, dx1, g1 = run(variant)
+	for m in range(2):
+		assert torch.equal(y0[m], y1[m]), "forward outputs must be bit-identical"
+		assert_close(dx1[m], dx0[m], f"{variant} dx[{m}]", rel_max=2e-3, rel_fro=1e-3)
+	for name in g0:
+		assert_close(g1[name], g0[name], f"{variant} grad {name}", rel_max=2e-3, rel_fro=1e-3)
+
+
+def test_engine_runs_1f1b_and_zbh1_streams():
+	"""The Engine interprets the filtered op stream of a middle stage (block 1 of pp = 4) and gives
+	the same gradients as the oracle stage driven by the same stream."""
+	from elf_amd.execution import Engine
+	from elf_amd.partitioners.utils import sequential_signatures
+	from elf_amd.registry import COMM_SCHEDULERS, SCHEDULERS
+	from elf_amd.scheduling import OperationType as T, add_comms
+
+	mb, nmb, placement = 2, 4, [0, 1, 2, 3]
+	for sched_name in ("1f1b", "zbh1"):
+		stage = _stage("llama")
+		R, cfg, ref = _oracle(stage, mb)
+		xs, dys = R.make_boundary(cfg, nmb, seed=31)
+		blk = _block(stage, mb)
+		blk.zero_grad()
+		blk.set_boundary(inputs=[x.cuda() for x in xs], grads=[d.cuda() for d in dys])
+		schedule = COMM_SCHEDULERS["pipelined"](add_comms(SCHEDULERS[sched_name](placement, nmb), sequential_signatures(placement)))
+		stream = [op for op in schedule if op.block_id == 1]
+		eng = Engine([blk])
+		result, losses, stats, detailed = eng.train_step(None, None, None, stream, [mb] * nmb)
+		for op in stream:
+			if op.op == T.FORWARD:
+				ref.forward(op.mb_id, xs[op.mb_id])
+			elif op.op == T.BACKWARD_INPUTS:
+				ref.backward_inputs(op.mb_id, dys[op.mb_id])
+			elif op.op == T.BACKWARD_PARAMS:
+				ref.backward_params(op.mb_id)
+			elif op.op == T.ALL_REDUCE_PARAM_GRADS:
+				ref.scale_grads(mb * nmb)
+		got, want = product_grads(stage), ref.grads()
+		for name in sorted(want):
+			assert_close(got[name], want[name], f"{sched_name} grad {name}")
+		assert list(detailed["memories"]) == [str(op) for op in stream]
+		assert set(stats) == {"total", "idle", "start_idle", "end_idle", "bubble"}
+
+
+def test_error_paths():
+	from elf_amd._lib import ElfStageError
+
+	stage = _stage("gpt")
+	blk = _block(stage, 2)
+	with pytest.raises(ElfStageError):
+		blk.backward_params(0)  # nothing stashed
+	blk.set_boundary(inputs=[torch.zeros(2, 128, 256, dtype=torch.float32, device="cuda")])
+	blk.recv_forward(0, 2, src=0)
+	with pytest.raises(ElfStageError):
+		blk.forward(0)  # wrong dtype
+	with pytest.raises(Exception):
+		blk.forward(1)  # empty slot
