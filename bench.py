@@ -1,0 +1,191 @@
+#!/usr/bin/env python3
+"""Stage throughput benchmark: one pass ("step") of a pipeline stage's operation stream
+(F, split B, deferred W, grad scale) over one batch of synthetic micro-batches on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
+
+Prints ONE JSON line.  ``value`` = tokens/s of the whole stream with weights, boundary
+activations and boundary gradients already resident in HBM.  ``roofline`` is for the dominant
+kernel family (the bf16 MFMA GEMM): algorithmic FLOPs (2MNK per launch) divided by the launch
+durations measured live with HIP events on the launch stream, against the published dense bf16
+peak.  ``cpu_baseline`` times the plain-PyTorch CPU restatement of the reference stage (oracle/)
+on a bounded sample (one micro-batch of F, B and W through ONE block, fp32) on the host cores.
+"""
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA peak
+PEAK_HBM_GBS = 8000.0
+
+WORKLOADS = {
+	# BASELINE.json configs[2]: Llama-3-8B-shaped stage, ZB-H1 stream of block 1 in a 4-stage pipeline
+	"llama3_8b_zbh1": dict(arch="llama", n_blocks=4, d=4096, heads=32, kv_heads=8, head_dim=128, ffn=14336, seq=4096, mb=2, n_mb=16,
+	                       scheduler="zbh1", causal=True, rope_theta=5e5),
+	# same stage under 1F1B
+	"llama3_8b_1f1b": dict(arch="llama", n_blocks=4, d=4096, heads=32, kv_heads=8, head_dim=128, ffn=14336, seq=4096, mb=2, n_mb=16,
+	                       scheduler="1f1b", causal=True, rope_theta=5e5),
+	# BASELINE.json configs[1]: GPT-2-small-shaped stage, 1F1B
+	"gpt2s_1f1b": dict(arch="gpt", n_blocks=3, d=768, heads=12, kv_heads=12, head_dim=64, ffn=3072, seq=1024, mb=8, n_mb=8,
+	                   scheduler="1f1b", causal=False),
+	# BASELINE.json configs[4]: Llama-3-70B-shaped stage, 1F1B with activation offload
+	"llama3_70b_offload": dict(arch="llama", n_blocks=2, d=8192, heads=64, kv_heads=8, head_dim=128, ffn=28672, seq=8192, mb=1, n_mb=8,
+	                           scheduler="1f1b", causal=True, rope_theta=5e5, offload=True),
+	# small shape for smoke runs
+	"tiny": dict(arch="llama", n_blocks=2, d=512, heads=4, kv_heads=2, head_dim=128, ffn=768, seq=256, mb=2, n_mb=4,
+	             scheduler="zbh1", causal=True, rope_theta=5e5),
+}
+PLACEMENT = [0, 1, 2, 3]
+BLOCK_ID = 1  # a middle stage: no embedding, no loss
+
+
+def stream_flops(w):
+	"""Algorithmic FLOPs of one step (F + B + W over all blocks and micro-batches); attention
+	backward counted as 4 matmuls, causal attention at half the square."""
+	T, d, F = w["mb"] * w["seq"], w["d"], w["ffn"]
+	nq, nkv = w["heads"] * w["head_dim"], w["kv_heads"] * w["head_dim"]
+	lin = 2.0 * T * (d * (nq + 2 * nkv) + nq * d + d * F * (3 if w["arch"] == "llama" else 2))
+	att = (2.0 if w["causal"] else 4.0) * w["mb"] * w["heads"] * w["seq"] ** 2 * w["head_dim"]
+	return (3 * lin + 3 * att) * w["n_blocks"] * w["n_mb"]
+
+
+def build_stage(w):
+	from elf_amd import models
+
+	if w["arch"] == "llama":
+		return models.llama_stage(w["n_blocks"], w["d"], w["heads"], w["kv_heads"], w["ffn"], w["seq"], head_dim=w["head_dim"], rope_theta=w["rope_theta"], seed=0)
+	return models.gpt_stage(w["n_blocks"], w["d"], w["heads"], w["ffn"], w["seq"], causal=w["causal"], seed=0)
+
+
+def op_stream(w):
+	from elf_amd.benchmark_utils import get_offloaded_scheduler
+	from elf_amd.partitioners.utils import sequential_signatures
+	from elf_amd.registry import COMM_SCHEDULERS, SCHEDULERS
+	from elf_amd.scheduling import add_comms, check_schedule_validity
+
+	sched = get_offloaded_scheduler(w["scheduler"], 1, 1) if w.get("offload") else SCHEDULERS[w["scheduler"]]
+	schedule = COMM_SCHEDULERS["pipelined"](add_comms(sched(PLACEMENT, w["n_mb"]), sequential_signatures(PLACEMENT)))
+	check_schedule_validity(schedule)
+	return [op for op in schedule if op.block_id == BLOCK_ID]
+
+
+def cpu_baseline(w, stage_module):
+	"""Oracle stage on the host cores: F, B, W of ONE micro-batch through ONE block, fp32."""
+	import torch
+	from oracle import stage_ref as R
+	from tests.helpers import cfg_from_stage, oracle_params_from_stage
+
+	cores = os.cpu_count() or 1
+	torch.set_num_threads(cores)
+	cfg = cfg_from_stage(stage_module, w["mb"])
+	cfg["n_blocks"] = 1
+	params = [{k: v.cpu() for k, v in oracle_params_from_stage(stage_module)[0].items()}]
+	ref = R.RefStage(cfg, params, compute_dtype=torch.float32, device="cpu", use_sdpa=True)
+	xs, dys = R.make_boundary(cfg, 1, seed=1)
+	t0 = time.perf_counter()
+	ref.forward(0, xs[0])
+	t1 = time.perf_counter()
+	ref.backward_inputs(0, dys[0])
+	t2 = time.perf_counter()
+	ref.backward_params(0)
+	t3 = time.perf_counter()
+	T = w["mb"] * w["seq"]
+	per_block = t3 - t0
+	return {
+		"value": T / (per_block * w["n_blocks"]), "unit": "tokens/s", "cores": cores, "kind": "port",
+		"sample": f"oracle/stage_ref.py RefStage on CPU, fp32, SDPA attention: 1 micro-batch ({T} tokens) of F+B+W through 1 of {w['n_blocks']} blocks "
+		          f"(F {t1 - t0:.2f}s, B {t2 - t1:.2f}s, W {t3 - t2:.2f}s), extrapolated to the {w['n_blocks']}-block stage; no warm-up",
+	}
+
+
+def main():
+	ap = argparse.ArgumentParser()
+	ap.add_argument("--gpus", type=int, default=1)
+	ap.add_argument("--steps", type=int, default=3)
+	ap.add_argument("--warmup", type=int, default=1)
+	ap.add_argument("--workload", default="llama3_8b_zbh1", choices=sorted(WORKLOADS))
+	ap.add_argument("--no-cpu-baseline", action="store_true")
+	args = ap.parse_args()
+	if args.gpus != 1:
+		print("bench.py: this build runs one stage on ONE GPU; --gpus must be 1 (multi-GPU sharding is design-only).", file=sys.stderr)
+		sys.exit(2)
+
+	import torch
+	from elf_amd import _lib
+	from elf_amd.execution import Engine, HipStageBlock
+	from elf_amd.partitioners.utils import sequential_signatures
+	from elf_amd.synthetic import make_boundary
+
+	if not torch.cuda.is_available():
+		print("bench.py: no GPU visible; the stage kernels have no CPU path.", file=sys.stderr)
+		sys.exit(1)
+	lib = _lib.load()
+	w = WORKLOADS[args.workload]
+	stage = build_stage(w)
+	cpu_stats = None
+	if not args.no_cpu_baseline:
+		cpu_stats = cpu_baseline(w, stage)
+	block = HipStageBlock(stage, BLOCK_ID, PLACEMENT, sequential_signatures(PLACEMENT)[BLOCK_ID], mb_size=w["mb"])
+	xs, dys = make_boundary(w["mb"], w["seq"], w["d"], w["n_mb"], seed=1, device="cuda")
+	block.set_boundary(inputs=xs, grads=dys)
+	stream = op_stream(w)
+	engine = Engine([block])
+	mb_sizes = [w["mb"]] * w["n_mb"]
+
+	def step():
+		block.zero_grad()
+		engine.train_step(None, None, None, stream, mb_sizes)
+
+	for _ in range(args.warmup):
+		step()
+	torch.cuda.synchronize()
+	lib.elf_prof_enable(1)
+	t0 = time.perf_counter()
+	for _ in range(args.steps):
+		step()
+	torch.cuda.synchronize()
+	elapsed = time.perf_counter() - t0
+	kinds = ["gemm", "attn_fwd", "attn_bwd", "norm_fwd", "norm_bwd", "act_fwd", "act_bwd", "rope", "grad_scale", "add"]
+	per_kernel = {}
+	for i, name in enumerate(kinds):
+		ms, work = ctypes.c_double(), ctypes.c_double()
+		n = lib.elf_prof_collect(i, ctypes.byref(ms), ctypes.byref(work))
+		if n > 0:
+			rate = work.value / (ms.value * 1e-3)
+			per_kernel[name] = {"launches": n, "avg_ms": ms.value / n, "total_ms": ms.value,
+			                    ("tflops" if i < 3 else "gbs"): rate / (1e12 if i < 3 else 1e9)}
+	lib.elf_prof_enable(0)
+	mem = block.mem_stats()
+	tokens = w["mb"] * w["seq"] * w["n_mb"]
+	ms_per_step = elapsed / args.steps * 1e3
+	g = per_kernel.get("gemm", {"tflops": 0.0, "launches": 0, "avg_ms": 0.0})
+	out = {
+		"metric": "stage tokens/sec (F+B+W) on 1 MI355X", "value": tokens / (elapsed / args.steps), "unit": "tokens/s", "n_gpus": 1,
+		"steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+		"vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+		"config": {
+			"workload": args.workload, "blocks": w["n_blocks"], "d_model": w["d"], "heads": w["heads"], "kv_heads": w["kv_heads"], "ffn": w["ffn"],
+			"seq_len": w["seq"], "micro_batch": w["mb"], "n_micro_batches": w["n_mb"], "op_stream": f"{w['scheduler']} block {BLOCK_ID} of placement {PLACEMENT}",
+			"tokens_per_step": tokens, "ops_per_step": len(stream), "offload": bool(w.get("offload")),
+		},
+		"roofline": {"bound": "mfma", "achieved": g["tflops"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": g["tflops"] / PEAK_BF16_TFLOPS, "traffic": None,
+		             "kernel": "elf::gemm_kernel (bf16 MFMA GEMM, all layouts)", "launches": g["launches"], "avg_launch_ms": g["avg_ms"]},
+		"stream_mfu": stream_flops(w) / (elapsed / args.steps) / (PEAK_BF16_TFLOPS * 1e12),
+		"kernels": per_kernel,
+		"peak_stage_memory_bytes": mem["peak_bytes"] + torch.cuda.max_memory_allocated(),
+		"stash_peak_bytes": mem["peak_bytes"], "offload_d2h_bytes": mem["d2h_bytes"], "offload_h2d_bytes": mem["h2d_bytes"],
+	}
+	if cpu_stats is not None:
+		out["cpu_baseline"] = cpu_stats
+	print(json.dumps(out))
+
+
+if __name__ == "__main__":
+	main()

@@ -577,6 +577,7 @@ int attn_fwd(const void* q, const void* k, const void* v, void* o, void* lse, in
 	ELF_REQUIRE(ldq % 8 == 0 && ldk % 8 == 0 && ldv % 8 == 0 && ldo % 8 == 0, "attn_fwd: strides must be multiples of 8");
 	ELF_REQUIRE(((uintptr_t)q % 16) == 0 && ((uintptr_t)k % 16) == 0 && ((uintptr_t)v % 16) == 0 && ((uintptr_t)o % 8) == 0,
 	            "attn_fwd: misaligned pointer");
+	ProfScope prof(PROF_ATTN_FWD, (causal ? 2.0 : 4.0) * B * Hq * (double)S * S * D, stream);
 	AttnArgs a{(const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, (bf16_t*)o, (float*)lse, ldq, ldk, ldv, ldo, B, S, Hq, Hkv, scale};
 	const dim3 grid((unsigned)((int64_t)B * Hq * (S / 128))), block(256);
 	int rc;
@@ -604,6 +605,7 @@ int attn_bwd(const void* q, const void* k, const void* v, const void* o, const v
 	                lddk % 8 == 0 && lddv % 8 == 0,
 	            "attn_bwd: strides must be multiples of 8");
 	ELF_REQUIRE(((uintptr_t)workspace % 16) == 0, "attn_bwd: misaligned workspace");
+	ProfScope prof(PROF_ATTN_BWD, (causal ? 4.0 : 8.0) * B * Hq * (double)S * S * D, stream);
 	const int64_t T = (int64_t)B * S;
 	float* dq_acc = (float*)workspace;
 	float* delta = dq_acc + T * Hq * D;

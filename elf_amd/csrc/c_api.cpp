@@ -60,4 +60,10 @@ int elf_attn_bwd(const void* q, const void* k, const void* v, const void* o, con
 	                     Hkv, D, causal, scale, S_(stream));
 }
 
+void elf_prof_enable(int on) { elf::prof_enable(on); }
+int elf_prof_collect(int kind, double* total_ms, double* total_work) {
+	if (kind < 0 || kind >= elf::PROF_COUNT) return -1;
+	return elf::prof_collect(kind, total_ms, total_work);
+}
+
 }  // extern "C"

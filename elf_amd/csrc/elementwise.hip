@@ -270,6 +270,7 @@ int norm_fwd(int kind, const void* x, const void* gamma, const void* beta, void*
              float eps, hipStream_t s) {
 	ELF_REQUIRE(T > 0 && d > 0 && d % 8 == 0 && d <= 8192, "norm_fwd: d must be a multiple of 8 and <= 8192 (d=%d)", d);
 	ELF_REQUIRE(x && gamma && y && stats, "norm_fwd: null pointer");
+	ProfScope prof(PROF_NORM_FWD, 4.0 * T * d, s);
 	if (kind == NORM_LAYER) {
 		ELF_REQUIRE(beta != nullptr, "norm_fwd: LayerNorm needs beta");
 		return norm_fwd_dispatch<true>(x, gamma, beta, y, stats, T, d, eps, s);
@@ -300,6 +301,7 @@ int norm_bwd(int kind, const void* dy, const void* x, const void* gamma, const v
              void* dx, float* dgamma, float* dbeta, float* workspace, int T, int d, hipStream_t s) {
 	ELF_REQUIRE(T > 0 && d > 0 && d % 8 == 0 && d <= 8192, "norm_bwd: d must be a multiple of 8 and <= 8192 (d=%d)", d);
 	ELF_REQUIRE(dy && x && gamma && stats && dx && dgamma && workspace, "norm_bwd: null pointer");
+	ProfScope prof(PROF_NORM_BWD, (dres ? 8.0 : 6.0) * T * d, s);
 	int rc;
 	if (kind == NORM_LAYER) {
 		ELF_REQUIRE(dbeta != nullptr, "norm_bwd: LayerNorm needs dbeta");
@@ -385,12 +387,14 @@ static inline int ew_grid(int64_t nchunks) {
 
 int gelu_fwd(const void* x, void* y, int64_t n, hipStream_t s) {
 	ELF_REQUIRE(n > 0 && n % 8 == 0 && x && y, "gelu_fwd: n must be a positive multiple of 8");
+	ProfScope prof(PROF_ACT_FWD, 4.0 * n, s);
 	hipLaunchKernelGGL(gelu_fwd_kernel, dim3(ew_grid(n / 8)), dim3(256), 0, s, (const bf16_t*)x, (bf16_t*)y, n / 8);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
 }
 int gelu_bwd(const void* dy, const void* x, void* dx, int64_t n, hipStream_t s) {
 	ELF_REQUIRE(n > 0 && n % 8 == 0 && x && dy && dx, "gelu_bwd: n must be a positive multiple of 8");
+	ProfScope prof(PROF_ACT_BWD, 6.0 * n, s);
 	hipLaunchKernelGGL(gelu_bwd_kernel, dim3(ew_grid(n / 8)), dim3(256), 0, s, (const bf16_t*)dy, (const bf16_t*)x,
 	                   (bf16_t*)dx, n / 8);
 	ELF_CHECK_HIP(hipGetLastError());
@@ -398,12 +402,14 @@ int gelu_bwd(const void* dy, const void* x, void* dx, int64_t n, hipStream_t s) 
 }
 int swiglu_fwd(const void* gu, void* h, int64_t T, int F, hipStream_t s) {
 	ELF_REQUIRE(T > 0 && F > 0 && F % 8 == 0 && gu && h, "swiglu_fwd: F must be a positive multiple of 8");
+	ProfScope prof(PROF_ACT_FWD, 6.0 * T * F, s);
 	hipLaunchKernelGGL(swiglu_fwd_kernel, dim3(ew_grid(T * (F / 8))), dim3(256), 0, s, (const bf16_t*)gu, (bf16_t*)h, T, F);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
 }
 int swiglu_bwd(const void* dh, const void* gu, void* dgu, int64_t T, int F, hipStream_t s) {
 	ELF_REQUIRE(T > 0 && F > 0 && F % 8 == 0 && gu && dh && dgu, "swiglu_bwd: F must be a positive multiple of 8");
+	ProfScope prof(PROF_ACT_BWD, 10.0 * T * F, s);
 	hipLaunchKernelGGL(swiglu_bwd_kernel, dim3(ew_grid(T * (F / 8))), dim3(256), 0, s, (const bf16_t*)dh,
 	                   (const bf16_t*)gu, (bf16_t*)dgu, T, F);
 	ELF_CHECK_HIP(hipGetLastError());
@@ -462,6 +468,7 @@ int rope_apply(void* buf, const void* cs, int64_t T, int S, int ld, int n_heads,
 	ELF_REQUIRE(buf && cs && T > 0 && S > 0 && T % S == 0, "rope: T must be a multiple of S");
 	ELF_REQUIRE(D % 16 == 0 && ld % 8 == 0 && n_heads * D <= ld, "rope: bad head layout");
 	const int64_t n = T * n_heads * (D / 16);
+	ProfScope prof(PROF_ROPE, 4.0 * T * n_heads * D, s);
 	hipLaunchKernelGGL(rope_kernel, dim3(ew_grid(n)), dim3(256), 0, s, (bf16_t*)buf, (const float2*)cs, T, S, ld, n_heads,
 	                   D, backward ? -1.f : 1.f);
 	ELF_CHECK_HIP(hipGetLastError());
@@ -495,6 +502,7 @@ __global__ __launch_bounds__(256) void scale_grads_kernel(float* __restrict__ ac
 int scale_grads(void* acc_f32, void* out_bf16, int64_t n, float scale, hipStream_t s) {
 	ELF_REQUIRE(acc_f32 && n > 0, "scale_grads: empty");
 	ELF_REQUIRE(((uintptr_t)acc_f32 % 16) == 0 && (!out_bf16 || ((uintptr_t)out_bf16 % 8) == 0), "scale_grads: misaligned");
+	ProfScope prof(PROF_SCALE, (out_bf16 ? 10.0 : 8.0) * n, s);
 	hipLaunchKernelGGL(scale_grads_kernel, dim3(ew_grid(n / 4 + 1)), dim3(256), 0, s, (float*)acc_f32, (bf16_t*)out_bf16,
 	                   n / 4, n, scale);
 	ELF_CHECK_HIP(hipGetLastError());
@@ -513,6 +521,7 @@ __global__ __launch_bounds__(256) void add_kernel(const bf16_t* __restrict__ a, 
 }
 int add_bf16(const void* a, const void* b, void* out, int64_t n, hipStream_t s) {
 	ELF_REQUIRE(n > 0 && n % 8 == 0 && a && b && out, "add: n must be a positive multiple of 8");
+	ProfScope prof(PROF_ADD, 6.0 * n, s);
 	hipLaunchKernelGGL(add_kernel, dim3(ew_grid(n / 8)), dim3(256), 0, s, (const bf16_t*)a, (const bf16_t*)b, (bf16_t*)out, n / 8);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;

@@ -306,6 +306,7 @@ int gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda,
 	ELF_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)B % 16) == 0, "gemm: operands must be 16-byte aligned");
 	ELF_REQUIRE(lda >= (a_t ? M : K) && ldb >= (b_t ? N : K) && ldc >= N, "gemm: leading dimension too small");
 	ELF_REQUIRE(epi != EPI_BF16_RESID || (R != nullptr && ldr >= N), "gemm: residual epilogue needs R");
+	ProfScope prof(PROF_GEMM, 2.0 * M * N * K, stream);
 	GemmArgs g;
 	g.A = (const bf16_t*)A;
 	g.B = (const bf16_t*)B;

@@ -42,4 +42,21 @@ int attn_bwd(const void* q, const void* k, const void* v, const void* o, const v
              int64_t lddq, int64_t lddk, int64_t lddv, int B, int S, int Hq, int Hkv, int D, int causal, float scale,
              hipStream_t stream);
 
+// Optional live timing of kernel launches: when enabled, every launcher brackets its launches
+// with an event pair on the launch stream and books the algorithmic work of the call.
+enum ProfKind {
+	PROF_GEMM = 0, PROF_ATTN_FWD, PROF_ATTN_BWD, PROF_NORM_FWD, PROF_NORM_BWD, PROF_ACT_FWD, PROF_ACT_BWD, PROF_ROPE,
+	PROF_SCALE, PROF_ADD, PROF_COUNT
+};
+void prof_enable(int on);
+bool prof_on();
+struct ProfScope {
+	ProfScope(int kind, double work, hipStream_t stream);
+	~ProfScope();
+	int slot;
+	hipStream_t stream;
+};
+// Waits for the recorded events; totals since the last prof_enable(1). Returns the launch count.
+int prof_collect(int kind, double* total_ms, double* total_work);
+
 }  // namespace elf

@@ -195,6 +195,17 @@ int elf_pinned_pool_n_parents(elf_pinned_pool_t* p);
 int elf_pinned_pool_n_free(elf_pinned_pool_t* p, int parent);
 int elf_pinned_pool_free_segment(elf_pinned_pool_t* p, int parent, int i, int64_t* offset, int64_t* length);
 
+/* ---------------------------------------------------------------------------------------------
+ * Live kernel timing for measurements (no counterpart in the reference, whose per-op Timer wraps
+ * whole F/B/W passes, elf/utils.py:249-324).  While enabled, every kernel launcher brackets its
+ * launch with a HIP event pair on the launch stream.  kind: 0 GEMM (work = 2MNK flops),
+ * 1 attention fwd, 2 attention bwd (algorithmic flops), 3 norm fwd, 4 norm bwd, 5 activation fwd,
+ * 6 activation bwd, 7 RoPE, 8 grad scale, 9 add (work = algorithmic bytes).
+ * elf_prof_collect waits for the events and returns the number of launches of that kind since
+ * elf_prof_enable(1), with their summed duration (ms) and summed work. */
+void elf_prof_enable(int on);
+int elf_prof_collect(int kind, double* total_ms, double* total_work);
+
 #ifdef __cplusplus
 }
 #endif
