@@ -229,18 +229,33 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(const bf16_t* __restrict_
 	}
 }
 
-// main_grad[c] += sum_b part[b][which][c]
-__global__ void norm_bwd_finalize_kernel(const float* __restrict__ part, int nparts, int d, float* __restrict__ dgamma,
-                                         float* __restrict__ dbeta) {
-	const int c = blockIdx.x * blockDim.x + threadIdx.x;
-	if (c >= d) return;
+// main_grad[c] += sum_b part[b][which][c].  One workgroup owns 32 columns; its 8 row groups
+// stride over the partial rows and are folded through LDS.
+__global__ __launch_bounds__(256) void norm_bwd_finalize_kernel(const float* __restrict__ part, int nparts, int d,
+                                                                float* __restrict__ dgamma, float* __restrict__ dbeta) {
+	__shared__ float red[2][8][32];
+	const int cl = threadIdx.x & 31, rg = threadIdx.x >> 5;
+	const int c = blockIdx.x * 32 + cl;
 	float sg = 0.f, sb = 0.f;
-	for (int b = 0; b < nparts; b++) {
-		sg += part[(int64_t)b * 2 * d + c];
-		if (dbeta) sb += part[(int64_t)b * 2 * d + d + c];
+	if (c < d) {
+		for (int b = rg; b < nparts; b += 8) {
+			sg += part[(int64_t)b * 2 * d + c];
+			if (dbeta) sb += part[(int64_t)b * 2 * d + d + c];
+		}
 	}
-	dgamma[c] += sg;
-	if (dbeta) dbeta[c] += sb;
+	red[0][rg][cl] = sg;
+	red[1][rg][cl] = sb;
+	__syncthreads();
+	if (rg == 0 && c < d) {
+		float tg = 0.f, tb = 0.f;
+#pragma unroll
+		for (int r = 0; r < 8; r++) {
+			tg += red[0][r][cl];
+			tb += red[1][r][cl];
+		}
+		dgamma[c] += tg;
+		if (dbeta) dbeta[c] += tb;
+	}
 }
 
 static inline int norm_bwd_blocks(int T, int d) {
@@ -310,7 +325,7 @@ int norm_bwd(int kind, const void* dy, const void* x, const void* gamma, const v
 		rc = norm_bwd_dispatch<false>(dy, x, gamma, stats, dres, dx, workspace, T, d, s);
 	}
 	if (rc) return rc;
-	hipLaunchKernelGGL(norm_bwd_finalize_kernel, dim3((d + 255) / 256), dim3(256), 0, s, workspace,
+	hipLaunchKernelGGL(norm_bwd_finalize_kernel, dim3((d + 31) / 32), dim3(256), 0, s, workspace,
 	                   norm_bwd_blocks(T, d), d, dgamma, kind == NORM_LAYER ? dbeta : nullptr);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;

@@ -90,27 +90,32 @@ class SplitLinearFn(torch.autograd.Function):
 
 # --------------------------------------------------------------------------------------------
 # ops
+def _up(t):
+	"""Math runs in fp32 for bf16 / fp16 / fp32 inputs and stays in fp64 for fp64 inputs."""
+	return t if t.dtype == torch.float64 else t.float()
+
+
 def rms_norm(x, g, eps):
-	xf = x.float()
-	return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * g.float()).to(x.dtype)
+	xf = _up(x)
+	return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * _up(g)).to(x.dtype)
 
 
 def layer_norm(x, g, b, eps):
-	return F.layer_norm(x.float(), (x.shape[-1],), g.float(), b.float(), eps).to(x.dtype)
+	return F.layer_norm(_up(x), (x.shape[-1],), _up(g), _up(b), eps).to(x.dtype)
 
 
 def rope_tables(S, D, theta, device):
 	"""cos/sin [S, D/2] in fp32 from fp64 angles: a = pos * theta^(-2i/D)."""
 	inv = theta ** (-torch.arange(0, D // 2, dtype=torch.float64, device=device) / (D // 2))
 	ang = torch.arange(S, dtype=torch.float64, device=device)[:, None] * inv[None, :]
-	return ang.cos().float(), ang.sin().float()
+	return ang.cos().float(), ang.sin().float()  # the tables themselves are fp32, as in the HIP path
 
 
 def rope(x, cos, sin):
 	"""x: [B, S, H, D]; half-split rotation (out_lo = lo*cos - hi*sin, out_hi = hi*cos + lo*sin)."""
 	D = x.shape[-1]
-	lo, hi = x[..., : D // 2].float(), x[..., D // 2 :].float()
-	c, s = cos[None, :, None, :], sin[None, :, None, :]
+	lo, hi = _up(x[..., : D // 2]), _up(x[..., D // 2 :])
+	c, s = cos[None, :, None, :].to(lo.dtype), sin[None, :, None, :].to(lo.dtype)
 	return torch.cat([lo * c - hi * s, hi * c + lo * s], dim=-1).to(x.dtype)
 
 
@@ -124,11 +129,11 @@ def attention(q, k, v, causal, use_sdpa=False):
 		return o.transpose(1, 2)
 	kt = kt.repeat_interleave(G, dim=1)
 	vt = vt.repeat_interleave(G, dim=1)
-	s = (qt.float() @ kt.float().transpose(-1, -2)) / math.sqrt(D)
+	s = (_up(qt) @ _up(kt).transpose(-1, -2)) / math.sqrt(D)
 	if causal:
 		s = s.masked_fill(~torch.ones(S, S, dtype=torch.bool, device=q.device).tril(), float("-inf"))
 	p = torch.softmax(s, dim=-1)
-	return (p @ vt.float()).to(q.dtype).transpose(1, 2)
+	return (p @ _up(vt)).to(q.dtype).transpose(1, 2)
 
 
 # --------------------------------------------------------------------------------------------

@@ -1,0 +1,297 @@
+"""Host scheduling logic against (1) the vectors the reference's own unit tests hold
+(tests/unit/scheduling/test_schedulers.py:9-34 AFAB, :38-83 1F1B, :86-201 validity matrix,
+:205-220 inference, :224-265 add_comms; test_comm_scheduling.py:22-60 DirectedGraph),
+(2) op lists dumped from the reference's generators (tests/golden/schedule_vectors.json, made by
+tests/golden/make_schedule_vectors.py), (3) closed forms and invariants."""
+
+import json
+import os
+
+import pytest
+
+from elf_amd.benchmark_utils import get_checkpointed_scheduler, get_offloaded_scheduler
+from elf_amd.partitioners.utils import sequential_signatures
+from elf_amd.registry import COMM_SCHEDULERS, PARTITIONERS, SCHEDULERS, TRACERS, resolve
+from elf_amd.scheduling import (
+	DirectedGraph, Operation, OperationType as T, OpOptions, add_comms, check_schedule_validity, comm_types, compute_types,
+	schedule_to_graph, schedule_to_str,
+)
+from elf_amd.scheduling.ilp import RematScheduler
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "schedule_vectors.json")
+
+
+def _seq(ops):
+	return [(op.op, op.block_id, op.mb_id, op.rank) for op in ops]
+
+
+# ---------------------------------------------------------------- vectors held by the reference's tests
+def test_afab_reference_vector():
+	F, B, W, LF, LB = T.FORWARD, T.BACKWARD_INPUTS, T.BACKWARD_PARAMS, T.LOSS_FORWARD, T.LOSS_BACKWARD
+	want = [(F, 0, 0, 0), (F, 0, 1, 0), (B, 0, 0, 0), (W, 0, 0, 0), (B, 0, 1, 0), (W, 0, 1, 0),
+	        (F, 1, 0, 1), (LF, 1, 0, 1), (F, 1, 1, 1), (LF, 1, 1, 1), (LB, 1, 0, 1), (B, 1, 0, 1), (W, 1, 0, 1), (LB, 1, 1, 1), (B, 1, 1, 1), (W, 1, 1, 1)]
+	assert _seq(SCHEDULERS["afab"]([0, 1], 2)) == want
+	assert SCHEDULERS["gpipe"] is SCHEDULERS["afab"]
+
+
+def test_1f1b_reference_vector():
+	F, B, W, LF, LB = T.FORWARD, T.BACKWARD_INPUTS, T.BACKWARD_PARAMS, T.LOSS_FORWARD, T.LOSS_BACKWARD
+	s = SCHEDULERS["1f1b"]([0, 1], 4)
+	r0 = [(o.op, o.mb_id) for o in s if o.rank == 0]
+	assert r0 == [(F, 0), (F, 1), (B, 0), (W, 0), (F, 2), (B, 1), (W, 1), (F, 3), (B, 2), (W, 2), (B, 3), (W, 3)]
+	r1 = [(o.op, o.mb_id) for o in s if o.rank == 1]
+	assert r1 == [x for m in range(4) for x in [(F, m), (LF, m), (LB, m), (B, m), (W, m)]]
+	# the reference compares with Operation.__eq__, which ignores block_id
+	assert [o for o in s if o.rank == 0][0] == Operation(99, 0, F, 0)
+
+
+def _check_validity(schedule, placement, nmb):
+	n_stages = len(placement)
+	count = lambda kind: sum(op.op == kind for op in schedule)
+	for kind in (T.FORWARD, T.BACKWARD_INPUTS, T.BACKWARD_PARAMS, T.SEND_FORWARD, T.SEND_BACKWARD, T.RECV_FORWARD, T.RECV_BACKWARD):
+		assert count(kind) == n_stages * nmb
+	assert count(T.LOSS_FORWARD) == count(T.LOSS_BACKWARD) == nmb
+	for blk in range(n_stages):
+		for kind in (T.FORWARD, T.BACKWARD_INPUTS, T.BACKWARD_PARAMS):
+			assert sum(op.op == kind and op.block_id == blk for op in schedule) == nmb
+	for mb in range(nmb):
+		for blk in range(n_stages):
+			order = [T.FORWARD] + ([T.LOSS_FORWARD, T.LOSS_BACKWARD] if blk == n_stages - 1 else []) + [T.BACKWARD_INPUTS, T.BACKWARD_PARAMS]
+			seen = [op.op for op in schedule if op.block_id == blk and op.mb_id == mb and op.op in order]
+			assert seen == order
+	for blk in range(n_stages):
+		w_seen = 0
+		for op in schedule:
+			if op.block_id != blk:
+				continue
+			w_seen += op.op == T.BACKWARD_PARAMS
+			if op.op == T.ALL_REDUCE_PARAM_GRADS:
+				assert w_seen == nmb
+	assert count(T.ALL_REDUCE_PARAM_GRADS) == n_stages
+
+
+VALIDITY_MATRIX = {
+	"gpipe": ([[0, 1], [0, 1, 2, 3], [0, 1, 2, 3, 0, 1, 2, 3]], [2, 4, 8]),
+	"1f1b": ([[0, 1], [0, 1, 2, 3], [0, 1, 2, 3, 0, 1, 2, 3]], [2, 4, 8]),
+	"hanayo": ([[0, 1, 2, 3, 3, 2, 1, 0], [0, 1, 2, 3, 4, 5, 6, 7, 7, 6, 5, 4, 3, 2, 1, 0], [0, 1, 2, 3, 3, 2, 1, 0, 0, 1, 2, 3, 3, 2, 1, 0]], [2, 4, 8]),
+	"zbh1": ([[0, 1], [0, 1, 2, 3]], [2, 4, 8]),
+	"zbh2": ([[0, 1], [0, 1, 2, 3]], [2, 4, 8]),
+	"zbv": ([[0, 1, 2, 3, 3, 2, 1, 0]], [8]),
+}
+
+
+@pytest.mark.parametrize("name", sorted(VALIDITY_MATRIX))
+def test_validity_matrix(name):
+	placements, nmbs = VALIDITY_MATRIX[name]
+	for placement in placements:
+		for nmb in nmbs:
+			schedule = add_comms(SCHEDULERS[name](placement, nmb), sequential_signatures(placement))
+			_check_validity(schedule, placement, nmb)
+
+
+def test_inference_has_no_backward():
+	s = SCHEDULERS["inference"]([0, 1, 2, 3], 4)
+	assert all(op.op == T.FORWARD for op in s) and len(s) == 16
+
+
+def test_add_comms_counts():
+	F, B, W = T.FORWARD, T.BACKWARD_INPUTS, T.BACKWARD_PARAMS
+	s = [Operation(0, 0, F, 0), Operation(0, 1, F, 0), Operation(0, 0, B, 0), Operation(0, 0, W, 0), Operation(0, 1, B, 0), Operation(0, 1, W, 0)]
+	s = add_comms(s, sequential_signatures([0, 1]))
+	for kind in (T.SEND_FORWARD, T.RECV_FORWARD, T.SEND_BACKWARD, T.RECV_BACKWARD):
+		ops = [op for op in s if op.op == kind]
+		assert len(ops) == 2 and all(op.block_id == 0 and op.rank == 0 for op in ops)
+	assert sum(op.op == T.ALL_REDUCE_PARAM_GRADS for op in s) == 1
+	# ends of the chain talk to nobody
+	assert [op.options for op in s if op.op == T.RECV_FORWARD] == [{"src": None}] * 2
+	assert [op.options for op in s if op.op == T.SEND_FORWARD] == [{"dst": 1}] * 2
+
+
+def test_directed_graph_reference_cases():
+	g = DirectedGraph(4)
+	g.add_edge(0, 1)
+	g.add_edge(1, 2)
+	assert g.has_edge(0, 1) and not g.has_edge(1, 0)
+	assert g.get_successors(0) == [1] and g.get_predecessors(2) == [1]
+	assert g.get_out_degree(1) == 1 and g.get_in_degree(1) == 1
+	g.remove_edge(0, 1)
+	assert not g.has_edge(0, 1) and g.get_successors(0) == []
+	two = DirectedGraph(2)
+	two.add_edge(0, 1)
+	two.add_edge(1, 0)
+	assert not two.has_cycle() and two.has_bidirectional_edge(0, 1) and not two.has_unidirectional_edge(0, 1)
+	three = DirectedGraph(3)
+	for a, b in ((0, 1), (1, 2), (2, 0)):
+		three.add_edge(a, b)
+	assert three.has_cycle()
+	with pytest.raises(ValueError):
+		DirectedGraph(0)
+	with pytest.raises(ValueError):
+		three.add_edge(1, 1)
+	with pytest.raises(ValueError):
+		three.add_edge(0, 3)
+
+
+# ---------------------------------------------------------------- golden op lists dumped from the reference
+def _decode(rec):
+	return (rec[0], rec[1], rec[2], rec[3], rec[4] if len(rec) > 4 else {})
+
+
+def _encode(op):
+	opts = {}
+	for k, v in op.options.items():
+		opts[str(k)] = ("fn:" + ",".join(n for n in ("", "x") if v(n, None))) if callable(v) else v
+	return (op.op.value, op.block_id, op.mb_id, op.rank, opts)
+
+
+def _golden_cases():
+	with open(GOLDEN) as f:
+		return json.load(f)
+
+
+def _produce(case):
+	name = case["name"]
+	placement, nmb = case["placement"], case["nmb"]
+	kind = name.split(":")[0]
+	if kind == "gen":
+		return SCHEDULERS[case["scheduler"]](placement, nmb)
+	if kind == "comm":
+		s = add_comms(SCHEDULERS[case["scheduler"]](placement, nmb), sequential_signatures(placement))
+		return COMM_SCHEDULERS[case["comm"]](s)
+	if kind in ("remat", "remat+comm"):
+		s = RematScheduler(SCHEDULERS[case["scheduler"]], case["solution"])(placement, nmb)
+		return s if kind == "remat" else COMM_SCHEDULERS["pipelined"](add_comms(s, sequential_signatures(placement)))
+	if kind in ("offload", "offload+comm"):
+		s = get_offloaded_scheduler(case["scheduler"], case["ratio"], case["prefetching_time"])(placement, nmb)
+		return s if kind == "offload" else COMM_SCHEDULERS["pipelined"](add_comms(s, sequential_signatures(placement)))
+	if kind == "ckpt":
+		return get_checkpointed_scheduler(case["scheduler"], case["type"])(placement, nmb)
+	raise AssertionError(name)
+
+
+@pytest.mark.parametrize("idx", range(32))
+def test_golden_op_lists_bit_exact(idx):
+	cases = _golden_cases()
+	assert len(cases) == 32
+	case = cases[idx]
+	got = [_encode(op) for op in _produce(case)]
+	want = [_decode(r) for r in case["ops"]]
+	assert len(got) == len(want), case["name"]
+	for i, (g, w) in enumerate(zip(got, want)):
+		assert g == w, f"{case['name']} {case.get('placement')} nmb={case.get('nmb')}: op {i}: {g} != {w}"
+
+
+# ---------------------------------------------------------------- closed forms and invariants
+@pytest.mark.parametrize("P,n", [(2, 4), (4, 8), (4, 3), (4, 16), (8, 8), (3, 1)])
+def test_1f1b_closed_form(P, n):
+	"""Rank r of P: min(n, P - r) forwards, then (B W F) while forwards remain, then (B W)."""
+	s = SCHEDULERS["1f1b"](list(range(P)), n)
+	for r in range(P):
+		got = [(o.op, o.mb_id) for o in s if o.rank == r and o.op in compute_types]
+		w = min(n, P - r)
+		want = [(T.FORWARD, m) for m in range(w)]
+		for i in range(n):
+			want += [(T.BACKWARD_INPUTS, i), (T.BACKWARD_PARAMS, i)]
+			if w + i < n:
+				want.append((T.FORWARD, w + i))
+		assert got == want
+
+
+def test_zbh1_block1_stream_of_the_benchmark():
+	"""P = 4, n = 16, block 1: F0 F1 F2 B0 F3 B1 | (W_i F_{i+4} B_{i+2}) ... | W14 | W15: W lags B by 2."""
+	s = [o for o in SCHEDULERS["zbh1"]([0, 1, 2, 3], 16) if o.block_id == 1]
+	letters = {T.FORWARD: "F", T.BACKWARD_INPUTS: "B", T.BACKWARD_PARAMS: "W"}
+	got = " ".join(f"{letters[o.op]}{o.mb_id}" for o in s)
+	want = ["F0", "F1", "F2", "B0", "F3", "B1"]
+	for i in range(16):
+		want.append(f"W{i}")
+		if i + 4 < 16:
+			want.append(f"F{i + 4}")
+		if i + 2 < 16:
+			want.append(f"B{i + 2}")
+	assert got == " ".join(want)
+
+
+@pytest.mark.parametrize("comm", ["pipelined", "simulation", "topo"])
+@pytest.mark.parametrize("sched,placement,nmb", [("1f1b", [0, 1, 2, 3], 8), ("zbh1", [0, 1, 2, 3], 6), ("zbh2", [0, 1, 2], 5), ("afab", [0, 1], 3), ("hanayo", [0, 1, 1, 0], 4)])
+def test_comm_schedulers_keep_compute_order_and_dependencies(comm, sched, placement, nmb):
+	base = add_comms(SCHEDULERS[sched](placement, nmb), sequential_signatures(placement))
+	out = COMM_SCHEDULERS[comm](list(base))
+	assert sorted(map(str, out)) == sorted(map(str, base)), "same multiset of ops"
+	for rank in set(placement):
+		keep = lambda ops: [(o.op, o.block_id, o.mb_id) for o in ops if o.rank == rank and o.op in compute_types]
+		assert keep(out) == keep(base), "compute order per rank is untouched"
+	pos = {id(op): i for i, op in enumerate(out)}
+	g = schedule_to_graph(base)
+	for i in range(len(base)):
+		for j in g.get_successors(i):
+			if g.has_unidirectional_edge(i, j):
+				assert pos[id(base[j])] < pos[id(base[i])], f"{base[i]} must come after {base[j]}"
+	check_schedule_validity(out)
+
+
+def test_operation_and_options_semantics():
+	a = Operation(0, 1, T.FORWARD, 2, **{OpOptions.SAVE: True})
+	assert a == Operation(5, 1, T.FORWARD, 2, save=True) and hash(a) != hash(Operation(5, 1, T.FORWARD, 2))
+	assert a != Operation(0, 1, T.FORWARD, 2)
+	assert str(a) == "[Block 0, mb 1]:forward({<OpOptions.SAVE: 'save'>: True})"
+	assert str(Operation(3, None, T.ALL_REDUCE_PARAM_GRADS, 1)) == "[Block 3, mb None]:all_reduce_param_grads({})"
+	assert [str(o) for o in OpOptions] == ["remat_strategy", "recompute_activations", "recompute_gradients", "activation_offload", "save", "offload_dw"]
+	assert a.options.get("save") is True and {"save": 1}[OpOptions.SAVE] == 1
+	assert (lambda **kw: kw)(**a.options) == {"save": True}
+	assert comm_types == {T.RECV_FORWARD, T.RECV_BACKWARD, T.SEND_FORWARD, T.SEND_BACKWARD}
+	assert T.LOSS_FORWARD not in compute_types and len(compute_types) == 5 and len(T) == 13
+
+
+def test_schedule_to_str():
+	s = add_comms(SCHEDULERS["1f1b"]([0, 1], 2), sequential_signatures([0, 1]))
+	assert schedule_to_str(s).splitlines() == ["Rank 0: f0-0 f0-1 b0-0 w0-0 b0-1 w0-1 (AR)0-", "Rank 1: f1-0 b1-0 w1-0 f1-1 b1-1 w1-1 (AR)1-"]
+	assert "rf0-0(None)" in schedule_to_str(s, print_comms=True) and "sf0-0(1)" in schedule_to_str(s, print_comms=True)
+	ck = get_checkpointed_scheduler("1f1b", "full")([0, 1], 1)
+	assert schedule_to_str(ck).splitlines()[0].startswith("Rank 0: F0-0")
+
+
+def test_registries():
+	assert SCHEDULERS.available() == ["1f1b", "afab", "auto", "fixed", "full_remat", "hanayo", "inference", "zbh1", "zbh2", "zbv"]
+	assert set(SCHEDULERS) >= {"gpipe", "megatron"} and SCHEDULERS["megatron"] is SCHEDULERS["1f1b"]
+	assert COMM_SCHEDULERS.available() == ["pipelined", "simulation", "topo"]
+	assert sorted(PARTITIONERS) == ["constrained", "dagP", "metis", "naive"] and sorted(TRACERS) == ["default", "export", "fx", "fx_safe"]
+	assert SCHEDULERS.get_key(SCHEDULERS["gpipe"]) == "afab"
+	assert resolve("zbh1", SCHEDULERS) is SCHEDULERS["zbh1"] and resolve(len, SCHEDULERS) is len
+	with pytest.raises(ValueError):
+		resolve("nope", SCHEDULERS)
+	with pytest.raises(KeyError):
+		SCHEDULERS["nope"]
+	with pytest.raises(KeyError):
+		SCHEDULERS.register("afab", len)
+	assert SCHEDULERS["auto"]([0, 1], 2) is None
+	with pytest.raises(NotImplementedError):
+		PARTITIONERS["naive"](None, None, None, 2)
+
+
+def test_fixed_schedule_and_validity_errors():
+	fixed = SCHEDULERS["fixed"]({"order": [("f", 0, 0), ("f", "1", "0"), ("b", 1, 0), ("w", 1, 0), ("b", 0, 0), ("w", 0, 0)]})
+	s = fixed([0, 1], 1)
+	assert [o.op for o in s] == [T.FORWARD, T.FORWARD, T.LOSS_FORWARD, T.LOSS_BACKWARD, T.BACKWARD_INPUTS, T.BACKWARD_PARAMS, T.BACKWARD_INPUTS, T.BACKWARD_PARAMS]
+	check_schedule_validity(s)
+	with pytest.raises(AssertionError):
+		check_schedule_validity([Operation(0, 0, T.BACKWARD_INPUTS, 0), Operation(0, 0, T.FORWARD, 0), Operation(0, 0, T.BACKWARD_PARAMS, 0)])
+	with pytest.raises(AssertionError):
+		check_schedule_validity([Operation(0, 0, T.FORWARD, 0), Operation(0, 0, T.BACKWARD_INPUTS, 0)])
+	with pytest.raises(ZeroDivisionError):
+		SCHEDULERS["1f1b"]([0], 2)  # a single device is not a pipeline (n_devices // 2 == 0)
+
+
+def test_offload_wrapper_hand_derived_case():
+	"""P = 4, n = 8, rank 1, ratio 1, prefetching_time 1: every F is marked; the prefetch of mb m sits
+	right before F(m+2) for m <= 5 and right before B(m-1) for m = 6, 7."""
+	s = [o for o in get_offloaded_scheduler("1f1b", 1, 1)([0, 1, 2, 3], 8) if o.rank == 1]
+	for m in range(8):
+		i = next(k for k, o in enumerate(s) if o.op == T.PREFETCH_ACTIVATIONS and o.mb_id == m)
+		nxt = s[i + 1]
+		assert (nxt.op, nxt.mb_id) == ((T.FORWARD, m + 2) if m <= 5 else (T.BACKWARD_INPUTS, m - 1))
+	assert all(o.options.get(OpOptions.ACTIVATION_OFFLOAD) for o in s if o.op in (T.FORWARD, T.BACKWARD_INPUTS))
+	# on the last stage B(m) directly follows F(m): no room to prefetch, offload is switched off
+	last = [o for o in get_offloaded_scheduler("1f1b", 1, 1)([0, 1, 2, 3], 8) if o.rank == 3]
+	assert not any(o.op == T.PREFETCH_ACTIVATIONS for o in last)
+	assert not any(o.options.get(OpOptions.ACTIVATION_OFFLOAD) for o in last)
