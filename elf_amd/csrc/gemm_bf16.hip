@@ -101,9 +101,11 @@ __global__ __launch_bounds__(WR* WC * 64) void gemm_kernel(GemmArgs g) {
 	constexpr int B_ELEMS = TileShape<BN, BT>::ELEMS;
 
 	extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-	bf16_t* smem = reinterpret_cast<bf16_t*>(smem_raw);
-	bf16_t* sA[2] = {smem, smem + A_ELEMS + B_ELEMS};
-	bf16_t* sB[2] = {smem + A_ELEMS, smem + 2 * A_ELEMS + B_ELEMS};
+	// Buffers are addressed as smem + integer offset (never through an array of pointers) so that
+	// every access stays a DS instruction; a generic pointer would turn them into FLAT accesses
+	// that also wait on the global-load counter.
+	bf16_t* const smem = reinterpret_cast<bf16_t*>(smem_raw);
+	constexpr int STAGE = A_ELEMS + B_ELEMS;
 
 	const int tid = threadIdx.x;
 	const int lane = tid & 63;
@@ -154,8 +156,8 @@ __global__ __launch_bounds__(WR* WC * 64) void gemm_kernel(GemmArgs g) {
 
 	la.load(Ap, g.lda, tid);
 	lb.load(Bp, g.ldb, tid);
-	la.store(sA[0], tid);
-	lb.store(sB[0], tid);
+	la.store(smem, tid);
+	lb.store(smem + A_ELEMS, tid);
 	__syncthreads();
 
 	for (int kt = kt_begin; kt < kt_end; kt++) {
@@ -167,8 +169,8 @@ __global__ __launch_bounds__(WR* WC * 64) void gemm_kernel(GemmArgs g) {
 			la.load(Ap, g.lda, tid);
 			lb.load(Bp, g.ldb, tid);
 		}
-		const bf16_t* a_s = sA[cur];
-		const bf16_t* b_s = sB[cur];
+		const bf16_t* a_s = smem + cur * STAGE;
+		const bf16_t* b_s = a_s + A_ELEMS;
 #pragma unroll
 		for (int ks = 0; ks < BK / 16; ks++) {
 			bf16x8 af[TM], bfr[TN];
@@ -183,8 +185,8 @@ __global__ __launch_bounds__(WR* WC * 64) void gemm_kernel(GemmArgs g) {
 					acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
 		}
 		if (more) {
-			la.store(sA[cur ^ 1], tid);
-			lb.store(sB[cur ^ 1], tid);
+			la.store(smem + (cur ^ 1) * STAGE, tid);
+			lb.store(smem + (cur ^ 1) * STAGE + A_ELEMS, tid);
 		}
 		__syncthreads();
 	}
