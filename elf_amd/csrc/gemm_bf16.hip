@@ -323,6 +323,14 @@ int gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda,
 	g.K = K;
 	g.tiles_m = g.tiles_n = 0;
 	g.k_splits = k_splits;
+	if (tile_cfg == 6) {
+		if (epi == EPI_F32_ACC && k_splits <= 0) {
+			const int64_t tiles = (int64_t)(M / 256) * (N / 256);
+			k_splits = 1;
+			while (tiles * k_splits < 256 && (K / 32) / (k_splits * 2) >= 16 && k_splits < 16) k_splits *= 2;
+		}
+		return gemm_bf16_dma(a_t, b_t, M, N, K, A, lda, B, ldb, C, ldc, epi, R, ldr, k_splits, stream);
+	}
 	if (!a_t && !b_t) return launch_epi<false, false>(g, epi, tile_cfg, stream);
 	if (!a_t && b_t) return launch_epi<false, true>(g, epi, tile_cfg, stream);
 	if (a_t && b_t) return launch_epi<true, true>(g, epi, tile_cfg, stream);

@@ -1,0 +1,271 @@
+// 256x256 bf16 MFMA GEMM tile kernel with direct global->LDS loads, for gfx950.
+//
+// Same contraction and layouts as gemm_bf16.hip (C (+)= sum_k A(m,k) B(n,k); "R" operands are
+// k-contiguous, "T" operands reduction-major), different data movement:
+//   * global_load_lds_dwordx4 moves 16 B per lane straight into LDS (no VGPR staging, no
+//     ds_write), so a 4-stage ring of 32-wide K slices (4 x 32 KiB) keeps three slices in
+//     flight while the fourth is being multiplied;
+//   * a wave instruction fills 1 KiB of LDS contiguously, so tiles cannot be padded; bank
+//     conflicts are avoided by an XOR swizzle of the 16-byte chunk index, applied on the global
+//     side when choosing which chunk a lane fetches and undone when fragments are read;
+//   * 4 waves, one per SIMD, each owning a 128x128 sub-tile (16 accumulator tiles): 8 fragment
+//     reads feed 16 MFMAs, half the LDS traffic per FLOP of the 128x64 arrangement.
+// The DMA loads are issued through inline assembly: the compiler cannot see that they write
+// LDS, which is what allows partial vmcnt waits (its own tracking would force vmcnt(0) before
+// every LDS read).  Ordering is explicit: s_waitcnt vmcnt(n) for this wave's slice, then a
+// workgroup barrier for the other waves' slices and for the reuse of the oldest stage.
+#include "common.h"
+#include "kernels.h"
+
+namespace elf {
+
+namespace dma {
+
+constexpr int BM = 256, BN = 256, BKS = 32, NST = 4, PD = NST - 1;
+constexpr int OPERAND_BYTES = 256 * BKS * 2;  // 16 KiB
+constexpr int STAGE_BYTES = 2 * OPERAND_BYTES;
+constexpr int LOADS_PER_STAGE = 8;  // wave instructions per wave per stage (4 per operand)
+
+struct Args {
+	const bf16_t* A;
+	const bf16_t* B;
+	void* C;
+	const bf16_t* R;
+	int64_t lda, ldb, ldc, ldr;
+	int M, N, K;
+	int tiles_m, tiles_n, k_splits;
+};
+
+// s_waitcnt with only vmcnt set (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt_hi[15:14])
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+	__builtin_amdgcn_s_waitcnt((N & 0xF) | (0x7 << 4) | (0xF << 8) | ((N >> 4) << 14));
+}
+
+// 16 bytes per lane from (base + byte_off) to LDS at lds_byte_addr + lane * 16 (base and LDS
+// address are wave-uniform and travel in scalar registers).
+__device__ __forceinline__ void dma16(const bf16_t* base, uint32_t byte_off, uint32_t lds_byte_addr) {
+	asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_byte_addr), "v"(byte_off), "s"(base) : "memory", "m0");
+}
+
+// Byte offsets (relative to the tile origin of the current K slice) of the four 16-byte
+// chunks this lane fetches for one operand (< 2^31: 256 rows of at most 64 K elements).
+template <bool T>
+__device__ __forceinline__ void lane_offsets(int wave, int lane, int64_t ld, uint32_t (&off)[4]) {
+#pragma unroll
+	for (int i = 0; i < 4; i++) {
+		const int q = wave * 4 + i;  // which 1 KiB piece of the operand's 16 KiB
+		if constexpr (!T) {
+			const int row = q * 16 + (lane >> 2), slot = lane & 3;
+			off[i] = (uint32_t)((row * ld + ((slot ^ ((row >> 2) & 3)) << 3)) * 2);
+		} else {
+			const int krow = q * 2 + (lane >> 5), slot = lane & 31;
+			off[i] = (uint32_t)((krow * ld + ((slot ^ ((krow & 7) << 1)) << 3)) * 2);
+		}
+	}
+}
+
+// MFMA operand fragment of the 32-row slab at `row0` for k16-step ks of the current stage.
+template <bool T>
+__device__ __forceinline__ bf16x8 frag(const unsigned char* base, int row0, int ks, int lane) {
+	if constexpr (!T) {
+		const int r = row0 + (lane & 31);
+		const int c = (2 * ks + (lane >> 5)) ^ ((r >> 2) & 3);
+		return *reinterpret_cast<const bf16x8*>(base + r * 64 + c * 16);
+	} else {
+		const int j = lane & 15;
+		const int m = row0 + 16 * ((lane & 31) >> 4) + 4 * (j & 3);
+		const int kk = ks * 16 + 8 * (lane >> 5) + (j >> 2);
+		// rows kk and kk+4 share (kk & 3) but not (kk & 7): compute both swizzles
+		const int c0 = (m >> 3) ^ ((kk & 7) << 1);
+		const int c1 = (m >> 3) ^ (((kk + 4) & 7) << 1);
+		const unsigned char* p0 = base + kk * 512 + c0 * 16 + (j & 1) * 8;
+		const unsigned char* p1 = base + (kk + 4) * 512 + c1 * 16 + (j & 1) * 8;
+		s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 ELF_LDS*)(p0));
+		s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 ELF_LDS*)(p1));
+		return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+	}
+}
+
+template <bool AT, bool BT, int EPI>
+__global__ __launch_bounds__(256) void gemm_dma_kernel(Args g) {
+	extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+	const int tid = threadIdx.x;
+	const int lane = tid & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+	const int wr = wave >> 1, wc = wave & 1;
+
+	// tile assignment (XCD-contiguous, grouped by 8 tile rows), optional K split
+	int pid = blockIdx.x;
+	const int ntiles = g.tiles_m * g.tiles_n;
+	int ksplit = 0;
+	if (g.k_splits > 1) {
+		ksplit = pid / ntiles;
+		pid = pid % ntiles;
+	}
+	if ((ntiles & 7) == 0) pid = (pid & 7) * (ntiles >> 3) + (pid >> 3);
+	constexpr int GROUP_M = 8;
+	const int per_group = GROUP_M * g.tiles_n;
+	const int first_m = (pid / per_group) * GROUP_M;
+	const int gsz = min(g.tiles_m - first_m, GROUP_M);
+	const int m0 = (first_m + (pid % per_group) % gsz) * BM;
+	const int n0 = ((pid % per_group) / gsz) * BN;
+
+	const int nk_total = g.K / BKS;
+	const int nk_per = (nk_total + g.k_splits - 1) / g.k_splits;
+	const int kt0 = ksplit * nk_per;
+	const int nk = min(nk_total, kt0 + nk_per) - kt0;
+	if (nk <= 0) return;
+
+	const bf16_t* Ap = AT ? g.A + (int64_t)kt0 * BKS * g.lda + m0 : g.A + (int64_t)m0 * g.lda + (int64_t)kt0 * BKS;
+	const bf16_t* Bp = BT ? g.B + (int64_t)kt0 * BKS * g.ldb + n0 : g.B + (int64_t)n0 * g.ldb + (int64_t)kt0 * BKS;
+	const int64_t a_step = AT ? (int64_t)BKS * g.lda : BKS;
+	const int64_t b_step = BT ? (int64_t)BKS * g.ldb : BKS;
+	uint32_t aoff[4], boff[4];
+	lane_offsets<AT>(wave, lane, g.lda, aoff);
+	lane_offsets<BT>(wave, lane, g.ldb, boff);
+
+	const uint32_t lds0 = (uint32_t)(uintptr_t)(unsigned char ELF_LDS*)smem + wave * 4096;  // this wave's first 1 KiB piece
+
+	auto issue = [&](int step) {
+		const uint32_t st = lds0 + (uint32_t)(step % NST) * STAGE_BYTES;
+		const bf16_t* a = Ap + (int64_t)step * a_step;
+		const bf16_t* b = Bp + (int64_t)step * b_step;
+#pragma unroll
+		for (int i = 0; i < 4; i++) dma16(a, aoff[i], __builtin_amdgcn_readfirstlane(st + i * 1024));
+#pragma unroll
+		for (int i = 0; i < 4; i++) dma16(b, boff[i], __builtin_amdgcn_readfirstlane(st + OPERAND_BYTES + i * 1024));
+	};
+
+	f32x16 acc[4][4];
+#pragma unroll
+	for (int i = 0; i < 4; i++)
+#pragma unroll
+		for (int j = 0; j < 4; j++)
+#pragma unroll
+			for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+#pragma unroll
+	for (int s = 0; s < PD; s++)
+		if (s < nk) issue(s);
+
+	for (int kt = 0; kt < nk; kt++) {
+		// slice kt of this wave has landed once at most the younger slices are outstanding
+		if (kt + PD - 1 < nk) wait_vmcnt<LOADS_PER_STAGE*(PD - 1)>();
+		else wait_vmcnt<0>();
+		__syncthreads();  // everyone's slice kt is in LDS; everyone is done reading slice kt-1
+		if (kt + PD < nk) issue(kt + PD);
+		const unsigned char* sa = smem + (kt % NST) * STAGE_BYTES;
+		const unsigned char* sb = sa + OPERAND_BYTES;
+#pragma unroll
+		for (int ks = 0; ks < BKS / 16; ks++) {
+			bf16x8 af[4], bfr[4];
+#pragma unroll
+			for (int i = 0; i < 4; i++) af[i] = frag<AT>(sa, wr * 128 + i * 32, ks, lane);
+#pragma unroll
+			for (int j = 0; j < 4; j++) bfr[j] = frag<BT>(sb, wc * 128 + j * 32, ks, lane);
+#pragma unroll
+			for (int i = 0; i < 4; i++)
+#pragma unroll
+				for (int j = 0; j < 4; j++)
+					acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+		}
+	}
+
+	// Epilogue through LDS (free once every wave has left the main loop).  Register r of a 32x32
+	// accumulator tile holds row (r/4)*8 + (lane/32)*4 + r%4, column lane%32; each wave parks one
+	// 32 x 128 fp32 strip at a time in its own LDS region (row pitch 136 floats: the two half-waves
+	// land on disjoint banks) and reads it back row-wise, so that global accesses are 16 bytes per
+	// lane over 256..512 contiguous bytes per row and accumulators leave the AGPRs only via ds_write.
+	__syncthreads();
+	constexpr int PITCH = 136;
+	float* ws = reinterpret_cast<float*>(smem) + wave * (32 * PITCH);
+	const int col_l = lane & 31;
+	const int row_l = (lane >> 5) * 4;
+#pragma unroll
+	for (int i = 0; i < 4; i++) {
+#pragma unroll
+		for (int j = 0; j < 4; j++)
+#pragma unroll
+			for (int r = 0; r < 16; r++) ws[((r >> 2) * 8 + row_l + (r & 3)) * PITCH + j * 32 + col_l] = acc[i][j][r];
+		const int grow0 = m0 + wr * 128 + i * 32;
+		const int gcol0 = n0 + wc * 128;
+		if constexpr (EPI == EPI_BF16 || EPI == EPI_BF16_RESID) {
+#pragma unroll
+			for (int it = 0; it < 8; it++) {
+				const int row = it * 4 + (lane >> 4), c8 = (lane & 15) * 8;
+				const f32x4 lo = *reinterpret_cast<const f32x4*>(ws + row * PITCH + c8);
+				const f32x4 hi = *reinterpret_cast<const f32x4*>(ws + row * PITCH + c8 + 4);
+				float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+				if constexpr (EPI == EPI_BF16_RESID) {
+					const bf16x8 rs = *reinterpret_cast<const bf16x8*>(g.R + (int64_t)(grow0 + row) * g.ldr + gcol0 + c8);
+#pragma unroll
+					for (int t = 0; t < 8; t++) v[t] += (float)rs[t];
+				}
+				bf16x8 o;
+#pragma unroll
+				for (int t = 0; t < 8; t++) o[t] = (bf16_t)v[t];
+				*reinterpret_cast<bf16x8*>(reinterpret_cast<bf16_t*>(g.C) + (int64_t)(grow0 + row) * g.ldc + gcol0 + c8) = o;
+			}
+		} else {
+#pragma unroll
+			for (int it = 0; it < 16; it++) {
+				const int row = it * 2 + (lane >> 5), c4 = (lane & 31) * 4;
+				f32x4 v = *reinterpret_cast<const f32x4*>(ws + row * PITCH + c4);
+				float* c = reinterpret_cast<float*>(g.C) + (int64_t)(grow0 + row) * g.ldc + gcol0 + c4;
+				if constexpr (EPI == EPI_F32_ACC) {
+					if (g.k_splits > 1) {
+#pragma unroll
+						for (int t = 0; t < 4; t++) unsafeAtomicAdd(c + t, v[t]);
+						continue;
+					}
+					v += *reinterpret_cast<const f32x4*>(c);
+				}
+				*reinterpret_cast<f32x4*>(c) = v;
+			}
+		}
+	}
+}
+
+template <bool AT, bool BT, int EPI>
+static int launch(const Args& a, hipStream_t stream) {
+	constexpr int smem = NST * STAGE_BYTES;
+	auto kern = gemm_dma_kernel<AT, BT, EPI>;
+	static bool attr_set = false;
+	if (!attr_set) {
+		ELF_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+		attr_set = true;
+	}
+	hipLaunchKernelGGL(kern, dim3(a.tiles_m * a.tiles_n * a.k_splits), dim3(256), smem, stream, a);
+	ELF_CHECK_HIP(hipGetLastError());
+	return 0;
+}
+
+template <bool AT, bool BT>
+static int launch_epi(const Args& a, int epi, hipStream_t stream) {
+	switch (epi) {
+		case EPI_BF16: return launch<AT, BT, EPI_BF16>(a, stream);
+		case EPI_BF16_RESID: return launch<AT, BT, EPI_BF16_RESID>(a, stream);
+		case EPI_F32_ACC: return launch<AT, BT, EPI_F32_ACC>(a, stream);
+		case EPI_F32_STORE: return launch<AT, BT, EPI_F32_STORE>(a, stream);
+	}
+	set_error("gemm: unknown epilogue %d", epi);
+	return -1;
+}
+
+}  // namespace dma
+
+// Arguments are validated by gemm_bf16() before it dispatches here.
+int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda, const void* B, int64_t ldb, void* C,
+                  int64_t ldc, int epi, const void* R, int64_t ldr, int k_splits, hipStream_t stream) {
+	ELF_REQUIRE(M % dma::BM == 0 && N % dma::BN == 0 && K % dma::BKS == 0, "gemm (dma tile): M, N multiples of 256 and K of 32 required");
+	dma::Args a{(const bf16_t*)A, (const bf16_t*)B, C, (const bf16_t*)R, lda, ldb, ldc, ldr, M, N, K, M / dma::BM, N / dma::BN, k_splits < 1 ? 1 : k_splits};
+	if (epi != EPI_F32_ACC) a.k_splits = 1;
+	if (!a_t && !b_t) return dma::launch_epi<false, false>(a, epi, stream);
+	if (!a_t && b_t) return dma::launch_epi<false, true>(a, epi, stream);
+	if (a_t && b_t) return dma::launch_epi<true, true>(a, epi, stream);
+	set_error("gemm: layout A=T,B=R is not used by any stage contraction");
+	return -1;
+}
+
+}  // namespace elf
