@@ -3,8 +3,8 @@
 // Same contraction and layouts as gemm_bf16.hip (C (+)= sum_k A(m,k) B(n,k); "R" operands are
 // k-contiguous, "T" operands reduction-major), different data movement:
 //   * global_load_lds_dwordx4 moves 16 B per lane straight into LDS (no VGPR staging, no
-//     ds_write), so a 4-stage ring of 32-wide K slices (4 x 32 KiB) keeps three slices in
-//     flight while the fourth is being multiplied;
+//     ds_write); two 64-wide K slices (2 x 64 KiB) alternate, the next slice being fetched while
+//     the current one is multiplied.  64 bf16 = one full 128-byte cache line per operand row;
 //   * a wave instruction fills 1 KiB of LDS contiguously, so tiles cannot be padded; bank
 //     conflicts are avoided by an XOR swizzle of the 16-byte chunk index, applied on the global
 //     side when choosing which chunk a lane fetches and undone when fragments are read;
@@ -21,10 +21,11 @@ namespace elf {
 
 namespace dma {
 
-constexpr int BM = 256, BN = 256, BKS = 32, NST = 4, PD = NST - 1;
-constexpr int OPERAND_BYTES = 256 * BKS * 2;  // 16 KiB
+constexpr int BM = 256, BN = 256, BKS = 64, NST = 2;
+constexpr int OPERAND_BYTES = 256 * BKS * 2;  // 32 KiB
 constexpr int STAGE_BYTES = 2 * OPERAND_BYTES;
-constexpr int LOADS_PER_STAGE = 8;  // wave instructions per wave per stage (4 per operand)
+constexpr int LOADS_PER_OPERAND = OPERAND_BYTES / 1024 / 4;  // wave instructions per wave per stage and operand
+constexpr int LOADS_PER_STAGE = 2 * LOADS_PER_OPERAND;
 
 struct Args {
 	const bf16_t* A;
@@ -48,16 +49,19 @@ __device__ __forceinline__ void dma16(const bf16_t* base, uint32_t byte_off, uin
 	asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_byte_addr), "v"(byte_off), "s"(base) : "memory", "m0");
 }
 
-// Byte offsets (relative to the tile origin of the current K slice) of the four 16-byte
-// chunks this lane fetches for one operand (< 2^31: 256 rows of at most 64 K elements).
+// Byte offsets (relative to the tile origin of the current K slice) of the 16-byte chunks this
+// lane fetches for one operand (< 2^31: 256 rows of at most 64 K elements).  "R" tiles are
+// [256 rows][128 B], "T" tiles [64 k][512 B]; LDS chunk slot s of a row holds global chunk
+// s ^ f(row) with f chosen so that 16 consecutive lanes of a fragment read hit 16 distinct
+// 16-byte bank groups.
 template <bool T>
-__device__ __forceinline__ void lane_offsets(int wave, int lane, int64_t ld, uint32_t (&off)[4]) {
+__device__ __forceinline__ void lane_offsets(int wave, int lane, int64_t ld, uint32_t (&off)[LOADS_PER_OPERAND]) {
 #pragma unroll
-	for (int i = 0; i < 4; i++) {
-		const int q = wave * 4 + i;  // which 1 KiB piece of the operand's 16 KiB
+	for (int i = 0; i < LOADS_PER_OPERAND; i++) {
+		const int q = wave * LOADS_PER_OPERAND + i;  // which 1 KiB piece of the operand tile
 		if constexpr (!T) {
-			const int row = q * 16 + (lane >> 2), slot = lane & 3;
-			off[i] = (uint32_t)((row * ld + ((slot ^ ((row >> 2) & 3)) << 3)) * 2);
+			const int row = q * 8 + (lane >> 3), slot = lane & 7;
+			off[i] = (uint32_t)((row * ld + ((slot ^ ((row >> 1) & 7)) << 3)) * 2);
 		} else {
 			const int krow = q * 2 + (lane >> 5), slot = lane & 31;
 			off[i] = (uint32_t)((krow * ld + ((slot ^ ((krow & 7) << 1)) << 3)) * 2);
@@ -70,8 +74,8 @@ template <bool T>
 __device__ __forceinline__ bf16x8 frag(const unsigned char* base, int row0, int ks, int lane) {
 	if constexpr (!T) {
 		const int r = row0 + (lane & 31);
-		const int c = (2 * ks + (lane >> 5)) ^ ((r >> 2) & 3);
-		return *reinterpret_cast<const bf16x8*>(base + r * 64 + c * 16);
+		const int c = (2 * ks + (lane >> 5)) ^ ((r >> 1) & 7);
+		return *reinterpret_cast<const bf16x8*>(base + r * 128 + c * 16);
 	} else {
 		const int j = lane & 15;
 		const int m = row0 + 16 * ((lane & 31) >> 4) + 4 * (j & 3);
@@ -121,20 +125,20 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(Args g) {
 	const bf16_t* Bp = BT ? g.B + (int64_t)kt0 * BKS * g.ldb + n0 : g.B + (int64_t)n0 * g.ldb + (int64_t)kt0 * BKS;
 	const int64_t a_step = AT ? (int64_t)BKS * g.lda : BKS;
 	const int64_t b_step = BT ? (int64_t)BKS * g.ldb : BKS;
-	uint32_t aoff[4], boff[4];
+	uint32_t aoff[LOADS_PER_OPERAND], boff[LOADS_PER_OPERAND];
 	lane_offsets<AT>(wave, lane, g.lda, aoff);
 	lane_offsets<BT>(wave, lane, g.ldb, boff);
 
-	const uint32_t lds0 = (uint32_t)(uintptr_t)(unsigned char ELF_LDS*)smem + wave * 4096;  // this wave's first 1 KiB piece
+	const uint32_t lds0 = (uint32_t)(uintptr_t)(unsigned char ELF_LDS*)smem + wave * (LOADS_PER_OPERAND * 1024);  // this wave's first 1 KiB piece
 
 	auto issue = [&](int step) {
 		const uint32_t st = lds0 + (uint32_t)(step % NST) * STAGE_BYTES;
 		const bf16_t* a = Ap + (int64_t)step * a_step;
 		const bf16_t* b = Bp + (int64_t)step * b_step;
 #pragma unroll
-		for (int i = 0; i < 4; i++) dma16(a, aoff[i], __builtin_amdgcn_readfirstlane(st + i * 1024));
+		for (int i = 0; i < LOADS_PER_OPERAND; i++) dma16(a, aoff[i], __builtin_amdgcn_readfirstlane(st + i * 1024));
 #pragma unroll
-		for (int i = 0; i < 4; i++) dma16(b, boff[i], __builtin_amdgcn_readfirstlane(st + OPERAND_BYTES + i * 1024));
+		for (int i = 0; i < LOADS_PER_OPERAND; i++) dma16(b, boff[i], __builtin_amdgcn_readfirstlane(st + OPERAND_BYTES + i * 1024));
 	};
 
 	f32x16 acc[4][4];
@@ -145,31 +149,53 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(Args g) {
 #pragma unroll
 			for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-#pragma unroll
-	for (int s = 0; s < PD; s++)
-		if (s < nk) issue(s);
+	// Software pipeline.  While the 16 MFMAs of one k16-step issue, the 8 fragment reads of the
+	// next step are in flight (one wave per SIMD: nothing else would hide the LDS latency).  The
+	// barrier that publishes slice kt+1 sits before the LAST k16-step of slice kt: by then every
+	// wave has read all of slice kt (its last fragments are in registers), so the same barrier
+	// frees that stage and the fetch of slice kt+2 starts a full slice ahead of its use.
+	issue(0);
+	if (nk > 1) {
+		issue(1);
+		wait_vmcnt<LOADS_PER_STAGE>();
+	} else {
+		wait_vmcnt<0>();
+	}
+	__syncthreads();
 
-	for (int kt = 0; kt < nk; kt++) {
-		// slice kt of this wave has landed once at most the younger slices are outstanding
-		if (kt + PD - 1 < nk) wait_vmcnt<LOADS_PER_STAGE*(PD - 1)>();
-		else wait_vmcnt<0>();
-		__syncthreads();  // everyone's slice kt is in LDS; everyone is done reading slice kt-1
-		if (kt + PD < nk) issue(kt + PD);
-		const unsigned char* sa = smem + (kt % NST) * STAGE_BYTES;
+	bf16x8 fa[2][4], fb[2][4];
+	auto load_frags = [&](int buf, int step, int ks) {
+		const unsigned char* sa = smem + (step % NST) * STAGE_BYTES;
 		const unsigned char* sb = sa + OPERAND_BYTES;
 #pragma unroll
-		for (int ks = 0; ks < BKS / 16; ks++) {
-			bf16x8 af[4], bfr[4];
+		for (int i = 0; i < 4; i++) fa[buf][i] = frag<AT>(sa, wr * 128 + i * 32, ks, lane);
 #pragma unroll
-			for (int i = 0; i < 4; i++) af[i] = frag<AT>(sa, wr * 128 + i * 32, ks, lane);
+		for (int j = 0; j < 4; j++) fb[buf][j] = frag<BT>(sb, wc * 128 + j * 32, ks, lane);
+	};
+	auto mfmas = [&](int buf) {
 #pragma unroll
-			for (int j = 0; j < 4; j++) bfr[j] = frag<BT>(sb, wc * 128 + j * 32, ks, lane);
+		for (int i = 0; i < 4; i++)
 #pragma unroll
-			for (int i = 0; i < 4; i++)
+			for (int j = 0; j < 4; j++)
+				acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][i], fb[buf][j], acc[i][j], 0, 0, 0);
+	};
+
+	load_frags(0, 0, 0);
+	for (int kt = 0; kt < nk; kt++) {
 #pragma unroll
-				for (int j = 0; j < 4; j++)
-					acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+		for (int ks = 0; ks < 3; ks++) {
+			load_frags((ks + 1) & 1, kt, ks + 1);
+			__builtin_amdgcn_sched_barrier(0);
+			mfmas(ks & 1);
+			__builtin_amdgcn_sched_barrier(0);
 		}
+		__builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0): slice kt+1 landed; lgkmcnt(0): slice kt fully read
+		__syncthreads();
+		if (kt + 2 < nk) issue(kt + 2);
+		load_frags(0, kt + 1, 0);  // past the end this reads a stale stage; the values are unused
+		__builtin_amdgcn_sched_barrier(0);
+		mfmas(1);
+		__builtin_amdgcn_sched_barrier(0);
 	}
 
 	// Epilogue through LDS (free once every wave has left the main loop).  Register r of a 32x32
@@ -258,7 +284,7 @@ static int launch_epi(const Args& a, int epi, hipStream_t stream) {
 // Arguments are validated by gemm_bf16() before it dispatches here.
 int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda, const void* B, int64_t ldb, void* C,
                   int64_t ldc, int epi, const void* R, int64_t ldr, int k_splits, hipStream_t stream) {
-	ELF_REQUIRE(M % dma::BM == 0 && N % dma::BN == 0 && K % dma::BKS == 0, "gemm (dma tile): M, N multiples of 256 and K of 32 required");
+	ELF_REQUIRE(M % dma::BM == 0 && N % dma::BN == 0 && K % dma::BKS == 0, "gemm (dma tile): M, N multiples of 256 and K of 64 required");
 	dma::Args a{(const bf16_t*)A, (const bf16_t*)B, C, (const bf16_t*)R, lda, ldb, ldc, ldr, M, N, K, M / dma::BM, N / dma::BN, k_splits < 1 ? 1 : k_splits};
 	if (epi != EPI_F32_ACC) a.k_splits = 1;
 	if (!a_t && !b_t) return dma::launch_epi<false, false>(a, epi, stream);
