@@ -16,6 +16,7 @@
 // workgroup barrier for the other waves' slices and for the reuse of the oldest stage.
 #include "common.h"
 #include "kernels.h"
+#include "lds_dma.h"
 
 namespace elf {
 
@@ -36,18 +37,6 @@ struct Args {
 	int M, N, K;
 	int tiles_m, tiles_n, k_splits;
 };
-
-// s_waitcnt with only vmcnt set (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt_hi[15:14])
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-	__builtin_amdgcn_s_waitcnt((N & 0xF) | (0x7 << 4) | (0xF << 8) | ((N >> 4) << 14));
-}
-
-// 16 bytes per lane from (base + byte_off) to LDS at lds_byte_addr + lane * 16 (base and LDS
-// address are wave-uniform and travel in scalar registers).
-__device__ __forceinline__ void dma16(const bf16_t* base, uint32_t byte_off, uint32_t lds_byte_addr) {
-	asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_byte_addr), "v"(byte_off), "s"(base) : "memory", "m0");
-}
 
 // Byte offsets (relative to the tile origin of the current K slice) of the 16-byte chunks this
 // lane fetches for one operand (< 2^31: 256 rows of at most 64 K elements).  "R" tiles are
@@ -129,7 +118,7 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(Args g) {
 	lane_offsets<AT>(wave, lane, g.lda, aoff);
 	lane_offsets<BT>(wave, lane, g.ldb, boff);
 
-	const uint32_t lds0 = (uint32_t)(uintptr_t)(unsigned char ELF_LDS*)smem + wave * (LOADS_PER_OPERAND * 1024);  // this wave's first 1 KiB piece
+	const uint32_t lds0 = lds_addr(smem) + wave * (LOADS_PER_OPERAND * 1024);  // this wave's first 1 KiB piece
 
 	auto issue = [&](int step) {
 		const uint32_t st = lds0 + (uint32_t)(step % NST) * STAGE_BYTES;
@@ -189,7 +178,7 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(Args g) {
 			mfmas(ks & 1);
 			__builtin_amdgcn_sched_barrier(0);
 		}
-		__builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0): slice kt+1 landed; lgkmcnt(0): slice kt fully read
+		wait_counters<0, 0>();  // vmcnt(0): slice kt+1 landed; lgkmcnt(0): slice kt fully read
 		__syncthreads();
 		if (kt + 2 < nk) issue(kt + 2);
 		load_frags(0, kt + 1, 0);  // past the end this reads a stale stage; the values are unused
