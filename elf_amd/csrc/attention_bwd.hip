@@ -1,0 +1,436 @@
+// Attention backward kernels (see attention_common.h for the layout conventions).
+#include "attention_common.h"
+
+namespace elf {
+namespace attn {
+
+// ------------------------------------------------------------------------------------------
+// delta[b,h,s] = sum_d dO * O and nlse2[b,h,s] = -lse * log2(e)   (one wave per token-head)
+__global__ __launch_bounds__(256) void attn_delta_kernel(const bf16_t* __restrict__ dO, const bf16_t* __restrict__ O,
+                                                         const float* __restrict__ lse, float* __restrict__ delta,
+                                                         float* __restrict__ nlse2, int64_t ldd, int64_t ldo, int B, int S,
+                                                         int Hq, int D) {
+	const int lane = threadIdx.x & 63;
+	const int64_t idx = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // token * Hq + h
+	if (idx >= (int64_t)B * S * Hq) return;
+	const int h = (int)(idx % Hq);
+	const int64_t tok = idx / Hq;
+	float s = 0.f;
+	for (int c = lane * 2; c < D; c += 128) {
+		bf16x2 x = *reinterpret_cast<const bf16x2*>(dO + tok * ldd + h * D + c);
+		bf16x2 y = *reinterpret_cast<const bf16x2*>(O + tok * ldo + h * D + c);
+		s += (float)x[0] * (float)y[0] + (float)x[1] * (float)y[1];
+	}
+	s = wave_sum(s);
+	if (lane == 0) {
+		const int64_t b = tok / S, sp = tok % S;
+		delta[(b * Hq + h) * S + sp] = s;
+		nlse2[(b * Hq + h) * S + sp] = -lse[(b * Hq + h) * S + sp] * LOG2E;
+	}
+}
+
+struct AttnBwdArgs {
+	const bf16_t* q;
+	const bf16_t* k;
+	const bf16_t* v;
+	const bf16_t* dO;
+	const float* nlse2;  // -lse * log2(e)
+	const float* delta;
+	float* dq_acc;  // fp32 [T, Hq*D], zero-initialised by the caller side of the launcher
+	bf16_t* dk;
+	bf16_t* dv;
+	int64_t ldq, ldk, ldv, lddo, lddk, lddv;
+	int B, S, Hq, Hkv;
+	float scale;
+};
+
+// Tiles fetched straight into LDS (lds_dma.h) are unpadded; the 16-byte chunk index of a row is
+// XOR-swizzled with a function of the row chosen so that both access patterns are conflict
+// free: row-wise fragment reads (16 consecutive rows, same chunk) and transpose reads (4
+// consecutive rows x 2 adjacent chunks).
+template <int D>
+struct BwdTile {
+	static constexpr int ROW_BYTES = D * 2;
+	static constexpr int CPR = D / 8;             // 16-byte chunks per row
+	static constexpr int RPI = 1024 / ROW_BYTES;  // rows per DMA wave instruction
+	__device__ static __forceinline__ int swz(int row) {
+		return D == 128 ? (((row & 7) << 1) | ((row >> 3) & 1)) : ((((row >> 1) & 3) << 1) | ((row >> 3) & 1));
+	}
+	// row-wise operand: rows row0 + lane%32, 8 consecutive columns from 16*ks + 8*(lane/32)
+	__device__ static __forceinline__ bf16x8 rows(const unsigned char* t, int row0, int ks, int lane) {
+		const int r = row0 + (lane & 31);
+		return *reinterpret_cast<const bf16x8*>(t + r * ROW_BYTES + (((2 * ks + (lane >> 5)) ^ swz(r)) << 4));
+	}
+	// transposed operand: column m0 + lane%32 at the rows {kA..kA+3, kA+second..+3}, kA = k0 + 4*(lane/32)
+	// (second = 8: accumulator row order) or kA = k0 + 8*(lane/32) (second = 4: natural order)
+	template <bool ACC_ORDER>
+	__device__ static __forceinline__ bf16x8 cols(const unsigned char* t, int k0, int m0, int lane) {
+		const int j = lane & 15;
+		const int kk = k0 + (ACC_ORDER ? 4 : 8) * (lane >> 5) + (j >> 2);
+		const int k2 = kk + (ACC_ORDER ? 8 : 4);
+		const int c = (m0 + 16 * ((lane & 31) >> 4) + 4 * (j & 3)) >> 3;
+		const unsigned char* p0 = t + kk * ROW_BYTES + ((c ^ swz(kk)) << 4) + (j & 1) * 8;
+		const unsigned char* p1 = t + k2 * ROW_BYTES + ((c ^ swz(k2)) << 4) + (j & 1) * 8;
+		s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 ELF_LDS*)(p0));
+		s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 ELF_LDS*)(p1));
+		return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+	}
+};
+
+// 4 bytes per lane from a per-lane global address to LDS at lds_byte_addr + lane * 4.
+__device__ __forceinline__ void dma4(const void* lane_addr, uint32_t lds_byte_addr) {
+	asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_byte_addr), "v"(lane_addr) : "memory", "m0");
+}
+
+// dS^T tile in LDS: [key][q] bf16 with 64-byte rows (32 queries); the 16-byte chunk index is
+// XOR-swizzled with (key >> 2) & 3 so that the 8-byte accumulator writes of 32 consecutive keys
+// and the transpose reads of 4 consecutive keys both spread over all banks.
+__device__ __forceinline__ int ds_t_offset(int key, int q) {  // q a multiple of 4
+	return key * 64 + (((q >> 3) ^ ((key >> 2) & 3)) << 4) + ((q >> 2) & 1) * 8;
+}
+// A operand from the dS^T tile: row q = lane%32, keys k0 + 8*(lane/32) .. +7
+__device__ __forceinline__ bf16x8 ds_t_frag(const unsigned char* t, int k0, int lane) {
+	const int j = lane & 15;
+	const int kk = k0 + 8 * (lane >> 5) + (j >> 2);
+	const int q = 16 * ((lane & 31) >> 4) + 4 * (j & 3);
+	s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 ELF_LDS*)(t + ds_t_offset(kk, q)));
+	s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 ELF_LDS*)(t + ds_t_offset(kk + 4, q)));
+	return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+}
+
+// One workgroup pass = 128 keys of one (batch, kv head); wave w owns keys [32w, 32w+32) and
+// keeps their K / V rows (MFMA B operands) and dK^T / dV^T accumulators in registers while the
+// workgroup walks over the 32-query tiles of every query head of the group.  Q and dO tiles
+// arrive by direct-to-LDS loads one tile ahead.  Per tile and wave:
+//   S = Q K^T, dP = dO V^T  (A operands: LDS rows)      P = exp2(S*sc - lse), dS = P (dP - delta)
+//   dV^T += dO^T P, dK^T += Q^T dS  (A operands: LDS transpose reads; B: P / dS from registers)
+// dS^T goes to LDS; after the next workgroup barrier each wave multiplies the whole 32x128 dS
+// by its slice of K (held in registers as B operands) to get its slice of the dQ tile.  That
+// product runs one tile behind, so a tile costs one barrier, and its atomic adds to the fp32
+// dQ accumulator are issued one more tile later, right after the barrier, because the
+// direct-to-LDS loads can only be awaited together with every other outstanding vector memory
+// operation of the wave.  The softmax scale of dK and dQ is applied by the epilogue / the
+// conversion kernel.  With a causal mask key tile kt meets 1 - kt/nkt of the query tiles, so
+// a workgroup takes the tiles kt and nkt-1-kt one after the other: every workgroup then does
+// the same amount of work.
+template <int D, bool CAUSAL>
+__global__ __launch_bounds__(256) void attn_bwd_kernel(AttnBwdArgs a) {
+	using TL = BwdTile<D>;
+	constexpr int BKV = 128, BQ = 32;
+	constexpr int NF = D / 16;  // fragments per operand tile
+	constexpr int DT = D / 32;
+	constexpr int KH = 4 / DT;  // key splits of the dQ product (4 waves = DT column slices x KH key ranges)
+	static_assert((BKV / 16) / KH == NF, "dQ fragment count");
+	constexpr int K_BYTES = BKV * TL::ROW_BYTES, Q_BYTES = BQ * TL::ROW_BYTES;
+	constexpr int STAGE = 2 * Q_BYTES + 256;  // Q tile, dO tile, 32 nlse2 + 32 delta floats
+	constexpr int DS_BYTES = BKV * BQ * 2;
+	constexpr int Q_LOADS = 8 / TL::RPI;  // DMA instructions per wave and tile (8 rows per wave)
+	extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
+	unsigned char* const sKt = smem_raw;            // K tile, [key][d]
+	unsigned char* const sStage = sKt + K_BYTES;    // 2 x {Q [q][d], dO [q][d], nlse2, delta}
+	unsigned char* const sdS = sStage + 2 * STAGE;  // 2 x dS^T [key][q]
+
+	const int tid = threadIdx.x, lane = tid & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+	const int g = lane >> 5, kl = lane & 31;
+	const int nkt = a.S / BKV;
+	const int npair = CAUSAL ? (nkt + 1) / 2 : nkt;
+	const int pair = blockIdx.x % npair;
+	const int bh = blockIdx.x / npair;
+	const int hk = bh % a.Hkv, b = bh / a.Hkv;
+	const int G = a.Hq / a.Hkv;
+	const int64_t tok0 = (int64_t)b * a.S;
+	const int64_t HqD = (int64_t)a.Hq * D;
+	const float sc = a.scale * LOG2E;
+	const int dq_dt = wave % DT, dq_ks0 = (wave / DT) * NF;  // this wave's share of the dQ product
+	const int key_l = wave * 32 + kl;                        // this lane's key within the tile
+	const int nqt_all = a.S / BQ;
+	const int dq_lane = (4 * g) * (int)HqD + dq_dt * 32 + kl;  // lane part of a dQ tile address (elements)
+
+	// DMA plan for one (Q, dO) tile pair: wave w moves rows [w*8, w*8+8) of each
+	uint32_t qoff[Q_LOADS], dooff[Q_LOADS];
+#pragma unroll
+	for (int i = 0; i < Q_LOADS; i++) {
+		const int row = wave * 8 + i * TL::RPI + lane / TL::CPR, slot = lane % TL::CPR;
+		qoff[i] = (uint32_t)((row * a.ldq + ((slot ^ TL::swz(row)) << 3)) * 2);
+		dooff[i] = (uint32_t)((row * a.lddo + ((slot ^ TL::swz(row)) << 3)) * 2);
+	}
+	auto zero_ds = [&](unsigned char* t) {
+#pragma unroll
+		for (int i = 0; i < 4; i++) *reinterpret_cast<u32x2*>(t + ds_t_offset(key_l, 8 * i + 4 * g)) = u32x2{0u, 0u};
+	};
+	auto atomics = [&](float* tile, const f32x16& v) {
+#pragma unroll
+		for (int r = 0; r < 16; r++) unsafeAtomicAdd(tile + ((r >> 2) * 8 + (r & 3)) * HqD + dq_lane, v[r]);
+	};
+
+	const int n_pass = (CAUSAL && nkt - 1 - pair != pair) ? 2 : 1;
+#pragma unroll 1
+	for (int pass = 0; pass < n_pass; pass++) {
+		const int kt_idx = pass == 0 ? pair : nkt - 1 - pair;
+		const int key0 = kt_idx * BKV;       // first key of the pass
+		const int wkey0 = key0 + wave * 32;  // first key of this wave
+		if (pass > 0) __syncthreads();       // every wave is done with the LDS of the previous pass
+
+		// K tile -> LDS; this wave moves rows [wave*32, wave*32+32)
+		{
+			const bf16_t* kb = a.k + (tok0 + key0) * a.ldk + hk * D;
+#pragma unroll
+			for (int i = 0; i < 32 / TL::RPI; i++) {
+				const int row = wave * 32 + i * TL::RPI + lane / TL::CPR, slot = lane % TL::CPR;
+				dma16(kb, (uint32_t)((row * a.ldk + ((slot ^ TL::swz(row)) << 3)) * 2),
+				      __builtin_amdgcn_readfirstlane(lds_addr(sKt) + (wave * 32 + i * TL::RPI) * TL::ROW_BYTES));
+			}
+		}
+		// own K and V rows as B operands (n = key, 8 consecutive d) in registers
+		bf16x8 kf[NF], vf[NF];
+		{
+			const bf16_t* kp = a.k + (tok0 + wkey0 + kl) * a.ldk + hk * D + 8 * g;
+			const bf16_t* vp = a.v + (tok0 + wkey0 + kl) * a.ldv + hk * D + 8 * g;
+#pragma unroll
+			for (int ks = 0; ks < NF; ks++) {
+				kf[ks] = *reinterpret_cast<const bf16x8*>(kp + ks * 16);
+				vf[ks] = *reinterpret_cast<const bf16x8*>(vp + ks * 16);
+			}
+		}
+		f32x16 acc_dk[DT], acc_dv[DT];
+#pragma unroll
+		for (int i = 0; i < DT; i++)
+#pragma unroll
+			for (int r = 0; r < 16; r++) acc_dk[i][r] = acc_dv[i][r] = 0.f;
+
+		// Walk over (query head in group, query tile); causal: only tiles that reach key0.
+		const int qt_first = CAUSAL ? key0 / BQ : 0;
+		const int n_iter = G * (nqt_all - qt_first);
+
+		// position of the tile whose loads are issued next
+		int ld_h = hk * G, ld_qt = qt_first;
+		auto issue = [&](int stage) {
+			const int q0 = ld_qt * BQ;
+			const uint32_t st = lds_addr(sStage) + (uint32_t)stage * STAGE;
+			const bf16_t* qb = a.q + (tok0 + q0) * a.ldq + ld_h * D;
+			const bf16_t* dob = a.dO + (tok0 + q0) * a.lddo + ld_h * D;
+#pragma unroll
+			for (int i = 0; i < Q_LOADS; i++) {
+				dma16(qb, qoff[i], __builtin_amdgcn_readfirstlane(st + (wave * 8 + i * TL::RPI) * TL::ROW_BYTES));
+				dma16(dob, dooff[i], __builtin_amdgcn_readfirstlane(st + Q_BYTES + (wave * 8 + i * TL::RPI) * TL::ROW_BYTES));
+			}
+			if (wave == 0) {
+				const int64_t base = ((int64_t)b * a.Hq + ld_h) * a.S + q0;
+				const float* src = (lane < 32 ? a.nlse2 : a.delta) + base + (lane & 31);
+				dma4(src, __builtin_amdgcn_readfirstlane(st + 2 * Q_BYTES));
+			}
+			if (++ld_qt == nqt_all) {
+				ld_qt = qt_first;
+				ld_h++;
+			}
+		};
+
+		issue(0);
+		zero_ds(sdS + DS_BYTES);  // the "previous tile" of the first iteration
+		wait_vmcnt<0>();
+		__syncthreads();
+		// this wave's slice of K as B operands of the dQ product (n = d column, k = key)
+		bf16x8 ktf[NF];
+#pragma unroll
+		for (int i = 0; i < NF; i++) ktf[i] = TL::template cols<false>(sKt, (dq_ks0 + i) * 16, dq_dt * 32, lane);
+
+		// position of the current tile; dq_prev_tile = where the dQ tile of iteration it-1 goes
+		int cur_h = hk * G, cur_qt = qt_first;
+		float* dq_prev_tile = a.dq_acc + (tok0 + qt_first * BQ) * HqD + cur_h * D;
+
+		for (int it = 0; it < n_iter; it++) {
+			if (it + 1 < n_iter) issue((it + 1) & 1);
+			const unsigned char* sQ = sStage + (it & 1) * STAGE;
+			const unsigned char* sdO = sQ + Q_BYTES;
+			const float* sLse = reinterpret_cast<const float*>(sdO + Q_BYTES);
+			const unsigned char* sdS_prev = sdS + ((it + 1) & 1) * DS_BYTES;
+			unsigned char* sdS_cur = sdS + (it & 1) * DS_BYTES;
+			const int q0 = cur_qt * BQ;
+
+			bf16x8 bA[NF], bC[NF];
+			f32x16 dq, s, dp;
+#pragma unroll
+			for (int r = 0; r < 16; r++) dq[r] = s[r] = dp[r] = 0.f;
+#pragma unroll
+			for (int i = 0; i < NF; i++) bC[i] = ds_t_frag(sdS_prev, (dq_ks0 + i) * 16, lane);
+#pragma unroll
+			for (int i = 0; i < NF; i++) bA[i] = TL::rows(sQ, 0, i, lane);
+			__builtin_amdgcn_sched_barrier(0);
+			// dQ product of the previous tile, interleaved with S of this one
+#pragma unroll
+			for (int i = 0; i < NF; i++) {
+				dq = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bC[i], ktf[i], dq, 0, 0, 0);
+				s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bA[i], kf[i], s, 0, 0, 0);
+			}
+			__builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+			for (int i = 0; i < NF; i++) bC[i] = TL::rows(sdO, 0, i, lane);
+			__builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+			for (int i = 0; i < NF; i++) dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bC[i], vf[i], dp, 0, 0, 0);
+			// dO^T fragments: rows d, k = queries in accumulator order
+#pragma unroll
+			for (int i = 0; i < NF; i++) bA[i] = TL::template cols<true>(sdO, (i / DT) * 16, (i % DT) * 32, lane);
+			atomics(dq_prev_tile, dq);
+			__builtin_amdgcn_sched_barrier(0);
+			// Q^T fragments
+#pragma unroll
+			for (int i = 0; i < NF; i++) bC[i] = TL::template cols<true>(sQ, (i / DT) * 16, (i % DT) * 32, lane);
+			// causal mask: key > query  <=>  row index of the accumulator register < key - q0
+			// (never true for a tile that lies wholly after the wave's keys; a wave whose keys lie
+			// wholly after the tile gets P = 0 everywhere)
+			const int kq = wkey0 + kl - q0 - 4 * g;
+#pragma unroll
+			for (int u = 0; u < 2; u++) {
+				float p[8], ds[8];
+#pragma unroll
+				for (int r4 = 2 * u; r4 < 2 * u + 2; r4++) {
+					const f32x4 l4 = *reinterpret_cast<const f32x4*>(sLse + r4 * 8 + 4 * g);
+					const f32x4 d4 = *reinterpret_cast<const f32x4*>(sLse + 32 + r4 * 8 + 4 * g);
+#pragma unroll
+					for (int t = 0; t < 4; t++) {
+						const int r = r4 * 4 + t;
+						float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(s[r], sc, l4[t]));
+						if (CAUSAL && r4 * 8 + t < kq) pr = 0.f;
+						p[r & 7] = pr;
+						ds[r & 7] = pr * (dp[r] - d4[t]);
+					}
+				}
+				const bf16x8 pf = pack8(p), dsf = pack8(ds);
+				// accumulator rows of register r: q = (r/4)*8 + 4g + r%4 -> two 8-byte groups per half
+				const u32x4 w = __builtin_bit_cast(u32x4, dsf);
+				*reinterpret_cast<u32x2*>(sdS_cur + ds_t_offset(key_l, 16 * u + 4 * g)) = u32x2{w[0], w[1]};
+				*reinterpret_cast<u32x2*>(sdS_cur + ds_t_offset(key_l, 16 * u + 8 + 4 * g)) = u32x2{w[2], w[3]};
+				if (u == 0) __builtin_amdgcn_sched_barrier(0);
+				// dV^T[d][key] += dO^T[d][q] P[q][key] ; dK^T[d][key] += Q^T[d][q] dS[q][key]
+#pragma unroll
+				for (int dt = 0; dt < DT; dt++) {
+					acc_dv[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bA[u * DT + dt], pf, acc_dv[dt], 0, 0, 0);
+					acc_dk[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bC[u * DT + dt], dsf, acc_dk[dt], 0, 0, 0);
+				}
+			}
+			dq_prev_tile = a.dq_acc + (tok0 + q0) * HqD + cur_h * D;
+			if (++cur_qt == nqt_all) {
+				cur_qt = qt_first;
+				cur_h++;
+			}
+			wait_vmcnt<0>();
+			__syncthreads();  // the next tile is in LDS, dS^T of this tile is complete, everyone is done with this tile
+		}
+		// drain: dQ product and atomics of the last tile
+		{
+			const unsigned char* sdS_prev = sdS + ((n_iter + 1) & 1) * DS_BYTES;
+			f32x16 dq;
+#pragma unroll
+			for (int r = 0; r < 16; r++) dq[r] = 0.f;
+#pragma unroll
+			for (int i = 0; i < NF; i++)
+				dq = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ds_t_frag(sdS_prev, (dq_ks0 + i) * 16, lane), ktf[i], dq, 0, 0, 0);
+			atomics(dq_prev_tile, dq);
+		}
+
+		// dK^T / dV^T accumulators: register r <-> d = dt*32 + (r/4)*8 + 4g + r%4, lane <-> key
+		bf16_t* dkp = a.dk + (tok0 + wkey0 + kl) * a.lddk + hk * D;
+		bf16_t* dvp = a.dv + (tok0 + wkey0 + kl) * a.lddv + hk * D;
+#pragma unroll
+		for (int dt = 0; dt < DT; dt++) {
+#pragma unroll
+			for (int r4 = 0; r4 < 4; r4++) {
+				bf16x4 k4, v4;
+#pragma unroll
+				for (int u = 0; u < 4; u++) {
+					k4[u] = (bf16_t)(acc_dk[dt][r4 * 4 + u] * a.scale);
+					v4[u] = (bf16_t)acc_dv[dt][r4 * 4 + u];
+				}
+				*reinterpret_cast<bf16x4*>(dkp + dt * 32 + r4 * 8 + 4 * g) = k4;
+				*reinterpret_cast<bf16x4*>(dvp + dt * 32 + r4 * 8 + 4 * g) = v4;
+			}
+		}
+	}
+}
+
+// dq(bf16, row stride ld) = scale * dq_acc(fp32, contiguous [T, cols])
+__global__ __launch_bounds__(256) void cvt_f32_bf16_kernel(const float* __restrict__ src, bf16_t* __restrict__ dst, int64_t T,
+                                                           int cols, int64_t ld, float scale) {
+	const int cpr = cols / 4;
+	const int64_t n = T * cpr;
+	for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+		const int64_t row = i / cpr;
+		const int c = (int)(i - row * cpr) * 4;
+		const f32x4 v = *reinterpret_cast<const f32x4*>(src + row * cols + c);
+		bf16x4 o;
+#pragma unroll
+		for (int t = 0; t < 4; t++) o[t] = (bf16_t)(v[t] * scale);
+		*reinterpret_cast<bf16x4*>(dst + row * ld + c) = o;
+	}
+}
+
+__global__ __launch_bounds__(256) void fill_zero_kernel(f32x4* __restrict__ p, int64_t n4) {
+	for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
+		f32x4 z = {0.f, 0.f, 0.f, 0.f};
+		p[i] = z;
+	}
+}
+
+template <int D, bool CAUSAL>
+int launch_bwd(const AttnBwdArgs& a, dim3 grid, hipStream_t stream) {
+	constexpr int smem = 128 * D * 2 + 2 * (2 * 32 * D * 2 + 256) + 2 * 128 * 32 * 2;
+	auto kern = attn_bwd_kernel<D, CAUSAL>;
+	static bool attr_set = false;
+	if (!attr_set) {
+		ELF_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+		attr_set = true;
+	}
+	hipLaunchKernelGGL(kern, grid, dim3(256), smem, stream, a);
+	ELF_CHECK_HIP(hipGetLastError());
+	return 0;
+}
+
+}  // namespace attn
+
+using namespace attn;
+
+int64_t attn_bwd_workspace_bytes(int B, int S, int Hq, int D) {
+	// fp32 dQ accumulator + delta + scaled log-sum-exp
+	return (int64_t)B * S * Hq * D * 4 + 2 * (int64_t)B * S * Hq * 4;
+}
+
+int attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* dO, const void* lse, void* dq,
+             void* dk, void* dv, void* workspace, int64_t ldq, int64_t ldk, int64_t ldv, int64_t ldo, int64_t lddo,
+             int64_t lddq, int64_t lddk, int64_t lddv, int B, int S, int Hq, int Hkv, int D, int causal, float scale,
+             hipStream_t stream) {
+	ELF_REQUIRE(q && k && v && o && dO && lse && dq && dk && dv && workspace, "attn_bwd: null pointer");
+	ELF_REQUIRE(B > 0 && S > 0 && S % 128 == 0, "attn_bwd: sequence length must be a multiple of 128 (S=%d)", S);
+	ELF_REQUIRE(Hkv > 0 && Hq % Hkv == 0, "attn_bwd: Hq must be a multiple of Hkv (Hq=%d Hkv=%d)", Hq, Hkv);
+	ELF_REQUIRE(D == 64 || D == 128, "attn_bwd: head_dim must be 64 or 128 (D=%d)", D);
+	ELF_REQUIRE(ldq % 8 == 0 && ldk % 8 == 0 && ldv % 8 == 0 && ldo % 8 == 0 && lddo % 8 == 0 && lddq % 8 == 0 &&
+	                lddk % 8 == 0 && lddv % 8 == 0,
+	            "attn_bwd: strides must be multiples of 8");
+	ELF_REQUIRE(((uintptr_t)workspace % 16) == 0, "attn_bwd: misaligned workspace");
+	ProfScope prof(PROF_ATTN_BWD, (causal ? 4.0 : 8.0) * B * Hq * (double)S * S * D, stream);
+	const int64_t T = (int64_t)B * S;
+	float* dq_acc = (float*)workspace;
+	float* delta = dq_acc + T * Hq * D;
+	float* nlse2 = delta + T * Hq;
+	// zero the dQ accumulator with a fill kernel (memset nodes misbehave under graph replay)
+	hipLaunchKernelGGL(fill_zero_kernel, dim3(2048), dim3(256), 0, stream, (f32x4*)dq_acc, T * Hq * D / 4);
+	hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)((T * Hq + 3) / 4)), dim3(256), 0, stream, (const bf16_t*)dO,
+	                   (const bf16_t*)o, (const float*)lse, delta, nlse2, lddo, ldo, B, S, Hq, D);
+	AttnBwdArgs a{(const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, (const bf16_t*)dO, nlse2, delta, dq_acc,
+	              (bf16_t*)dk, (bf16_t*)dv, ldq, ldk, ldv, lddo, lddk, lddv, B, S, Hq, Hkv, scale};
+	const int nkt = S / 128;
+	const dim3 grid((unsigned)((int64_t)B * Hkv * (causal ? (nkt + 1) / 2 : nkt))), block(256);
+	int rc;
+	if (D == 128) rc = causal ? launch_bwd<128, true>(a, grid, stream) : launch_bwd<128, false>(a, grid, stream);
+	else rc = causal ? launch_bwd<64, true>(a, grid, stream) : launch_bwd<64, false>(a, grid, stream);
+	if (rc) return rc;
+	const int64_t n4 = T * (Hq * D / 4);
+	const int64_t blocks = (n4 + 255) / 256;
+	hipLaunchKernelGGL(cvt_f32_bf16_kernel, dim3((unsigned)(blocks < 4096 ? blocks : 4096)), dim3(256), 0, stream, dq_acc,
+	                   (bf16_t*)dq, T, Hq * D, lddq, scale);
+	ELF_CHECK_HIP(hipGetLastError());
+	return 0;
+}
+
+}  // namespace elf
