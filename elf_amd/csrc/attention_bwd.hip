@@ -119,8 +119,7 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(AttnBwdArgs a) {
 	constexpr int BKV = 128, BQ = 32;
 	constexpr int NF = D / 16;  // fragments per operand tile
 	constexpr int DT = D / 32;
-	constexpr int KH = 4 / DT;  // key splits of the dQ product (4 waves = DT column slices x KH key ranges)
-	static_assert((BKV / 16) / KH == NF, "dQ fragment count");
+	constexpr int NQ = BKV / 16;  // fragments of the dQ product (all 128 keys); waves 0..DT-1 own one 32-column slice each
 	constexpr int K_BYTES = BKV * TL::ROW_BYTES, Q_BYTES = BQ * TL::ROW_BYTES;
 	constexpr int STAGE = 2 * Q_BYTES + 256;  // Q tile, dO tile, 32 nlse2 + 32 delta floats
 	constexpr int DS_BYTES = BKV * BQ * 2;
@@ -142,7 +141,8 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(AttnBwdArgs a) {
 	const int64_t tok0 = (int64_t)b * a.S;
 	const int64_t HqD = (int64_t)a.Hq * D;
 	const float sc = a.scale * LOG2E;
-	const int dq_dt = wave % DT, dq_ks0 = (wave / DT) * NF;  // this wave's share of the dQ product
+	const bool dq_wave = DT == 4 || wave < DT;  // head_dim 64: two slices, waves 2 and 3 have no dQ share
+	const int dq_dt = wave % DT;
 	const int key_l = wave * 32 + kl;                        // this lane's key within the tile
 	const int nqt_all = a.S / BQ;
 	const int dq_lane = (4 * g) * (int)HqD + dq_dt * 32 + kl;  // lane part of a dQ tile address (elements)
@@ -159,9 +159,13 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(AttnBwdArgs a) {
 #pragma unroll
 		for (int i = 0; i < 4; i++) *reinterpret_cast<u32x2*>(t + ds_t_offset(key_l, 8 * i + 4 * g)) = u32x2{0u, 0u};
 	};
-	auto atomics = [&](float* tile, const f32x16& v) {
+	// registers [r_lo, r_hi) of a dQ accumulator tile -> fp32 atomics (issued a few at a time between
+	// other work: a long burst backs up the memory pipeline and stalls the wave)
+	auto atomics = [&](float* tile, const f32x16& v, int r_lo, int r_hi) {
+		if (!dq_wave) return;
 #pragma unroll
-		for (int r = 0; r < 16; r++) unsafeAtomicAdd(tile + ((r >> 2) * 8 + (r & 3)) * HqD + dq_lane, v[r]);
+		for (int r = 0; r < 16; r++)
+			if (r >= r_lo && r < r_hi) unsafeAtomicAdd(tile + ((r >> 2) * 8 + (r & 3)) * HqD + dq_lane, v[r]);
 	};
 
 	const int n_pass = (CAUSAL && nkt - 1 - pair != pair) ? 2 : 1;
@@ -203,26 +207,35 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(AttnBwdArgs a) {
 		const int qt_first = CAUSAL ? key0 / BQ : 0;
 		const int n_iter = G * (nqt_all - qt_first);
 
-		// position of the tile whose loads are issued next
+		// tile whose loads are issued next: running pointers, recomputed when the walk moves to the next head
 		int ld_h = hk * G, ld_qt = qt_first;
+		const bf16_t* ld_q;
+		const bf16_t* ld_do;
+		const float* ld_stat;  // lanes 0..31: nlse2 of the tile's queries, lanes 32..63: delta
+		auto seek = [&]() {
+			const int64_t row = tok0 + ld_qt * BQ;
+			ld_q = a.q + row * a.ldq + ld_h * D;
+			ld_do = a.dO + row * a.lddo + ld_h * D;
+			ld_stat = (lane < 32 ? a.nlse2 : a.delta) + ((int64_t)b * a.Hq + ld_h) * a.S + ld_qt * BQ + (lane & 31);
+		};
+		seek();
+		const uint32_t lds_stage = lds_addr(sStage) + wave * 8 * TL::ROW_BYTES;
 		auto issue = [&](int stage) {
-			const int q0 = ld_qt * BQ;
-			const uint32_t st = lds_addr(sStage) + (uint32_t)stage * STAGE;
-			const bf16_t* qb = a.q + (tok0 + q0) * a.ldq + ld_h * D;
-			const bf16_t* dob = a.dO + (tok0 + q0) * a.lddo + ld_h * D;
+			const uint32_t st = lds_stage + (uint32_t)stage * STAGE;
 #pragma unroll
 			for (int i = 0; i < Q_LOADS; i++) {
-				dma16(qb, qoff[i], __builtin_amdgcn_readfirstlane(st + (wave * 8 + i * TL::RPI) * TL::ROW_BYTES));
-				dma16(dob, dooff[i], __builtin_amdgcn_readfirstlane(st + Q_BYTES + (wave * 8 + i * TL::RPI) * TL::ROW_BYTES));
+				dma16(ld_q, qoff[i], __builtin_amdgcn_readfirstlane(st + i * TL::RPI * TL::ROW_BYTES));
+				dma16(ld_do, dooff[i], __builtin_amdgcn_readfirstlane(st + Q_BYTES + i * TL::RPI * TL::ROW_BYTES));
 			}
-			if (wave == 0) {
-				const int64_t base = ((int64_t)b * a.Hq + ld_h) * a.S + q0;
-				const float* src = (lane < 32 ? a.nlse2 : a.delta) + base + (lane & 31);
-				dma4(src, __builtin_amdgcn_readfirstlane(st + 2 * Q_BYTES));
-			}
+			if (wave == 0) dma4(ld_stat, __builtin_amdgcn_readfirstlane(st + 2 * Q_BYTES));
 			if (++ld_qt == nqt_all) {
 				ld_qt = qt_first;
 				ld_h++;
+				seek();
+			} else {
+				ld_q += BQ * a.ldq;
+				ld_do += BQ * a.lddo;
+				ld_stat += BQ;
 			}
 		};
 
@@ -231,9 +244,9 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(AttnBwdArgs a) {
 		wait_vmcnt<0>();
 		__syncthreads();
 		// this wave's slice of K as B operands of the dQ product (n = d column, k = key)
-		bf16x8 ktf[NF];
+		bf16x8 ktf[NQ];
 #pragma unroll
-		for (int i = 0; i < NF; i++) ktf[i] = TL::template cols<false>(sKt, (dq_ks0 + i) * 16, dq_dt * 32, lane);
+		for (int i = 0; i < NQ; i++) ktf[i] = TL::template cols<false>(sKt, i * 16, dq_dt * 32, lane);
 
 		// position of the current tile; dq_prev_tile = where the dQ tile of iteration it-1 goes
 		int cur_h = hk * G, cur_qt = qt_first;
@@ -252,64 +265,88 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(AttnBwdArgs a) {
 			f32x16 dq, s, dp;
 #pragma unroll
 			for (int r = 0; r < 16; r++) dq[r] = s[r] = dp[r] = 0.f;
+			if constexpr (DT == 4) {
 #pragma unroll
-			for (int i = 0; i < NF; i++) bC[i] = ds_t_frag(sdS_prev, (dq_ks0 + i) * 16, lane);
+				for (int i = 0; i < NF; i++) bC[i] = ds_t_frag(sdS_prev, i * 16, lane);
 #pragma unroll
-			for (int i = 0; i < NF; i++) bA[i] = TL::rows(sQ, 0, i, lane);
-			__builtin_amdgcn_sched_barrier(0);
-			// dQ product of the previous tile, interleaved with S of this one
+				for (int i = 0; i < NF; i++) bA[i] = TL::rows(sQ, 0, i, lane);
+				__builtin_amdgcn_sched_barrier(0);
+				// dQ product of the previous tile, interleaved with S of this one
 #pragma unroll
-			for (int i = 0; i < NF; i++) {
-				dq = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bC[i], ktf[i], dq, 0, 0, 0);
-				s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bA[i], kf[i], s, 0, 0, 0);
+				for (int i = 0; i < NF; i++) {
+					dq = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bC[i], ktf[i], dq, 0, 0, 0);
+					s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bA[i], kf[i], s, 0, 0, 0);
+				}
+			} else {
+#pragma unroll
+				for (int i = 0; i < NF; i++) bA[i] = TL::rows(sQ, 0, i, lane);
+				if (dq_wave) {
+					bf16x8 bD[NQ];
+#pragma unroll
+					for (int i = 0; i < NQ; i++) bD[i] = ds_t_frag(sdS_prev, i * 16, lane);
+#pragma unroll
+					for (int i = 0; i < NQ; i++) dq = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bD[i], ktf[i], dq, 0, 0, 0);
+				}
+#pragma unroll
+				for (int i = 0; i < NF; i++) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bA[i], kf[i], s, 0, 0, 0);
 			}
 			__builtin_amdgcn_sched_barrier(0);
 #pragma unroll
 			for (int i = 0; i < NF; i++) bC[i] = TL::rows(sdO, 0, i, lane);
+			atomics(dq_prev_tile, dq, 0, 4);
 			__builtin_amdgcn_sched_barrier(0);
+			// dP = dO V^T on the matrix pipe while the vector pipe turns S into P
 #pragma unroll
 			for (int i = 0; i < NF; i++) dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bC[i], vf[i], dp, 0, 0, 0);
 			// dO^T fragments: rows d, k = queries in accumulator order
 #pragma unroll
 			for (int i = 0; i < NF; i++) bA[i] = TL::template cols<true>(sdO, (i / DT) * 16, (i % DT) * 32, lane);
-			atomics(dq_prev_tile, dq);
-			__builtin_amdgcn_sched_barrier(0);
-			// Q^T fragments
-#pragma unroll
-			for (int i = 0; i < NF; i++) bC[i] = TL::template cols<true>(sQ, (i / DT) * 16, (i % DT) * 32, lane);
 			// causal mask: key > query  <=>  row index of the accumulator register < key - q0
 			// (never true for a tile that lies wholly after the wave's keys; a wave whose keys lie
 			// wholly after the tile gets P = 0 everywhere)
 			const int kq = wkey0 + kl - q0 - 4 * g;
+			float p[16];
 #pragma unroll
-			for (int u = 0; u < 2; u++) {
-				float p[8], ds[8];
+			for (int r4 = 0; r4 < 4; r4++) {
+				const f32x4 l4 = *reinterpret_cast<const f32x4*>(sLse + r4 * 8 + 4 * g);
 #pragma unroll
-				for (int r4 = 2 * u; r4 < 2 * u + 2; r4++) {
-					const f32x4 l4 = *reinterpret_cast<const f32x4*>(sLse + r4 * 8 + 4 * g);
-					const f32x4 d4 = *reinterpret_cast<const f32x4*>(sLse + 32 + r4 * 8 + 4 * g);
-#pragma unroll
-					for (int t = 0; t < 4; t++) {
-						const int r = r4 * 4 + t;
-						float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(s[r], sc, l4[t]));
-						if (CAUSAL && r4 * 8 + t < kq) pr = 0.f;
-						p[r & 7] = pr;
-						ds[r & 7] = pr * (dp[r] - d4[t]);
-					}
-				}
-				const bf16x8 pf = pack8(p), dsf = pack8(ds);
-				// accumulator rows of register r: q = (r/4)*8 + 4g + r%4 -> two 8-byte groups per half
-				const u32x4 w = __builtin_bit_cast(u32x4, dsf);
-				*reinterpret_cast<u32x2*>(sdS_cur + ds_t_offset(key_l, 16 * u + 4 * g)) = u32x2{w[0], w[1]};
-				*reinterpret_cast<u32x2*>(sdS_cur + ds_t_offset(key_l, 16 * u + 8 + 4 * g)) = u32x2{w[2], w[3]};
-				if (u == 0) __builtin_amdgcn_sched_barrier(0);
-				// dV^T[d][key] += dO^T[d][q] P[q][key] ; dK^T[d][key] += Q^T[d][q] dS[q][key]
-#pragma unroll
-				for (int dt = 0; dt < DT; dt++) {
-					acc_dv[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bA[u * DT + dt], pf, acc_dv[dt], 0, 0, 0);
-					acc_dk[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bC[u * DT + dt], dsf, acc_dk[dt], 0, 0, 0);
+				for (int t = 0; t < 4; t++) {
+					float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(s[r4 * 4 + t], sc, l4[t]));
+					if (CAUSAL && r4 * 8 + t < kq) pr = 0.f;
+					p[r4 * 4 + t] = pr;
 				}
 			}
+			const bf16x8 pf[2] = {pack8(p), pack8(p + 8)};
+			atomics(dq_prev_tile, dq, 4, 8);
+			__builtin_amdgcn_sched_barrier(0);
+			// dV^T[d][key] += dO^T[d][q] P[q][key] while the vector pipe forms dS = P (dP - delta)
+#pragma unroll
+			for (int i = 0; i < NF; i++) bC[i] = TL::template cols<true>(sQ, (i / DT) * 16, (i % DT) * 32, lane);
+#pragma unroll
+			for (int i = 0; i < NF; i++)
+				acc_dv[i % DT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bA[i], pf[i / DT], acc_dv[i % DT], 0, 0, 0);
+			float ds[16];
+#pragma unroll
+			for (int r4 = 0; r4 < 4; r4++) {
+				const f32x4 d4 = *reinterpret_cast<const f32x4*>(sLse + 32 + r4 * 8 + 4 * g);
+#pragma unroll
+				for (int t = 0; t < 4; t++) ds[r4 * 4 + t] = p[r4 * 4 + t] * (dp[r4 * 4 + t] - d4[t]);
+			}
+			const bf16x8 dsf[2] = {pack8(ds), pack8(ds + 8)};
+			// accumulator rows of register r: q = (r/4)*8 + 4g + r%4 -> four 8-byte groups per lane
+#pragma unroll
+			for (int u = 0; u < 2; u++) {
+				const u32x4 w = __builtin_bit_cast(u32x4, dsf[u]);
+				*reinterpret_cast<u32x2*>(sdS_cur + ds_t_offset(key_l, 16 * u + 4 * g)) = u32x2{w[0], w[1]};
+				*reinterpret_cast<u32x2*>(sdS_cur + ds_t_offset(key_l, 16 * u + 8 + 4 * g)) = u32x2{w[2], w[3]};
+			}
+			atomics(dq_prev_tile, dq, 8, 12);
+			__builtin_amdgcn_sched_barrier(0);
+			// dK^T[d][key] += Q^T[d][q] dS[q][key]
+#pragma unroll
+			for (int i = 0; i < NF; i++)
+				acc_dk[i % DT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bC[i], dsf[i / DT], acc_dk[i % DT], 0, 0, 0);
+			atomics(dq_prev_tile, dq, 12, 16);
 			dq_prev_tile = a.dq_acc + (tok0 + q0) * HqD + cur_h * D;
 			if (++cur_qt == nqt_all) {
 				cur_qt = qt_first;
@@ -325,9 +362,9 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(AttnBwdArgs a) {
 #pragma unroll
 			for (int r = 0; r < 16; r++) dq[r] = 0.f;
 #pragma unroll
-			for (int i = 0; i < NF; i++)
-				dq = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ds_t_frag(sdS_prev, (dq_ks0 + i) * 16, lane), ktf[i], dq, 0, 0, 0);
-			atomics(dq_prev_tile, dq);
+			for (int i = 0; i < NQ; i++)
+				dq = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ds_t_frag(sdS_prev, i * 16, lane), ktf[i], dq, 0, 0, 0);
+			atomics(dq_prev_tile, dq, 0, 16);
 		}
 
 		// dK^T / dV^T accumulators: register r <-> d = dt*32 + (r/4)*8 + 4g + r%4, lane <-> key
