@@ -120,14 +120,23 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(Args g) {
 
 	const uint32_t lds0 = lds_addr(smem) + wave * (LOADS_PER_OPERAND * 1024);  // this wave's first 1 KiB piece
 
+	// One 1 KiB piece of a slice: pieces 0..7 belong to A, 8..15 to B.  A piece of a slice past the
+	// end of K is fetched from the last slice into a scratch area behind the ring instead, so that
+	// the main loop needs no branches around its loads (the accumulators stay put in registers).
+	const uint32_t lds_dummy = lds_addr(smem) + NST * STAGE_BYTES + wave * 1024;
+	auto issue_piece = [&](int step, int piece) {
+		const bool ok = step < nk;
+		const int sc = ok ? step : nk - 1;
+		const uint32_t st = lds0 + (uint32_t)(sc % NST) * STAGE_BYTES;
+		if (piece < LOADS_PER_OPERAND)
+			dma16(Ap + (int64_t)sc * a_step, aoff[piece], __builtin_amdgcn_readfirstlane(ok ? st + piece * 1024 : lds_dummy));
+		else
+			dma16(Bp + (int64_t)sc * b_step, boff[piece - LOADS_PER_OPERAND],
+			      __builtin_amdgcn_readfirstlane(ok ? st + OPERAND_BYTES + (piece - LOADS_PER_OPERAND) * 1024 : lds_dummy));
+	};
 	auto issue = [&](int step) {
-		const uint32_t st = lds0 + (uint32_t)(step % NST) * STAGE_BYTES;
-		const bf16_t* a = Ap + (int64_t)step * a_step;
-		const bf16_t* b = Bp + (int64_t)step * b_step;
 #pragma unroll
-		for (int i = 0; i < LOADS_PER_OPERAND; i++) dma16(a, aoff[i], __builtin_amdgcn_readfirstlane(st + i * 1024));
-#pragma unroll
-		for (int i = 0; i < LOADS_PER_OPERAND; i++) dma16(b, boff[i], __builtin_amdgcn_readfirstlane(st + OPERAND_BYTES + i * 1024));
+		for (int i = 0; i < LOADS_PER_STAGE; i++) issue_piece(step, i);
 	};
 
 	f32x16 acc[4][4];
@@ -144,12 +153,9 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(Args g) {
 	// wave has read all of slice kt (its last fragments are in registers), so the same barrier
 	// frees that stage and the fetch of slice kt+2 starts a full slice ahead of its use.
 	issue(0);
-	if (nk > 1) {
-		issue(1);
-		wait_vmcnt<LOADS_PER_STAGE>();
-	} else {
-		wait_vmcnt<0>();
-	}
+#pragma unroll
+	for (int i = 0; i < LOADS_PER_STAGE / 2; i++) issue_piece(1, i);
+	wait_vmcnt<LOADS_PER_STAGE / 2>();
 	__syncthreads();
 
 	bf16x8 fa[2][4], fb[2][4];
@@ -169,10 +175,31 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(Args g) {
 				acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][i], fb[buf][j], acc[i][j], 0, 0, 0);
 	};
 
+	// 16 MFMAs of one k16-step with half of a slice's loads (8 pieces from `piece0`) dealt between
+	// them: the four waves' loads of a slice are 64 KiB through a 64 B/clk path, and a wave that
+	// issues them in one burst sits in the queue for ~1000 cycles with its MFMAs behind it.
+	auto mfmas_dma = [&](int buf, int step, int piece0) {
+#pragma unroll
+		for (int i = 0; i < 4; i++)
+#pragma unroll
+			for (int j = 0; j < 4; j++) {
+				acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][i], fb[buf][j], acc[i][j], 0, 0, 0);
+				if (j & 1) {
+					issue_piece(step, piece0 + i * 2 + (j >> 1));
+					__builtin_amdgcn_sched_barrier(0);
+				}
+			}
+	};
+
 	load_frags(0, 0, 0);
 	for (int kt = 0; kt < nk; kt++) {
+		// k16-step 0, with the second half of slice kt+1's loads
+		load_frags(1, kt, 1);
+		__builtin_amdgcn_sched_barrier(0);
+		mfmas_dma(0, kt + 1, LOADS_PER_STAGE / 2);
+		__builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-		for (int ks = 0; ks < 3; ks++) {
+		for (int ks = 1; ks < 3; ks++) {
 			load_frags((ks + 1) & 1, kt, ks + 1);
 			__builtin_amdgcn_sched_barrier(0);
 			mfmas(ks & 1);
@@ -180,10 +207,10 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(Args g) {
 		}
 		wait_counters<0, 0>();  // vmcnt(0): slice kt+1 landed; lgkmcnt(0): slice kt fully read
 		__syncthreads();
-		if (kt + 2 < nk) issue(kt + 2);
 		load_frags(0, kt + 1, 0);  // past the end this reads a stale stage; the values are unused
 		__builtin_amdgcn_sched_barrier(0);
-		mfmas(1);
+		// k16-step 3, with the first half of slice kt+2's loads into the stage the barrier just freed
+		mfmas_dma(1, kt + 2, 0);
 		__builtin_amdgcn_sched_barrier(0);
 	}
 
@@ -244,7 +271,7 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(Args g) {
 
 template <bool AT, bool BT, int EPI>
 static int launch(const Args& a, hipStream_t stream) {
-	constexpr int smem = NST * STAGE_BYTES;
+	constexpr int smem = NST * STAGE_BYTES + 4 * 1024;  // ring + scratch target of the loads past the end of K
 	auto kern = gemm_dma_kernel<AT, BT, EPI>;
 	static bool attr_set = false;
 	if (!attr_set) {
