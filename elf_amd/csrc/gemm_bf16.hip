@@ -325,14 +325,14 @@ int gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda,
 	g.k_splits = k_splits;
 	// Tile choice when the caller leaves it open: the direct-to-LDS 256x256 kernel whenever its
 	// tiles can fill the chip, the register-staged kernels (smaller tiles) otherwise.
-	if (tile_cfg <= 0 && M % 256 == 0 && N % 256 == 0 && (int64_t)(M / 256) * (N / 256) >= 192) tile_cfg = 6;
-	if (tile_cfg == 6) {
+	if (tile_cfg <= 0 && M % 256 == 0 && N % 256 == 0 && (int64_t)(M / 256) * (N / 256) >= 192) tile_cfg = 7;
+	if (tile_cfg == 6 || tile_cfg == 7) {
 		if (epi == EPI_F32_ACC && k_splits <= 0) {
 			const int64_t tiles = (int64_t)(M / 256) * (N / 256);
 			k_splits = 1;
 			while (tiles * k_splits < 256 && (K / 64) / (k_splits * 2) >= 8 && k_splits < 16) k_splits *= 2;
 		}
-		return gemm_bf16_dma(a_t, b_t, M, N, K, A, lda, B, ldb, C, ldc, epi, R, ldr, k_splits, stream);
+		return gemm_bf16_dma(a_t, b_t, M, N, K, A, lda, B, ldb, C, ldc, epi, R, ldr, k_splits, tile_cfg == 7 ? 8 : 4, stream);
 	}
 	if (!a_t && !b_t) return launch_epi<false, false>(g, epi, tile_cfg, stream);
 	if (!a_t && b_t) return launch_epi<false, true>(g, epi, tile_cfg, stream);

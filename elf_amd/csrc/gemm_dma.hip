@@ -25,8 +25,7 @@ namespace dma {
 constexpr int BM = 256, BN = 256, BKS = 64, NST = 2;
 constexpr int OPERAND_BYTES = 256 * BKS * 2;  // 32 KiB
 constexpr int STAGE_BYTES = 2 * OPERAND_BYTES;
-constexpr int LOADS_PER_OPERAND = OPERAND_BYTES / 1024 / 4;  // wave instructions per wave per stage and operand
-constexpr int LOADS_PER_STAGE = 2 * LOADS_PER_OPERAND;
+constexpr int PIECES_PER_OPERAND = OPERAND_BYTES / 1024;  // 1 KiB pieces (one wave instruction each) per stage and operand
 
 struct Args {
 	const bf16_t* A;
@@ -43,11 +42,11 @@ struct Args {
 // [256 rows][128 B], "T" tiles [64 k][512 B]; LDS chunk slot s of a row holds global chunk
 // s ^ f(row) with f chosen so that 16 consecutive lanes of a fragment read hit 16 distinct
 // 16-byte bank groups.
-template <bool T>
-__device__ __forceinline__ void lane_offsets(int wave, int lane, int64_t ld, uint32_t (&off)[LOADS_PER_OPERAND]) {
+template <bool T, int LPO>
+__device__ __forceinline__ void lane_offsets(int wave, int lane, int64_t ld, uint32_t (&off)[LPO]) {
 #pragma unroll
-	for (int i = 0; i < LOADS_PER_OPERAND; i++) {
-		const int q = wave * LOADS_PER_OPERAND + i;  // which 1 KiB piece of the operand tile
+	for (int i = 0; i < LPO; i++) {
+		const int q = wave * LPO + i;  // which 1 KiB piece of the operand tile
 		if constexpr (!T) {
 			const int row = q * 8 + (lane >> 3), slot = lane & 7;
 			off[i] = (uint32_t)((row * ld + ((slot ^ ((row >> 1) & 7)) << 3)) * 2);
@@ -80,8 +79,15 @@ __device__ __forceinline__ bf16x8 frag(const unsigned char* base, int row0, int 
 	}
 }
 
-template <bool AT, bool BT, int EPI>
-__global__ __launch_bounds__(256) void gemm_dma_kernel(Args g) {
+// NW = 4: one wave per SIMD, 128x128 wave tiles (16 accumulator tiles, 8 fragment reads per 16
+// MFMAs).  NW = 8: two waves per SIMD, 64x128 wave tiles (8 accumulator tiles, 6 reads per 8
+// MFMAs): more LDS traffic per FLOP, but the two waves fill each other's issue gaps (every
+// non-MFMA instruction of a lone wave delays its MFMA stream by a few cycles) and barrier waits.
+template <int NW, bool AT, bool BT, int EPI>
+__global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
+	constexpr int RT = 16 / NW;                       // 32-row accumulator tiles per wave (x 4 column tiles)
+	constexpr int LOADS_PER_OPERAND = PIECES_PER_OPERAND / NW;  // wave instructions per wave per stage and operand
+	constexpr int LOADS_PER_STAGE = 2 * LOADS_PER_OPERAND;
 	extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 	const int tid = threadIdx.x;
 	const int lane = tid & 63;
@@ -115,12 +121,12 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(Args g) {
 	const int64_t a_step = AT ? (int64_t)BKS * g.lda : BKS;
 	const int64_t b_step = BT ? (int64_t)BKS * g.ldb : BKS;
 	uint32_t aoff[LOADS_PER_OPERAND], boff[LOADS_PER_OPERAND];
-	lane_offsets<AT>(wave, lane, g.lda, aoff);
-	lane_offsets<BT>(wave, lane, g.ldb, boff);
+	lane_offsets<AT, LOADS_PER_OPERAND>(wave, lane, g.lda, aoff);
+	lane_offsets<BT, LOADS_PER_OPERAND>(wave, lane, g.ldb, boff);
 
 	const uint32_t lds0 = lds_addr(smem) + wave * (LOADS_PER_OPERAND * 1024);  // this wave's first 1 KiB piece
 
-	// One 1 KiB piece of a slice: pieces 0..7 belong to A, 8..15 to B.  A piece of a slice past the
+	// One 1 KiB piece of a slice: the first LOADS_PER_OPERAND pieces belong to A, the rest to B.  A piece of a slice past the
 	// end of K is fetched from the last slice into a scratch area behind the ring instead, so that
 	// the main loop needs no branches around its loads (the accumulators stay put in registers).
 	const uint32_t lds_dummy = lds_addr(smem) + NST * STAGE_BYTES + wave * 1024;
@@ -139,9 +145,9 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(Args g) {
 		for (int i = 0; i < LOADS_PER_STAGE; i++) issue_piece(step, i);
 	};
 
-	f32x16 acc[4][4];
+	f32x16 acc[RT][4];
 #pragma unroll
-	for (int i = 0; i < 4; i++)
+	for (int i = 0; i < RT; i++)
 #pragma unroll
 		for (int j = 0; j < 4; j++)
 #pragma unroll
@@ -158,29 +164,29 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(Args g) {
 	wait_vmcnt<LOADS_PER_STAGE / 2>();
 	__syncthreads();
 
-	bf16x8 fa[2][4], fb[2][4];
+	bf16x8 fa[2][RT], fb[2][4];
 	auto load_frags = [&](int buf, int step, int ks) {
 		const unsigned char* sa = smem + (step % NST) * STAGE_BYTES;
 		const unsigned char* sb = sa + OPERAND_BYTES;
 #pragma unroll
-		for (int i = 0; i < 4; i++) fa[buf][i] = frag<AT>(sa, wr * 128 + i * 32, ks, lane);
+		for (int i = 0; i < RT; i++) fa[buf][i] = frag<AT>(sa, wr * (RT * 32) + i * 32, ks, lane);
 #pragma unroll
 		for (int j = 0; j < 4; j++) fb[buf][j] = frag<BT>(sb, wc * 128 + j * 32, ks, lane);
 	};
 	auto mfmas = [&](int buf) {
 #pragma unroll
-		for (int i = 0; i < 4; i++)
+		for (int i = 0; i < RT; i++)
 #pragma unroll
 			for (int j = 0; j < 4; j++)
 				acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][i], fb[buf][j], acc[i][j], 0, 0, 0);
 	};
 
-	// 16 MFMAs of one k16-step with half of a slice's loads (8 pieces from `piece0`) dealt between
+	// The MFMAs of one k16-step with half of this wave's loads of a slice (from `piece0`) dealt between
 	// them: the four waves' loads of a slice are 64 KiB through a 64 B/clk path, and a wave that
 	// issues them in one burst sits in the queue for ~1000 cycles with its MFMAs behind it.
 	auto mfmas_dma = [&](int buf, int step, int piece0) {
 #pragma unroll
-		for (int i = 0; i < 4; i++)
+		for (int i = 0; i < RT; i++)
 #pragma unroll
 			for (int j = 0; j < 4; j++) {
 				acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][i], fb[buf][j], acc[i][j], 0, 0, 0);
@@ -225,12 +231,12 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(Args g) {
 	const int col_l = lane & 31;
 	const int row_l = (lane >> 5) * 4;
 #pragma unroll
-	for (int i = 0; i < 4; i++) {
+	for (int i = 0; i < RT; i++) {
 #pragma unroll
 		for (int j = 0; j < 4; j++)
 #pragma unroll
 			for (int r = 0; r < 16; r++) ws[((r >> 2) * 8 + row_l + (r & 3)) * PITCH + j * 32 + col_l] = acc[i][j][r];
-		const int grow0 = m0 + wr * 128 + i * 32;
+		const int grow0 = m0 + wr * (RT * 32) + i * 32;
 		const int gcol0 = n0 + wc * 128;
 		if constexpr (EPI == EPI_BF16 || EPI == EPI_BF16_RESID) {
 #pragma unroll
@@ -269,27 +275,30 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(Args g) {
 	}
 }
 
-template <bool AT, bool BT, int EPI>
+template <int NW, bool AT, bool BT, int EPI>
 static int launch(const Args& a, hipStream_t stream) {
-	constexpr int smem = NST * STAGE_BYTES + 4 * 1024;  // ring + scratch target of the loads past the end of K
-	auto kern = gemm_dma_kernel<AT, BT, EPI>;
+	// ring + 1 KiB per wave as the target of the loads past the end of K; the epilogue needs a
+	// 32 x 136 fp32 strip per wave
+	constexpr int ring = NST * STAGE_BYTES + NW * 1024, epi = NW * 32 * 136 * 4;
+	constexpr int smem = ring > epi ? ring : epi;
+	auto kern = gemm_dma_kernel<NW, AT, BT, EPI>;
 	static bool attr_set = false;
 	if (!attr_set) {
 		ELF_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
 		attr_set = true;
 	}
-	hipLaunchKernelGGL(kern, dim3(a.tiles_m * a.tiles_n * a.k_splits), dim3(256), smem, stream, a);
+	hipLaunchKernelGGL(kern, dim3(a.tiles_m * a.tiles_n * a.k_splits), dim3(NW * 64), smem, stream, a);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
 }
 
-template <bool AT, bool BT>
+template <int NW, bool AT, bool BT>
 static int launch_epi(const Args& a, int epi, hipStream_t stream) {
 	switch (epi) {
-		case EPI_BF16: return launch<AT, BT, EPI_BF16>(a, stream);
-		case EPI_BF16_RESID: return launch<AT, BT, EPI_BF16_RESID>(a, stream);
-		case EPI_F32_ACC: return launch<AT, BT, EPI_F32_ACC>(a, stream);
-		case EPI_F32_STORE: return launch<AT, BT, EPI_F32_STORE>(a, stream);
+		case EPI_BF16: return launch<NW, AT, BT, EPI_BF16>(a, stream);
+		case EPI_BF16_RESID: return launch<NW, AT, BT, EPI_BF16_RESID>(a, stream);
+		case EPI_F32_ACC: return launch<NW, AT, BT, EPI_F32_ACC>(a, stream);
+		case EPI_F32_STORE: return launch<NW, AT, BT, EPI_F32_STORE>(a, stream);
 	}
 	set_error("gemm: unknown epilogue %d", epi);
 	return -1;
@@ -299,13 +308,20 @@ static int launch_epi(const Args& a, int epi, hipStream_t stream) {
 
 // Arguments are validated by gemm_bf16() before it dispatches here.
 int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda, const void* B, int64_t ldb, void* C,
-                  int64_t ldc, int epi, const void* R, int64_t ldr, int k_splits, hipStream_t stream) {
+                  int64_t ldc, int epi, const void* R, int64_t ldr, int k_splits, int waves, hipStream_t stream) {
+	ELF_REQUIRE(waves == 4 || waves == 8, "gemm (dma tile): 4 or 8 waves");
 	ELF_REQUIRE(M % dma::BM == 0 && N % dma::BN == 0 && K % dma::BKS == 0, "gemm (dma tile): M, N multiples of 256 and K of 64 required");
 	dma::Args a{(const bf16_t*)A, (const bf16_t*)B, C, (const bf16_t*)R, lda, ldb, ldc, ldr, M, N, K, M / dma::BM, N / dma::BN, k_splits < 1 ? 1 : k_splits};
 	if (epi != EPI_F32_ACC) a.k_splits = 1;
-	if (!a_t && !b_t) return dma::launch_epi<false, false>(a, epi, stream);
-	if (!a_t && b_t) return dma::launch_epi<false, true>(a, epi, stream);
-	if (a_t && b_t) return dma::launch_epi<true, true>(a, epi, stream);
+	if (waves == 4) {
+		if (!a_t && !b_t) return dma::launch_epi<4, false, false>(a, epi, stream);
+		if (!a_t && b_t) return dma::launch_epi<4, false, true>(a, epi, stream);
+		if (a_t && b_t) return dma::launch_epi<4, true, true>(a, epi, stream);
+	} else {
+		if (!a_t && !b_t) return dma::launch_epi<8, false, false>(a, epi, stream);
+		if (!a_t && b_t) return dma::launch_epi<8, false, true>(a, epi, stream);
+		if (a_t && b_t) return dma::launch_epi<8, true, true>(a, epi, stream);
+	}
 	set_error("gemm: layout A=T,B=R is not used by any stage contraction");
 	return -1;
 }

@@ -40,10 +40,10 @@ def K():
 
 @pytest.mark.parametrize("layout", ["nt", "nn", "tn"])
 @pytest.mark.parametrize("shape", [(256, 256, 64), (512, 768, 256), (1024, 2304, 768), (2048, 1024, 4096)])
-@pytest.mark.parametrize("tile_cfg", [0, 1, 2, 3, 5])
+@pytest.mark.parametrize("tile_cfg", [0, 1, 2, 3, 5, 6, 7])
 def test_gemm_layouts(K, layout, shape, tile_cfg):
 	M, N, Kd = shape
-	if tile_cfg in (1, 5) and (M % 256 or N % 256):
+	if tile_cfg in (1, 5, 6, 7) and (M % 256 or N % 256):
 		pytest.skip("tile does not divide")
 	A = _randn(M, Kd, seed=1)
 	B = _randn(N, Kd, seed=2, scale=0.05)
