@@ -24,6 +24,10 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA peak
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per GEMM launch (mean over the launches of one step), from rocprofv3 --pmc FETCH_SIZE and
+# --pmc WRITE_SIZE runs of this script scaled by the same counters' reading for a copy kernel of known
+# size (--calibration-copy); measured per workload, None where it was not.
+GEMM_TRAFFIC_BYTES = {"llama3_8b_zbh1": 1.588e9}
 
 WORKLOADS = {
 	# BASELINE.json configs[2]: Llama-3-8B-shaped stage, ZB-H1 stream of block 1 in a 4-stage pipeline
@@ -112,6 +116,8 @@ def main():
 	ap.add_argument("--warmup", type=int, default=1)
 	ap.add_argument("--workload", default="llama3_8b_zbh1", choices=sorted(WORKLOADS))
 	ap.add_argument("--no-cpu-baseline", action="store_true")
+	ap.add_argument("--calibration-copy", action="store_true",
+	                help="also launch one elf::add_kernel over 2 x 128 MiB in, 128 MiB out: a kernel of known HBM traffic to scale profiler byte counters with")
 	args = ap.parse_args()
 	if args.gpus != 1:
 		print("bench.py: this build runs one stage on ONE GPU; --gpus must be 1 (multi-GPU sharding is design-only).", file=sys.stderr)
@@ -143,6 +149,14 @@ def main():
 		block.zero_grad()
 		engine.train_step(None, None, None, stream, mb_sizes)
 
+	if args.calibration_copy:
+		from elf_amd import kernels
+		n = 64 * 1024 * 1024
+		ca = torch.ones(n, dtype=torch.bfloat16, device="cuda")
+		cb = torch.ones(n, dtype=torch.bfloat16, device="cuda")
+		kernels.add(ca, cb)
+		torch.cuda.synchronize()
+		del ca, cb
 	for _ in range(args.warmup):
 		step()
 	torch.cuda.synchronize()
@@ -175,8 +189,8 @@ def main():
 			"seq_len": w["seq"], "micro_batch": w["mb"], "n_micro_batches": w["n_mb"], "op_stream": f"{w['scheduler']} block {BLOCK_ID} of placement {PLACEMENT}",
 			"tokens_per_step": tokens, "ops_per_step": len(stream), "offload": bool(w.get("offload")),
 		},
-		"roofline": {"bound": "mfma", "achieved": g["tflops"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": g["tflops"] / PEAK_BF16_TFLOPS, "traffic": None,
-		             "kernel": "elf::gemm_kernel (bf16 MFMA GEMM, all layouts)", "launches": g["launches"], "avg_launch_ms": g["avg_ms"]},
+		"roofline": {"bound": "mfma", "achieved": g["tflops"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": g["tflops"] / PEAK_BF16_TFLOPS, "traffic": GEMM_TRAFFIC_BYTES.get(args.workload),
+		             "kernel": "elf::dma::gemm_dma_kernel / elf::gemm_kernel (bf16 MFMA GEMM, all layouts)", "launches": g["launches"], "avg_launch_ms": g["avg_ms"]},
 		"stream_mfu": stream_flops(w) / (elapsed / args.steps) / (PEAK_BF16_TFLOPS * 1e12),
 		"kernels": per_kernel,
 		"peak_stage_memory_bytes": mem["peak_bytes"] + torch.cuda.max_memory_allocated(),
