@@ -74,7 +74,7 @@ def op_stream(w):
 	from elf_amd.registry import COMM_SCHEDULERS, SCHEDULERS
 	from elf_amd.scheduling import add_comms, check_schedule_validity
 
-	sched = get_offloaded_scheduler(w["scheduler"], 1, 1) if w.get("offload") else SCHEDULERS[w["scheduler"]]
+	sched = get_offloaded_scheduler(w["scheduler"], 1, w.get("prefetching_time", 1)) if w.get("offload") else SCHEDULERS[w["scheduler"]]
 	schedule = COMM_SCHEDULERS["pipelined"](add_comms(sched(PLACEMENT, w["n_mb"]), sequential_signatures(PLACEMENT)))
 	check_schedule_validity(schedule)
 	return [op for op in schedule if op.block_id == BLOCK_ID]
@@ -116,6 +116,8 @@ def main():
 	ap.add_argument("--warmup", type=int, default=1)
 	ap.add_argument("--workload", default="llama3_8b_zbh1", choices=sorted(WORKLOADS))
 	ap.add_argument("--no-cpu-baseline", action="store_true")
+	ap.add_argument("--prefetching-time", type=int, default=None,
+	                help="offload workloads: how many compute ops before its B a micro-batch's PREFETCH_ACTIVATIONS is placed (reference default 1)")
 	ap.add_argument("--calibration-copy", action="store_true",
 	                help="also launch one elf::add_kernel over 2 x 128 MiB in, 128 MiB out: a kernel of known HBM traffic to scale profiler byte counters with")
 	args = ap.parse_args()
@@ -133,7 +135,9 @@ def main():
 		print("bench.py: no GPU visible; the stage kernels have no CPU path.", file=sys.stderr)
 		sys.exit(1)
 	lib = _lib.load()
-	w = WORKLOADS[args.workload]
+	w = dict(WORKLOADS[args.workload])
+	if args.prefetching_time is not None:
+		w["prefetching_time"] = args.prefetching_time
 	stage = build_stage(w)
 	cpu_stats = None
 	if not args.no_cpu_baseline:
@@ -161,6 +165,7 @@ def main():
 		step()
 	torch.cuda.synchronize()
 	lib.elf_prof_enable(1)
+	mem_before = block.mem_stats()
 	t0 = time.perf_counter()
 	for _ in range(args.steps):
 		step()
@@ -196,6 +201,13 @@ def main():
 		"peak_stage_memory_bytes": mem["peak_bytes"] + torch.cuda.max_memory_allocated(),
 		"stash_peak_bytes": mem["peak_bytes"], "offload_d2h_bytes": mem["d2h_bytes"], "offload_h2d_bytes": mem["h2d_bytes"],
 	}
+	if w.get("offload"):
+		# bytes moved by the side-stream copies of the timed steps over the steps' wall time: the
+		# rate the host link sustained while overlapped with the kernels (both directions at once)
+		d2h = mem["d2h_bytes"] - mem_before["d2h_bytes"]
+		h2d = mem["h2d_bytes"] - mem_before["h2d_bytes"]
+		out["host_link"] = {"d2h_gbs": d2h / elapsed / 1e9, "h2d_gbs": h2d / elapsed / 1e9, "d2h_bytes_per_step": d2h / args.steps,
+		                    "h2d_bytes_per_step": h2d / args.steps, "prefetching_time": w.get("prefetching_time", 1)}
 	if cpu_stats is not None:
 		out["cpu_baseline"] = cpu_stats
 	print(json.dumps(out))

@@ -57,6 +57,9 @@ struct Buf {
 
 struct BlockState {
 	Buf b[B_COUNT];
+	// offload copies run block by block: this block's device->host copies are done at off_ev,
+	// its host->device copies at pre_ev
+	hipEvent_t off_ev = nullptr, pre_ev = nullptr;
 };
 
 struct MbState {
@@ -64,7 +67,6 @@ struct MbState {
 	bool has_acts = false, has_win = false, has_wgrad = false;
 	bool remat_root = false;  // forward kept nothing: B re-runs it
 	bool offloaded = false, prefetched = false;
-	hipEvent_t off_ev = nullptr, pre_ev = nullptr;
 };
 
 struct BlockParams {
@@ -137,13 +139,17 @@ static MbState& mb_state(Stage* s, int mb) {
 }
 
 static void destroy_events(MbState& m) {
-	if (m.off_ev) (void)hipEventDestroy(m.off_ev);
-	if (m.pre_ev) (void)hipEventDestroy(m.pre_ev);
-	m.off_ev = m.pre_ev = nullptr;
+	for (auto& bs : m.blk) {
+		if (bs.off_ev) (void)hipEventDestroy(bs.off_ev);
+		if (bs.pre_ev) (void)hipEventDestroy(bs.pre_ev);
+		bs.off_ev = bs.pre_ev = nullptr;
+	}
 }
 
+static int do_offload_block(Stage* s, BlockState& bs, hipStream_t st);
+
 // ---------------------------------------------------------------------------------------------
-static int run_forward(Stage* s, MbState& m, const void* x, void* y, FwdMode mode, hipStream_t st) {
+static int run_forward(Stage* s, MbState& m, const void* x, void* y, FwdMode mode, hipStream_t st, bool offload = false) {
 	const int nb = s->cfg.n_blocks;
 	const int T = s->T, d = s->d, F = s->F;
 	const int norm_kind = s->llama ? NORM_RMS : NORM_LAYER;
@@ -195,9 +201,15 @@ static int run_forward(Stage* s, MbState& m, const void* x, void* y, FwdMode mod
 			for (int id = 0; id < B_COUNT; id++)
 				if ((ACT_MASK & (1u << id)) && !(keep & (1u << id))) buf_free(s, bs, id);
 		}
+		// the block's stash starts its way to the host while the next block computes
+		if (offload && mode == SAVE_ALL) ELF_TRY(do_offload_block(s, bs, st));
 	}
 	m.has_acts = mode == SAVE_ALL;
 	m.has_win = mode != SAVE_NONE;
+	if (offload && mode == SAVE_ALL) {
+		m.offloaded = true;
+		m.prefetched = false;
+	}
 	return 0;
 }
 
@@ -218,6 +230,7 @@ static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool gra
 			bs.b[B_DY].bytes = s->buf_bytes(B_DY);
 		}
 		const void* dyin = bs.b[B_DY].p;
+		if (m.offloaded && m.prefetched && bs.pre_ev) ELF_CHECK_HIP(hipStreamWaitEvent(st, bs.pre_ev, 0));
 		// FFN
 		void* d_a = s->pool.alloc((size_t)T * F * 2);
 		if (!d_a) return -3;
@@ -291,30 +304,33 @@ static int run_backward_params(Stage* s, MbState& m, hipStream_t st) {
 // Offload (elf/execution/offload.py:228-268, 330-390): every stage-owned activation buffer of
 // more than 1 MiB goes to the pinned arena on the offload stream; the device copy returns to the
 // pool once that copy has finished.
-static int do_offload(Stage* s, MbState& m, hipStream_t st) {
-	if (!m.has_acts || m.offloaded) return 0;
+static int do_offload_block(Stage* s, BlockState& bs, hipStream_t st) {
 	hipEvent_t ready;
 	ELF_CHECK_HIP(hipEventCreateWithFlags(&ready, hipEventDisableTiming));
 	ELF_CHECK_HIP(hipEventRecord(ready, st));
 	ELF_CHECK_HIP(hipStreamWaitEvent(s->offload_stream, ready, 0));
 	ELF_CHECK_HIP(hipEventDestroy(ready));
-	if (!m.off_ev) ELF_CHECK_HIP(hipEventCreateWithFlags(&m.off_ev, hipEventDisableTiming));
+	if (!bs.off_ev) ELF_CHECK_HIP(hipEventCreateWithFlags(&bs.off_ev, hipEventDisableTiming));
 	std::vector<void*> to_free;
-	for (auto& bs : m.blk) {
-		for (int id = 0; id < B_COUNT; id++) {
-			Buf& b = bs.b[id];
-			if (!(ACT_MASK & (1u << id)) || !b.p || !b.owned || b.bytes <= (size_t(1) << 20)) continue;
-			if (!s->pinned->allocate((int64_t)(b.bytes / 2), 2, /*bf16*/ 1, &b.host)) return -3;
-			ELF_CHECK_HIP(hipMemcpyAsync(b.host.ptr, b.p, b.bytes, hipMemcpyDeviceToHost, s->offload_stream));
-			s->d2h_bytes += (int64_t)b.bytes;
-			to_free.push_back(b.p);
-			b.p = nullptr;
-			b.owned = false;
-			b.offloaded = true;
-		}
+	for (int id = 0; id < B_COUNT; id++) {
+		Buf& b = bs.b[id];
+		if (!(ACT_MASK & (1u << id)) || !b.p || !b.owned || b.bytes <= (size_t(1) << 20)) continue;
+		if (!s->pinned->allocate((int64_t)(b.bytes / 2), 2, /*bf16*/ 1, &b.host)) return -3;
+		ELF_CHECK_HIP(hipMemcpyAsync(b.host.ptr, b.p, b.bytes, hipMemcpyDeviceToHost, s->offload_stream));
+		s->d2h_bytes += (int64_t)b.bytes;
+		to_free.push_back(b.p);
+		b.p = nullptr;
+		b.owned = false;
+		b.offloaded = true;
 	}
-	ELF_CHECK_HIP(hipEventRecord(m.off_ev, s->offload_stream));
-	for (void* p : to_free) s->pool.free_after(p, m.off_ev);
+	ELF_CHECK_HIP(hipEventRecord(bs.off_ev, s->offload_stream));
+	for (void* p : to_free) s->pool.free_after(p, bs.off_ev);
+	return 0;
+}
+
+static int do_offload(Stage* s, MbState& m, hipStream_t st) {
+	if (!m.has_acts || m.offloaded) return 0;
+	for (auto& bs : m.blk) ELF_TRY(do_offload_block(s, bs, st));
 	m.offloaded = true;
 	m.prefetched = false;
 	return 0;
@@ -322,7 +338,8 @@ static int do_offload(Stage* s, MbState& m, hipStream_t st) {
 
 // Bring offloaded buffers back: on the prefetch stream (async = true, PREFETCH_ACTIVATIONS) or on
 // the compute stream when B finds them still on the host (the reference restores synchronously
-// in that case, offload.py:281-283).
+// in that case, offload.py:281-283).  Blocks come back in the order B walks them (last first),
+// each with its own event, so B starts on the last block while the first is still on the link.
 static int do_restore(Stage* s, MbState& m, bool async, hipStream_t st) {
 	if (!m.offloaded || m.prefetched) return 0;
 	hipStream_t cs = async ? s->prefetch_stream : st;
@@ -342,17 +359,22 @@ static int do_restore(Stage* s, MbState& m, bool async, hipStream_t st) {
 		ELF_CHECK_HIP(hipStreamWaitEvent(cs, now, 0));
 		ELF_CHECK_HIP(hipEventDestroy(now));
 	}
-	ELF_CHECK_HIP(hipStreamWaitEvent(cs, m.off_ev, 0));
-	for (auto& bs : m.blk)
+	for (int i = (int)m.blk.size() - 1; i >= 0; i--) {
+		BlockState& bs = m.blk[i];
+		if (bs.off_ev) ELF_CHECK_HIP(hipStreamWaitEvent(cs, bs.off_ev, 0));
 		for (int id = 0; id < B_COUNT; id++) {
 			Buf& b = bs.b[id];
 			if (!b.offloaded) continue;
 			ELF_CHECK_HIP(hipMemcpyAsync(b.p, b.host.ptr, b.bytes, hipMemcpyHostToDevice, cs));
 			s->h2d_bytes += (int64_t)b.bytes;
 		}
-	if (async) {
-		if (!m.pre_ev) ELF_CHECK_HIP(hipEventCreateWithFlags(&m.pre_ev, hipEventDisableTiming));
-		ELF_CHECK_HIP(hipEventRecord(m.pre_ev, cs));
+		if (async) {
+			if (!bs.pre_ev) ELF_CHECK_HIP(hipEventCreateWithFlags(&bs.pre_ev, hipEventDisableTiming));
+			ELF_CHECK_HIP(hipEventRecord(bs.pre_ev, cs));
+		} else if (bs.pre_ev) {
+			(void)hipEventDestroy(bs.pre_ev);
+			bs.pre_ev = nullptr;
+		}
 	}
 	m.prefetched = true;
 	return 0;
@@ -360,8 +382,10 @@ static int do_restore(Stage* s, MbState& m, bool async, hipStream_t st) {
 
 static int do_release(Stage* s, MbState& m) {
 	if (!m.offloaded) return 0;
-	if (m.pre_ev) ELF_CHECK_HIP(hipEventSynchronize(m.pre_ev));
-	else if (m.off_ev && !m.prefetched) ELF_CHECK_HIP(hipEventSynchronize(m.off_ev));
+	for (auto& bs : m.blk) {
+		if (m.prefetched && bs.pre_ev) ELF_CHECK_HIP(hipEventSynchronize(bs.pre_ev));
+		else if (bs.off_ev) ELF_CHECK_HIP(hipEventSynchronize(bs.off_ev));
+	}
 	for (auto& bs : m.blk)
 		for (int id = 0; id < B_COUNT; id++) {
 			Buf& b = bs.b[id];
@@ -473,10 +497,9 @@ int elf_stage_forward(elf_stage_t* h, int mb, const void* x, void* y, uint32_t f
 	MbState& m = mb_state(s, mb);
 	ELF_REQUIRE(!m.has_acts && !m.has_win && !m.has_wgrad && !m.remat_root, "elf_stage_forward: micro-batch %d is already in flight", mb);
 	const bool root = flags & ELF_FWD_REMAT_ROOT;
-	ELF_TRY(run_forward(s, m, x, y, root ? SAVE_NONE : SAVE_ALL, (hipStream_t)stream));
+	ELF_TRY(run_forward(s, m, x, y, root ? SAVE_NONE : SAVE_ALL, (hipStream_t)stream, (flags & ELF_FWD_OFFLOAD) && !root));
 	m.remat_root = root;
 	if (root) m.has_win = false;
-	if ((flags & ELF_FWD_OFFLOAD) && !root) ELF_TRY(do_offload(s, m, (hipStream_t)stream));
 	return 0;
 }
 
@@ -499,8 +522,7 @@ int elf_stage_backward_inputs(elf_stage_t* h, int mb, const void* x, const void*
 	}
 	ELF_REQUIRE(m.has_acts, "elf_stage_backward_inputs: micro-batch %d has no saved activations", mb);
 	if (m.offloaded) {
-		if (m.prefetched && m.pre_ev) ELF_CHECK_HIP(hipStreamWaitEvent(st, m.pre_ev, 0));
-		else ELF_TRY(do_restore(s, m, false, st));
+		if (!m.prefetched) ELF_TRY(do_restore(s, m, false, st));  // run_backward waits block by block otherwise
 	}
 	if (x) m.blk[0].b[B_X].p = const_cast<void*>(x);
 	ELF_TRY(run_backward(s, m, dy, dx, false, st));
