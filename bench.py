@@ -42,6 +42,11 @@ WORKLOADS = {
 	# BASELINE.json configs[4]: Llama-3-70B-shaped stage, 1F1B with activation offload
 	"llama3_70b_offload": dict(arch="llama", n_blocks=2, d=8192, heads=64, kv_heads=8, head_dim=128, ffn=28672, seq=8192, mb=1, n_mb=8,
 	                           scheduler="1f1b", causal=True, rope_theta=5e5, offload=True),
+	# BASELINE.json configs[3]: the Llama-3-8B-shaped stage with 8 blocks at seq 8192 under a 48 GB budget: the stage is
+	# profiled on the native executor, the remat ILP is solved for a pipeline of 8 such stages (the other stages are
+	# copies of the measured one) and block 1's rewritten 1F1B stream runs
+	"llama3_8b_remat": dict(arch="llama", n_blocks=8, d=4096, heads=32, kv_heads=8, head_dim=128, ffn=14336, seq=8192, mb=1, n_mb=16,
+	                        scheduler="1f1b", causal=True, rope_theta=5e5, placement=list(range(8)), memory_budget_mib=48e9 / 2**20),
 	# small shape for smoke runs
 	"tiny": dict(arch="llama", n_blocks=2, d=512, heads=4, kv_heads=2, head_dim=128, ffn=768, seq=256, mb=2, n_mb=4,
 	             scheduler="zbh1", causal=True, rope_theta=5e5),
@@ -68,14 +73,16 @@ def build_stage(w):
 	return models.gpt_stage(w["n_blocks"], w["d"], w["heads"], w["ffn"], w["seq"], causal=w["causal"], seed=0)
 
 
-def op_stream(w):
+def op_stream(w, sched=None):
 	from elf_amd.benchmark_utils import get_offloaded_scheduler
 	from elf_amd.partitioners.utils import sequential_signatures
 	from elf_amd.registry import COMM_SCHEDULERS, SCHEDULERS
 	from elf_amd.scheduling import add_comms, check_schedule_validity
 
-	sched = get_offloaded_scheduler(w["scheduler"], 1, w.get("prefetching_time", 1)) if w.get("offload") else SCHEDULERS[w["scheduler"]]
-	schedule = COMM_SCHEDULERS["pipelined"](add_comms(sched(PLACEMENT, w["n_mb"]), sequential_signatures(PLACEMENT)))
+	placement = w.get("placement", PLACEMENT)
+	if sched is None:
+		sched = get_offloaded_scheduler(w["scheduler"], 1, w.get("prefetching_time", 1)) if w.get("offload") else SCHEDULERS[w["scheduler"]]
+	schedule = COMM_SCHEDULERS["pipelined"](add_comms(sched(placement, w["n_mb"]), sequential_signatures(placement)))
 	check_schedule_validity(schedule)
 	return [op for op in schedule if op.block_id == BLOCK_ID]
 
@@ -142,10 +149,28 @@ def main():
 	cpu_stats = None
 	if not args.no_cpu_baseline:
 		cpu_stats = cpu_baseline(w, stage)
-	block = HipStageBlock(stage, BLOCK_ID, PLACEMENT, sequential_signatures(PLACEMENT)[BLOCK_ID], mb_size=w["mb"])
+	placement = w.get("placement", PLACEMENT)
+	block = HipStageBlock(stage, BLOCK_ID, placement, sequential_signatures(placement)[BLOCK_ID], mb_size=w["mb"])
 	xs, dys = make_boundary(w["mb"], w["seq"], w["d"], w["n_mb"], seed=1, device="cuda")
 	block.set_boundary(inputs=xs, grads=dys)
-	stream = op_stream(w)
+	remat = None
+	if w.get("memory_budget_mib"):
+		from elf_amd.registry import SCHEDULERS
+		from elf_amd.scheduling.ilp import RematScheduler, profile_stage, solve_remat
+
+		stats, _ = profile_stage(block, n_iter=3)
+		t_ilp = time.perf_counter()
+		solution = solve_remat([stats] * len(placement), placement, SCHEDULERS[w["scheduler"]], w["n_mb"], w["memory_budget_mib"])
+		t_ilp = time.perf_counter() - t_ilp
+		remat = {
+			"memory_budget_mib": w["memory_budget_mib"], "ilp_seconds": t_ilp, "ilp_makespan_ms": solution["objective"],
+			"ilp_peak_mib_rank": solution["peak_mems"][placement[BLOCK_ID]],
+			"decisions_block": {k: int(sum(solution[k][BLOCK_ID])) for k in ("full_fwd", "activations_bwd", "full_bwd")},
+			"profile": {k: stats[k] for k in ("T", "M", "Mpeak", "Mpeak_ckpt", "Mparams", "Mba", "Mbg", "Minput")},
+		}
+		stream = op_stream(w, RematScheduler(SCHEDULERS[w["scheduler"]], solution))
+	else:
+		stream = op_stream(w)
 	engine = Engine([block])
 	mb_sizes = [w["mb"]] * w["n_mb"]
 
@@ -191,7 +216,7 @@ def main():
 		"vs_baseline": None, "dtype": "bf16", "data": "synthetic",
 		"config": {
 			"workload": args.workload, "blocks": w["n_blocks"], "d_model": w["d"], "heads": w["heads"], "kv_heads": w["kv_heads"], "ffn": w["ffn"],
-			"seq_len": w["seq"], "micro_batch": w["mb"], "n_micro_batches": w["n_mb"], "op_stream": f"{w['scheduler']} block {BLOCK_ID} of placement {PLACEMENT}",
+			"seq_len": w["seq"], "micro_batch": w["mb"], "n_micro_batches": w["n_mb"], "op_stream": f"{w['scheduler']} block {BLOCK_ID} of placement {placement}",
 			"tokens_per_step": tokens, "ops_per_step": len(stream), "offload": bool(w.get("offload")),
 		},
 		"roofline": {"bound": "mfma", "achieved": g["tflops"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": g["tflops"] / PEAK_BF16_TFLOPS, "traffic": GEMM_TRAFFIC_BYTES.get(args.workload),
@@ -201,6 +226,8 @@ def main():
 		"peak_stage_memory_bytes": mem["peak_bytes"] + torch.cuda.max_memory_allocated(),
 		"stash_peak_bytes": mem["peak_bytes"], "offload_d2h_bytes": mem["d2h_bytes"], "offload_h2d_bytes": mem["h2d_bytes"],
 	}
+	if remat is not None:
+		out["remat"] = remat
 	if w.get("offload"):
 		# bytes moved by the side-stream copies of the timed steps over the steps' wall time: the
 		# rate the host link sustained while overlapped with the kernels (both directions at once)

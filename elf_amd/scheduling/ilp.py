@@ -22,7 +22,7 @@ from .scheduling import Operation, OperationType, OpOptions
 
 logger = logging.getLogger("ilp")
 
-__all__ = ["build_ilp_params", "solve_remat", "evaluate_remat", "RematScheduler", "stagerematify", "AutoScheduler", "RematOption"]
+__all__ = ["build_ilp_params", "solve_remat", "evaluate_remat", "RematScheduler", "stagerematify", "AutoScheduler", "RematOption", "profile_stage"]
 
 _OPS = ("f", "b", "w")
 _KIND = {OperationType.FORWARD: "f", OperationType.BACKWARD_INPUTS: "b", OperationType.BACKWARD_PARAMS: "w"}
@@ -34,6 +34,132 @@ class RematOption:
 
 	def __repr__(self):
 		return f"RematOption({self.name!r}, {self.type!r}, mem_freed={self.mem_freed}, time_overhead={self.time_overhead})"
+
+
+def profile_stage(stage, sample_metadata=None, n_iter=10):
+	"""Profiling record of one stage for the ILP, measured on the native executor
+	(elf/scheduling/ilp.py:50-126 ``_measure_full_pass``, :224-254 ``profile_stage``).
+
+	``stage`` is a ``HipStageBlock``.  One warm-up pass, then ``n_iter`` passes of F, B, W on a
+	reserved micro-batch slot with N(0,1) boundary tensors; medians are reported:
+
+	T[f|b|w]      ms, event pairs on the launch stream
+	M[f|b|w]      MiB still held after the op, relative to before F (after F: output + stash;
+	              after B: the W stash; after W: 0)
+	Mpeak[f|b|w]  MiB high-water mark during the op (relative to before F for f, to before the op
+	              for b and w, as in the reference)
+	Mpeak_ckpt    the same for a forward that keeps nothing (whole-stage checkpoint)
+	Mba / Mbg     the two halves of the W stash after B: layer inputs / output gradients
+	Minput, Moutput  boundary tensor sizes;  Tcomm 0 (no transfers on one GPU)
+	Mparams       MiB of the bf16 weights x 1.5: the ILP charges 2 x Mparams per stage for weights +
+	              gradients, and this executor keeps bf16 weights plus fp32 accumulators (6 B/param)
+
+	Memory = bytes held by the stage library (stash + temporaries) + torch's allocator (boundary
+	tensors).  Returns ``(stats, next_stage_input)`` like the reference (warm-up output on the CPU).
+	"""
+	import ctypes
+
+	import torch
+
+	from .. import _lib
+	from ..execution.block import BWD_RECOMPUTE_GRADIENTS, FWD_REMAT_ROOT
+
+	block, lib = stage, stage.lib
+	h = block._handle
+	mb = 1 << 20  # a slot no schedule uses
+	stream = torch.cuda.current_stream().cuda_stream
+	MiB = 1024.0 * 1024.0
+	x = torch.randn(block.T, block.d, device="cuda").to(torch.bfloat16)
+	dy = torch.randn_like(x, dtype=torch.float32).to(torch.bfloat16)
+
+	def held():
+		return torch.cuda.memory_allocated() + block.mem_stats()["live_bytes"]
+
+	def peak():
+		return torch.cuda.max_memory_allocated() + block.mem_stats()["peak_bytes"]
+
+	def reset():
+		torch.cuda.reset_peak_memory_stats()
+		block.reset_peak()
+
+	def timed(fn):
+		e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+		e0.record()
+		fn()
+		e1.record()
+		e1.synchronize()
+		return e0.elapsed_time(e1)
+
+	def fwd(y, flags=0):
+		_lib.check(lib.elf_stage_forward(h, mb, x.data_ptr(), y.data_ptr(), flags, stream), "elf_stage_forward")
+
+	def bwd(dx, flags=0):
+		_lib.check(lib.elf_stage_backward_inputs(h, mb, x.data_ptr(), dy.data_ptr(), dx.data_ptr(), flags, stream), "elf_stage_backward_inputs")
+
+	def wgrad():
+		_lib.check(lib.elf_stage_backward_params(h, mb, stream), "elf_stage_backward_params")
+
+	saved_grads = [g.clone() for g in block._fused_g]  # the passes below accumulate into main_grad
+	y = torch.empty_like(x)
+	fwd(y)
+	warmup_output = y.detach().cpu()
+	dx = torch.empty_like(x)
+	bwd(dx)
+	wgrad()
+	del y, dx
+	torch.cuda.synchronize()
+
+	times, mems, peaks = ({k: [] for k in _OPS} for _ in range(3))
+	for _ in range(n_iter):
+		reset()
+		start = held()
+		y = torch.empty_like(x)
+		times["f"].append(timed(lambda: fwd(y)))
+		mems["f"].append((held() - start) / MiB)
+		peaks["f"].append((peak() - start) / MiB)
+		reset()
+		before = held()
+		dx = torch.empty_like(x)
+		times["b"].append(timed(lambda: bwd(dx)))
+		del y, dx
+		mems["b"].append((held() - start) / MiB)
+		peaks["b"].append((peak() - before) / MiB)
+		reset()
+		before = held()
+		times["w"].append(timed(wgrad))
+		mems["w"].append((held() - start) / MiB)
+		peaks["w"].append((peak() - before) / MiB)
+	med = lambda d: {k: float(np.median(v)) for k, v in d.items()}
+	T, M, Mpeak = med(times), med(mems), med(peaks)
+
+	# whole-stage checkpoint forward
+	reset()
+	start = held()
+	y = torch.empty_like(x)
+	fwd(y, FWD_REMAT_ROOT)
+	torch.cuda.synchronize()
+	peak_ckpt = (peak() - start) / MiB
+	# B re-runs the forward of a checkpointed micro-batch; with recompute_gradients it leaves only the
+	# layer-input half of the W stash behind: that is Mba
+	start = held() - y.numel() * 2
+	dx = torch.empty_like(x)
+	bwd(dx, BWD_RECOMPUTE_GRADIENTS)
+	torch.cuda.synchronize()
+	del dx, y
+	mba = (held() - start) / MiB
+	_lib.check(lib.elf_stage_clear(h), "elf_stage_clear")
+	for g, keep in zip(block._fused_g, saved_grads):
+		g.copy_(keep)
+	torch.cuda.synchronize()
+
+	nbytes = x.numel() * 2
+	stats = {
+		"T": T, "M": M, "Mpeak": Mpeak, "Mpeak_ckpt": peak_ckpt,
+		"Mparams": 1.5 * sum(w.numel() * 2 for w in block._fused_w) / MiB,
+		"Mba": mba, "Mbg": M["b"] - mba, "Minput": nbytes / MiB, "Moutput": nbytes / MiB, "Tcomm": 0.0,
+		"forward_remat_options": [], "backward_remat_options": [],
+	}
+	return stats, warmup_output
 
 
 def _simplified_schedule(placement, n_micro_batches, scheduler):

@@ -185,6 +185,65 @@ def test_engine_runs_1f1b_and_zbh1_streams():
 		assert set(stats) == {"total", "idle", "start_idle", "end_idle", "bubble"}
 
 
+def test_profile_stage_feeds_the_remat_ilp_and_the_stream_fits_the_budget():
+	"""profile_stage on the native executor (reference: elf/scheduling/ilp.py:50-126, 224-254): the
+	record is self-consistent, the ILP solved from it picks remat under a budget between the
+	full-remat and no-remat peaks, and block 1's rewritten stream runs within that budget with the
+	gradients of the plain stream."""
+	from elf_amd.execution import Engine
+	from elf_amd.partitioners.utils import sequential_signatures
+	from elf_amd.registry import COMM_SCHEDULERS, SCHEDULERS
+	from elf_amd.scheduling import add_comms
+	from elf_amd.scheduling.ilp import RematScheduler, evaluate_remat, build_ilp_params, profile_stage, solve_remat
+
+	mb, nmb, placement = 2, 6, [0, 1, 2, 3]
+	stage = _stage("llama")
+	blk = _block(stage, mb)
+	blk.zero_grad()
+	stats, nxt = profile_stage(blk, n_iter=2)
+	assert tuple(nxt.shape) == (blk.T, blk.d) and nxt.device.type == "cpu"
+	assert all(stats["T"][k] > 0 for k in "fbw")
+	assert stats["M"]["w"] == 0.0 and stats["Mpeak"]["f"] >= stats["M"]["f"] > stats["Mpeak_ckpt"] > 0
+	assert stats["Mba"] > 0 and stats["Mbg"] > 0 and abs(stats["Mba"] + stats["Mbg"] - stats["M"]["b"]) < 1e-6
+	assert all(float(g.abs().max()) == 0.0 for g in blk._fused_g), "profiling must leave the accumulators as it found them"
+	assert blk.mem_stats()["live_bytes"] == 0
+
+	base = SCHEDULERS["1f1b"]
+	statistics = [stats] * len(placement)
+	params = build_ilp_params(statistics, placement, base, nmb, 1e9)
+	zeros = {k: [[0.0] * nmb for _ in placement] for k in ("full_fwd", "activations_bwd", "full_bwd")}
+	ones = dict(zeros, full_fwd=[[1.0] * nmb for _ in placement])
+	peak_plain, peak_remat = max(evaluate_remat(params, zeros)[1]), max(evaluate_remat(params, ones)[1])
+	assert peak_remat < peak_plain
+	budget = 0.5 * (peak_plain + peak_remat)
+	solution = solve_remat(statistics, placement, base, nmb, budget, time_limit=20)
+	assert max(solution["peak_mems"]) <= budget + 1e-6
+	assert sum(map(sum, solution["full_fwd"])) + sum(map(sum, solution["activations_bwd"])) + sum(map(sum, solution["full_bwd"])) > 0
+
+	def run(scheduler):
+		b = _block(_stage("llama"), mb)
+		b.zero_grad()
+		xs, dys = b_xs
+		b.set_boundary(inputs=xs, grads=dys)
+		schedule = COMM_SCHEDULERS["pipelined"](add_comms(scheduler(placement, nmb), sequential_signatures(placement)))
+		stream = [op for op in schedule if op.block_id == 1]
+		b.reset_peak()
+		Engine([b]).train_step(None, None, None, stream, [mb] * nmb)
+		torch.cuda.synchronize()
+		return product_grads(b.model), b.mem_stats()["peak_bytes"]
+
+	from elf_amd.synthetic import make_boundary
+
+	b_xs = make_boundary(mb, stage.seq_len, blk.d, nmb, seed=5, device="cuda")
+	g_plain, peak_plain_run = run(base)
+	g_remat, peak_remat_run = run(RematScheduler(base, solution))
+	assert peak_remat_run < peak_plain_run
+	# what the library held at its high-water mark + weights and accumulators stays under the budget
+	assert peak_remat_run / 2**20 + 2 * stats["Mparams"] <= budget + 1.0
+	for name in sorted(g_plain):
+		assert_close(g_remat[name], g_plain[name], f"remat grad {name}", rel_max=2e-3, rel_fro=2e-3)
+
+
 def test_error_paths():
 	from elf_amd._lib import ElfStageError
 
