@@ -1,0 +1,89 @@
+"""``Pipeline`` over the native stage executor (reference API: elf/pipeline.py:97-295): two stages on
+one rank under AFAB, and one stage under ZB-H1, against the oracle stages driven by hand with the
+same loss.  Tolerances as for the stage tests (rel 2e-2 of max, 1e-2 Frobenius)."""
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from tests.helpers import assert_close, cfg_from_stage, oracle_params_from_stage, perturb_norms, product_grads
+
+pytestmark = pytest.mark.gpu
+
+
+def _stages(n):
+	from elf_amd import models
+
+	out = []
+	for i in range(n):
+		st = models.llama_stage(1, 256, 2, 1, 512, 128, head_dim=128, seed=20 + i)
+		perturb_norms(st)
+		out.append(st)
+	return out
+
+
+@pytest.mark.parametrize("case", [("afab", [0, 0]), ("zbh1", [0])])
+def test_pipeline_step_matches_oracle(case):
+	from elf_amd.pipeline import Pipeline, PipelineConfig
+	from oracle import stage_ref as R
+
+	sched, placement = case
+	mb, nmb = 2, 3
+	stages = _stages(len(placement))
+	refs = [R.RefStage(cfg_from_stage(st, mb), oracle_params_from_stage(st), device="cuda") for st in stages]
+	S, d = stages[0].seq_len, 256
+	g = torch.Generator().manual_seed(7)
+	batch = torch.randn(mb * nmb, S, d, generator=g).to(torch.bfloat16).cuda()
+	target = torch.randn(mb * nmb, S, d, generator=g).to(torch.bfloat16).cuda()
+
+	pipe = Pipeline(stages if len(stages) > 1 else stages[0], batch[:mb], config=PipelineConfig(scheduler=sched, partitioner=False, placement=placement))
+	assert pipe.is_first() and pipe.is_last() and [b.id for b in pipe.blocks] == list(range(len(placement)))
+	pipe.zero_grad()
+	result, loss = pipe(batch, target, F.mse_loss, split_size=mb)
+	assert len(result) == nmb and pipe.last_nmb == nmb
+	assert set(pipe.stats) == {"total", "idle", "start_idle", "end_idle", "bubble"}
+	assert list(pipe.detailed_stats["memories"]) == [str(op) for op in pipe.schedule]
+
+	want_loss = 0.0
+	for m in range(nmb):
+		x = batch[m * mb:(m + 1) * mb]
+		for ref in refs:
+			x = ref.forward(m, x)
+		y = x.detach().float().requires_grad_()
+		t = target[m * mb:(m + 1) * mb].float()
+		l = F.mse_loss(y, t, reduction="sum") / (S * d)
+		l.backward()
+		want_loss += float(l.detach())
+		assert_close(result[m].reshape(mb, S, d), x, f"{sched} output[{m}]")
+		dy = y.grad.to(torch.bfloat16)
+		for ref in reversed(refs):
+			dy = ref.backward_inputs(m, dy)
+		for ref in refs:
+			ref.backward_params(m)
+	for ref in refs:
+		ref.scale_grads(mb * nmb)
+	assert abs(float(loss) - want_loss / (mb * nmb)) <= 2e-2 * abs(want_loss / (mb * nmb))
+	for st, ref in zip(stages, refs):
+		got, want = product_grads(st), ref.grads()
+		for name in sorted(want):
+			assert_close(got[name], want[name], f"{sched} grad {name}")
+
+	# a second step with the same batch reuses the schedule and gives the same loss
+	pipe.zero_grad()
+	_, loss2 = pipe(batch, target, F.mse_loss, split_size=mb)
+	assert abs(float(loss2) - float(loss)) <= 1e-3 * abs(float(loss))
+	assert sum(p.numel() for p in pipe.parameters()) == sum(p.numel() for st in stages for p in st.parameters())
+	pipe.clear()
+
+
+def test_pipeline_rejects_what_this_build_does_not_run():
+	from elf_amd.pipeline import Pipeline
+
+	st = _stages(1)[0]
+	with pytest.raises(NotImplementedError):
+		Pipeline(st, torch.zeros(2, 128, 256), scheduler="afab", placement=[0])  # default partitioner needs a tracer
+	with pytest.raises(ValueError):
+		Pipeline(st, None, scheduler="afab", partitioner=False, placement=[0])  # no sample, no mb_size
+	pipe = Pipeline(st, None, scheduler="afab", partitioner=False, placement=[0], mb_size=2)
+	with pytest.raises(ValueError):
+		pipe(torch.zeros(6, 128, 256, dtype=torch.bfloat16, device="cuda"), None, None, split_size=3)
