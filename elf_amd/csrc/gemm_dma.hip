@@ -225,6 +225,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	// 32 x 128 fp32 strip at a time in its own LDS region (row pitch 136 floats: the two half-waves
 	// land on disjoint banks) and reads it back row-wise, so that global accesses are 16 bytes per
 	// lane over 256..512 contiguous bytes per row and accumulators leave the AGPRs only via ds_write.
+	wait_vmcnt<0>();  // the loads past the end of K issued by the last iterations land in LDS too
 	__syncthreads();
 	constexpr int PITCH = 136;
 	float* ws = reinterpret_cast<float*>(smem) + wave * (32 * PITCH);

@@ -1,0 +1,130 @@
+"""Properties that do not depend on size, checked at the benchmark's full shapes (Llama-3-8B-shaped
+stage: 8192 tokens per micro-batch, d_model 4096, 32 query / 8 kv heads of 128, FFN 14336), where
+an oracle run would take minutes.  Each property is one a wrong tile index, a dropped K slice, a
+mis-masked attention tile or a lost accumulation would break."""
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+T, D_MODEL, HQ, HKV, HD, FFN, SEQ = 8192, 4096, 32, 8, 128, 14336, 4096
+
+
+def _randn(*shape, seed=0, scale=1.0):
+	g = torch.Generator(device="cuda").manual_seed(seed)
+	return (torch.randn(*shape, generator=g, device="cuda") * scale).to(torch.bfloat16)
+
+
+@pytest.fixture(scope="module")
+def K():
+	from elf_amd import kernels
+
+	return kernels
+
+
+@pytest.mark.parametrize("layout", ["nt", "nn", "tn"])
+def test_gemm_row_and_column_probes_at_full_size(K, layout):
+	"""C = A B^T at 8192 x 14336 x 4096 (and the dW shape for tn): 64 sampled rows and columns of
+	the result equal their fp32 dot products; a one-hot A row selects a B column exactly."""
+	M, N, Kd = (T, FFN, D_MODEL) if layout != "tn" else (D_MODEL, FFN, T)
+	A = _randn(M, Kd, seed=1)
+	B = _randn(N, Kd, seed=2, scale=0.05)
+	A[7].zero_()
+	A[7, 1234] = 1.0  # row 7 of C must be column 1234 of B, bit for bit
+	if layout == "nt":
+		C = K.gemm(A, B)
+	elif layout == "nn":
+		C = K.gemm(A, B.t().contiguous(), b_t=True)
+	else:
+		C = K.gemm(A.t().contiguous(), B.t().contiguous(), a_t=True, b_t=True)
+	assert torch.equal(C[7], B[:, 1234])
+	rows = torch.randint(0, M, (64,), generator=torch.Generator().manual_seed(3)).cuda()
+	cols = torch.randint(0, N, (64,), generator=torch.Generator().manual_seed(4)).cuda()
+	ref_r = A[rows].float() @ B.float().t()
+	ref_c = A.float() @ B[cols].float().t()
+	for got, ref in ((C[rows].float(), ref_r), (C[:, cols].float(), ref_c)):
+		assert (got - ref).abs().max().item() <= 2e-2 * ref.abs().max().item()
+		assert ((got - ref).norm() / ref.norm()).item() <= 5e-3
+
+
+def test_gemm_fp32_accumulation_is_additive_at_full_size(K):
+	"""The deferred weight-gradient epilogue: three calls into one fp32 buffer = 3 x one call,
+	and the K-split variant (fp32 atomics) agrees with the unsplit one."""
+	dY = _randn(T, D_MODEL, seed=5, scale=0.1)
+	X = _randn(T, FFN, seed=6)
+	one = torch.zeros(D_MODEL, FFN, dtype=torch.float32, device="cuda")
+	K.gemm(dY, X, a_t=True, b_t=True, out=one, epilogue=K.EPI_F32_ACC, k_splits=1)
+	acc = torch.zeros_like(one)
+	for _ in range(3):
+		K.gemm(dY, X, a_t=True, b_t=True, out=acc, epilogue=K.EPI_F32_ACC, k_splits=1)
+	assert ((acc - 3 * one).abs().max() <= 1e-5 * one.abs().max()).item()
+	split = torch.zeros_like(one)
+	K.gemm(dY, X, a_t=True, b_t=True, out=split, epilogue=K.EPI_F32_ACC, k_splits=4)
+	assert ((split - one).norm() / one.norm()).item() <= 1e-5
+
+
+def test_attention_properties_at_full_size(K):
+	"""Causal GQA attention at batch 2 x seq 4096: (1) with V = 1 every output is 1 (rows of P sum
+	to one); (2) changing keys / values / queries after position p leaves outputs up to p unchanged
+	bit for bit; (3) dQ, dK, dV are linear in dO; (4) with dO = 0 all gradients vanish."""
+	B = 2
+	nq, nkv = HQ * HD, HKV * HD
+	qkv = _randn(B * SEQ, nq + 2 * nkv, seed=7, scale=0.5)
+	ones = qkv.clone()
+	ones[:, nq + nkv:] = 1.0
+	o, _ = K.attn_fwd(ones, B, SEQ, HQ, HKV, HD, True)
+	assert (o.float() - 1.0).abs().max().item() <= 1e-2
+	o_ref, lse = K.attn_fwd(qkv, B, SEQ, HQ, HKV, HD, True)
+	p = 2500
+	pert = qkv.clone()
+	pert.view(B, SEQ, -1)[:, p + 1:] = _randn(B, SEQ - p - 1, nq + 2 * nkv, seed=8)
+	o_pert, lse_pert = K.attn_fwd(pert, B, SEQ, HQ, HKV, HD, True)
+	assert torch.equal(o_pert.view(B, SEQ, -1)[:, :p + 1], o_ref.view(B, SEQ, -1)[:, :p + 1])
+	assert torch.equal(lse_pert[:, :, :p + 1], lse[:, :, :p + 1])
+	do1 = _randn(B * SEQ, nq, seed=9)
+	do2 = _randn(B * SEQ, nq, seed=10)
+	g1 = K.attn_bwd(qkv, o_ref, do1, lse, B, SEQ, HQ, HKV, HD, True).float()
+	g2 = K.attn_bwd(qkv, o_ref, do2, lse, B, SEQ, HQ, HKV, HD, True).float()
+	g12 = K.attn_bwd(qkv, o_ref, (do1.float() + do2.float()).to(torch.bfloat16), lse, B, SEQ, HQ, HKV, HD, True).float()
+	for name, sl in (("dq", slice(0, nq)), ("dk", slice(nq, nq + nkv)), ("dv", slice(nq + nkv, None))):
+		want = g1[:, sl] + g2[:, sl]
+		assert ((g12[:, sl] - want).norm() / want.norm()).item() <= 1.5e-2, name
+	g0 = K.attn_bwd(qkv, o_ref, torch.zeros_like(do1), lse, B, SEQ, HQ, HKV, HD, True)
+	assert g0.abs().max().item() == 0.0
+	# causality of the backward: a gradient that arrives only at positions <= p gives no dK / dV after p
+	do_head = do1.clone()
+	do_head.view(B, SEQ, -1)[:, p + 1:] = 0
+	gh = K.attn_bwd(qkv, o_ref, do_head, lse, B, SEQ, HQ, HKV, HD, True).view(B, SEQ, -1)
+	assert gh[:, p + 1:].abs().max().item() == 0.0
+
+
+def test_bandwidth_kernels_at_full_size(K):
+	"""RMSNorm output has unit RMS under gamma = 1; SwiGLU of (g, u) with u = 1 is silu(g); RoPE
+	keeps the norm of every (x_i, x_{i+D/2}) pair and its backward undoes its forward; the gradient
+	scale is exact in fp32."""
+	x = _randn(T, D_MODEL, seed=11) * 3.0
+	x = x.to(torch.bfloat16)
+	y, stats = K.norm_fwd(K.NORM_RMS, x, torch.ones(D_MODEL, dtype=torch.bfloat16, device="cuda"), None, 1e-5)
+	rms = y.float().pow(2).mean(-1).sqrt()
+	assert (rms - 1).abs().max().item() <= 5e-3
+	gu = _randn(T, 2 * FFN, seed=12)
+	gu[:, FFN:] = 1.0
+	h = K.swiglu_fwd(gu)
+	assert (h.float() - torch.nn.functional.silu(gu[:, :FFN].float())).abs().max().item() <= 2e-2
+	qkv = _randn(2 * SEQ, (HQ + 2 * HKV) * HD, seed=13)
+	before = qkv.clone()
+	cs = K.rope_table(SEQ, HD, 5e5)
+	K.rope_apply_(qkv, cs, SEQ, HQ + HKV, HD)
+	v0 = before[:, : (HQ + HKV) * HD].float().view(2 * SEQ, HQ + HKV, 2, HD // 2)
+	v1 = qkv[:, : (HQ + HKV) * HD].float().view(2 * SEQ, HQ + HKV, 2, HD // 2)
+	n0, n1 = v0.pow(2).sum(2), v1.pow(2).sum(2)
+	assert ((n1 - n0).abs() <= 2e-2 * n0 + 1e-3).all().item()
+	assert torch.equal(qkv[:, (HQ + HKV) * HD:], before[:, (HQ + HKV) * HD:])  # V untouched
+	K.rope_apply_(qkv, cs, SEQ, HQ + HKV, HD, backward=True)
+	assert (qkv.float() - before.float()).abs().max().item() <= 3e-2 * before.float().abs().max().item()
+	acc = torch.randn(D_MODEL, FFN, device="cuda", generator=torch.Generator(device="cuda").manual_seed(14))
+	want = acc / 32
+	out = torch.empty(D_MODEL, FFN, dtype=torch.bfloat16, device="cuda")
+	K.scale_grads_(acc, out, 1.0 / 32)
+	assert torch.equal(acc, want) and torch.equal(out, want.to(torch.bfloat16))

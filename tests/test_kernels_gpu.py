@@ -73,6 +73,33 @@ def test_gemm_epilogues(K):
 		_close(acc, 3 * ref + 0.25, rel_fro=1e-5, rel_max=1e-5, what=f"f32 acc ks={ks}")
 
 
+@pytest.mark.parametrize("tile_cfg", [6, 7])
+@pytest.mark.parametrize("layout", ["nt", "tn"])
+def test_gemm_direct_to_lds_epilogues_and_k_split(K, tile_cfg, layout):
+	"""The 256x256 direct-to-LDS kernels (4- and 8-wave): every epilogue, short K (1 and 2 slices:
+	the loop's loads past the end of K), and the K split with fp32 atomics."""
+	M, N = 512, 768
+	for Kd in (64, 128, 1024):
+		A = _randn(M, Kd, seed=21)
+		B = _randn(N, Kd, seed=22, scale=0.05)
+		R = _randn(M, N, seed=23)
+		ref = A.float() @ B.float().t()
+		if layout == "nt":
+			kw = dict(tile_cfg=tile_cfg)
+			a, b = A, B
+		else:
+			kw = dict(tile_cfg=tile_cfg, a_t=True, b_t=True)
+			a, b = A.t().contiguous(), B.t().contiguous()
+		_close(K.gemm(a, b, **kw), ref, what=f"bf16 K={Kd}")
+		_close(K.gemm(a, b, epilogue=K.EPI_BF16_RESID, residual=R, **kw), ref + R.float(), what=f"resid K={Kd}")
+		_close(K.gemm(a, b, epilogue=K.EPI_F32_STORE, **kw), ref, rel_fro=1e-5, rel_max=1e-5, what=f"f32 store K={Kd}")
+		for ks in (1, 2, 4):
+			acc = torch.full((M, N), 0.25, dtype=torch.float32, device="cuda")
+			for _ in range(2):
+				K.gemm(a, b, out=acc, epilogue=K.EPI_F32_ACC, k_splits=ks, **kw)
+			_close(acc, 2 * ref + 0.25, rel_fro=1e-5, rel_max=1e-5, what=f"f32 acc K={Kd} ks={ks}")
+
+
 def test_gemm_strided_views(K):
 	# operands that are column slices of wider buffers (leading dimension > row length)
 	big = _randn(512, 1024, seed=6)
