@@ -30,19 +30,19 @@ PEAK_HBM_GBS = 8000.0
 GEMM_TRAFFIC_BYTES = {"llama3_8b_zbh1": 1.588e9}
 
 WORKLOADS = {
-	# BASELINE.json configs[2]: Llama-3-8B-shaped stage, ZB-H1 stream of block 1 in a 4-stage pipeline
+	# headline configuration: Llama-3-8B-shaped stage, ZB-H1 stream of block 1 in a 4-stage pipeline
 	"llama3_8b_zbh1": dict(arch="llama", n_blocks=4, d=4096, heads=32, kv_heads=8, head_dim=128, ffn=14336, seq=4096, mb=2, n_mb=16,
 	                       scheduler="zbh1", causal=True, rope_theta=5e5),
 	# same stage under 1F1B
 	"llama3_8b_1f1b": dict(arch="llama", n_blocks=4, d=4096, heads=32, kv_heads=8, head_dim=128, ffn=14336, seq=4096, mb=2, n_mb=16,
 	                       scheduler="1f1b", causal=True, rope_theta=5e5),
-	# BASELINE.json configs[1]: GPT-2-small-shaped stage, 1F1B
+	# small configuration: GPT-2-small-shaped stage, 1F1B
 	"gpt2s_1f1b": dict(arch="gpt", n_blocks=3, d=768, heads=12, kv_heads=12, head_dim=64, ffn=3072, seq=1024, mb=8, n_mb=8,
 	                   scheduler="1f1b", causal=False),
-	# BASELINE.json configs[4]: Llama-3-70B-shaped stage, 1F1B with activation offload
+	# offload configuration: Llama-3-70B-shaped stage, 1F1B with activation offload
 	"llama3_70b_offload": dict(arch="llama", n_blocks=2, d=8192, heads=64, kv_heads=8, head_dim=128, ffn=28672, seq=8192, mb=1, n_mb=8,
 	                           scheduler="1f1b", causal=True, rope_theta=5e5, offload=True),
-	# BASELINE.json configs[3]: the Llama-3-8B-shaped stage with 8 blocks at seq 8192 under a 48 GB budget: the stage is
+	# remat configuration: the Llama-3-8B-shaped stage with 8 blocks at seq 8192 under a 48 GB budget: the stage is
 	# profiled on the native executor, the remat ILP is solved for a pipeline of 8 such stages (the other stages are
 	# copies of the measured one) and block 1's rewritten 1F1B stream runs
 	"llama3_8b_remat": dict(arch="llama", n_blocks=8, d=4096, heads=32, kv_heads=8, head_dim=128, ffn=14336, seq=8192, mb=1, n_mb=16,
