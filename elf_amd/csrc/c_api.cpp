@@ -47,6 +47,12 @@ int elf_scale_grads(void* acc_f32, void* out_bf16, int64_t n, float scale, void*
 int elf_add_bf16(const void* a, const void* b, void* out, int64_t n, void* stream) {
 	return elf::add_bf16(a, b, out, n, S_(stream));
 }
+int elf_embedding_fwd(const void* ids, const void* table, void* out, int64_t T, int d, int V, void* stream) {
+	return elf::embedding_fwd(ids, table, out, T, d, V, S_(stream));
+}
+int elf_embedding_bwd(const void* ids, const void* dx, void* dtable_f32, int64_t T, int d, int V, void* stream) {
+	return elf::embedding_bwd(ids, dx, dtable_f32, T, d, V, S_(stream));
+}
 int elf_attn_fwd(const void* q, const void* k, const void* v, void* o, void* lse, int64_t ldq, int64_t ldk, int64_t ldv,
                  int64_t ldo, int B, int S, int Hq, int Hkv, int D, int causal, float scale, void* stream) {
 	return elf::attn_fwd(q, k, v, o, lse, ldq, ldk, ldv, ldo, B, S, Hq, Hkv, D, causal, scale, S_(stream));

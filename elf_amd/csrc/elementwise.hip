@@ -542,4 +542,59 @@ int add_bf16(const void* a, const void* b, void* out, int64_t n, hipStream_t s) 
 	return 0;
 }
 
+// ------------------------------------------------------------------------------------------
+// Token embedding of a pipeline's first stage (benchmarks/models/simple.py:496, 502):
+// out[t, :] = table[ids[t], :].  One 16-byte chunk per lane; rows of ids outside [0, V) give a
+// zero row (the host cannot check ids without a device round trip).
+__global__ __launch_bounds__(256) void embedding_fwd_kernel(const int64_t* __restrict__ ids, const bf16_t* __restrict__ table,
+                                                            bf16_t* __restrict__ out, int64_t T, int d, int V) {
+	const int cpr = d / 8;
+	const int64_t n = T * cpr;
+	for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+		const int64_t t = i / cpr;
+		const int c = (int)(i - t * cpr) * 8;
+		const int64_t id = ids[t];
+		Chunk x;
+		if (id >= 0 && id < V) {
+			x = load8(table + id * d + c);
+		} else {
+#pragma unroll
+			for (int j = 0; j < 8; j++) x.v[j] = 0.f;
+		}
+		store8(out + t * d + c, x);
+	}
+}
+// dtable[ids[t], :] += dx[t, :] in fp32 (tokens repeat within a micro-batch: atomics).
+__global__ __launch_bounds__(256) void embedding_bwd_kernel(const int64_t* __restrict__ ids, const bf16_t* __restrict__ dx,
+                                                            float* __restrict__ dtable, int64_t T, int d, int V) {
+	const int cpr = d / 8;
+	const int64_t n = T * cpr;
+	for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+		const int64_t t = i / cpr;
+		const int c = (int)(i - t * cpr) * 8;
+		const int64_t id = ids[t];
+		if (id < 0 || id >= V) continue;
+		const Chunk x = load8(dx + t * d + c);
+		float* g = dtable + id * d + c;
+#pragma unroll
+		for (int j = 0; j < 8; j++) unsafeAtomicAdd(g + j, x.v[j]);
+	}
+}
+int embedding_fwd(const void* ids, const void* table, void* out, int64_t T, int d, int V, hipStream_t s) {
+	ELF_REQUIRE(ids && table && out && T > 0 && V > 0 && d > 0 && d % 8 == 0, "embedding_fwd: bad argument (d must be a multiple of 8)");
+	ProfScope prof(PROF_EMBED, 4.0 * T * d, s);
+	hipLaunchKernelGGL(embedding_fwd_kernel, dim3(ew_grid(T * (d / 8))), dim3(256), 0, s, (const int64_t*)ids, (const bf16_t*)table,
+	                   (bf16_t*)out, T, d, V);
+	ELF_CHECK_HIP(hipGetLastError());
+	return 0;
+}
+int embedding_bwd(const void* ids, const void* dx, void* dtable_f32, int64_t T, int d, int V, hipStream_t s) {
+	ELF_REQUIRE(ids && dx && dtable_f32 && T > 0 && V > 0 && d > 0 && d % 8 == 0, "embedding_bwd: bad argument (d must be a multiple of 8)");
+	ProfScope prof(PROF_EMBED, 10.0 * T * d, s);
+	hipLaunchKernelGGL(embedding_bwd_kernel, dim3(ew_grid(T * (d / 8))), dim3(256), 0, s, (const int64_t*)ids, (const bf16_t*)dx,
+	                   (float*)dtable_f32, T, d, V);
+	ELF_CHECK_HIP(hipGetLastError());
+	return 0;
+}
+
 }  // namespace elf

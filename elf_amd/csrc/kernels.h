@@ -36,6 +36,9 @@ int rope_table(void* cs, int S, int D, double theta, hipStream_t s);
 int rope_apply(void* buf, const void* cs, int64_t T, int S, int ld, int n_heads, int D, int backward, hipStream_t s);
 int scale_grads(void* acc_f32, void* out_bf16, int64_t n, float scale, hipStream_t s);
 int add_bf16(const void* a, const void* b, void* out, int64_t n, hipStream_t s);
+// ids: int64 [T]; table bf16 [V, d]; dtable fp32 [V, d] (+=)
+int embedding_fwd(const void* ids, const void* table, void* out, int64_t T, int d, int V, hipStream_t s);
+int embedding_bwd(const void* ids, const void* dx, void* dtable_f32, int64_t T, int d, int V, hipStream_t s);
 
 // Attention over the packed projection layout; lse is [B, Hq, S] fp32 (natural log).
 int attn_fwd(const void* q, const void* k, const void* v, void* o, void* lse, int64_t ldq, int64_t ldk, int64_t ldv,
@@ -50,7 +53,7 @@ int attn_bwd(const void* q, const void* k, const void* v, const void* o, const v
 // with an event pair on the launch stream and books the algorithmic work of the call.
 enum ProfKind {
 	PROF_GEMM = 0, PROF_ATTN_FWD, PROF_ATTN_BWD, PROF_NORM_FWD, PROF_NORM_BWD, PROF_ACT_FWD, PROF_ACT_BWD, PROF_ROPE,
-	PROF_SCALE, PROF_ADD, PROF_COUNT
+	PROF_SCALE, PROF_ADD, PROF_EMBED, PROF_COUNT
 };
 void prof_enable(int on);
 bool prof_on();

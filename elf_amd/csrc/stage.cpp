@@ -46,6 +46,8 @@ static const unsigned WIN_MASK = (1u << B_H1) | (1u << B_O) | (1u << B_H2) | (1u
 static const unsigned WGRAD_MASK = (1u << B_DY) | (1u << B_DGU) | (1u << B_DX2) | (1u << B_DQKV);
 
 enum ParamId { P_NORM1_G = 0, P_NORM1_B, P_WQKV, P_WO, P_NORM2_G, P_NORM2_B, P_W1, P_W2, P_COUNT };
+// stage-level parameters of a first / last pipeline stage (ELF_P_EMBED .. ELF_P_HEAD - ELF_P_EMBED)
+enum EndParamId { XP_EMBED = 0, XP_FNORM_G, XP_FNORM_B, XP_HEAD, XP_COUNT };
 
 struct Buf {
 	void* p = nullptr;
@@ -64,6 +66,11 @@ struct BlockState {
 
 struct MbState {
 	std::vector<BlockState> blk;
+	// last stage: the output head.  B_X / B_ST1 = input and statistics of the final norm, B_H1 = input
+	// of the head linear (the last block's output when there is no final norm), B_DQKV = gradient of
+	// the logits (caller-owned, like the stage's dY)
+	BlockState head;
+	const void* ids = nullptr;  // first stage: the token ids of the micro-batch (caller-owned)
 	bool has_acts = false, has_win = false, has_wgrad = false;
 	bool remat_root = false;  // forward kept nothing: B re-runs it
 	bool offloaded = false, prefetched = false;
@@ -81,6 +88,12 @@ struct Stage {
 	int T, d, Hq, Hkv, D, F, S, B, nqkv, ffn_in;
 	bool llama;
 	std::vector<BlockParams> params;
+	// first / last stage of a pipeline (elf_stage_set_ends): token embedding in front of block 0,
+	// optional final norm + output head behind the last block (logits [T, vld], vld >= vocab_out)
+	int vocab_in = 0, vocab_out = 0, vld = 0;
+	bool final_norm = false;
+	void* xw[XP_COUNT] = {};
+	float* xg[XP_COUNT] = {};
 	std::map<int, MbState> mbs;
 	DevicePool pool;
 	std::unique_ptr<PinnedPool> pinned;
@@ -127,6 +140,8 @@ static void buf_free(Stage* s, BlockState& bs, int id) {
 	b.owned = false;
 }
 static void free_mask(Stage* s, MbState& m, unsigned mask) {
+	for (int id = 0; id < B_COUNT; id++)
+		if (mask & (1u << id)) buf_free(s, m.head, id);
 	for (auto& bs : m.blk)
 		for (int id = 0; id < B_COUNT; id++)
 			if (mask & (1u << id)) buf_free(s, bs, id);
@@ -158,9 +173,15 @@ static int run_forward(Stage* s, MbState& m, const void* x, void* y, FwdMode mod
 		BlockState& bs = m.blk[i];
 		const BlockParams& p = s->params[i];
 		if (i == 0) {
-			bs.b[B_X].p = const_cast<void*>(x);
-			bs.b[B_X].owned = false;
-			bs.b[B_X].bytes = s->buf_bytes(B_X);
+			if (s->vocab_in) {
+				m.ids = x;
+				ELF_TRY(buf_alloc(s, bs, B_X));
+				ELF_TRY(embedding_fwd(x, s->xw[XP_EMBED], bs.b[B_X].p, T, d, s->vocab_in, st));
+			} else {
+				bs.b[B_X].p = const_cast<void*>(x);
+				bs.b[B_X].owned = false;
+				bs.b[B_X].bytes = s->buf_bytes(B_X);
+			}
 		}
 		const void* xin = bs.b[B_X].p;
 		ELF_TRY(buf_alloc(s, bs, B_ST1));
@@ -187,7 +208,11 @@ static int run_forward(Stage* s, MbState& m, const void* x, void* y, FwdMode mod
 		if (s->llama) ELF_TRY(swiglu_fwd(bs.b[B_GU].p, bs.b[B_A].p, T, F, st));
 		else ELF_TRY(gelu_fwd(bs.b[B_GU].p, bs.b[B_A].p, (int64_t)T * F, st));
 		void* yout;
-		if (i == nb - 1) {
+		if (i == nb - 1 && s->vocab_out) {
+			const int id = s->final_norm ? B_X : B_H1;
+			ELF_TRY(buf_alloc(s, m.head, id));
+			yout = m.head.b[id].p;
+		} else if (i == nb - 1) {
 			yout = y;
 		} else {
 			BlockState& nx = m.blk[i + 1];
@@ -203,6 +228,21 @@ static int run_forward(Stage* s, MbState& m, const void* x, void* y, FwdMode mod
 		}
 		// the block's stash starts its way to the host while the next block computes
 		if (offload && mode == SAVE_ALL) ELF_TRY(do_offload_block(s, bs, st));
+	}
+	if (s->vocab_out) {
+		// last stage: (final norm,) logits = h W_head^T   (benchmarks/models/simple.py:497, 508)
+		BlockState& hd = m.head;
+		if (s->final_norm) {
+			ELF_TRY(buf_alloc(s, hd, B_ST1));
+			ELF_TRY(buf_alloc(s, hd, B_H1));
+			ELF_TRY(norm_fwd(norm_kind, hd.b[B_X].p, s->xw[XP_FNORM_G], s->xw[XP_FNORM_B], hd.b[B_H1].p, hd.b[B_ST1].p, T, d, s->cfg.eps, st));
+		}
+		ELF_TRY(gemm_bf16(0, 0, T, s->vld, d, hd.b[B_H1].p, d, s->xw[XP_HEAD], d, y, s->vld, EPI_BF16, nullptr, 0, 0, 0, st));
+		if (mode != SAVE_ALL) {
+			const unsigned keep = mode == SAVE_WIN ? WIN_MASK : 0u;
+			for (int id = 0; id < B_COUNT; id++)
+				if ((ACT_MASK & (1u << id)) && !(keep & (1u << id))) buf_free(s, hd, id);
+		}
 	}
 	m.has_acts = mode == SAVE_ALL;
 	m.has_win = mode != SAVE_NONE;
@@ -221,10 +261,31 @@ static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool gra
 	const int T = s->T, d = s->d, F = s->F;
 	const int norm_kind = s->llama ? NORM_RMS : NORM_LAYER;
 	const float scale = 1.0f / sqrtf((float)s->D);
+	if (s->vocab_out) {
+		// last stage: dy is the gradient of the logits; it is the dY of the head linear's W stash
+		BlockState& hd = m.head;
+		hd.b[B_DQKV].p = const_cast<void*>(dy);
+		hd.b[B_DQKV].owned = false;
+		hd.b[B_DQKV].bytes = (size_t)T * s->vld * 2;
+		BlockState& last = m.blk[nb - 1];
+		ELF_TRY(buf_alloc(s, last, B_DY));
+		if (s->final_norm) {
+			void* d_hn = s->pool.alloc((size_t)T * d * 2);
+			if (!d_hn) return -3;
+			ELF_TRY(gemm_bf16(0, 1, T, d, s->vld, dy, s->vld, s->xw[XP_HEAD], d, d_hn, d, EPI_BF16, nullptr, 0, 0, 0, st));
+			ELF_TRY(norm_bwd(norm_kind, d_hn, hd.b[B_X].p, s->xw[XP_FNORM_G], hd.b[B_ST1].p, nullptr, last.b[B_DY].p,
+			                 grads_only ? s->dummy_grad : s->xg[XP_FNORM_G], grads_only ? s->dummy_grad + d : s->xg[XP_FNORM_B], s->norm_ws, T, d, st));
+			s->pool.free(d_hn);
+		} else {
+			ELF_TRY(gemm_bf16(0, 1, T, d, s->vld, dy, s->vld, s->xw[XP_HEAD], d, last.b[B_DY].p, d, EPI_BF16, nullptr, 0, 0, 0, st));
+		}
+		for (int id = 0; id < B_COUNT; id++)
+			if ((ACT_MASK & (1u << id)) && !(WIN_MASK & (1u << id))) buf_free(s, hd, id);
+	}
 	for (int i = nb - 1; i >= 0; i--) {
 		BlockState& bs = m.blk[i];
 		const BlockParams& p = s->params[i];
-		if (i == nb - 1) {
+		if (i == nb - 1 && !s->vocab_out) {
 			bs.b[B_DY].p = const_cast<void*>(dy);
 			bs.b[B_DY].owned = false;
 			bs.b[B_DY].bytes = s->buf_bytes(B_DY);
@@ -262,7 +323,12 @@ static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool gra
 		if (!(grads_only && i == 0)) {
 			ELF_TRY(gemm_bf16(0, 1, T, d, s->nqkv, bs.b[B_DQKV].p, s->nqkv, p.w[P_WQKV], d, d_h, d, EPI_BF16, nullptr, 0, 0, 0, st));
 			void* dxout;
-			if (i == 0) {
+			void* d_emb = nullptr;
+			if (i == 0 && s->vocab_in) {
+				d_emb = s->pool.alloc((size_t)T * d * 2);
+				if (!d_emb) return -3;
+				dxout = d_emb;
+			} else if (i == 0) {
 				dxout = dx;
 			} else {
 				BlockState& pv = m.blk[i - 1];
@@ -271,6 +337,11 @@ static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool gra
 			}
 			ELF_TRY(norm_bwd(norm_kind, d_h, bs.b[B_X].p, p.w[P_NORM1_G], bs.b[B_ST1].p, bs.b[B_DX2].p, dxout,
 			                 grads_only ? s->dummy_grad : p.g[P_NORM1_G], grads_only ? s->dummy_grad + d : p.g[P_NORM1_B], s->norm_ws, T, d, st));
+			if (d_emb) {
+				// first stage: the embedding is not a split layer, its gradient accumulates inside B
+				if (!grads_only) ELF_TRY(embedding_bwd(m.ids, d_emb, s->xg[XP_EMBED], T, d, s->vocab_in, st));
+				s->pool.free(d_emb);
+			}
 		}
 		s->pool.free(d_h);
 		// B consumed the activation stash; what is left is the W stash
@@ -295,6 +366,8 @@ static int run_backward_params(Stage* s, MbState& m, hipStream_t st) {
 		ELF_TRY(gemm_bf16(1, 1, d, hd, T, bs.b[B_DX2].p, d, bs.b[B_O].p, hd, p.g[P_WO], hd, EPI_F32_ACC, nullptr, 0, 0, 0, st));
 		ELF_TRY(gemm_bf16(1, 1, s->nqkv, d, T, bs.b[B_DQKV].p, s->nqkv, bs.b[B_H1].p, d, p.g[P_WQKV], d, EPI_F32_ACC, nullptr, 0, 0, 0, st));
 	}
+	if (s->vocab_out)
+		ELF_TRY(gemm_bf16(1, 1, s->vld, d, T, m.head.b[B_DQKV].p, s->vld, m.head.b[B_H1].p, d, s->xg[XP_HEAD], d, EPI_F32_ACC, nullptr, 0, 0, 0, st));
 	free_mask(s, m, WIN_MASK | WGRAD_MASK);
 	m.has_win = m.has_wgrad = false;
 	return 0;
@@ -472,10 +545,16 @@ void elf_stage_destroy(elf_stage_t* h) {
 int elf_stage_bind_param(elf_stage_t* h, int block, int which, void* weight_bf16, void* grad_f32) {
 	Stage* s = (Stage*)h;
 	ELF_REQUIRE(s, "elf_stage_bind_param: null stage");
-	ELF_REQUIRE(block >= 0 && block < s->cfg.n_blocks, "elf_stage_bind_param: block %d out of range", block);
-	ELF_REQUIRE(which >= 0 && which < P_COUNT, "elf_stage_bind_param: parameter id %d out of range", which);
 	ELF_REQUIRE(weight_bf16 && grad_f32, "elf_stage_bind_param: null pointer");
 	ELF_REQUIRE(((uintptr_t)weight_bf16 % 16) == 0 && ((uintptr_t)grad_f32 % 16) == 0, "elf_stage_bind_param: pointers must be 16-byte aligned");
+	if (block == -1) {
+		ELF_REQUIRE(which >= ELF_P_EMBED && which <= ELF_P_HEAD, "elf_stage_bind_param: stage-level parameter id %d out of range", which);
+		s->xw[which - ELF_P_EMBED] = weight_bf16;
+		s->xg[which - ELF_P_EMBED] = (float*)grad_f32;
+		return 0;
+	}
+	ELF_REQUIRE(block >= 0 && block < s->cfg.n_blocks, "elf_stage_bind_param: block %d out of range", block);
+	ELF_REQUIRE(which >= 0 && which < P_COUNT, "elf_stage_bind_param: parameter id %d out of range", which);
 	s->params[block].w[which] = weight_bf16;
 	s->params[block].g[which] = (float*)grad_f32;
 	return 0;
@@ -487,6 +566,24 @@ static int check_bound(Stage* s) {
 			if (s->llama && (w == P_NORM1_B || w == P_NORM2_B)) continue;
 			ELF_REQUIRE(s->params[i].w[w] != nullptr, "stage: parameter %d of block %d is not bound", w, i);
 		}
+	ELF_REQUIRE(!s->vocab_in || s->xw[XP_EMBED], "stage: the embedding table is not bound");
+	ELF_REQUIRE(!s->vocab_out || s->xw[XP_HEAD], "stage: the output head is not bound");
+	ELF_REQUIRE(!s->final_norm || (s->xw[XP_FNORM_G] && (s->llama || s->xw[XP_FNORM_B])), "stage: the final norm is not bound");
+	return 0;
+}
+
+int elf_stage_set_ends(elf_stage_t* h, int vocab_in, int vocab_out, int vocab_out_ld, int final_norm) {
+	Stage* s = (Stage*)h;
+	ELF_REQUIRE(s, "elf_stage_set_ends: null stage");
+	ELF_REQUIRE(s->mbs.empty(), "elf_stage_set_ends: call it before the first forward");
+	ELF_REQUIRE(vocab_in >= 0 && vocab_out >= 0, "elf_stage_set_ends: negative vocabulary size");
+	ELF_REQUIRE(!vocab_out || (vocab_out_ld >= vocab_out && vocab_out_ld % 64 == 0),
+	            "elf_stage_set_ends: the logits row stride must be a multiple of 64 and at least vocab_out (%d, %d)", vocab_out_ld, vocab_out);
+	ELF_REQUIRE(!final_norm || vocab_out, "elf_stage_set_ends: a final norm needs an output head");
+	s->vocab_in = vocab_in;
+	s->vocab_out = vocab_out;
+	s->vld = vocab_out ? vocab_out_ld : 0;
+	s->final_norm = final_norm != 0;
 	return 0;
 }
 
@@ -505,7 +602,7 @@ int elf_stage_forward(elf_stage_t* h, int mb, const void* x, void* y, uint32_t f
 
 int elf_stage_backward_inputs(elf_stage_t* h, int mb, const void* x, const void* dy, void* dx, uint32_t flags, void* stream) {
 	Stage* s = (Stage*)h;
-	ELF_REQUIRE(s && dy && dx && mb >= 0, "elf_stage_backward_inputs: bad argument");
+	ELF_REQUIRE(s && dy && (dx || s->vocab_in) && mb >= 0, "elf_stage_backward_inputs: bad argument");
 	auto it = s->mbs.find(mb);
 	ELF_REQUIRE(it != s->mbs.end(), "elf_stage_backward_inputs: no forward was run for micro-batch %d", mb);
 	MbState& m = it->second;
@@ -513,7 +610,7 @@ int elf_stage_backward_inputs(elf_stage_t* h, int mb, const void* x, const void*
 	if (m.remat_root) {
 		// the forward kept only the stage input: re-run it, this time keeping the stash
 		ELF_REQUIRE(x != nullptr, "elf_stage_backward_inputs: micro-batch %d was checkpointed, the stage input is needed", mb);
-		void* ytmp = s->pool.alloc((size_t)s->T * s->d * 2);
+		void* ytmp = s->pool.alloc((size_t)s->T * (s->vocab_out ? s->vld : s->d) * 2);
 		if (!ytmp) return -3;
 		int rc = run_forward(s, m, x, ytmp, SAVE_ALL, st);
 		s->pool.free(ytmp);
@@ -524,7 +621,8 @@ int elf_stage_backward_inputs(elf_stage_t* h, int mb, const void* x, const void*
 	if (m.offloaded) {
 		if (!m.prefetched) ELF_TRY(do_restore(s, m, false, st));  // run_backward waits block by block otherwise
 	}
-	if (x) m.blk[0].b[B_X].p = const_cast<void*>(x);
+	if (x && s->vocab_in) m.ids = x;
+	else if (x) m.blk[0].b[B_X].p = const_cast<void*>(x);
 	ELF_TRY(run_backward(s, m, dy, dx, false, st));
 	if (flags & ELF_BWD_RECOMPUTE_GRADIENTS) free_mask(s, m, WGRAD_MASK), m.has_wgrad = false;
 	if (flags & ELF_BWD_RECOMPUTE_ACTIVATIONS) free_mask(s, m, WIN_MASK), m.has_win = false;
@@ -539,6 +637,7 @@ int elf_stage_backward_params(elf_stage_t* h, int mb, void* stream) {
 	            "elf_stage_backward_params: micro-batch %d has no saved inputs / output gradients (run B, or the recompute ops, first)", mb);
 	for (int i = 0; i < s->cfg.n_blocks; i++)
 		for (int w : {P_WQKV, P_WO, P_W1, P_W2}) ELF_REQUIRE(s->params[i].g[w] != nullptr, "elf_stage_backward_params: gradient buffer not bound");
+	ELF_REQUIRE(!s->vocab_out || s->xg[XP_HEAD], "elf_stage_backward_params: gradient buffer of the output head not bound");
 	ELF_TRY(run_backward_params(s, it->second, (hipStream_t)stream));
 	return 0;
 }
@@ -551,7 +650,7 @@ int elf_stage_recompute_forward(elf_stage_t* h, int mb, const void* x, int save,
 	MbState& m = it->second;
 	ELF_REQUIRE(!m.has_acts && !m.has_win, "elf_stage_recompute_forward: micro-batch %d still holds its activations", mb);
 	hipStream_t st = (hipStream_t)stream;
-	void* ytmp = s->pool.alloc((size_t)s->T * s->d * 2);
+	void* ytmp = s->pool.alloc((size_t)s->T * (s->vocab_out ? s->vld : s->d) * 2);
 	if (!ytmp) return -3;
 	int rc = run_forward(s, m, x, ytmp, save ? SAVE_ALL : SAVE_WIN, st);
 	s->pool.free(ytmp);

@@ -14,7 +14,7 @@ import logging
 import torch
 
 from .. import _lib
-from ..models import LlamaBlock, TransformerBlock
+from ..models import EndStage, LlamaBlock, TransformerBlock
 from ..scheduling import OpOptions
 from ..utils import Timer
 
@@ -94,6 +94,7 @@ for _name, _ret, _args in [
 	("elf_stage_create", _I, [ctypes.POINTER(StageConfig), ctypes.POINTER(_P)]),
 	("elf_stage_destroy", None, [_P]),
 	("elf_stage_bind_param", _I, [_P, _I, _I, _P, _P]),
+	("elf_stage_set_ends", _I, [_P, _I, _I, _I, _I]),
 	("elf_stage_forward", _I, [_P, _I, _P, _P, ctypes.c_uint32, _P]),
 	("elf_stage_backward_inputs", _I, [_P, _I, _P, _P, _P, ctypes.c_uint32, _P]),
 	("elf_stage_backward_params", _I, [_P, _I, _P]),
@@ -113,6 +114,7 @@ FWD_REMAT_ROOT, FWD_OFFLOAD = 1, 4
 BWD_RECOMPUTE_ACTIVATIONS, BWD_RECOMPUTE_GRADIENTS = 1, 2
 # parameter ids of elf_stage_bind_param
 P_NORM1_G, P_NORM1_B, P_WQKV, P_WO, P_NORM2_G, P_NORM2_B, P_W1, P_W2 = range(8)
+P_EMBED, P_FNORM_G, P_FNORM_B, P_HEAD = 8, 9, 10, 11  # stage-level, bound with block = -1
 
 
 def _stream():
@@ -155,12 +157,14 @@ class HipStageBlock:
 
 	# ------------------------------------------------------------------ set-up
 	def _build(self, mb_size, seq_len):
-		blocks = list(self.model.children()) if not isinstance(self.model, (TransformerBlock, LlamaBlock)) else [self.model]
+		core = self.model.blocks if isinstance(self.model, EndStage) else self.model
+		self.ends = self.model if isinstance(self.model, EndStage) else None
+		blocks = list(core.children()) if not isinstance(core, (TransformerBlock, LlamaBlock)) else [core]
 		if not blocks or not all(isinstance(b, (TransformerBlock, LlamaBlock)) for b in blocks) or len({type(b) for b in blocks}) != 1:
 			raise _lib.ElfStageError("HipStageBlock: the stage must be a chain of TransformerBlock or of LlamaBlock modules")
 		b0 = blocks[0]
 		llama = isinstance(b0, LlamaBlock)
-		seq = seq_len or getattr(self.model, "seq_len", None)
+		seq = seq_len or getattr(core, "seq_len", None)
 		if seq is None:
 			raise _lib.ElfStageError("HipStageBlock: seq_len is required (StageModule carries it)")
 		att = b0.attn
@@ -178,10 +182,11 @@ class HipStageBlock:
 		_lib.check(self.lib.elf_stage_create(ctypes.byref(cfg), ctypes.byref(handle)), "elf_stage_create")
 		self._handle = handle
 
-		def fuse(params):
-			"""Move `params` (row blocks of one matrix) into one bf16 buffer + one fp32 grad buffer."""
-			rows = sum(p.shape[0] for p in params)
-			w = torch.empty((rows,) + tuple(params[0].shape[1:]), dtype=torch.bfloat16, device=dev)
+		def fuse(params, pad_rows=0):
+			"""Move `params` (row blocks of one matrix) into one bf16 buffer + one fp32 grad buffer
+			(`pad_rows` extra zero rows at the end)."""
+			rows = sum(p.shape[0] for p in params) + pad_rows
+			w = torch.zeros((rows,) + tuple(params[0].shape[1:]), dtype=torch.bfloat16, device=dev)
 			g = torch.zeros(w.shape, dtype=torch.float32, device=dev)
 			r = 0
 			for p in params:
@@ -215,6 +220,29 @@ class HipStageBlock:
 				_lib.check(self.lib.elf_stage_bind_param(self._handle, i, pid, w.data_ptr(), g.data_ptr()), "elf_stage_bind_param")
 		self.T = mb_size * seq
 		self.d = b0.dim
+		self.mb_size, self.seq = mb_size, seq
+		# first / last stage of a pipeline: token embedding, (final norm,) output head
+		self.vocab_in = self.vocab_out = self.vld = 0
+		if self.ends is not None:
+			e = self.ends
+			stage_level = {}
+			if e.embed is not None:
+				self.vocab_in = e.embed.num_embeddings
+				stage_level[P_EMBED] = ([e.embed.weight], 0)
+			if e.head is not None:
+				self.vocab_out = e.head.out_features
+				self.vld = -(-self.vocab_out // 64) * 64
+				stage_level[P_HEAD] = ([e.head.weight], self.vld - self.vocab_out)
+			if e.norm_f is not None:
+				stage_level[P_FNORM_G] = ([e.norm_f.weight], 0)
+				if not llama:
+					stage_level[P_FNORM_B] = ([e.norm_f.bias], 0)
+			_lib.check(self.lib.elf_stage_set_ends(self._handle, self.vocab_in, self.vocab_out, self.vld, int(e.norm_f is not None)), "elf_stage_set_ends")
+			for pid, (params, pad) in stage_level.items():
+				if any(p.dtype != torch.bfloat16 for p in params):
+					raise _lib.ElfStageError("HipStageBlock: parameters must be bf16")
+				w, g = fuse(params, pad)
+				_lib.check(self.lib.elf_stage_bind_param(self._handle, -1, pid, w.data_ptr(), g.data_ptr()), "elf_stage_bind_param")
 
 	def __del__(self):
 		try:
@@ -232,6 +260,35 @@ class HipStageBlock:
 			raise _lib.ElfStageError(f"{self}: {what} must be a bf16 GPU tensor of {self.T}x{self.d} elements, got {tuple(t.shape)} {t.dtype} {t.device}")
 		return t.contiguous()
 
+	def _check_ids(self, t):
+		if t.dtype != torch.int64 or not t.is_cuda or t.numel() != self.T:
+			raise _lib.ElfStageError(f"{self}: the input of a first stage must be an int64 GPU tensor of {self.T} token ids, got {tuple(t.shape)} {t.dtype} {t.device}")
+		return t.contiguous()
+
+	def _new_output(self, x):
+		"""(buffer the library writes, tensor handed on).  Last stage: logits [T, vld] with the
+		padding columns hidden from the caller; otherwise activations shaped like the input."""
+		if self.vocab_out:
+			buf = torch.empty(self.T, self.vld, dtype=torch.bfloat16, device=x.device)
+			return buf, buf.view(self.mb_size, self.seq, self.vld)[..., : self.vocab_out]
+		if self.vocab_in:
+			buf = torch.empty(self.mb_size, self.seq, self.d, dtype=torch.bfloat16, device=x.device)
+			return buf, buf
+		buf = torch.empty_like(x)
+		return buf, buf
+
+	def _check_dy(self, dy):
+		"""Gradient of the stage output in the layout the library reads."""
+		if not self.vocab_out:
+			return self._check_io(dy, "output gradient")
+		if dy.dtype != torch.bfloat16 or not dy.is_cuda or dy.numel() != self.T * self.vocab_out:
+			raise _lib.ElfStageError(f"{self}: the gradient of the logits must be a bf16 GPU tensor of {self.T}x{self.vocab_out} elements, got {tuple(dy.shape)} {dy.dtype} {dy.device}")
+		if self.vld == self.vocab_out:
+			return dy.contiguous()
+		pad = torch.zeros(self.T, self.vld, dtype=torch.bfloat16, device=dy.device)
+		pad[:, : self.vocab_out] = dy.reshape(self.T, self.vocab_out)
+		return pad
+
 	def _timed(self, name):
 		t = Timer(name=name)
 		self.compute_time.append(t)
@@ -243,12 +300,13 @@ class HipStageBlock:
 		is kept: whole-stage checkpoint) and ``activation_offload`` (handled by the offloader the
 		engine wraps around this call)."""
 		var = self.input_variables[0]
-		x = self._check_io(var.wait_and_pop(mb_id), "stage input")
+		x = var.wait_and_pop(mb_id)
+		x = self._check_ids(x) if self.vocab_in else self._check_io(x, "stage input")
 		strategy = options.get(OpOptions.REMAT_STRATEGY)
 		flags = FWD_REMAT_ROOT if (strategy is not None and strategy("", self.model)) else 0
-		y = torch.empty_like(x)
+		ybuf, y = self._new_output(x)
 		with self._timed(f"forward({self.id}:{mb_id})"):
-			_lib.check(self.lib.elf_stage_forward(self._handle, mb_id, x.data_ptr(), y.data_ptr(), flags, _stream()), "elf_stage_forward")
+			_lib.check(self.lib.elf_stage_forward(self._handle, mb_id, x.data_ptr(), ybuf.data_ptr(), flags, _stream()), "elf_stage_forward")
 		self._kept.setdefault(mb_id, {})["x"] = x
 		for dst in self.output_variables[0]:
 			dst.set(dst.to_send, mb_id, y)
@@ -267,18 +325,19 @@ class HipStageBlock:
 		dy = outs[0].wait_and_pop(mb_id)
 		for dst in outs[1:]:
 			dy = dy + dst.wait_and_pop(mb_id)
-		dy = self._check_io(dy, "output gradient")
+		dy = self._check_dy(dy)
 		ra = bool(options.get(OpOptions.RECOMPUTE_ACTIVATIONS, False))
 		rg = bool(options.get(OpOptions.RECOMPUTE_GRADIENTS, False))
 		flags = (BWD_RECOMPUTE_ACTIVATIONS if ra else 0) | (BWD_RECOMPUTE_GRADIENTS if rg else 0)
-		dx = torch.empty_like(x)
+		dx = None if self.vocab_in else torch.empty_like(x)  # token ids have no gradient
 		with self._timed(f"backward_inputs({self.id}:{mb_id})"):
-			_lib.check(self.lib.elf_stage_backward_inputs(self._handle, mb_id, x.data_ptr(), dy.data_ptr(), dx.data_ptr(), flags, _stream()), "elf_stage_backward_inputs")
+			_lib.check(self.lib.elf_stage_backward_inputs(self._handle, mb_id, x.data_ptr(), dy.data_ptr(), dx.data_ptr() if dx is not None else None, flags, _stream()), "elf_stage_backward_inputs")
 		kept = self._kept.setdefault(mb_id, {})
 		kept["dy"] = dy  # the last block's dY of the W stash is this tensor
 		if not ra:
 			kept.pop("x", None)
-		var.set(var.to_send, mb_id, dx)
+		if dx is not None:
+			var.set(var.to_send, mb_id, dx)
 		if ra:
 			var.set(var.saved, mb_id, x)
 		if rg:
@@ -366,7 +425,7 @@ class HipStageBlock:
 
 	def send_backward(self, mb_id, **options):
 		dst = options.get("dst")
-		if self._remote(dst):
+		if self._remote(dst) and not self.vocab_in:  # token ids have no gradient to send
 			var = self.input_variables[0]
 			if var.peer == dst:
 				dx = var.get(var.to_send, mb_id)

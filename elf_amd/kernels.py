@@ -117,6 +117,26 @@ def add(a, b):
 	return out
 
 
+def embedding_fwd(ids, table):
+	"""ids: int64 [T] (any shape, flattened); table: bf16 [V, d] -> bf16 [T, d]."""
+	_need(table, torch.bfloat16, "embedding.table")
+	if ids.dtype != torch.int64 or not ids.is_cuda:
+		raise _lib.ElfStageError("embedding.ids must be an int64 GPU tensor")
+	ids = ids.contiguous()
+	out = torch.empty(ids.numel(), table.shape[1], dtype=torch.bfloat16, device=table.device)
+	_lib.check(_lib.load().elf_embedding_fwd(_ptr(ids), _ptr(table), _ptr(out), ids.numel(), table.shape[1], table.shape[0], _stream()), "elf_embedding_fwd")
+	return out
+
+
+def embedding_bwd_(ids, dx, dtable):
+	"""dtable (fp32 [V, d]) += scatter of dx (bf16 [T, d]) by ids."""
+	_need(dx, torch.bfloat16, "embedding.dx")
+	_need(dtable, torch.float32, "embedding.dtable")
+	ids = ids.contiguous()
+	_lib.check(_lib.load().elf_embedding_bwd(_ptr(ids), _ptr(dx), _ptr(dtable), ids.numel(), dtable.shape[1], dtable.shape[0], _stream()), "elf_embedding_bwd")
+	return dtable
+
+
 def attn_fwd(qkv, B, S, Hq, Hkv, D, causal, scale=None):
 	"""qkv: [B*S, (Hq+2*Hkv)*D] packed projections. Returns (o [B*S, Hq*D], lse [B,Hq,S])."""
 	_need(qkv, torch.bfloat16, "attn.qkv")

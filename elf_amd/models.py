@@ -17,7 +17,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-__all__ = ["TransformerBlock", "LlamaBlock", "StageModule", "RMSNorm", "gpt_stage", "llama_stage"]
+__all__ = ["TransformerBlock", "LlamaBlock", "StageModule", "EndStage", "RMSNorm", "gpt_stage", "llama_stage", "gpt_end_stage"]
 
 
 class Attention(nn.Module):
@@ -141,10 +141,37 @@ class StageModule(nn.Sequential):
 		self.seq_len = seq_len
 
 
+class EndStage(nn.Module):
+	"""First and / or last stage of a decoder: token embedding in front of the blocks, (final norm
+	and) output head behind them, with the attribute names of the reference's FullTransformer
+	(benchmarks/models/simple.py:470-509: ``embed``, ``head``; it has no final norm, ``norm_f`` is an
+	option for Llama-style models)."""
+
+	def __init__(self, blocks, vocab_in=None, vocab_out=None, final_norm=False):
+		super().__init__()
+		b0 = blocks[0]
+		self.blocks = blocks
+		self.seq_len = blocks.seq_len
+		self.embed = nn.Embedding(vocab_in, b0.dim) if vocab_in else None
+		self.norm_f = None
+		if final_norm:
+			assert vocab_out, "a final norm needs an output head"
+			self.norm_f = RMSNorm(b0.dim, b0.eps) if isinstance(b0, LlamaBlock) else nn.LayerNorm(b0.dim, eps=b0.eps)
+		self.head = nn.Linear(b0.dim, vocab_out, bias=False) if vocab_out else None
+
+	def forward(self, x):
+		if self.embed is not None:
+			x = self.embed(x)
+		x = self.blocks(x)
+		if self.norm_f is not None:
+			x = self.norm_f(x)
+		return self.head(x) if self.head is not None else x
+
+
 def _init(module, seed, dtype):
 	g = torch.Generator(device="cpu").manual_seed(seed)
 	for m in module.modules():
-		if isinstance(m, nn.Linear):
+		if isinstance(m, (nn.Linear, nn.Embedding)):
 			with torch.no_grad():
 				m.weight.copy_(torch.randn(m.weight.shape, generator=g) * 0.02)
 	return module.to(dtype)
@@ -157,3 +184,9 @@ def gpt_stage(n_blocks, dim, num_heads, ffn_dim, seq_len, causal=False, seed=0, 
 def llama_stage(n_blocks, dim, num_heads, num_kv_heads, ffn_dim, seq_len, head_dim=None, rope_theta=5e5, seed=0, dtype=torch.bfloat16):
 	blocks = [LlamaBlock(dim, num_heads, num_kv_heads, ffn_dim, head_dim, True, rope_theta) for _ in range(n_blocks)]
 	return _init(StageModule(blocks, seq_len), seed, dtype)
+
+
+def gpt_end_stage(n_blocks, dim, num_heads, ffn_dim, seq_len, vocab_in=None, vocab_out=None, causal=True, final_norm=False, seed=0, dtype=torch.bfloat16):
+	"""GPT-style first / last / only stage: (embedding +) blocks (+ final norm + head)."""
+	blocks = StageModule([TransformerBlock(dim, num_heads, ffn_dim, causal) for _ in range(n_blocks)], seq_len)
+	return _init(EndStage(blocks, vocab_in, vocab_out, final_norm), seed, dtype)

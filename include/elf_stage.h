@@ -79,6 +79,12 @@ int elf_scale_grads(void* acc_f32, void* out_bf16, int64_t n, float scale, void*
  * (elf/execution/block.py:651-655) and residual adds (simple.py:460,466). */
 int elf_add_bf16(const void* a, const void* b, void* out, int64_t n, void* stream);
 
+/* Token embedding of a first pipeline stage: out[t, :] = table[ids[t], :] (ids: int64 [T], table: bf16
+ * [V, d], d % 8 == 0; an id outside [0, V) gives a zero row) and its weight gradient dtable[ids[t], :] +=
+ * dx[t, :] in fp32.  Replaces nn.Embedding forward / backward (benchmarks/models/simple.py:496, 502). */
+int elf_embedding_fwd(const void* ids, const void* table, void* out, int64_t T, int d, int V, void* stream);
+int elf_embedding_bwd(const void* ids, const void* dx, void* dtable_f32, int64_t T, int d, int V, void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Attention on the packed projection layout: q/k/v/o are column slices of [T, ld*] bf16 buffers,
  * T = B*S tokens, head h at columns [h*D, (h+1)*D).  Hq % Hkv == 0 (grouped-query attention),
@@ -133,6 +139,10 @@ typedef struct elf_stage_cfg {
  *  3 Wo [d, Hq*D]      4 norm2 gamma    5 norm2 beta (GPT only)
  *  6 W1 [F, d] (GPT fc1)  or  [2F, d] (Llama: gate rows then up rows)     7 W2 [d, F] */
 enum { ELF_P_NORM1_G = 0, ELF_P_NORM1_B, ELF_P_WQKV, ELF_P_WO, ELF_P_NORM2_G, ELF_P_NORM2_B, ELF_P_W1, ELF_P_W2, ELF_P_COUNT };
+/* Stage-level parameters of a first / last pipeline stage, bound with block = -1:
+ *  8 token embedding [vocab_in, d]   9 final norm gamma [d]   10 final norm beta [d] (GPT only)
+ *  11 output head [vocab_out_ld, d] (rows >= vocab_out are padding and must be zero) */
+enum { ELF_P_EMBED = 8, ELF_P_FNORM_G, ELF_P_FNORM_B, ELF_P_HEAD };
 
 /* Forward flags (FORWARD options, elf/scheduling/scheduling.py:58-86):
  *  REMAT_ROOT: remat_strategy selects the whole stage (name == ""), i.e. full checkpointing: only
@@ -157,6 +167,13 @@ int elf_stage_create(const elf_stage_cfg* cfg, elf_stage_t** out);
 void elf_stage_destroy(elf_stage_t* s);
 /* torch keeps ownership; grad_f32 is the fp32 accumulator of the same shape as the weight. */
 int elf_stage_bind_param(elf_stage_t* s, int block, int which, void* weight_bf16, void* grad_f32);
+/* First / last stage of a pipeline (FullTransformer.embed / .head, benchmarks/models/simple.py:496-509);
+ * call once after elf_stage_create.  vocab_in > 0: the stage input x of F / B / RF is int64 token ids [T]
+ * instead of activations, B adds the embedding gradient to its fp32 accumulator and writes no dx (dx may be
+ * NULL).  vocab_out > 0: the stage output y is bf16 logits [T, vocab_out_ld] (vocab_out_ld a multiple of
+ * 64, columns >= vocab_out are zero) and dy is their gradient in the same layout; final_norm != 0 puts a
+ * norm of the architecture's kind in front of the head. */
+int elf_stage_set_ends(elf_stage_t* s, int vocab_in, int vocab_out, int vocab_out_ld, int final_norm);
 /* F: PipelineBlock.forward (block.py:210-279). x, y: bf16 [T, d_model]. */
 int elf_stage_forward(elf_stage_t* s, int mb, const void* x, void* y, uint32_t flags, void* stream);
 /* B: PipelineBlock.backward_inputs (block.py:624-694, 281-306). dy, dx: bf16 [T, d_model]; x is the

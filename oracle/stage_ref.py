@@ -15,6 +15,11 @@ What is restated, and from where (paths are into the reference repository):
   inv_freq = theta^(-2i/D), grouped-query attention = repeat K/V heads, SwiGLU silu(g)*u.
 * ``RefStage``    - PipelineBlock F / B / W / RF / RB* and their slot semantics,
   elf/execution/block.py:210-391, 624-694; full-stage checkpointing elf/execution/remat.py:26-74.
+  ``ends`` adds what the first / last stage of the reference's FullTransformer own
+  (benchmarks/models/simple.py:496-509): ``embed`` = nn.Embedding in front of the blocks (a plain
+  autograd leaf: its gradient accumulates in B), ``head`` = bias-free nn.Linear behind them (a
+  split linear like the others), ``normf_g`` / ``normf_b`` = an optional final norm (no reference
+  module; textbook definition as for the blocks' norms).
 
 Parity pins (tests/test_oracle_cpu.py): SplitLinear against the closed-form 2x2 example held by
 the reference's tests/distributed/distributed_test_block.py:16-55; B-then-W against fused
@@ -219,7 +224,7 @@ class RefStage:
 	acc_dtype: dtype of the dW accumulators (the reference accumulates in the parameter dtype,
 	zb_utils.py:241-244; the HIP path in fp32)."""
 
-	def __init__(self, cfg, params, compute_dtype=torch.float32, acc_dtype=torch.float32, device="cpu", use_sdpa=False):
+	def __init__(self, cfg, params, compute_dtype=torch.float32, acc_dtype=torch.float32, device="cpu", use_sdpa=False, ends=None):
 		self.cfg = dict(cfg)
 		self.device = device
 		self.compute_dtype = compute_dtype
@@ -236,18 +241,34 @@ class RefStage:
 			self.blocks.append(b)
 		self.saved_in, self.saved_out, self.kept_grad = {}, {}, {}
 		self.block_fn = llama_block if cfg["arch"] == ARCH_LLAMA else gpt_block
+		self.ends = {}
+		for name, t in (ends or {}).items():
+			leaf = t.to(device=device, dtype=compute_dtype).clone().requires_grad_(name != "head")
+			self.ends[name] = SplitLinear(leaf) if name == "head" else leaf
 
 	def _linears(self):
-		return [b[n] for b in self.blocks for n in LINEARS]
+		return [b[n] for b in self.blocks for n in LINEARS] + ([self.ends["head"]] if "head" in self.ends else [])
 
 	def _model(self, x):
+		if "embed" in self.ends:
+			x = F.embedding(x, self.ends["embed"])
 		for b in self.blocks:
 			x = self.block_fn(x, b, self.cfg, self.use_sdpa)
+		if "normf_g" in self.ends:
+			e = self.ends
+			x = rms_norm(x, e["normf_g"], self.cfg["eps"]) if self.cfg["arch"] == ARCH_LLAMA else layer_norm(x, e["normf_g"], e["normf_b"], self.cfg["eps"])
+		if "head" in self.ends:
+			x = self.ends["head"](x)
 		return x
+
+	def _as_input(self, x):
+		if "embed" in self.ends:
+			return x.to(device=self.device)  # token ids: no gradient
+		return x.to(device=self.device, dtype=self.compute_dtype).detach().requires_grad_(True)
 
 	# F (block.py:210-263)
 	def forward(self, mb, x, remat_root=False):
-		x = x.to(device=self.device, dtype=self.compute_dtype).detach().requires_grad_(True)
+		x = self._as_input(x)
 		y = checkpoint(self._model, x, use_reentrant=False) if remat_root else self._model(x)
 		for lin in self._linears():
 			lin.move_last("input", mb)
@@ -273,13 +294,13 @@ class RefStage:
 			self.saved_in[mb] = x
 		if recompute_gradients:
 			self.kept_grad[mb] = dy
-		return x.grad.detach()
+		return x.grad.detach() if x.is_floating_point() else None
 
 	# RF (block.py:308-338)
 	def recompute_forward(self, mb, save=False):
 		x = self.saved_in.pop(mb)
 		if save:
-			x = x.detach().requires_grad_(True)
+			x = self._as_input(x)
 			y = self._model(x)
 			self.saved_in[mb], self.saved_out[mb] = x, y
 		else:
@@ -292,7 +313,8 @@ class RefStage:
 	# gradients of the norms must not be accumulated a second time.
 	def recompute_backward_inputs(self, mb):
 		x, y, dy = self.saved_in.pop(mb), self.saved_out.pop(mb), self.kept_grad.pop(mb)
-		torch.autograd.grad(y, [x], dy, allow_unused=True)
+		# only the graph walk matters (it refills the split linears' dY); no .grad is touched
+		torch.autograd.grad(y, [x] if x.is_floating_point() else [self.ends["embed"]], dy, allow_unused=True)
 		for lin in self._linears():
 			lin.move_last("grad_output", mb)
 
@@ -314,9 +336,14 @@ class RefStage:
 				g = v.grad
 				if g is not None:
 					out[f"{i}.{name}"] = g
+		for name, v in self.ends.items():
+			if v.grad is not None:
+				out[f"ends.{name}"] = v.grad
 		return out
 
 	def zero_grad(self):
 		for b in self.blocks:
 			for v in b.values():
 				v.grad = None
+		for v in self.ends.values():
+			v.grad = None

@@ -1,0 +1,173 @@
+"""First / last stage of a decoder on the native executor: token embedding in front of the blocks,
+(final norm,) output head behind them (reference modules: FullTransformer.embed / .head,
+benchmarks/models/simple.py:470-524), against the oracle stage; and the reference's own small
+configuration (4-layer GPT-style decoder, d 256, 4 heads, FFN 1024, seq 128, vocabulary 1000,
+micro-batch 4 x 8, cross-entropy) run through ``Pipeline`` as two stages on one rank against plain
+fp32 autograd over the same weights.  Tolerances: the stage bar (rel 2e-2 of max, 1e-2 Frobenius)."""
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from tests.helpers import assert_close, cfg_from_stage, oracle_params_from_stage, perturb_norms, product_grads
+
+pytestmark = pytest.mark.gpu
+
+
+def test_embedding_kernels_match_torch():
+	from elf_amd import kernels as K
+
+	V, d, T = 1000, 256, 4096
+	g = torch.Generator().manual_seed(1)
+	table = (torch.randn(V, d, generator=g) * 0.5).to(torch.bfloat16).cuda()
+	ids = torch.randint(0, V, (T,), generator=g).cuda()
+	ids[:64] = 7  # a token that repeats: its gradient rows must add up
+	out = K.embedding_fwd(ids, table)
+	assert torch.equal(out, table[ids])
+	bad = ids.clone()
+	bad[3], bad[5] = -1, V
+	out_bad = K.embedding_fwd(bad, table)
+	assert out_bad[3].abs().max().item() == 0 and out_bad[5].abs().max().item() == 0 and torch.equal(out_bad[6:], out[6:])
+	dx = torch.randn(T, d, generator=g).to(torch.bfloat16).cuda()
+	dtab = torch.full((V, d), 0.25, dtype=torch.float32, device="cuda")
+	K.embedding_bwd_(ids, dx, dtab)
+	want = torch.full((V, d), 0.25, dtype=torch.float32, device="cuda").index_add_(0, ids, dx.float())
+	assert_close(dtab, want, "embedding dtable", rel_max=1e-5, rel_fro=1e-5)
+	K.embedding_bwd_(bad, dx, dtab.zero_())
+	assert dtab.abs().sum().item() > 0  # out-of-range ids are skipped, the rest still lands
+
+
+def _end_stage(kind, vocab_in, vocab_out, final_norm, seed):
+	from elf_amd import models
+
+	if kind == "gpt":
+		st = models.gpt_end_stage(1, 256, 4, 512, 128, vocab_in=vocab_in, vocab_out=vocab_out, causal=True, final_norm=final_norm, seed=seed)
+	else:
+		blocks = models.StageModule([models.LlamaBlock(256, 2, 1, 512, 128, True, 5e5)], 128)
+		st = models._init(models.EndStage(blocks, vocab_in, vocab_out, final_norm), seed, torch.bfloat16)
+	perturb_norms(st.blocks)
+	if st.norm_f is not None:
+		with torch.no_grad():
+			st.norm_f.weight.add_(0.1 * torch.randn(st.norm_f.weight.shape).to(torch.bfloat16))
+	return st
+
+
+def _ends_params(st):
+	out = {}
+	if st.embed is not None:
+		out["embed"] = st.embed.weight.detach().clone()
+	if st.head is not None:
+		out["head"] = st.head.weight.detach().clone()
+	if st.norm_f is not None:
+		out["normf_g"] = st.norm_f.weight.detach().clone()
+		if getattr(st.norm_f, "bias", None) is not None:
+			out["normf_b"] = st.norm_f.bias.detach().clone()
+	return out
+
+
+def _ends_grads(st):
+	out = {}
+	for name, mod in (("embed", st.embed), ("head", st.head), ("normf_g", st.norm_f)):
+		if mod is not None:
+			out[f"ends.{name}"] = mod.weight.main_grad
+	if st.norm_f is not None and getattr(st.norm_f, "bias", None) is not None:
+		out["ends.normf_b"] = st.norm_f.bias.main_grad
+	return out
+
+
+@pytest.mark.parametrize("case", [("gpt", 1000, None, False), ("gpt", None, 1000, False), ("gpt", None, 1024, True), ("llama", 512, 320, True)])
+@pytest.mark.parametrize("variant", ["plain", "full_fwd", "full_bwd"])
+def test_first_and_last_stage_match_oracle(case, variant):
+	"""F, B, W (and the remat variants) of a stage with an embedding and / or a head, driven
+	directly through the block's ops with hand-fed boundaries."""
+	from elf_amd.execution import HipStageBlock
+	from elf_amd.partitioners.utils import sequential_signatures
+	from elf_amd.scheduling import OpOptions
+	from oracle import stage_ref as R
+
+	kind, vin, vout, fnorm = case
+	mb, nmb, S, d = 2, 2, 128, 256
+	st = _end_stage(kind, vin, vout, fnorm, seed=31)
+	cfg = cfg_from_stage(st.blocks, mb)
+	ref = R.RefStage(cfg, oracle_params_from_stage(st.blocks), device="cuda", ends=_ends_params(st))
+	placement = [0, 1, 2]
+	blk = HipStageBlock(st, 1, placement, sequential_signatures(placement)[1], mb_size=mb)
+	blk.zero_grad()
+	g = torch.Generator().manual_seed(5)
+	xs = [torch.randint(0, vin, (mb, S), generator=g).cuda() if vin else torch.randn(mb, S, d, generator=g).to(torch.bfloat16).cuda() for _ in range(nmb)]
+	dys = [(torch.randn(mb, S, vout or d, generator=g) * (0.1 if vout else 1.0)).to(torch.bfloat16).cuda() for _ in range(nmb)]
+	blk.set_boundary(inputs=xs, grads=dys, keep_sent=True)
+	root = (lambda name, module: name == "") if variant == "full_fwd" else None
+	for m in range(nmb):
+		blk.recv_forward(m, mb, src=0)
+		blk.forward(m, **({OpOptions.REMAT_STRATEGY: root} if root else {}))
+		blk.send_forward(m, dst=2)
+		y = blk.sent_forward[m]
+		assert tuple(y.shape) == (mb, S, vout or d)
+		assert_close(y, ref.forward(m, xs[m], remat_root=root is not None), f"{case} y[{m}]")
+	for m in range(nmb):
+		blk.recv_backward(m, mb, src=2)
+		full_bwd = variant == "full_bwd"
+		blk.backward_inputs(m, **({OpOptions.RECOMPUTE_ACTIVATIONS: True, OpOptions.RECOMPUTE_GRADIENTS: True} if full_bwd else {}))
+		blk.send_backward(m, dst=0)
+		want_dx = ref.backward_inputs(m, dys[m], recompute_activations=full_bwd, recompute_gradients=full_bwd)
+		if vin:
+			assert want_dx is None and m not in blk.sent_backward
+		else:
+			assert_close(blk.sent_backward[m], want_dx, f"{case} dx[{m}]")
+		if full_bwd:
+			blk.recompute_forward(m, **{OpOptions.SAVE: True})
+			blk.recompute_backward_inputs(m)
+			ref.recompute_forward(m, save=True)
+			ref.recompute_backward_inputs(m)
+		blk.backward_params(m)
+		ref.backward_params(m)
+	torch.cuda.synchronize()
+	got = dict(product_grads(st.blocks), **_ends_grads(st))
+	want = ref.grads()
+	assert set(want) <= set(got)
+	for name in sorted(want):
+		assert_close(got[name], want[name], f"{case} {variant} grad {name}")
+	if vout and blk.vld != vout:  # the padding rows of the head never receive a gradient
+		assert blk._fused_g[blk._param_loc[st.head.weight][0]][vout:].abs().max().item() == 0
+	assert blk.mem_stats()["live_bytes"] == 0
+
+
+def test_reference_small_configuration_through_pipeline():
+	"""4-layer GPT-style decoder, d 256, 4 heads, FFN 1024 GELU, LayerNorm, seq 128, vocabulary 1000,
+	micro-batch 4 x 8 micro-batches, cross-entropy on fp32 logits flattened over the sequence
+	(FullTransformer.loss_fn, benchmarks/models/simple.py:519-523), as two stages on one rank."""
+	from elf_amd import models
+	from elf_amd.pipeline import Pipeline
+
+	V, d, S, mb, nmb = 1000, 256, 128, 4, 8
+	first = models.gpt_end_stage(2, d, 4, 1024, S, vocab_in=V, causal=True, seed=41)
+	last = models.gpt_end_stage(2, d, 4, 1024, S, vocab_out=V, causal=True, seed=42)
+	for st in (first, last):
+		perturb_norms(st.blocks)
+
+	def loss_fn(pred, target, *args, **kwargs):
+		return F.cross_entropy(pred.to(torch.float32).view(-1, V), target.view(-1), *args, **kwargs)
+
+	# plain autograd in fp32 over the same (bf16-rounded) weights, whole batch at once
+	import copy
+
+	ref_first, ref_last = copy.deepcopy(first).float().cuda(), copy.deepcopy(last).float().cuda()
+	g = torch.Generator().manual_seed(9)
+	ids = torch.randint(0, V, (mb * nmb, S), generator=g).cuda()
+	tgt = torch.randint(0, V, (mb * nmb, S), generator=g).cuda()
+	logits = ref_last(ref_first(ids))
+	want_loss = F.cross_entropy(logits.view(-1, V), tgt.view(-1), reduction="sum") / (S * mb * nmb)
+	want_loss.backward()
+
+	pipe = Pipeline([first, last], ids[:mb], scheduler="afab", partitioner=False, placement=[0, 0])
+	pipe.zero_grad()
+	result, loss = pipe(ids, tgt, loss_fn, split_size=mb)
+	assert len(result) == nmb and tuple(result[0].shape) == (mb, S, V)
+	assert_close(torch.cat([r.float() for r in result]), logits.detach(), "logits")
+	assert abs(float(loss) - float(want_loss.detach())) <= 1e-2 * float(want_loss.detach())
+	for mod, ref_mod in ((first, ref_first), (last, ref_last)):
+		ref_params = dict(ref_mod.named_parameters())
+		for name, p in mod.named_parameters():
+			assert_close(p.main_grad, ref_params[name].grad, f"grad {name}", rel_max=3e-2, rel_fro=2e-2)
+			assert_close(p.grad, ref_params[name].grad, f"bf16 grad {name}", rel_max=4e-2, rel_fro=2e-2)

@@ -219,3 +219,59 @@ def test_product_modules_agree_with_the_oracle_blocks():
 		ref = R.RefStage(cfg, oracle_params_from_stage(stage))
 		x = torch.randn(2, 8, 32)
 		assert torch.allclose(stage(x), ref.forward(0, x), atol=2e-5)
+
+
+@pytest.mark.parametrize("kind", ["gpt", "llama"])
+def test_stage_ends_equal_library_embedding_and_linear(kind):
+	"""The oracle's first / last stage pieces against library routines on the whole batch: the
+	embedding is F.embedding (its gradient an index_add of the block-0 input gradient), the head
+	a plain matmul behind the (closed-form) final norm; F/B/W over 3 micro-batches in any order sum
+	to the full-batch gradients, and every remat variant gives them too."""
+	cfg = CFG[kind]
+	V_in, V_out, d = 37, 29, cfg["d_model"]
+	params = R.make_params(cfg, seed=5, dtype=torch.float64)
+	g = torch.Generator().manual_seed(6)
+	ends = {"embed": torch.randn(V_in, d, generator=g, dtype=torch.float64), "head": torch.randn(V_out, d, generator=g, dtype=torch.float64) * 0.1,
+	        "normf_g": 1 + 0.1 * torch.randn(d, generator=g, dtype=torch.float64)}
+	if kind == "gpt":
+		ends["normf_b"] = 0.1 * torch.randn(d, generator=g, dtype=torch.float64)
+	ids = [torch.randint(0, V_in, (cfg["mb"], cfg["seq"]), generator=g) for _ in range(3)]
+	ids[0][0, :4] = 3  # repeated token
+	dls = [torch.randn(cfg["mb"], cfg["seq"], V_out, generator=g, dtype=torch.float64) for _ in range(3)]
+
+	# whole batch with library routines around the (already pinned) block chain
+	emb = ends["embed"].clone().requires_grad_(True)
+	head = ends["head"].clone().requires_grad_(True)
+	ng = ends["normf_g"].clone().requires_grad_(True)
+	nb = ends["normf_b"].clone().requires_grad_(True) if kind == "gpt" else None
+	x0 = F.embedding(torch.cat(ids), emb)
+	x0.retain_grad()
+	inner = R.RefStage(cfg, params, compute_dtype=torch.float64, acc_dtype=torch.float64)
+	h = inner._model(x0)
+	hn = F.layer_norm(h, (d,), ng, nb, cfg["eps"]) if kind == "gpt" else h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + cfg["eps"]) * ng
+	logits = hn @ head.t()
+	logits.backward(torch.cat(dls))
+	want_embed = torch.zeros(V_in, d, dtype=torch.float64).index_add_(0, torch.cat(ids).reshape(-1), x0.grad.reshape(-1, d))
+	assert torch.allclose(emb.grad, want_embed, atol=1e-10)
+
+	for variant in ("plain", "full_fwd", "full_bwd"):
+		ref = R.RefStage(cfg, params, compute_dtype=torch.float64, acc_dtype=torch.float64, ends=ends)
+		ys = [ref.forward(m, ids[m], remat_root=variant == "full_fwd") for m in range(3)]
+		assert torch.allclose(torch.cat(ys), logits.detach(), atol=1e-9)
+		for m in (2, 0, 1):
+			fb = variant == "full_bwd"
+			assert ref.backward_inputs(m, dls[m], recompute_activations=fb, recompute_gradients=fb) is None
+			if fb:
+				ref.recompute_forward(m, save=True)
+				ref.recompute_backward_inputs(m)
+			ref.backward_params(m)
+		got = ref.grads()
+		assert torch.allclose(got["ends.embed"], emb.grad, atol=1e-8), variant
+		assert torch.allclose(got["ends.head"], head.grad, atol=1e-8), variant
+		assert torch.allclose(got["ends.normf_g"], ng.grad, atol=1e-8), variant
+		if kind == "gpt":
+			assert torch.allclose(got["ends.normf_b"], nb.grad, atol=1e-8), variant
+		inner_grads = {f"{i}.{k}": (v.weight.grad if isinstance(v, R.SplitLinear) else v.grad) for i, b in enumerate(inner.blocks) for k, v in b.items()}
+		for name, gr in inner_grads.items():
+			if gr is not None:  # norm gains / biases of the blocks (their linears are split: no autograd .grad)
+				assert torch.allclose(got[name], gr, atol=1e-8), (variant, name)
