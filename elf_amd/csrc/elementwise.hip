@@ -229,8 +229,9 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(const bf16_t* __restrict_
 	}
 }
 
-// main_grad[c] += sum_b part[b][which][c].  One workgroup owns 32 columns; its 8 row groups
-// stride over the partial rows and are folded through LDS.
+// main_grad[c] += sum_b part[b][which][c].  A workgroup owns 32 columns and one of gridDim.y slices
+// of the partial rows; its 8 row groups stride over the slice and are folded through LDS, the
+// slices meet in the accumulator through fp32 atomics (a few thousand per call).
 __global__ __launch_bounds__(256) void norm_bwd_finalize_kernel(const float* __restrict__ part, int nparts, int d,
                                                                 float* __restrict__ dgamma, float* __restrict__ dbeta) {
 	__shared__ float red[2][8][32];
@@ -238,7 +239,7 @@ __global__ __launch_bounds__(256) void norm_bwd_finalize_kernel(const float* __r
 	const int c = blockIdx.x * 32 + cl;
 	float sg = 0.f, sb = 0.f;
 	if (c < d) {
-		for (int b = rg; b < nparts; b += 8) {
+		for (int b = blockIdx.y * 8 + rg; b < nparts; b += 8 * gridDim.y) {
 			sg += part[(int64_t)b * 2 * d + c];
 			if (dbeta) sb += part[(int64_t)b * 2 * d + d + c];
 		}
@@ -253,8 +254,8 @@ __global__ __launch_bounds__(256) void norm_bwd_finalize_kernel(const float* __r
 			tg += red[0][r][cl];
 			tb += red[1][r][cl];
 		}
-		dgamma[c] += tg;
-		if (dbeta) dbeta[c] += tb;
+		unsafeAtomicAdd(dgamma + c, tg);
+		if (dbeta) unsafeAtomicAdd(dbeta + c, tb);
 	}
 }
 
@@ -325,8 +326,13 @@ int norm_bwd(int kind, const void* dy, const void* x, const void* gamma, const v
 		rc = norm_bwd_dispatch<false>(dy, x, gamma, stats, dres, dx, workspace, T, d, s);
 	}
 	if (rc) return rc;
-	hipLaunchKernelGGL(norm_bwd_finalize_kernel, dim3((d + 31) / 32), dim3(256), 0, s, workspace,
-	                   norm_bwd_blocks(T, d), d, dgamma, kind == NORM_LAYER ? dbeta : nullptr);
+	const int nparts = norm_bwd_blocks(T, d);
+	const int col_blocks = (d + 31) / 32;
+	int slices = (512 + col_blocks - 1) / col_blocks;  // about two workgroups per CU
+	if (slices > (nparts + 7) / 8) slices = (nparts + 7) / 8;
+	if (slices < 1) slices = 1;
+	hipLaunchKernelGGL(norm_bwd_finalize_kernel, dim3(col_blocks, slices), dim3(256), 0, s, workspace, nparts, d, dgamma,
+	                   kind == NORM_LAYER ? dbeta : nullptr);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
 }
