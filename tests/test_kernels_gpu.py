@@ -240,6 +240,7 @@ def _attn_ref(qkv, B, S, Hq, Hkv, D, causal, do=None):
 @pytest.mark.parametrize("cfg", [
 	(1, 128, 2, 2, 64, False), (2, 256, 4, 4, 64, False), (2, 256, 4, 2, 128, True),
 	(1, 512, 8, 2, 128, True), (1, 384, 2, 1, 64, True), (2, 128, 4, 4, 128, False),
+	(1, 1024, 4, 1, 128, True), (1, 1024, 3, 3, 64, False), (1, 640, 2, 2, 128, True),
 ])
 def test_attention_fwd_bwd(K, cfg):
 	B, S, Hq, Hkv, D, causal = cfg
