@@ -16,6 +16,7 @@ hand tensors over locally, as in the reference engine), and no process groups ar
 """
 
 import logging
+import os
 from dataclasses import asdict, dataclass, field, fields
 from typing import Any, List
 
@@ -183,6 +184,48 @@ class Pipeline:
 		torch.cuda.synchronize()
 		for block in self.blocks:
 			block.clear()
+
+	# ------------------------------------------------------------------ checkpoints (elf/pipeline.py:346-451)
+	def checkpoint(self, epoch="init", dir_path="./"):
+		"""One file per rank, ``{dir_path}/{epoch}/dp{dp}_pp{pp}.pt`` holding ``rank``, ``pp``, ``dp``,
+		``epoch`` and one ``state_dict_{block id}`` per owned block: the reference's format."""
+		dp, pp = self.rank // self.pp, self.rank % self.pp
+		state = {"rank": self.rank, "pp": pp, "dp": dp, "epoch": epoch}
+		for block in self.blocks:
+			state[f"state_dict_{block.id}"] = {k: v.data.clone() for k, v in block.model.state_dict().items()}
+		dir_path = f"{dir_path}/{epoch}/"
+		os.makedirs(dir_path, exist_ok=True)
+		torch.save(state, f"{dir_path}/dp{dp}_pp{pp}.pt")
+
+	def load_checkpoint(self, epoch="init", dir_path="./"):
+		"""Reads this rank's file back into the owned blocks (the values land in the fused weight
+		buffers the library reads, since the modules' parameters are views of them)."""
+		dp, pp = self.rank // self.pp, self.rank % self.pp
+		state = torch.load(f"{dir_path}/{epoch}/dp{dp}_pp{pp}.pt", map_location="cuda", weights_only=True)
+		for block in self.blocks:
+			with torch.no_grad():
+				for k, v in block.model.state_dict().items():
+					v.copy_(state[f"state_dict_{block.id}"][k])
+
+	def gather_parameters(self, dst=0):
+		"""{parameter name: tensor} of every block (all of them live on this rank); a name that occurs in
+		several blocks keeps its first occurrence, as in the reference."""
+		if self.rank != dst:
+			return {}
+		out = {}
+		for block in self.blocks:
+			for name, param in block.model.named_parameters():
+				if name not in out:
+					out[name] = param.data
+				else:
+					logger.warning(f"Duplicate parameter {name} found in block {block.id}, using first occurrence")
+		return out
+
+	def save(self, path, worker=0):
+		"""All parameters of the pipeline on the CPU in one file."""
+		if self.rank == worker:
+			torch.save({name: p.detach().cpu() for name, p in self.named_parameters()}, path)
+			logger.info(f"Saved model to {path}")
 
 	def is_first(self):
 		return self.placement.is_head(self.rank)
