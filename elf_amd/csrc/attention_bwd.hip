@@ -5,27 +5,30 @@ namespace elf {
 namespace attn {
 
 // ------------------------------------------------------------------------------------------
-// delta[b,h,s] = sum_d dO * O and nlse2[b,h,s] = -lse * log2(e)   (one wave per token-head)
+// delta[b,h,s] = sum_d dO * O and nlse2[b,h,s] = -lse * log2(e).  D/8 lanes share one (token, head)
+// row, 16 bytes each, so a wave covers 4 (D = 128) or 8 (D = 64) rows per step.
 __global__ __launch_bounds__(256) void attn_delta_kernel(const bf16_t* __restrict__ dO, const bf16_t* __restrict__ O,
                                                          const float* __restrict__ lse, float* __restrict__ delta,
                                                          float* __restrict__ nlse2, int64_t ldd, int64_t ldo, int B, int S,
                                                          int Hq, int D) {
-	const int lane = threadIdx.x & 63;
-	const int64_t idx = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // token * Hq + h
-	if (idx >= (int64_t)B * S * Hq) return;
-	const int h = (int)(idx % Hq);
-	const int64_t tok = idx / Hq;
-	float s = 0.f;
-	for (int c = lane * 2; c < D; c += 128) {
-		bf16x2 x = *reinterpret_cast<const bf16x2*>(dO + tok * ldd + h * D + c);
-		bf16x2 y = *reinterpret_cast<const bf16x2*>(O + tok * ldo + h * D + c);
-		s += (float)x[0] * (float)y[0] + (float)x[1] * (float)y[1];
-	}
-	s = wave_sum(s);
-	if (lane == 0) {
-		const int64_t b = tok / S, sp = tok % S;
-		delta[(b * Hq + h) * S + sp] = s;
-		nlse2[(b * Hq + h) * S + sp] = -lse[(b * Hq + h) * S + sp] * LOG2E;
+	const int lpr = D / 8;  // lanes per row: 8 or 16
+	const int rows_per_block = 256 / lpr;
+	const int sub = threadIdx.x % lpr;
+	const int64_t n = (int64_t)B * S * Hq;
+	for (int64_t idx = (int64_t)blockIdx.x * rows_per_block + threadIdx.x / lpr; idx < n; idx += (int64_t)gridDim.x * rows_per_block) {
+		const int h = (int)(idx % Hq);
+		const int64_t tok = idx / Hq;
+		const bf16x8 x = *reinterpret_cast<const bf16x8*>(dO + tok * ldd + h * D + sub * 8);
+		const bf16x8 y = *reinterpret_cast<const bf16x8*>(O + tok * ldo + h * D + sub * 8);
+		float s = 0.f;
+#pragma unroll
+		for (int j = 0; j < 8; j++) s += (float)x[j] * (float)y[j];
+		for (int o = lpr >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+		if (sub == 0) {
+			const int64_t b = tok / S, sp = tok % S;
+			delta[(b * Hq + h) * S + sp] = s;
+			nlse2[(b * Hq + h) * S + sp] = -lse[(b * Hq + h) * S + sp] * LOG2E;
+		}
 	}
 }
 
@@ -445,6 +448,7 @@ int attn_bwd(const void* q, const void* k, const void* v, const void* o, const v
 	                lddk % 8 == 0 && lddv % 8 == 0,
 	            "attn_bwd: strides must be multiples of 8");
 	ELF_REQUIRE(((uintptr_t)workspace % 16) == 0, "attn_bwd: misaligned workspace");
+	ELF_REQUIRE(((uintptr_t)o % 16) == 0 && ((uintptr_t)dO % 16) == 0, "attn_bwd: o and dO must be 16-byte aligned");
 	ProfScope prof(PROF_ATTN_BWD, (causal ? 4.0 : 8.0) * B * Hq * (double)S * S * D, stream);
 	const int64_t T = (int64_t)B * S;
 	float* dq_acc = (float*)workspace;
@@ -452,8 +456,12 @@ int attn_bwd(const void* q, const void* k, const void* v, const void* o, const v
 	float* nlse2 = delta + T * Hq;
 	// zero the dQ accumulator with a fill kernel (memset nodes misbehave under graph replay)
 	hipLaunchKernelGGL(fill_zero_kernel, dim3(2048), dim3(256), 0, stream, (f32x4*)dq_acc, T * Hq * D / 4);
-	hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)((T * Hq + 3) / 4)), dim3(256), 0, stream, (const bf16_t*)dO,
+	{
+		const int64_t rows = T * Hq, per_block = 256 / (D / 8);
+		const int64_t want = (rows + per_block - 1) / per_block;
+		hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)(want < 8192 ? want : 8192)), dim3(256), 0, stream, (const bf16_t*)dO,
 	                   (const bf16_t*)o, (const float*)lse, delta, nlse2, lddo, ldo, B, S, Hq, D);
+	}
 	AttnBwdArgs a{(const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, (const bf16_t*)dO, nlse2, delta, dq_acc,
 	              (bf16_t*)dk, (bf16_t*)dv, ldq, ldk, ldv, lddo, lddk, lddv, B, S, Hq, Hkv, scale};
 	const int nkt = S / 128;
