@@ -275,9 +275,6 @@ static int launch_layout(GemmArgs& g, int tile_cfg, hipStream_t stream) {
 		case 3:
 			ELF_REQUIRE(M % 64 == 0 && N % 64 == 0, "gemm: M and N must be multiples of 64 (M=%d N=%d)", M, N);
 			return launch_cfg<64, 64, 2, 2, AT, BT, EPI>(g, stream);
-		case 4:
-			ELF_REQUIRE(M % 256 == 0 && N % 256 == 0, "gemm: tile 256 needs M,N multiples of 256 (M=%d N=%d)", M, N);
-			return launch_cfg<256, 256, 2, 2, AT, BT, EPI>(g, stream);
 		case 5:
 			ELF_REQUIRE(M % 256 == 0 && N % 128 == 0, "gemm: tile 256x128 needs M%%256==0, N%%128==0 (M=%d N=%d)", M, N);
 			return launch_cfg<256, 128, 2, 2, AT, BT, EPI>(g, stream);
