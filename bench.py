@@ -196,7 +196,7 @@ def main():
 		step()
 	torch.cuda.synchronize()
 	elapsed = time.perf_counter() - t0
-	kinds = ["gemm", "attn_fwd", "attn_bwd", "norm_fwd", "norm_bwd", "act_fwd", "act_bwd", "rope", "grad_scale", "add", "embed"]
+	kinds = ["gemm", "attn_fwd", "attn_bwd", "norm_fwd", "norm_bwd", "act_fwd", "act_bwd", "rope", "grad_scale", "add", "embed", "loss"]
 	per_kernel = {}
 	for i, name in enumerate(kinds):
 		ms, work = ctypes.c_double(), ctypes.c_double()

@@ -33,6 +33,8 @@ _SIGNATURES = {
 	"elf_add_bf16": (c_int, [_P, _P, _P, c_int64, _P]),
 	"elf_embedding_fwd": (c_int, [_P, _P, _P, c_int64, c_int, c_int, _P]),
 	"elf_embedding_bwd": (c_int, [_P, _P, _P, c_int64, c_int, c_int, _P]),
+	"elf_cross_entropy": (c_int, [_P, c_int64, _P, c_int64, c_int64, c_int64, c_float, _P, _P, _P, c_int64, _P]),
+	"elf_cross_entropy_reduce": (c_int, [_P, _P, c_int64, c_int64, _P, _P]),
 	"elf_attn_fwd": (c_int, [_P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_float, _P]),
 	"elf_attn_bwd_workspace_bytes": (c_int64, [c_int, c_int, c_int, c_int]),
 	"elf_prof_enable": (None, [c_int]),

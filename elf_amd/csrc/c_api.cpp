@@ -53,6 +53,13 @@ int elf_embedding_fwd(const void* ids, const void* table, void* out, int64_t T, 
 int elf_embedding_bwd(const void* ids, const void* dx, void* dtable_f32, int64_t T, int d, int V, void* stream) {
 	return elf::embedding_bwd(ids, dx, dtable_f32, T, d, V, S_(stream));
 }
+int elf_cross_entropy(const void* logits, int64_t ld, const void* target, int64_t rows, int64_t V, int64_t ignore_index, float scale,
+                      const void* dev_div, void* row_loss, void* dlogits, int64_t ld_out, void* stream) {
+	return elf::cross_entropy(logits, ld, target, rows, V, ignore_index, scale, dev_div, row_loss, dlogits, ld_out, S_(stream));
+}
+int elf_cross_entropy_reduce(const void* row_loss, const void* target, int64_t rows, int64_t ignore_index, void* out2, void* stream) {
+	return elf::cross_entropy_reduce(row_loss, target, rows, ignore_index, out2, S_(stream));
+}
 int elf_attn_fwd(const void* q, const void* k, const void* v, void* o, void* lse, int64_t ldq, int64_t ldk, int64_t ldv,
                  int64_t ldo, int B, int S, int Hq, int Hkv, int D, int causal, float scale, void* stream) {
 	return elf::attn_fwd(q, k, v, o, lse, ldq, ldk, ldv, ldo, B, S, Hq, Hkv, D, causal, scale, S_(stream));

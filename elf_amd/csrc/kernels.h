@@ -39,6 +39,10 @@ int add_bf16(const void* a, const void* b, void* out, int64_t n, hipStream_t s);
 // ids: int64 [T]; table bf16 [V, d]; dtable fp32 [V, d] (+=)
 int embedding_fwd(const void* ids, const void* table, void* out, int64_t T, int d, int V, hipStream_t s);
 int embedding_bwd(const void* ids, const void* dx, void* dtable_f32, int64_t T, int d, int V, hipStream_t s);
+// Cross-entropy over bf16 logits [rows, V] (row stride ld), loss and gradient in one pass; target int64 [rows].
+int cross_entropy(const void* logits, int64_t ld, const void* target, int64_t rows, int64_t V, int64_t ignore_index, float scale,
+                  const void* dev_div, void* row_loss, void* dlogits, int64_t ld_out, hipStream_t s);
+int cross_entropy_reduce(const void* row_loss, const void* target, int64_t rows, int64_t ignore_index, void* out2, hipStream_t s);
 
 // Attention over the packed projection layout; lse is [B, Hq, S] fp32 (natural log).
 int attn_fwd(const void* q, const void* k, const void* v, void* o, void* lse, int64_t ldq, int64_t ldk, int64_t ldv,
@@ -53,7 +57,7 @@ int attn_bwd(const void* q, const void* k, const void* v, const void* o, const v
 // with an event pair on the launch stream and books the algorithmic work of the call.
 enum ProfKind {
 	PROF_GEMM = 0, PROF_ATTN_FWD, PROF_ATTN_BWD, PROF_NORM_FWD, PROF_NORM_BWD, PROF_ACT_FWD, PROF_ACT_BWD, PROF_ROPE,
-	PROF_SCALE, PROF_ADD, PROF_EMBED, PROF_COUNT
+	PROF_SCALE, PROF_ADD, PROF_EMBED, PROF_LOSS, PROF_COUNT
 };
 void prof_enable(int on);
 bool prof_on();

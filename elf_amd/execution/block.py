@@ -285,9 +285,28 @@ class HipStageBlock:
 			raise _lib.ElfStageError(f"{self}: the gradient of the logits must be a bf16 GPU tensor of {self.T}x{self.vocab_out} elements, got {tuple(dy.shape)} {dy.dtype} {dy.device}")
 		if self.vld == self.vocab_out:
 			return dy.contiguous()
+		if self._rows_padded(dy):
+			# rows already sit vld apart (the layout elf_amd.losses writes): read in place, with the
+			# columns past the vocabulary cleared so they add nothing to dX and dW
+			buf = torch.as_strided(dy, (self.T, self.vld), (self.vld, 1))
+			buf[:, self.vocab_out :].zero_()
+			return buf
 		pad = torch.zeros(self.T, self.vld, dtype=torch.bfloat16, device=dy.device)
 		pad[:, : self.vocab_out] = dy.reshape(self.T, self.vocab_out)
 		return pad
+
+	def _rows_padded(self, dy):
+		"""Whether ``dy`` is a [..., vocab_out] view whose rows are exactly ``vld`` elements apart inside
+		one allocation that holds all ``T * vld`` of them."""
+		if dy.dim() < 2 or dy.stride(-1) != 1 or dy.stride(-2) != self.vld or dy.data_ptr() % 16:
+			return False
+		expect = self.vld
+		for size, stride in zip(reversed(dy.shape[:-1]), reversed(dy.stride()[:-1])):
+			if size != 1 and stride != expect:
+				return False
+			expect *= size
+		room = dy.untyped_storage().nbytes() // dy.element_size() - dy.storage_offset()
+		return room >= self.T * self.vld
 
 	def _timed(self, name):
 		t = Timer(name=name)

@@ -222,6 +222,14 @@ def compute_loss(block, output, target, loss_fn):
 	the closure that back-propagates it to the block output."""
 	if not isinstance(output, torch.Tensor) or not isinstance(target, torch.Tensor):
 		logger.warning("Loss computation with non-tensor output or target")
+	elems = target.numel() // target.size(0)
+	fused = getattr(loss_fn, "loss_and_grad", None)
+	if fused is not None:
+		# loss and gradient from one kernel (elf_amd.losses): nothing for autograd to record
+		with Timer(name="loss_forward") as timer:
+			loss, grad = fused(output.detach(), target, reduction="sum", scale=1.0 / elems)
+		block.compute_time.append(timer)
+		return (loss / elems).detach(), lambda: (grad,)
 	output = output.detach().requires_grad_()
 	with Timer(name="loss_forward") as timer:
 		try:
@@ -229,7 +237,7 @@ def compute_loss(block, output, target, loss_fn):
 		except TypeError:
 			loss = loss_fn(output, target)
 	block.compute_time.append(timer)
-	loss = loss / (target.numel() // target.size(0))
+	loss = loss / elems
 
 	def grad_fn():
 		loss.backward()

@@ -86,6 +86,24 @@ int elf_add_bf16(const void* a, const void* b, void* out, int64_t n, void* strea
 int elf_embedding_fwd(const void* ids, const void* table, void* out, int64_t T, int d, int V, void* stream);
 int elf_embedding_bwd(const void* ids, const void* dx, void* dtable_f32, int64_t T, int d, int V, void* stream);
 
+/* Cross-entropy of a last pipeline stage, loss and gradient in one pass over the logits.  Replaces the
+ * reference's loss function (benchmarks/models/simple.py:520-524: upcast to fp32, flatten,
+ * torch.nn.functional.cross_entropy) and its backward as Engine.compute_loss runs them
+ * (elf/execution/engine.py:374-410).
+ *   logits   bf16 [rows, V], row stride ld elements (ld % 8 == 0, base 16-byte aligned)
+ *   target   int64 [rows]; rows with target == ignore_index contribute no loss and a zero gradient;
+ *            any other target outside [0, V) makes that row's loss NaN
+ *   row_loss fp32 [rows] or NULL:  logsumexp(logits[r, :]) - logits[r, target[r]], arithmetic in fp32
+ *   dlogits  bf16 [rows, ld_out] or NULL (ld_out % 8 == 0, >= V; must not overlap logits):
+ *            (softmax(logits[r, :]) - onehot(target[r])) * scale / (dev_div ? *dev_div : 1), columns
+ *            V .. ld_out-1 are written as zeros
+ *   dev_div  optional device fp32 scalar (e.g. the count of non-ignored rows for reduction="mean")
+ * elf_cross_entropy_reduce: out2[0] = sum of row_loss (untouched when row_loss is NULL), out2[1] =
+ * number of rows whose target is not ignore_index; fixed summation order (bit-reproducible). */
+int elf_cross_entropy(const void* logits, int64_t ld, const void* target, int64_t rows, int64_t V, int64_t ignore_index, float scale,
+                      const void* dev_div, void* row_loss, void* dlogits, int64_t ld_out, void* stream);
+int elf_cross_entropy_reduce(const void* row_loss, const void* target, int64_t rows, int64_t ignore_index, void* out2, void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Attention on the packed projection layout: q/k/v/o are column slices of [T, ld*] bf16 buffers,
  * T = B*S tokens, head h at columns [h*D, (h+1)*D).  Hq % Hkv == 0 (grouped-query attention),

@@ -133,10 +133,12 @@ def test_first_and_last_stage_match_oracle(case, variant):
 	assert blk.mem_stats()["live_bytes"] == 0
 
 
-def test_reference_small_configuration_through_pipeline():
+@pytest.mark.parametrize("loss_kind", ["torch", "fused"])
+def test_reference_small_configuration_through_pipeline(loss_kind):
 	"""4-layer GPT-style decoder, d 256, 4 heads, FFN 1024 GELU, LayerNorm, seq 128, vocabulary 1000,
 	micro-batch 4 x 8 micro-batches, cross-entropy on fp32 logits flattened over the sequence
-	(FullTransformer.loss_fn, benchmarks/models/simple.py:519-523), as two stages on one rank."""
+	(FullTransformer.loss_fn, benchmarks/models/simple.py:519-523), as two stages on one rank; once with
+	that torch loss under autograd and once with the library's one-kernel cross-entropy."""
 	from elf_amd import models
 	from elf_amd.pipeline import Pipeline
 
@@ -148,6 +150,9 @@ def test_reference_small_configuration_through_pipeline():
 
 	def loss_fn(pred, target, *args, **kwargs):
 		return F.cross_entropy(pred.to(torch.float32).view(-1, V), target.view(-1), *args, **kwargs)
+
+	if loss_kind == "fused":
+		from elf_amd.losses import cross_entropy as loss_fn
 
 	# plain autograd in fp32 over the same (bf16-rounded) weights, whole batch at once
 	import copy

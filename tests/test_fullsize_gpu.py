@@ -128,3 +128,33 @@ def test_bandwidth_kernels_at_full_size(K):
 	out = torch.empty(D_MODEL, FFN, dtype=torch.bfloat16, device="cuda")
 	K.scale_grads_(acc, out, 1.0 / 32)
 	assert torch.equal(acc, want) and torch.equal(out, want.to(torch.bfloat16))
+
+
+def test_cross_entropy_at_the_llama_vocabulary(K):
+	"""One micro-batch of logits at the Llama-3 vocabulary (8192 x 128256): rows whose logits are zero
+	except b at the target have the closed-form loss log(1 + (V-1) e^-b); every gradient row sums to
+	zero (softmax - onehot) within bf16 rounding; a sample of random rows matches the CPU oracle."""
+	import math
+
+	from elf_amd import losses
+	from oracle import loss_ref as L
+
+	V, b = 128256, 5.0
+	g = torch.Generator(device="cuda").manual_seed(21)
+	x = (torch.randn(T, V, device="cuda", generator=g) * 2.0).to(torch.bfloat16)
+	t = torch.randint(0, V, (T,), device="cuda", generator=g)
+	x[:256] = 0
+	x[torch.arange(256, device="cuda"), t[:256]] = b
+	loss, grad = losses.cross_entropy.loss_and_grad(x, t, reduction="sum", scale=1.0)
+	rows = losses.cross_entropy(x, t, reduction="none")
+	assert float(loss) == pytest.approx(float(rows.double().sum()), rel=1e-5)
+	assert torch.allclose(rows[:256], torch.full((256,), math.log1p((V - 1) * math.exp(-b)), device="cuda"), rtol=1e-5)
+	row_sums = grad.float().sum(-1)
+	assert row_sums.abs().max().item() <= 2e-2  # |sum| of V values each rounded to bf16
+	pick = torch.arange(256, T, 131, device="cuda")
+	xs, ts = x[pick].cpu(), t[pick].cpu()
+	assert torch.allclose(rows[pick].cpu(), L.cross_entropy_ref(xs, ts, "none"), rtol=1e-5, atol=2e-5)
+	xf = xs.float().requires_grad_()
+	L.cross_entropy_ref(xf, ts, "sum").backward()
+	err = (grad[pick].float().cpu() - xf.grad).abs()
+	assert bool((err <= xf.grad.abs() * 2.0**-7 + 1e-6).all())

@@ -275,3 +275,37 @@ def test_stage_ends_equal_library_embedding_and_linear(kind):
 		for name, gr in inner_grads.items():
 			if gr is not None:  # norm gains / biases of the blocks (their linears are split: no autograd .grad)
 				assert torch.allclose(got[name], gr, atol=1e-8), (variant, name)
+
+
+def test_loss_oracle_against_fp64_loops():
+	"""-log softmax(x)[t] and its gradient softmax(x) - onehot(t), row by row in fp64 Python loops:
+	pins sum / mean / none reductions, ignored rows and the engine's division by elements per sample."""
+	from oracle import loss_ref as L
+
+	torch.manual_seed(3)
+	mb, S, V = 2, 5, 7
+	x = (torch.randn(mb, S, V) * 3).to(torch.bfloat16)
+	t = torch.randint(0, V, (mb, S))
+	t[0, 1] = -100
+	t[1, 4] = -100
+	rows, grads = [], []
+	for b in range(mb):
+		for s in range(S):
+			v = [float(x[b, s, c]) for c in range(V)]
+			mx = max(v)
+			den = sum(math.exp(a - mx) for a in v)
+			if t[b, s] == -100:
+				rows.append(0.0)
+				grads.append([0.0] * V)
+				continue
+			rows.append(mx + math.log(den) - v[int(t[b, s])])
+			grads.append([math.exp(a - mx) / den - (1.0 if c == int(t[b, s]) else 0.0) for c, a in enumerate(v)])
+	live = sum(1 for r in t.view(-1) if r != -100)
+	assert L.cross_entropy_ref(x, t, "none").tolist() == pytest.approx(rows, rel=1e-5, abs=1e-6)
+	assert float(L.cross_entropy_ref(x, t, "sum")) == pytest.approx(sum(rows), rel=1e-5)
+	assert float(L.cross_entropy_ref(x, t, "mean")) == pytest.approx(sum(rows) / live, rel=1e-5)
+	loss, g = L.compute_loss_ref(x, t)
+	assert g.dtype == torch.bfloat16 and g.shape == x.shape
+	assert float(loss) == pytest.approx(sum(rows) / S, rel=1e-5)
+	want = torch.tensor(grads).view(mb, S, V) / S
+	assert torch.allclose(g.float(), want, rtol=1e-2, atol=1e-4)  # bf16 rounding of the gradient
