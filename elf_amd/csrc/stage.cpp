@@ -95,6 +95,9 @@ struct Stage {
 	void* xw[XP_COUNT] = {};
 	float* xg[XP_COUNT] = {};
 	std::map<int, MbState> mbs;
+	// micro-batches with fewer sequences than cfg.mb (the last one of a batch the split size does not
+	// divide): T and B above are set from here at every entry point (one host thread per stage)
+	std::map<int, int> mb_samples;
 	DevicePool pool;
 	std::unique_ptr<PinnedPool> pinned;
 	hipStream_t offload_stream = nullptr, prefetch_stream = nullptr;
@@ -151,6 +154,12 @@ static MbState& mb_state(Stage* s, int mb) {
 	MbState& m = s->mbs[mb];
 	if (m.blk.empty()) m.blk.resize(s->cfg.n_blocks);
 	return m;
+}
+
+static void use_mb(Stage* s, int mb) {
+	auto it = s->mb_samples.find(mb);
+	s->B = it == s->mb_samples.end() ? s->cfg.mb : it->second;
+	s->T = s->B * s->S;
 }
 
 static void destroy_events(MbState& m) {
@@ -587,12 +596,27 @@ int elf_stage_set_ends(elf_stage_t* h, int vocab_in, int vocab_out, int vocab_ou
 	return 0;
 }
 
+int elf_stage_set_mb_samples(elf_stage_t* h, int mb, int samples) {
+	Stage* s = (Stage*)h;
+	ELF_REQUIRE(s && mb >= 0, "elf_stage_set_mb_samples: bad argument");
+	ELF_REQUIRE(samples >= 1 && samples <= s->cfg.mb, "elf_stage_set_mb_samples: micro-batch %d has %d sequences, the stage was created for 1..%d", mb, samples, s->cfg.mb);
+	auto it = s->mbs.find(mb);
+	if (it != s->mbs.end()) {
+		const MbState& m = it->second;
+		ELF_REQUIRE(!m.has_acts && !m.has_win && !m.has_wgrad && !m.remat_root, "elf_stage_set_mb_samples: micro-batch %d is in flight", mb);
+	}
+	if (samples == s->cfg.mb) s->mb_samples.erase(mb);
+	else s->mb_samples[mb] = samples;
+	return 0;
+}
+
 int elf_stage_forward(elf_stage_t* h, int mb, const void* x, void* y, uint32_t flags, void* stream) {
 	Stage* s = (Stage*)h;
 	ELF_REQUIRE(s && x && y && mb >= 0, "elf_stage_forward: bad argument");
 	ELF_TRY(check_bound(s));
 	MbState& m = mb_state(s, mb);
 	ELF_REQUIRE(!m.has_acts && !m.has_win && !m.has_wgrad && !m.remat_root, "elf_stage_forward: micro-batch %d is already in flight", mb);
+	use_mb(s, mb);
 	const bool root = flags & ELF_FWD_REMAT_ROOT;
 	ELF_TRY(run_forward(s, m, x, y, root ? SAVE_NONE : SAVE_ALL, (hipStream_t)stream, (flags & ELF_FWD_OFFLOAD) && !root));
 	m.remat_root = root;
@@ -607,6 +631,7 @@ int elf_stage_backward_inputs(elf_stage_t* h, int mb, const void* x, const void*
 	ELF_REQUIRE(it != s->mbs.end(), "elf_stage_backward_inputs: no forward was run for micro-batch %d", mb);
 	MbState& m = it->second;
 	hipStream_t st = (hipStream_t)stream;
+	use_mb(s, mb);
 	if (m.remat_root) {
 		// the forward kept only the stage input: re-run it, this time keeping the stash
 		ELF_REQUIRE(x != nullptr, "elf_stage_backward_inputs: micro-batch %d was checkpointed, the stage input is needed", mb);
@@ -638,6 +663,7 @@ int elf_stage_backward_params(elf_stage_t* h, int mb, void* stream) {
 	for (int i = 0; i < s->cfg.n_blocks; i++)
 		for (int w : {P_WQKV, P_WO, P_W1, P_W2}) ELF_REQUIRE(s->params[i].g[w] != nullptr, "elf_stage_backward_params: gradient buffer not bound");
 	ELF_REQUIRE(!s->vocab_out || s->xg[XP_HEAD], "elf_stage_backward_params: gradient buffer of the output head not bound");
+	use_mb(s, mb);
 	ELF_TRY(run_backward_params(s, it->second, (hipStream_t)stream));
 	return 0;
 }
@@ -650,6 +676,7 @@ int elf_stage_recompute_forward(elf_stage_t* h, int mb, const void* x, int save,
 	MbState& m = it->second;
 	ELF_REQUIRE(!m.has_acts && !m.has_win, "elf_stage_recompute_forward: micro-batch %d still holds its activations", mb);
 	hipStream_t st = (hipStream_t)stream;
+	use_mb(s, mb);
 	void* ytmp = s->pool.alloc((size_t)s->T * (s->vocab_out ? s->vld : s->d) * 2);
 	if (!ytmp) return -3;
 	int rc = run_forward(s, m, x, ytmp, save ? SAVE_ALL : SAVE_WIN, st);
@@ -663,6 +690,7 @@ int elf_stage_recompute_backward_inputs(elf_stage_t* h, int mb, const void* dy, 
 	auto it = s->mbs.find(mb);
 	ELF_REQUIRE(it != s->mbs.end() && it->second.has_acts,
 	            "elf_stage_recompute_backward_inputs: micro-batch %d has no saved graph (run recompute_forward with save first)", mb);
+	use_mb(s, mb);
 	return run_backward(s, it->second, dy, nullptr, true, (hipStream_t)stream);
 }
 
@@ -700,6 +728,7 @@ int elf_stage_clear(elf_stage_t* h) {
 		destroy_events(kv.second);
 	}
 	s->mbs.clear();
+	s->mb_samples.clear();
 	return 0;
 }
 

@@ -95,6 +95,7 @@ for _name, _ret, _args in [
 	("elf_stage_destroy", None, [_P]),
 	("elf_stage_bind_param", _I, [_P, _I, _I, _P, _P]),
 	("elf_stage_set_ends", _I, [_P, _I, _I, _I, _I]),
+	("elf_stage_set_mb_samples", _I, [_P, _I, _I]),
 	("elf_stage_forward", _I, [_P, _I, _P, _P, ctypes.c_uint32, _P]),
 	("elf_stage_backward_inputs", _I, [_P, _I, _P, _P, _P, ctypes.c_uint32, _P]),
 	("elf_stage_backward_params", _I, [_P, _I, _P]),
@@ -152,6 +153,7 @@ class HipStageBlock:
 		self.compute_time = []
 		self.send_ops = []
 		self._handle = None
+		self._samples = {}  # mb -> sequences in it, where fewer than mb_size
 		self._kept = {}  # mb -> external tensors the library still points at (x until B/recompute, dy until W)
 		self._build(mb_size, seq_len)
 
@@ -255,49 +257,70 @@ class HipStageBlock:
 	def __str__(self):
 		return f"Rank {self.rank} - Layer {self.id}"
 
-	def _check_io(self, t, what):
-		if t.dtype != torch.bfloat16 or not t.is_cuda or t.numel() != self.T * self.d:
-			raise _lib.ElfStageError(f"{self}: {what} must be a bf16 GPU tensor of {self.T}x{self.d} elements, got {tuple(t.shape)} {t.dtype} {t.device}")
+	def _rows(self, mb_id):
+		"""Tokens in micro-batch ``mb_id`` (fewer than ``T`` for a short last micro-batch)."""
+		return self._samples.get(mb_id, self.mb_size) * self.seq
+
+	def _set_samples(self, mb_id, t, per_sample):
+		"""Tell the library how many sequences the incoming micro-batch holds (block.py:210-263 takes
+		whatever batch arrives; here the stage was sized for ``mb_size`` and accepts 1..mb_size)."""
+		n, rem = divmod(t.numel(), per_sample)
+		if rem or not 1 <= n <= self.mb_size:
+			raise _lib.ElfStageError(f"{self}: stage input of {tuple(t.shape)} is not 1..{self.mb_size} sequences of {self.seq} tokens")
+		if n != self._samples.get(mb_id, self.mb_size):
+			_lib.check(self.lib.elf_stage_set_mb_samples(self._handle, mb_id, n), "elf_stage_set_mb_samples")
+			if n == self.mb_size:
+				self._samples.pop(mb_id, None)
+			else:
+				self._samples[mb_id] = n
+
+	def _check_io(self, t, what, mb_id):
+		rows = self._rows(mb_id)
+		if t.dtype != torch.bfloat16 or not t.is_cuda or t.numel() != rows * self.d:
+			raise _lib.ElfStageError(f"{self}: {what} must be a bf16 GPU tensor of {rows}x{self.d} elements, got {tuple(t.shape)} {t.dtype} {t.device}")
 		return t.contiguous()
 
-	def _check_ids(self, t):
-		if t.dtype != torch.int64 or not t.is_cuda or t.numel() != self.T:
-			raise _lib.ElfStageError(f"{self}: the input of a first stage must be an int64 GPU tensor of {self.T} token ids, got {tuple(t.shape)} {t.dtype} {t.device}")
+	def _check_ids(self, t, mb_id):
+		rows = self._rows(mb_id)
+		if t.dtype != torch.int64 or not t.is_cuda or t.numel() != rows:
+			raise _lib.ElfStageError(f"{self}: the input of a first stage must be an int64 GPU tensor of {rows} token ids, got {tuple(t.shape)} {t.dtype} {t.device}")
 		return t.contiguous()
 
-	def _new_output(self, x):
-		"""(buffer the library writes, tensor handed on).  Last stage: logits [T, vld] with the
+	def _new_output(self, x, mb_id):
+		"""(buffer the library writes, tensor handed on).  Last stage: logits [rows, vld] with the
 		padding columns hidden from the caller; otherwise activations shaped like the input."""
+		n = self._samples.get(mb_id, self.mb_size)
 		if self.vocab_out:
-			buf = torch.empty(self.T, self.vld, dtype=torch.bfloat16, device=x.device)
-			return buf, buf.view(self.mb_size, self.seq, self.vld)[..., : self.vocab_out]
+			buf = torch.empty(n * self.seq, self.vld, dtype=torch.bfloat16, device=x.device)
+			return buf, buf.view(n, self.seq, self.vld)[..., : self.vocab_out]
 		if self.vocab_in:
-			buf = torch.empty(self.mb_size, self.seq, self.d, dtype=torch.bfloat16, device=x.device)
+			buf = torch.empty(n, self.seq, self.d, dtype=torch.bfloat16, device=x.device)
 			return buf, buf
 		buf = torch.empty_like(x)
 		return buf, buf
 
-	def _check_dy(self, dy):
+	def _check_dy(self, dy, mb_id):
 		"""Gradient of the stage output in the layout the library reads."""
 		if not self.vocab_out:
-			return self._check_io(dy, "output gradient")
-		if dy.dtype != torch.bfloat16 or not dy.is_cuda or dy.numel() != self.T * self.vocab_out:
-			raise _lib.ElfStageError(f"{self}: the gradient of the logits must be a bf16 GPU tensor of {self.T}x{self.vocab_out} elements, got {tuple(dy.shape)} {dy.dtype} {dy.device}")
+			return self._check_io(dy, "output gradient", mb_id)
+		rows = self._rows(mb_id)
+		if dy.dtype != torch.bfloat16 or not dy.is_cuda or dy.numel() != rows * self.vocab_out:
+			raise _lib.ElfStageError(f"{self}: the gradient of the logits must be a bf16 GPU tensor of {rows}x{self.vocab_out} elements, got {tuple(dy.shape)} {dy.dtype} {dy.device}")
 		if self.vld == self.vocab_out:
 			return dy.contiguous()
-		if self._rows_padded(dy):
+		if self._rows_padded(dy, rows):
 			# rows already sit vld apart (the layout elf_amd.losses writes): read in place, with the
 			# columns past the vocabulary cleared so they add nothing to dX and dW
-			buf = torch.as_strided(dy, (self.T, self.vld), (self.vld, 1))
+			buf = torch.as_strided(dy, (rows, self.vld), (self.vld, 1))
 			buf[:, self.vocab_out :].zero_()
 			return buf
-		pad = torch.zeros(self.T, self.vld, dtype=torch.bfloat16, device=dy.device)
-		pad[:, : self.vocab_out] = dy.reshape(self.T, self.vocab_out)
+		pad = torch.zeros(rows, self.vld, dtype=torch.bfloat16, device=dy.device)
+		pad[:, : self.vocab_out] = dy.reshape(rows, self.vocab_out)
 		return pad
 
-	def _rows_padded(self, dy):
+	def _rows_padded(self, dy, rows):
 		"""Whether ``dy`` is a [..., vocab_out] view whose rows are exactly ``vld`` elements apart inside
-		one allocation that holds all ``T * vld`` of them."""
+		one allocation that holds all ``rows * vld`` of them."""
 		if dy.dim() < 2 or dy.stride(-1) != 1 or dy.stride(-2) != self.vld or dy.data_ptr() % 16:
 			return False
 		expect = self.vld
@@ -306,7 +329,7 @@ class HipStageBlock:
 				return False
 			expect *= size
 		room = dy.untyped_storage().nbytes() // dy.element_size() - dy.storage_offset()
-		return room >= self.T * self.vld
+		return room >= rows * self.vld
 
 	def _timed(self, name):
 		t = Timer(name=name)
@@ -320,10 +343,11 @@ class HipStageBlock:
 		engine wraps around this call)."""
 		var = self.input_variables[0]
 		x = var.wait_and_pop(mb_id)
-		x = self._check_ids(x) if self.vocab_in else self._check_io(x, "stage input")
+		self._set_samples(mb_id, x, self.seq if self.vocab_in else self.seq * self.d)
+		x = self._check_ids(x, mb_id) if self.vocab_in else self._check_io(x, "stage input", mb_id)
 		strategy = options.get(OpOptions.REMAT_STRATEGY)
 		flags = FWD_REMAT_ROOT if (strategy is not None and strategy("", self.model)) else 0
-		ybuf, y = self._new_output(x)
+		ybuf, y = self._new_output(x, mb_id)
 		with self._timed(f"forward({self.id}:{mb_id})"):
 			_lib.check(self.lib.elf_stage_forward(self._handle, mb_id, x.data_ptr(), ybuf.data_ptr(), flags, _stream()), "elf_stage_forward")
 		self._kept.setdefault(mb_id, {})["x"] = x
@@ -344,7 +368,7 @@ class HipStageBlock:
 		dy = outs[0].wait_and_pop(mb_id)
 		for dst in outs[1:]:
 			dy = dy + dst.wait_and_pop(mb_id)
-		dy = self._check_dy(dy)
+		dy = self._check_dy(dy, mb_id)
 		ra = bool(options.get(OpOptions.RECOMPUTE_ACTIVATIONS, False))
 		rg = bool(options.get(OpOptions.RECOMPUTE_GRADIENTS, False))
 		flags = (BWD_RECOMPUTE_ACTIVATIONS if ra else 0) | (BWD_RECOMPUTE_GRADIENTS if rg else 0)
@@ -484,6 +508,7 @@ class HipStageBlock:
 		"""Drop every micro-batch state held by the library and the tensors pinned for it."""
 		_lib.check(self.lib.elf_stage_clear(self._handle), "elf_stage_clear")
 		self._kept.clear()
+		self._samples.clear()
 
 	def mem_stats(self):
 		st = MemStats()

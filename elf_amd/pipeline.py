@@ -136,8 +136,8 @@ class Pipeline:
 		if batch is not None and isinstance(batch, torch.Tensor):
 			batch = [batch]
 		mb_sizes = self._get_mb_sizes(split_size, batch)
-		if any(m != self.mb_size for m in mb_sizes):
-			raise ValueError(f"Pipeline: the stage buffers are sized for micro-batches of {self.mb_size} samples, got sizes {sorted(set(mb_sizes))}")
+		if any(not 1 <= m <= self.mb_size for m in mb_sizes):
+			raise ValueError(f"Pipeline: the stage buffers are sized for micro-batches of 1..{self.mb_size} samples, got sizes {sorted(set(mb_sizes))}")
 		n_micro_batches = len(mb_sizes)
 		regenerate = scheduler is not None or n_micro_batches != self.last_nmb
 		scheduler = self.scheduler if scheduler is None else resolve(scheduler, SCHEDULERS)

@@ -193,6 +193,12 @@ int elf_stage_bind_param(elf_stage_t* s, int block, int which, void* weight_bf16
  * 64, columns >= vocab_out are zero) and dy is their gradient in the same layout; final_norm != 0 puts a
  * norm of the architecture's kind in front of the head. */
 int elf_stage_set_ends(elf_stage_t* s, int vocab_in, int vocab_out, int vocab_out_ld, int final_norm);
+/* Number of sequences in micro-batch mb when it is smaller than cfg.mb: the last micro-batch of a
+ * batch that the split size does not divide, or an explicit list of sizes (Pipeline._get_mb_sizes,
+ * elf/pipeline.py:477-504; Engine.train_step splits the batch by those sizes, engine.py:123-160).
+ * Every buffer of that micro-batch then has T = samples * seq rows.  Call before the micro-batch's F;
+ * the value holds until it is set again or elf_stage_clear; unset micro-batches have cfg.mb. */
+int elf_stage_set_mb_samples(elf_stage_t* s, int mb, int samples);
 /* F: PipelineBlock.forward (block.py:210-279). x, y: bf16 [T, d_model]. */
 int elf_stage_forward(elf_stage_t* s, int mb, const void* x, void* y, uint32_t flags, void* stream);
 /* B: PipelineBlock.backward_inputs (block.py:624-694, 281-306). dy, dx: bf16 [T, d_model]; x is the

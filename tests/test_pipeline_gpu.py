@@ -22,47 +22,51 @@ def _stages(n):
 	return out
 
 
-@pytest.mark.parametrize("case", [("afab", [0, 0]), ("zbh1", [0])])
+# (scheduler, placement, total batch, split): an even split, a batch the split size does not divide (short
+# last micro-batch: elf/pipeline.py:497-500) and an explicit list of sizes (elf/pipeline.py:501-503)
+@pytest.mark.parametrize("case", [("afab", [0, 0], 6, 2), ("zbh1", [0], 6, 2), ("afab", [0, 0], 5, 2), ("zbh1", [0], 5, [1, 2, 2])])
 def test_pipeline_step_matches_oracle(case):
 	from elf_amd.pipeline import Pipeline, PipelineConfig
 	from oracle import stage_ref as R
 
-	sched, placement = case
-	mb, nmb = 2, 3
+	sched, placement, total, split = case
+	mb = 2
+	sizes = split if isinstance(split, list) else [mb] * (total // mb) + ([total % mb] if total % mb else [])
+	nmb, starts = len(sizes), [sum(sizes[:i]) for i in range(len(sizes))]
 	stages = _stages(len(placement))
 	refs = [R.RefStage(cfg_from_stage(st, mb), oracle_params_from_stage(st), device="cuda") for st in stages]
 	S, d = stages[0].seq_len, 256
 	g = torch.Generator().manual_seed(7)
-	batch = torch.randn(mb * nmb, S, d, generator=g).to(torch.bfloat16).cuda()
-	target = torch.randn(mb * nmb, S, d, generator=g).to(torch.bfloat16).cuda()
+	batch = torch.randn(total, S, d, generator=g).to(torch.bfloat16).cuda()
+	target = torch.randn(total, S, d, generator=g).to(torch.bfloat16).cuda()
 
 	pipe = Pipeline(stages if len(stages) > 1 else stages[0], batch[:mb], config=PipelineConfig(scheduler=sched, partitioner=False, placement=placement))
 	assert pipe.is_first() and pipe.is_last() and [b.id for b in pipe.blocks] == list(range(len(placement)))
 	pipe.zero_grad()
-	result, loss = pipe(batch, target, F.mse_loss, split_size=mb)
+	result, loss = pipe(batch, target, F.mse_loss, split_size=split)
 	assert len(result) == nmb and pipe.last_nmb == nmb
 	assert set(pipe.stats) == {"total", "idle", "start_idle", "end_idle", "bubble"}
 	assert list(pipe.detailed_stats["memories"]) == [str(op) for op in pipe.schedule]
 
 	want_loss = 0.0
 	for m in range(nmb):
-		x = batch[m * mb:(m + 1) * mb]
+		x = batch[starts[m]:starts[m] + sizes[m]]
 		for ref in refs:
 			x = ref.forward(m, x)
 		y = x.detach().float().requires_grad_()
-		t = target[m * mb:(m + 1) * mb].float()
+		t = target[starts[m]:starts[m] + sizes[m]].float()
 		l = F.mse_loss(y, t, reduction="sum") / (S * d)
 		l.backward()
 		want_loss += float(l.detach())
-		assert_close(result[m].reshape(mb, S, d), x, f"{sched} output[{m}]")
+		assert_close(result[m].reshape(sizes[m], S, d), x, f"{sched} output[{m}]")
 		dy = y.grad.to(torch.bfloat16)
 		for ref in reversed(refs):
 			dy = ref.backward_inputs(m, dy)
 		for ref in refs:
 			ref.backward_params(m)
 	for ref in refs:
-		ref.scale_grads(mb * nmb)
-	assert abs(float(loss) - want_loss / (mb * nmb)) <= 2e-2 * abs(want_loss / (mb * nmb))
+		ref.scale_grads(total)
+	assert abs(float(loss) - want_loss / total) <= 2e-2 * abs(want_loss / total)
 	for st, ref in zip(stages, refs):
 		got, want = product_grads(st), ref.grads()
 		for name in sorted(want):
@@ -70,7 +74,7 @@ def test_pipeline_step_matches_oracle(case):
 
 	# a second step with the same batch reuses the schedule and gives the same loss
 	pipe.zero_grad()
-	_, loss2 = pipe(batch, target, F.mse_loss, split_size=mb)
+	_, loss2 = pipe(batch, target, F.mse_loss, split_size=split)
 	assert abs(float(loss2) - float(loss)) <= 1e-3 * abs(float(loss))
 	assert sum(p.numel() for p in pipe.parameters()) == sum(p.numel() for st in stages for p in st.parameters())
 	pipe.clear()
@@ -113,4 +117,4 @@ def test_pipeline_rejects_what_this_build_does_not_run():
 		Pipeline(st, None, scheduler="afab", partitioner=False, placement=[0])  # no sample, no mb_size
 	pipe = Pipeline(st, None, scheduler="afab", partitioner=False, placement=[0], mb_size=2)
 	with pytest.raises(ValueError):
-		pipe(torch.zeros(6, 128, 256, dtype=torch.bfloat16, device="cuda"), None, None, split_size=3)
+		pipe(torch.zeros(6, 128, 256, dtype=torch.bfloat16, device="cuda"), None, None, split_size=3)  # larger than the stage was sized for

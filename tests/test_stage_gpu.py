@@ -81,6 +81,45 @@ def test_fbw_matches_oracle(kind):
 
 
 @pytest.mark.parametrize("kind", ["gpt", "llama"])
+def test_short_micro_batches_share_a_stage(kind):
+	"""Micro-batches of 3, 1 and 2 sequences on a stage sized for 3 (an uneven split of the batch,
+	elf/pipeline.py:497-503): each against the oracle, with a recompute of the short one, and the slot
+	of the short micro-batch reused by a full one in the next step."""
+	mb, sizes = 3, [3, 1, 2]
+	stage = _stage(kind)
+	R, cfg, ref = _oracle(stage, mb)
+	blk = _block(stage, mb)
+	xs, dys = R.make_boundary(cfg, len(sizes), seed=13)
+	xs = [x[:n].contiguous() for x, n in zip(xs, sizes)]
+	dys = [d[:n].contiguous() for d, n in zip(dys, sizes)]
+	blk.set_boundary(inputs=[x.cuda() for x in xs], grads=[d.cuda() for d in dys], keep_sent=True)
+	for m, n in enumerate(sizes):
+		blk.recv_forward(m, n, src=0)
+		blk.forward(m, **({"remat_strategy": (lambda name, module: name == "")} if m == 1 else {}))
+		blk.send_forward(m, dst=2)
+		assert_close(blk.sent_forward[m], ref.forward(m, xs[m]), f"{kind} y[{m}] ({n} sequences)")
+	for m, n in enumerate(sizes):
+		blk.recv_backward(m, n, src=2)
+		blk.backward_inputs(m)
+		blk.send_backward(m, dst=0)
+		assert_close(blk.sent_backward[m], ref.backward_inputs(m, dys[m]), f"{kind} dx[{m}] ({n} sequences)")
+		blk.backward_params(m)
+		ref.backward_params(m)
+	got, want = product_grads(stage), ref.grads()
+	for name in sorted(want):
+		assert_close(got[name], want[name], f"{kind} grad {name}")
+	assert blk.mem_stats()["live_bytes"] == 0
+	# next step: slot 1 now carries a full micro-batch
+	full = R.make_boundary(cfg, 1, seed=14)[0][0]
+	blk.set_boundary(inputs={1: full.cuda()}.__getitem__, keep_sent=True)
+	blk.recv_forward(1, mb, src=0)
+	blk.forward(1)
+	blk.send_forward(1, dst=2)
+	assert_close(blk.sent_forward[1], R.RefStage(cfg, oracle_params_from_stage(stage), device="cuda").forward(1, full), f"{kind} full micro-batch in a slot that was short")
+	blk.clear()
+
+
+@pytest.mark.parametrize("kind", ["gpt", "llama"])
 @pytest.mark.parametrize("variant", ["full_fwd", "activations_bwd", "full_bwd", "offload", "offload_no_prefetch"])
 def test_remat_and_offload_variants_equal_plain(kind, variant):
 	"""Every remat / offload variant must give the results of the plain F-B-W sequence (same
@@ -257,3 +296,7 @@ def test_error_paths():
 		blk.forward(0)  # wrong dtype
 	with pytest.raises(Exception):
 		blk.forward(1)  # empty slot
+	blk.set_boundary(inputs=[None, None, torch.zeros(3, 128, 256, dtype=torch.bfloat16, device="cuda")])
+	blk.recv_forward(2, 3, src=0)
+	with pytest.raises(ElfStageError):
+		blk.forward(2)  # more sequences than the stage was sized for
