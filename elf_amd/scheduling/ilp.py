@@ -69,8 +69,19 @@ def profile_stage(stage, sample_metadata=None, n_iter=10):
 	mb = 1 << 20  # a slot no schedule uses
 	stream = torch.cuda.current_stream().cuda_stream
 	MiB = 1024.0 * 1024.0
-	x = torch.randn(block.T, block.d, device="cuda").to(torch.bfloat16)
-	dy = torch.randn_like(x, dtype=torch.float32).to(torch.bfloat16)
+	# a first stage reads token ids and sends no input gradient; a last stage writes logits (rows padded
+	# to vld columns) and reads their gradient in the same layout
+	vin, vout = getattr(block, "vocab_in", 0), getattr(block, "vocab_out", 0)
+	if vin:
+		x = torch.randint(0, vin, (block.T,), device="cuda")
+	else:
+		x = torch.randn(block.T, block.d, device="cuda").to(torch.bfloat16)
+	out_cols = block.vld if vout else block.d
+	dy = torch.randn(block.T, out_cols, device="cuda").to(torch.bfloat16)
+	if vout:
+		dy[:, vout:] = 0
+	new_y = lambda: torch.empty(block.T, out_cols, dtype=torch.bfloat16, device="cuda")
+	new_dx = lambda: None if vin else torch.empty_like(x)
 
 	def held():
 		return torch.cuda.memory_allocated() + block.mem_stats()["live_bytes"]
@@ -94,16 +105,16 @@ def profile_stage(stage, sample_metadata=None, n_iter=10):
 		_lib.check(lib.elf_stage_forward(h, mb, x.data_ptr(), y.data_ptr(), flags, stream), "elf_stage_forward")
 
 	def bwd(dx, flags=0):
-		_lib.check(lib.elf_stage_backward_inputs(h, mb, x.data_ptr(), dy.data_ptr(), dx.data_ptr(), flags, stream), "elf_stage_backward_inputs")
+		_lib.check(lib.elf_stage_backward_inputs(h, mb, x.data_ptr(), dy.data_ptr(), dx.data_ptr() if dx is not None else None, flags, stream), "elf_stage_backward_inputs")
 
 	def wgrad():
 		_lib.check(lib.elf_stage_backward_params(h, mb, stream), "elf_stage_backward_params")
 
 	saved_grads = [g.clone() for g in block._fused_g]  # the passes below accumulate into main_grad
-	y = torch.empty_like(x)
+	y = new_y()
 	fwd(y)
-	warmup_output = y.detach().cpu()
-	dx = torch.empty_like(x)
+	warmup_output = (y[:, :vout] if vout else y).detach().cpu()
+	dx = new_dx()
 	bwd(dx)
 	wgrad()
 	del y, dx
@@ -113,13 +124,13 @@ def profile_stage(stage, sample_metadata=None, n_iter=10):
 	for _ in range(n_iter):
 		reset()
 		start = held()
-		y = torch.empty_like(x)
+		y = new_y()
 		times["f"].append(timed(lambda: fwd(y)))
 		mems["f"].append((held() - start) / MiB)
 		peaks["f"].append((peak() - start) / MiB)
 		reset()
 		before = held()
-		dx = torch.empty_like(x)
+		dx = new_dx()
 		times["b"].append(timed(lambda: bwd(dx)))
 		del y, dx
 		mems["b"].append((held() - start) / MiB)
@@ -135,14 +146,14 @@ def profile_stage(stage, sample_metadata=None, n_iter=10):
 	# whole-stage checkpoint forward
 	reset()
 	start = held()
-	y = torch.empty_like(x)
+	y = new_y()
 	fwd(y, FWD_REMAT_ROOT)
 	torch.cuda.synchronize()
 	peak_ckpt = (peak() - start) / MiB
 	# B re-runs the forward of a checkpointed micro-batch; with recompute_gradients it leaves only the
 	# layer-input half of the W stash behind: that is Mba
 	start = held() - y.numel() * 2
-	dx = torch.empty_like(x)
+	dx = new_dx()
 	bwd(dx, BWD_RECOMPUTE_GRADIENTS)
 	torch.cuda.synchronize()
 	del dx, y
@@ -152,11 +163,10 @@ def profile_stage(stage, sample_metadata=None, n_iter=10):
 		g.copy_(keep)
 	torch.cuda.synchronize()
 
-	nbytes = x.numel() * 2
 	stats = {
 		"T": T, "M": M, "Mpeak": Mpeak, "Mpeak_ckpt": peak_ckpt,
 		"Mparams": 1.5 * sum(w.numel() * 2 for w in block._fused_w) / MiB,
-		"Mba": mba, "Mbg": M["b"] - mba, "Minput": nbytes / MiB, "Moutput": nbytes / MiB, "Tcomm": 0.0,
+		"Mba": mba, "Mbg": M["b"] - mba, "Minput": x.numel() * x.element_size() / MiB, "Moutput": dy.numel() * 2 / MiB, "Tcomm": 0.0,
 		"forward_remat_options": [], "backward_remat_options": [],
 	}
 	return stats, warmup_output

@@ -176,3 +176,49 @@ def test_reference_small_configuration_through_pipeline(loss_kind):
 		for name, p in mod.named_parameters():
 			assert_close(p.main_grad, ref_params[name].grad, f"grad {name}", rel_max=3e-2, rel_fro=2e-2)
 			assert_close(p.grad, ref_params[name].grad, f"bf16 grad {name}", rel_max=4e-2, rel_fro=2e-2)
+
+
+def test_memory_budget_with_first_and_last_stage():
+	"""``Pipeline(..., memory_budget=)`` on stages that own the embedding and the head: profile_stage
+	feeds token ids to the first stage and padded logits gradients to the last one, the ILP solved from
+	those records rewrites the schedule under a tight budget, and the step gives the loss and gradients
+	of the unconstrained one."""
+	from elf_amd import losses, models
+	from elf_amd.pipeline import Pipeline
+	from elf_amd.scheduling import OperationType, OpOptions
+	from elf_amd.scheduling.ilp import profile_stage
+
+	V, d, S, mb, nmb = 1000, 256, 128, 4, 6
+	g = torch.Generator().manual_seed(9)
+	ids = torch.randint(0, V, (mb * nmb, S), generator=g).cuda()
+	tgt = torch.randint(0, V, (mb * nmb, S), generator=g).cuda()
+
+	def build(**kw):
+		first = models.gpt_end_stage(2, d, 4, 1024, S, vocab_in=V, causal=True, seed=41)
+		last = models.gpt_end_stage(2, d, 4, 1024, S, vocab_out=V, causal=True, seed=42)
+		return Pipeline([first, last], ids[:mb], scheduler="afab", partitioner=False, placement=[0, 0], **kw), (first, last)
+
+	plain, plain_mods = build()
+	rec_first, nxt = profile_stage(plain.blocks[0], n_iter=2)
+	rec_last, logits = profile_stage(plain.blocks[1], n_iter=2)
+	T = mb * S
+	assert tuple(nxt.shape) == (T, d) and tuple(logits.shape) == (T, V)
+	assert rec_first["Minput"] == pytest.approx(T * 8 / 2**20) and rec_first["Moutput"] == pytest.approx(T * d * 2 / 2**20)
+	assert rec_last["Moutput"] == pytest.approx(T * 1024 * 2 / 2**20)  # rows padded to 1024 columns
+	for rec in (rec_first, rec_last):
+		assert all(rec["T"][k] > 0 for k in "fbw") and rec["M"]["w"] == 0.0 and rec["M"]["f"] > rec["Mpeak_ckpt"] > 0
+	plain.zero_grad()
+	_, loss_plain = plain(ids, tgt, losses.cross_entropy, split_size=mb)
+
+	# AFAB holds every micro-batch's stash at once: a budget of two thirds of that forces remat
+	need = 2 * (rec_first["Mparams"] + rec_last["Mparams"]) + nmb * (rec_first["M"]["f"] + rec_last["M"]["f"])
+	tight, tight_mods = build(memory_budget=0.67 * need)
+	tight.zero_grad()
+	_, loss_tight = tight(ids, tgt, losses.cross_entropy, split_size=mb)
+	remat_ops = [op for op in tight.schedule if op.op in (OperationType.RECOMPUTE_FORWARD, OperationType.RECOMPUTE_BACKWARD_INPUTS) or op.options.get(OpOptions.REMAT_STRATEGY) is not None]
+	assert remat_ops, "the budget must have forced rematerialisation"
+	assert float(loss_tight) == pytest.approx(float(loss_plain), rel=1e-3)
+	for mod_p, mod_t in zip(plain_mods, tight_mods):
+		want = dict(mod_p.named_parameters())
+		for name, p in mod_t.named_parameters():
+			assert_close(p.main_grad, want[name].main_grad, f"grad {name} under the budget", rel_max=2e-3, rel_fro=2e-3)
