@@ -324,12 +324,23 @@ int gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda,
 	// tiles can fill the chip, the register-staged kernels (smaller tiles) otherwise.
 	if (tile_cfg <= 0 && M % 256 == 0 && N % 256 == 0 && (int64_t)(M / 256) * (N / 256) >= 192) tile_cfg = 7;
 	if (tile_cfg == 6 || tile_cfg == 7) {
+		int tail_tiles = -1;  // an explicit k_splits splits every tile
 		if (epi == EPI_F32_ACC && k_splits <= 0) {
 			const int64_t tiles = (int64_t)(M / 256) * (N / 256);
+			const int nk = K / 64;
 			k_splits = 1;
-			while (tiles * k_splits < 256 && (K / 64) / (k_splits * 2) >= 8 && k_splits < 16) k_splits *= 2;
+			if (tiles < 256) {
+				// too few tiles for the chip: split them all
+				while (tiles * k_splits < 256 && nk / (k_splits * 2) >= 8 && k_splits < 16) k_splits *= 2;
+			} else if (const int rem = (int)(tiles % 256); rem != 0 && rem <= 128) {
+				// the last round of workgroups would leave at least half of the CUs idle: split just those
+				// tiles so that they fill it with proportionally shorter workgroups
+				k_splits = rem <= 64 ? 4 : 2;
+				tail_tiles = rem;
+				if (nk / k_splits < 16) k_splits = 1;
+			}
 		}
-		return gemm_bf16_dma(a_t, b_t, M, N, K, A, lda, B, ldb, C, ldc, epi, R, ldr, k_splits, tile_cfg == 7 ? 8 : 4, stream);
+		return gemm_bf16_dma(a_t, b_t, M, N, K, A, lda, B, ldb, C, ldc, epi, R, ldr, k_splits, tail_tiles, tile_cfg == 7 ? 8 : 4, stream);
 	}
 	if (!a_t && !b_t) return launch_epi<false, false>(g, epi, tile_cfg, stream);
 	if (!a_t && b_t) return launch_epi<false, true>(g, epi, tile_cfg, stream);

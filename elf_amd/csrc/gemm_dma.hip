@@ -34,7 +34,9 @@ struct Args {
 	const bf16_t* R;
 	int64_t lda, ldb, ldc, ldr;
 	int M, N, K;
-	int tiles_m, tiles_n, k_splits;
+	int tiles_m, tiles_n;
+	int k_splits;    // K is split this many ways (fp32 atomics epilogue) for the last tail_tiles tiles
+	int tail_tiles;  // tiles_m * tiles_n for a uniform split, 0 when nothing is split
 };
 
 // Byte offsets (relative to the tile origin of the current K slice) of the 16-byte chunks this
@@ -94,13 +96,24 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int wr = wave >> 1, wc = wave & 1;
 
-	// tile assignment (XCD-contiguous, grouped by 8 tile rows), optional K split
-	int pid = blockIdx.x;
+	// Tile assignment (XCD-contiguous, grouped by 8 tile rows).  The first ntiles - tail_tiles tiles
+	// are computed whole, one workgroup each; each of the last tail_tiles is shared by k_splits
+	// workgroups that take a K range each and add their part with atomics.  Splitting only the tail
+	// turns the last, partly filled round of workgroups of a launch into a full round of shorter ones.
 	const int ntiles = g.tiles_m * g.tiles_n;
-	int ksplit = 0;
-	if (g.k_splits > 1) {
-		ksplit = pid / ntiles;
-		pid = pid % ntiles;
+	const int full = ntiles - g.tail_tiles;
+	int pid = blockIdx.x, ksplit = 0, splits = 1;
+	if (pid >= full) {
+		const int q = pid - full;
+		splits = g.k_splits;
+		if (((ntiles | full) & 7) == 0) {  // keep workgroup index = tile index (mod 8): same XCD as its neighbours
+			const int rest = q >> 3;
+			ksplit = rest % splits;
+			pid = full + (rest / splits) * 8 + (q & 7);
+		} else {
+			ksplit = q % splits;
+			pid = full + q / splits;
+		}
 	}
 	if ((ntiles & 7) == 0) pid = (pid & 7) * (ntiles >> 3) + (pid >> 3);
 	constexpr int GROUP_M = 8;
@@ -111,7 +124,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	const int n0 = ((pid % per_group) / gsz) * BN;
 
 	const int nk_total = g.K / BKS;
-	const int nk_per = (nk_total + g.k_splits - 1) / g.k_splits;
+	const int nk_per = (nk_total + splits - 1) / splits;
 	const int kt0 = ksplit * nk_per;
 	const int nk = min(nk_total, kt0 + nk_per) - kt0;
 	if (nk <= 0) return;
@@ -231,6 +244,22 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	float* ws = reinterpret_cast<float*>(smem) + wave * (32 * PITCH);
 	const int col_l = lane & 31;
 	const int row_l = (lane >> 5) * 4;
+	if constexpr (EPI == EPI_F32_ACC) {
+		if (splits > 1) {
+			// several workgroups add into this tile: fp32 atomics straight from the accumulators, in the
+			// accumulator layout, where a wave instruction covers two full 128-byte rows of 32 columns
+			// (the row-wise 16-byte layout below would touch a quarter of eight lines per instruction)
+			float* cbase = reinterpret_cast<float*>(g.C) + (int64_t)(m0 + wr * (RT * 32) + row_l) * g.ldc + n0 + wc * 128 + col_l;
+#pragma unroll
+			for (int i = 0; i < RT; i++)
+#pragma unroll
+				for (int j = 0; j < 4; j++)
+#pragma unroll
+					for (int r = 0; r < 16; r++)
+						unsafeAtomicAdd(cbase + (int64_t)(i * 32 + (r >> 2) * 8 + (r & 3)) * g.ldc + j * 32, acc[i][j][r]);
+			return;
+		}
+	}
 #pragma unroll
 	for (int i = 0; i < RT; i++) {
 #pragma unroll
@@ -262,14 +291,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 				const int row = it * 2 + (lane >> 5), c4 = (lane & 31) * 4;
 				f32x4 v = *reinterpret_cast<const f32x4*>(ws + row * PITCH + c4);
 				float* c = reinterpret_cast<float*>(g.C) + (int64_t)(grow0 + row) * g.ldc + gcol0 + c4;
-				if constexpr (EPI == EPI_F32_ACC) {
-					if (g.k_splits > 1) {
-#pragma unroll
-						for (int t = 0; t < 4; t++) unsafeAtomicAdd(c + t, v[t]);
-						continue;
-					}
-					v += *reinterpret_cast<const f32x4*>(c);
-				}
+				if constexpr (EPI == EPI_F32_ACC) v += *reinterpret_cast<const f32x4*>(c);
 				*reinterpret_cast<f32x4*>(c) = v;
 			}
 		}
@@ -288,7 +310,7 @@ static int launch(const Args& a, hipStream_t stream) {
 		ELF_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
 		attr_set = true;
 	}
-	hipLaunchKernelGGL(kern, dim3(a.tiles_m * a.tiles_n * a.k_splits), dim3(NW * 64), smem, stream, a);
+	hipLaunchKernelGGL(kern, dim3(a.tiles_m * a.tiles_n + a.tail_tiles * (a.k_splits - 1)), dim3(NW * 64), smem, stream, a);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
 }
@@ -309,11 +331,13 @@ static int launch_epi(const Args& a, int epi, hipStream_t stream) {
 
 // Arguments are validated by gemm_bf16() before it dispatches here.
 int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda, const void* B, int64_t ldb, void* C,
-                  int64_t ldc, int epi, const void* R, int64_t ldr, int k_splits, int waves, hipStream_t stream) {
+                  int64_t ldc, int epi, const void* R, int64_t ldr, int k_splits, int tail_tiles, int waves, hipStream_t stream) {
 	ELF_REQUIRE(waves == 4 || waves == 8, "gemm (dma tile): 4 or 8 waves");
 	ELF_REQUIRE(M % dma::BM == 0 && N % dma::BN == 0 && K % dma::BKS == 0, "gemm (dma tile): M, N multiples of 256 and K of 64 required");
-	dma::Args a{(const bf16_t*)A, (const bf16_t*)B, C, (const bf16_t*)R, lda, ldb, ldc, ldr, M, N, K, M / dma::BM, N / dma::BN, k_splits < 1 ? 1 : k_splits};
-	if (epi != EPI_F32_ACC) a.k_splits = 1;
+	const int ntiles = (M / dma::BM) * (N / dma::BN);
+	dma::Args a{(const bf16_t*)A, (const bf16_t*)B, C, (const bf16_t*)R, lda, ldb, ldc, ldr, M, N, K, M / dma::BM, N / dma::BN, k_splits < 1 ? 1 : k_splits,
+	            tail_tiles < 0 || tail_tiles > ntiles ? ntiles : tail_tiles};
+	if (epi != EPI_F32_ACC || a.k_splits == 1) a.k_splits = 1, a.tail_tiles = 0;
 	if (waves == 4) {
 		if (!a_t && !b_t) return dma::launch_epi<4, false, false>(a, epi, stream);
 		if (!a_t && b_t) return dma::launch_epi<4, false, true>(a, epi, stream);
