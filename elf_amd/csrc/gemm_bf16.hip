@@ -322,7 +322,11 @@ int gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda,
 	g.k_splits = k_splits;
 	// Tile choice when the caller leaves it open: the direct-to-LDS 256x256 kernel whenever its
 	// tiles can fill the chip, the register-staged kernels (smaller tiles) otherwise.
-	if (tile_cfg <= 0 && M % 256 == 0 && N % 256 == 0 && (int64_t)(M / 256) * (N / 256) >= 192) tile_cfg = 7;
+	if (tile_cfg <= 0 && M % 256 == 0 && N % 256 == 0) {
+		const int64_t tiles = (int64_t)(M / 256) * (N / 256);
+		// weight gradients (long K, fp32 accumulate) also when the tiles are few: K is split instead
+		if (tiles >= 192 || (epi == EPI_F32_ACC && tiles >= 24 && K >= 4096)) tile_cfg = 7;
+	}
 	if (tile_cfg == 6 || tile_cfg == 7) {
 		int tail_tiles = -1;  // an explicit k_splits splits every tile
 		if (epi == EPI_F32_ACC && k_splits <= 0) {
@@ -330,8 +334,9 @@ int gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda,
 			const int nk = K / 64;
 			k_splits = 1;
 			if (tiles < 256) {
-				// too few tiles for the chip: split them all
-				while (tiles * k_splits < 256 && nk / (k_splits * 2) >= 8 && k_splits < 16) k_splits *= 2;
+				// too few tiles for the chip: split them all, down to 32 slices per workgroup (shorter
+				// ranges pay more in pipeline fill and atomics than the extra workgroups bring)
+				while (tiles * k_splits * 2 <= 256 && nk / (k_splits * 2) >= 32 && k_splits < 16) k_splits *= 2;
 			} else if (const int rem = (int)(tiles % 256); rem != 0 && rem <= 128) {
 				// the last round of workgroups would leave at least half of the CUs idle: split just those
 				// tiles so that they fill it with proportionally shorter workgroups
