@@ -1,4 +1,4 @@
-// 256x256 bf16 MFMA GEMM tile kernel with direct global->LDS loads, for gfx950.
+// 256x256 (and 128x256) bf16 MFMA GEMM tile kernel with direct global->LDS loads, for gfx950.
 //
 // Same contraction and layouts as gemm_bf16.hip (C (+)= sum_k A(m,k) B(n,k); "R" operands are
 // k-contiguous, "T" operands reduction-major), different data movement:
@@ -22,10 +22,21 @@ namespace elf {
 
 namespace dma {
 
-constexpr int BM = 256, BN = 256, BKS = 64, NST = 2;
-constexpr int OPERAND_BYTES = 256 * BKS * 2;  // 32 KiB
-constexpr int STAGE_BYTES = 2 * OPERAND_BYTES;
-constexpr int PIECES_PER_OPERAND = OPERAND_BYTES / 1024;  // 1 KiB pieces (one wave instruction each) per stage and operand
+constexpr int BN = 256, BKS = 64, NST = 2;
+constexpr int B_BYTES = BN * BKS * 2;  // 32 KiB per stage
+
+// Shape of one workgroup: NW waves arranged (NW / 2) x 2, each owning RT x 4 accumulator tiles of
+// 32 x 32, so the workgroup tile is BM x 256 with BM = (NW / 2) * RT * 32.
+template <int NW, int RT>
+struct Shape {
+	static constexpr int BM = (NW / 2) * RT * 32;
+	static constexpr int A_BYTES = BM * BKS * 2;
+	static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+	// 1 KiB pieces (one wave instruction each) per wave, stage and operand
+	static constexpr int LOADS_A = A_BYTES / 1024 / NW, LOADS_B = B_BYTES / 1024 / NW;
+	static constexpr int LOADS_PER_STAGE = LOADS_A + LOADS_B;
+	static_assert(LOADS_PER_STAGE % 2 == 0, "the loads of a slice are issued in two halves");
+};
 
 struct Args {
 	const bf16_t* A;
@@ -81,15 +92,18 @@ __device__ __forceinline__ bf16x8 frag(const unsigned char* base, int row0, int 
 	}
 }
 
-// NW = 4: one wave per SIMD, 128x128 wave tiles (16 accumulator tiles, 8 fragment reads per 16
-// MFMAs).  NW = 8: two waves per SIMD, 64x128 wave tiles (8 accumulator tiles, 6 reads per 8
-// MFMAs): more LDS traffic per FLOP, but the two waves fill each other's issue gaps (every
+// NW = 4, RT = 4: one wave per SIMD, 128x128 wave tiles (16 accumulator tiles, 8 fragment reads per
+// 16 MFMAs).  NW = 8, RT = 2: two waves per SIMD, 64x128 wave tiles (8 accumulator tiles, 6 reads per
+// 8 MFMAs): more LDS traffic per FLOP, but the two waves fill each other's issue gaps (every
 // non-MFMA instruction of a lone wave delays its MFMA stream by a few cycles) and barrier waits.
-template <int NW, bool AT, bool BT, int EPI>
+// NW = 4, RT = 2: 128x256 workgroup tile for outputs with too few 256x256 tiles to fill the chip
+// (A must be k-contiguous: the reduction-major tile layout below assumes 256 rows).
+template <int NW, int RT, bool AT, bool BT, int EPI>
 __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
-	constexpr int RT = 16 / NW;                       // 32-row accumulator tiles per wave (x 4 column tiles)
-	constexpr int LOADS_PER_OPERAND = PIECES_PER_OPERAND / NW;  // wave instructions per wave per stage and operand
-	constexpr int LOADS_PER_STAGE = 2 * LOADS_PER_OPERAND;
+	using Sh = Shape<NW, RT>;
+	constexpr int BM = Sh::BM, A_BYTES = Sh::A_BYTES, STAGE_BYTES = Sh::STAGE_BYTES;
+	constexpr int LOADS_A = Sh::LOADS_A, LOADS_B = Sh::LOADS_B, LOADS_PER_STAGE = Sh::LOADS_PER_STAGE;
+	static_assert(BM == 256 || !AT, "reduction-major A tiles are laid out for 256 rows");
 	extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 	const int tid = threadIdx.x;
 	const int lane = tid & 63;
@@ -133,25 +147,27 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	const bf16_t* Bp = BT ? g.B + (int64_t)kt0 * BKS * g.ldb + n0 : g.B + (int64_t)n0 * g.ldb + (int64_t)kt0 * BKS;
 	const int64_t a_step = AT ? (int64_t)BKS * g.lda : BKS;
 	const int64_t b_step = BT ? (int64_t)BKS * g.ldb : BKS;
-	uint32_t aoff[LOADS_PER_OPERAND], boff[LOADS_PER_OPERAND];
-	lane_offsets<AT, LOADS_PER_OPERAND>(wave, lane, g.lda, aoff);
-	lane_offsets<BT, LOADS_PER_OPERAND>(wave, lane, g.ldb, boff);
+	uint32_t aoff[LOADS_A], boff[LOADS_B];
+	lane_offsets<AT, LOADS_A>(wave, lane, g.lda, aoff);
+	lane_offsets<BT, LOADS_B>(wave, lane, g.ldb, boff);
 
-	const uint32_t lds0 = lds_addr(smem) + wave * (LOADS_PER_OPERAND * 1024);  // this wave's first 1 KiB piece
+	// this wave's first 1 KiB piece of each operand in stage 0
+	const uint32_t lds_a = lds_addr(smem) + wave * (LOADS_A * 1024);
+	const uint32_t lds_b = lds_addr(smem) + A_BYTES + wave * (LOADS_B * 1024);
 
-	// One 1 KiB piece of a slice: the first LOADS_PER_OPERAND pieces belong to A, the rest to B.  A piece of a slice past the
+	// One 1 KiB piece of a slice: the first LOADS_A pieces belong to A, the rest to B.  A piece of a slice past the
 	// end of K is fetched from the last slice into a scratch area behind the ring instead, so that
 	// the main loop needs no branches around its loads (the accumulators stay put in registers).
 	const uint32_t lds_dummy = lds_addr(smem) + NST * STAGE_BYTES + wave * 1024;
 	auto issue_piece = [&](int step, int piece) {
 		const bool ok = step < nk;
 		const int sc = ok ? step : nk - 1;
-		const uint32_t st = lds0 + (uint32_t)(sc % NST) * STAGE_BYTES;
-		if (piece < LOADS_PER_OPERAND)
-			dma16(Ap + (int64_t)sc * a_step, aoff[piece], __builtin_amdgcn_readfirstlane(ok ? st + piece * 1024 : lds_dummy));
+		const uint32_t st = (uint32_t)(sc % NST) * STAGE_BYTES;
+		if (piece < LOADS_A)
+			dma16(Ap + (int64_t)sc * a_step, aoff[piece], __builtin_amdgcn_readfirstlane(ok ? lds_a + st + piece * 1024 : lds_dummy));
 		else
-			dma16(Bp + (int64_t)sc * b_step, boff[piece - LOADS_PER_OPERAND],
-			      __builtin_amdgcn_readfirstlane(ok ? st + OPERAND_BYTES + (piece - LOADS_PER_OPERAND) * 1024 : lds_dummy));
+			dma16(Bp + (int64_t)sc * b_step, boff[piece - LOADS_A],
+			      __builtin_amdgcn_readfirstlane(ok ? lds_b + st + (piece - LOADS_A) * 1024 : lds_dummy));
 	};
 	auto issue = [&](int step) {
 #pragma unroll
@@ -180,7 +196,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	bf16x8 fa[2][RT], fb[2][4];
 	auto load_frags = [&](int buf, int step, int ks) {
 		const unsigned char* sa = smem + (step % NST) * STAGE_BYTES;
-		const unsigned char* sb = sa + OPERAND_BYTES;
+		const unsigned char* sb = sa + A_BYTES;
 #pragma unroll
 		for (int i = 0; i < RT; i++) fa[buf][i] = frag<AT>(sa, wr * (RT * 32) + i * 32, ks, lane);
 #pragma unroll
@@ -198,13 +214,15 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	// them: the four waves' loads of a slice are 64 KiB through a 64 B/clk path, and a wave that
 	// issues them in one burst sits in the queue for ~1000 cycles with its MFMAs behind it.
 	auto mfmas_dma = [&](int buf, int step, int piece0) {
+		constexpr int HALF = LOADS_PER_STAGE / 2, NM = RT * 4;  // HALF loads spread evenly over NM MFMAs
 #pragma unroll
 		for (int i = 0; i < RT; i++)
 #pragma unroll
 			for (int j = 0; j < 4; j++) {
 				acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][i], fb[buf][j], acc[i][j], 0, 0, 0);
-				if (j & 1) {
-					issue_piece(step, piece0 + i * 2 + (j >> 1));
+				const int n = i * 4 + j;
+				if ((n + 1) * HALF / NM != n * HALF / NM) {
+					issue_piece(step, piece0 + n * HALF / NM);
 					__builtin_amdgcn_sched_barrier(0);
 				}
 			}
@@ -298,13 +316,13 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	}
 }
 
-template <int NW, bool AT, bool BT, int EPI>
+template <int NW, int RT, bool AT, bool BT, int EPI>
 static int launch(const Args& a, hipStream_t stream) {
 	// ring + 1 KiB per wave as the target of the loads past the end of K; the epilogue needs a
 	// 32 x 136 fp32 strip per wave
-	constexpr int ring = NST * STAGE_BYTES + NW * 1024, epi = NW * 32 * 136 * 4;
+	constexpr int ring = NST * Shape<NW, RT>::STAGE_BYTES + NW * 1024, epi = NW * 32 * 136 * 4;
 	constexpr int smem = ring > epi ? ring : epi;
-	auto kern = gemm_dma_kernel<NW, AT, BT, EPI>;
+	auto kern = gemm_dma_kernel<NW, RT, AT, BT, EPI>;
 	static bool attr_set = false;
 	if (!attr_set) {
 		ELF_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
@@ -315,13 +333,13 @@ static int launch(const Args& a, hipStream_t stream) {
 	return 0;
 }
 
-template <int NW, bool AT, bool BT>
+template <int NW, int RT, bool AT, bool BT>
 static int launch_epi(const Args& a, int epi, hipStream_t stream) {
 	switch (epi) {
-		case EPI_BF16: return launch<NW, AT, BT, EPI_BF16>(a, stream);
-		case EPI_BF16_RESID: return launch<NW, AT, BT, EPI_BF16_RESID>(a, stream);
-		case EPI_F32_ACC: return launch<NW, AT, BT, EPI_F32_ACC>(a, stream);
-		case EPI_F32_STORE: return launch<NW, AT, BT, EPI_F32_STORE>(a, stream);
+		case EPI_BF16: return launch<NW, RT, AT, BT, EPI_BF16>(a, stream);
+		case EPI_BF16_RESID: return launch<NW, RT, AT, BT, EPI_BF16_RESID>(a, stream);
+		case EPI_F32_ACC: return launch<NW, RT, AT, BT, EPI_F32_ACC>(a, stream);
+		case EPI_F32_STORE: return launch<NW, RT, AT, BT, EPI_F32_STORE>(a, stream);
 	}
 	set_error("gemm: unknown epilogue %d", epi);
 	return -1;
@@ -331,21 +349,26 @@ static int launch_epi(const Args& a, int epi, hipStream_t stream) {
 
 // Arguments are validated by gemm_bf16() before it dispatches here.
 int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda, const void* B, int64_t ldb, void* C,
-                  int64_t ldc, int epi, const void* R, int64_t ldr, int k_splits, int tail_tiles, int waves, hipStream_t stream) {
-	ELF_REQUIRE(waves == 4 || waves == 8, "gemm (dma tile): 4 or 8 waves");
-	ELF_REQUIRE(M % dma::BM == 0 && N % dma::BN == 0 && K % dma::BKS == 0, "gemm (dma tile): M, N multiples of 256 and K of 64 required");
-	const int ntiles = (M / dma::BM) * (N / dma::BN);
-	dma::Args a{(const bf16_t*)A, (const bf16_t*)B, C, (const bf16_t*)R, lda, ldb, ldc, ldr, M, N, K, M / dma::BM, N / dma::BN, k_splits < 1 ? 1 : k_splits,
+                  int64_t ldc, int epi, const void* R, int64_t ldr, int k_splits, int tail_tiles, int waves, int bm, hipStream_t stream) {
+	ELF_REQUIRE((waves == 4 || waves == 8) && (bm == 256 || (bm == 128 && waves == 4)), "gemm (dma tile): 256-row tiles with 4 or 8 waves, 128-row tiles with 4");
+	ELF_REQUIRE(M % bm == 0 && N % dma::BN == 0 && K % dma::BKS == 0, "gemm (dma tile): M multiple of %d, N of 256 and K of 64 required", bm);
+	ELF_REQUIRE(bm == 256 || !a_t, "gemm (dma tile): 128-row tiles need a k-contiguous A");
+	const int ntiles = (M / bm) * (N / dma::BN);
+	dma::Args a{(const bf16_t*)A, (const bf16_t*)B, C, (const bf16_t*)R, lda, ldb, ldc, ldr, M, N, K, M / bm, N / dma::BN, k_splits < 1 ? 1 : k_splits,
 	            tail_tiles < 0 || tail_tiles > ntiles ? ntiles : tail_tiles};
 	if (epi != EPI_F32_ACC || a.k_splits == 1) a.k_splits = 1, a.tail_tiles = 0;
+	if (bm == 128) {
+		if (!b_t) return dma::launch_epi<4, 2, false, false>(a, epi, stream);
+		return dma::launch_epi<4, 2, false, true>(a, epi, stream);
+	}
 	if (waves == 4) {
-		if (!a_t && !b_t) return dma::launch_epi<4, false, false>(a, epi, stream);
-		if (!a_t && b_t) return dma::launch_epi<4, false, true>(a, epi, stream);
-		if (a_t && b_t) return dma::launch_epi<4, true, true>(a, epi, stream);
+		if (!a_t && !b_t) return dma::launch_epi<4, 4, false, false>(a, epi, stream);
+		if (!a_t && b_t) return dma::launch_epi<4, 4, false, true>(a, epi, stream);
+		if (a_t && b_t) return dma::launch_epi<4, 4, true, true>(a, epi, stream);
 	} else {
-		if (!a_t && !b_t) return dma::launch_epi<8, false, false>(a, epi, stream);
-		if (!a_t && b_t) return dma::launch_epi<8, false, true>(a, epi, stream);
-		if (a_t && b_t) return dma::launch_epi<8, true, true>(a, epi, stream);
+		if (!a_t && !b_t) return dma::launch_epi<8, 2, false, false>(a, epi, stream);
+		if (!a_t && b_t) return dma::launch_epi<8, 2, false, true>(a, epi, stream);
+		if (a_t && b_t) return dma::launch_epi<8, 2, true, true>(a, epi, stream);
 	}
 	set_error("gemm: layout A=T,B=R is not used by any stage contraction");
 	return -1;

@@ -40,11 +40,13 @@ def K():
 
 @pytest.mark.parametrize("layout", ["nt", "nn", "tn"])
 @pytest.mark.parametrize("shape", [(256, 256, 64), (512, 768, 256), (1024, 2304, 768), (2048, 1024, 4096)])
-@pytest.mark.parametrize("tile_cfg", [0, 1, 2, 3, 5, 6, 7])
+@pytest.mark.parametrize("tile_cfg", [0, 1, 2, 3, 5, 6, 7, 8])
 def test_gemm_layouts(K, layout, shape, tile_cfg):
 	M, N, Kd = shape
 	if tile_cfg in (1, 5, 6, 7) and (M % 256 or N % 256):
 		pytest.skip("tile does not divide")
+	if tile_cfg == 8 and (layout == "tn" or N % 256):
+		pytest.skip("the 128x256 direct-to-LDS tile needs a k-contiguous A and N % 256 == 0")
 	A = _randn(M, Kd, seed=1)
 	B = _randn(N, Kd, seed=2, scale=0.05)
 	ref = A.float() @ B.float().t()
@@ -73,12 +75,14 @@ def test_gemm_epilogues(K):
 		_close(acc, 3 * ref + 0.25, rel_fro=1e-5, rel_max=1e-5, what=f"f32 acc ks={ks}")
 
 
-@pytest.mark.parametrize("tile_cfg", [6, 7])
-@pytest.mark.parametrize("layout", ["nt", "tn"])
+@pytest.mark.parametrize("tile_cfg", [6, 7, 8])
+@pytest.mark.parametrize("layout", ["nt", "tn", "nn"])
 def test_gemm_direct_to_lds_epilogues_and_k_split(K, tile_cfg, layout):
-	"""The 256x256 direct-to-LDS kernels (4- and 8-wave): every epilogue, short K (1 and 2 slices:
-	the loop's loads past the end of K), and the K split with fp32 atomics."""
-	M, N = 512, 768
+	"""The direct-to-LDS kernels (256x256 with 4 and 8 waves, 128x256): every epilogue, short K (1 and
+	2 slices: the loop's loads past the end of K), and the K split with fp32 atomics."""
+	if tile_cfg == 8 and layout == "tn":
+		pytest.skip("the 128x256 tile needs a k-contiguous A")
+	M, N = (384, 768) if tile_cfg == 8 else (512, 768)
 	for Kd in (64, 128, 1024):
 		A = _randn(M, Kd, seed=21)
 		B = _randn(N, Kd, seed=22, scale=0.05)
@@ -87,13 +91,16 @@ def test_gemm_direct_to_lds_epilogues_and_k_split(K, tile_cfg, layout):
 		if layout == "nt":
 			kw = dict(tile_cfg=tile_cfg)
 			a, b = A, B
+		elif layout == "nn":
+			kw = dict(tile_cfg=tile_cfg, b_t=True)
+			a, b = A, B.t().contiguous()
 		else:
 			kw = dict(tile_cfg=tile_cfg, a_t=True, b_t=True)
 			a, b = A.t().contiguous(), B.t().contiguous()
 		_close(K.gemm(a, b, **kw), ref, what=f"bf16 K={Kd}")
 		_close(K.gemm(a, b, epilogue=K.EPI_BF16_RESID, residual=R, **kw), ref + R.float(), what=f"resid K={Kd}")
 		_close(K.gemm(a, b, epilogue=K.EPI_F32_STORE, **kw), ref, rel_fro=1e-5, rel_max=1e-5, what=f"f32 store K={Kd}")
-		for ks in (1, 2, 4):
+		for ks in (1, 2, 4):  # the 128x256 tile never splits K: it runs ks = 1 whatever is asked
 			acc = torch.full((M, N), 0.25, dtype=torch.float32, device="cuda")
 			for _ in range(2):
 				K.gemm(a, b, out=acc, epilogue=K.EPI_F32_ACC, k_splits=ks, **kw)
