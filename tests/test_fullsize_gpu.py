@@ -23,11 +23,14 @@ def K():
 	return kernels
 
 
+# the Llama-3-8B FFN shapes (256x256 tiles; for tn the dW shape whose 896 tiles get a K-split tail) and
+# the GPT-2-small ones (N = 768: 128x256 tiles; dW with 36 tiles: K split over all of them)
+@pytest.mark.parametrize("dims", [(T, FFN, D_MODEL), (T, 768, 3072)])
 @pytest.mark.parametrize("layout", ["nt", "nn", "tn"])
-def test_gemm_row_and_column_probes_at_full_size(K, layout):
-	"""C = A B^T at 8192 x 14336 x 4096 (and the dW shape for tn): 64 sampled rows and columns of
-	the result equal their fp32 dot products; a one-hot A row selects a B column exactly."""
-	M, N, Kd = (T, FFN, D_MODEL) if layout != "tn" else (D_MODEL, FFN, T)
+def test_gemm_row_and_column_probes_at_full_size(K, layout, dims):
+	"""C = A B^T (for tn the matching dW shape, K = tokens): 64 sampled rows and columns of the result
+	equal their fp32 dot products; a one-hot A row selects a B column exactly."""
+	M, N, Kd = dims if layout != "tn" else (dims[2], dims[1], dims[0])
 	A = _randn(M, Kd, seed=1)
 	B = _randn(N, Kd, seed=2, scale=0.05)
 	A[7].zero_()
@@ -37,8 +40,9 @@ def test_gemm_row_and_column_probes_at_full_size(K, layout):
 	elif layout == "nn":
 		C = K.gemm(A, B.t().contiguous(), b_t=True)
 	else:
-		C = K.gemm(A.t().contiguous(), B.t().contiguous(), a_t=True, b_t=True)
-	assert torch.equal(C[7], B[:, 1234])
+		C = torch.zeros(M, N, dtype=torch.float32, device="cuda")
+		K.gemm(A.t().contiguous(), B.t().contiguous(), a_t=True, b_t=True, out=C, epilogue=K.EPI_F32_ACC)
+	assert torch.equal(C[7].to(torch.bfloat16), B[:, 1234])
 	rows = torch.randint(0, M, (64,), generator=torch.Generator().manual_seed(3)).cuda()
 	cols = torch.randint(0, N, (64,), generator=torch.Generator().manual_seed(4)).cuda()
 	ref_r = A[rows].float() @ B.float().t()
