@@ -125,6 +125,9 @@ def main():
 	ap.add_argument("--no-cpu-baseline", action="store_true")
 	ap.add_argument("--prefetching-time", type=int, default=None,
 	                help="offload workloads: how many compute ops before its B a micro-batch's PREFETCH_ACTIVATIONS is placed (reference default 1)")
+	ap.add_argument("--graph", action="store_true",
+	                help="time replays of the step captured as one HIP graph (Engine.capture) instead of eager steps; the per-kernel figures "
+	                     "then come from one extra eager step after the timed region (a replay runs no host code that could bracket launches)")
 	ap.add_argument("--calibration-copy", action="store_true",
 	                help="also launch one elf::add_kernel over 2 x 128 MiB in, 128 MiB out: a kernel of known HBM traffic to scale profiler byte counters with")
 	args = ap.parse_args()
@@ -189,13 +192,28 @@ def main():
 	for _ in range(args.warmup):
 		step()
 	torch.cuda.synchronize()
-	lib.elf_prof_enable(1)
+	eager_step = step
+	if args.graph:
+		graphed = engine.capture(None, None, None, stream, mb_sizes)
+
+		def step():
+			block.zero_grad()
+			graphed.replay()
+
+		step()
+		torch.cuda.synchronize()
+	else:
+		lib.elf_prof_enable(1)
 	mem_before = block.mem_stats()
 	t0 = time.perf_counter()
 	for _ in range(args.steps):
 		step()
 	torch.cuda.synchronize()
 	elapsed = time.perf_counter() - t0
+	if args.graph:
+		lib.elf_prof_enable(1)
+		eager_step()
+		torch.cuda.synchronize()
 	kinds = ["gemm", "attn_fwd", "attn_bwd", "norm_fwd", "norm_bwd", "act_fwd", "act_bwd", "rope", "grad_scale", "add", "embed", "loss"]
 	per_kernel = {}
 	for i, name in enumerate(kinds):
@@ -217,7 +235,7 @@ def main():
 		"config": {
 			"workload": args.workload, "blocks": w["n_blocks"], "d_model": w["d"], "heads": w["heads"], "kv_heads": w["kv_heads"], "ffn": w["ffn"],
 			"seq_len": w["seq"], "micro_batch": w["mb"], "n_micro_batches": w["n_mb"], "op_stream": f"{w['scheduler']} block {BLOCK_ID} of placement {placement}",
-			"tokens_per_step": tokens, "ops_per_step": len(stream), "offload": bool(w.get("offload")),
+			"tokens_per_step": tokens, "ops_per_step": len(stream), "offload": bool(w.get("offload")), "hip_graph": bool(args.graph),
 		},
 		"roofline": {"bound": "mfma", "achieved": g["tflops"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": g["tflops"] / PEAK_BF16_TFLOPS, "traffic": GEMM_TRAFFIC_BYTES.get(args.workload),
 		             "kernel": "elf::dma::gemm_dma_kernel / elf::gemm_kernel (bf16 MFMA GEMM, all layouts)", "launches": g["launches"], "avg_launch_ms": g["avg_ms"]},

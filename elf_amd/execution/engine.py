@@ -25,7 +25,7 @@ logger = logging.getLogger("engine")
 precise_timings = os.environ.get("ELF_TIMINGS", False)
 precise_memory = os.environ.get("ELF_MEMORY", False)
 
-__all__ = ["Engine", "compute_loss"]
+__all__ = ["Engine", "GraphedStep", "compute_loss"]
 
 _GPU = torch.cuda.is_available
 
@@ -35,8 +35,12 @@ def _fake_p2p(data):
 	return [None, data.detach()]
 
 
+def _capturing():
+	return _GPU() and torch.cuda.is_current_stream_capturing()
+
+
 def _sync():
-	if _GPU():
+	if _GPU() and not _capturing():
 		torch.cuda.synchronize()
 
 
@@ -157,7 +161,7 @@ class Engine:
 				with Timer(name=f"backward({block.id}:{op.mb_id})") as timer:
 					grads = grad_fns.popleft()()
 				block.compute_time.append(timer)
-				if self.offload_stream is not None:
+				if self.offload_stream is not None and not _capturing():  # a captured step keeps its outputs on the GPU
 					self.offload_stream.wait_stream(torch.cuda.current_stream())
 					with torch.cuda.stream(self.offload_stream), torch.no_grad():
 						result[op.mb_id] = result[op.mb_id].to("cpu", non_blocking=True)
@@ -209,11 +213,75 @@ class Engine:
 		detailed_stats = {"all_events": all_events, "memories": memories, "peak_memory": peak_memories}
 		for block in self.blocks:
 			block.compute_time.clear()
-		if self.offload_stream is not None:
+		if self.offload_stream is not None and not _capturing():
 			torch.cuda.current_stream().wait_stream(self.offload_stream)
 		for off in offloaders.values():
 			off.release()
 		return result, losses, stats, detailed_stats
+
+	def capture(self, batch, target, loss_fn, schedule, mb_sizes, warmup=1):
+		"""Record one ``train_step`` as a HIP graph and return a ``GraphedStep`` that replays it.
+
+		A stage step is a fixed sequence of kernel launches (hundreds to thousands per step: one op is
+		40-50 launches); replaying it as a graph takes the Python interpreter, the slot bookkeeping
+		and the per-launch driver work out of the step.  The reference has no counterpart (its ops
+		build autograd graphs on the fly).  Conditions: the schedule must not offload activations
+		(copies to pinned memory on side streams stay eager), and between replays nothing else may
+		run stage ops of these blocks.  ``warmup`` eager steps run first so that every pool and
+		workspace has its final size (nothing may allocate device memory while capturing); the
+		gradient accumulators are put back as they were, so the capture itself adds no gradient.
+		"""
+		for op in schedule:
+			if op.op == OperationType.PREFETCH_ACTIVATIONS or op.options.get(OpOptions.ACTIVATION_OFFLOAD):
+				raise NotImplementedError("Engine.capture: schedules with activation offload are not captured")
+		static_batch = None if batch is None else [t.clone() for t in batch]
+		static_target = None if target is None else target.clone()
+		kept = [[g.clone() for g in getattr(b, "_fused_g", [])] for b in self.blocks]
+		side = torch.cuda.Stream()
+		side.wait_stream(torch.cuda.current_stream())
+		with torch.cuda.stream(side):
+			for _ in range(max(1, warmup)):
+				self.train_step(static_batch, static_target, loss_fn, schedule, mb_sizes)
+				self._reset_slots()
+		torch.cuda.current_stream().wait_stream(side)
+		torch.cuda.synchronize()
+		for b, gs in zip(self.blocks, kept):
+			for g, keep in zip(getattr(b, "_fused_g", []), gs):
+				g.copy_(keep)
+		graph = torch.cuda.CUDAGraph()
+		with torch.cuda.graph(graph):
+			result, losses, _, _ = self.train_step(static_batch, static_target, loss_fn, schedule, mb_sizes)
+		self._reset_slots()
+		return GraphedStep(graph, static_batch, static_target, result, losses)
+
+	def _reset_slots(self):
+		"""Empty the per-micro-batch slot lists of every block (what Pipeline.step does after a step)."""
+		for block in self.blocks:
+			block._wait_for_send_ops()
+			for var in block.input_variables:
+				var.clear()
+			for var in block.output_variables:
+				for dst in var:
+					dst.clear()
+
+
+class GraphedStep:
+	"""A captured ``Engine.train_step``.  ``replay(batch, target)`` copies the new data into the
+	buffers the graph reads, launches the graph and returns ``(result, losses)``: the same GPU tensors
+	every time (an eager step moves its outputs to the host), overwritten by each replay.  Weight gradients accumulate into the blocks' ``main_grad``
+	buffers exactly as in an eager step (zero them between steps as usual)."""
+
+	def __init__(self, graph, batch, target, result, losses):
+		self.graph, self.batch, self.target, self.result, self.losses = graph, batch, target, result, losses
+
+	def replay(self, batch=None, target=None):
+		if batch is not None:
+			for dst, src in zip(self.batch, [batch] if isinstance(batch, torch.Tensor) else batch):
+				dst.copy_(src)
+		if target is not None:
+			self.target.copy_(target)
+		self.graph.replay()
+		return self.result, self.losses
 
 
 def compute_loss(block, output, target, loss_fn):

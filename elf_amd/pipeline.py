@@ -133,17 +133,7 @@ class Pipeline:
 		"""One pass of the schedule over ``batch`` (elf/pipeline.py:209-295).  Returns
 		``(outputs per micro-batch, loss)`` when this process owns the last stage, else ``(None, None)``;
 		the loss is the sum of the micro-batch losses divided by the batch size."""
-		if batch is not None and isinstance(batch, torch.Tensor):
-			batch = [batch]
-		mb_sizes = self._get_mb_sizes(split_size, batch)
-		if any(not 1 <= m <= self.mb_size for m in mb_sizes):
-			raise ValueError(f"Pipeline: the stage buffers are sized for micro-batches of 1..{self.mb_size} samples, got sizes {sorted(set(mb_sizes))}")
-		n_micro_batches = len(mb_sizes)
-		regenerate = scheduler is not None or n_micro_batches != self.last_nmb
-		scheduler = self.scheduler if scheduler is None else resolve(scheduler, SCHEDULERS)
-		if regenerate:
-			self._generate_schedule(n_micro_batches, scheduler, self.cfg.comm_scheduler, mb_sizes)
-			self.last_nmb = n_micro_batches
+		batch, mb_sizes = self._prepare(batch, split_size, scheduler)
 
 		result, losses, stats, detailed_stats = self.engine.train_step(batch, target, loss_fn, self.schedule, mb_sizes, profile)
 
@@ -164,6 +154,41 @@ class Pipeline:
 
 	def __call__(self, *args, **kwargs):
 		return self.step(*args, **kwargs)
+
+	def _prepare(self, batch, split_size, scheduler):
+		"""Micro-batch sizes of ``batch`` and, when their number changed (or a scheduler is given), a new
+		schedule (elf/pipeline.py:237-252)."""
+		if batch is not None and isinstance(batch, torch.Tensor):
+			batch = [batch]
+		mb_sizes = self._get_mb_sizes(split_size, batch)
+		if any(not 1 <= m <= self.mb_size for m in mb_sizes):
+			raise ValueError(f"Pipeline: the stage buffers are sized for micro-batches of 1..{self.mb_size} samples, got sizes {sorted(set(mb_sizes))}")
+		n_micro_batches = len(mb_sizes)
+		regenerate = scheduler is not None or n_micro_batches != self.last_nmb
+		scheduler = self.scheduler if scheduler is None else resolve(scheduler, SCHEDULERS)
+		if regenerate:
+			self._generate_schedule(n_micro_batches, scheduler, self.cfg.comm_scheduler, mb_sizes)
+			self.last_nmb = n_micro_batches
+		return batch, mb_sizes
+
+	def capture_step(self, batch, target, loss_fn, split_size=0, scheduler=None, warmup=1):
+		"""``step`` recorded once as a HIP graph (``Engine.capture``).  Returns a callable
+		``replay(batch=None, target=None) -> (outputs per micro-batch, loss)`` with the shapes of the
+		captured call; outputs and loss are the same tensors at every replay.  No counterpart in the
+		reference; for steps whose kernels are short enough that launching them is what takes the time."""
+		batch, mb_sizes = self._prepare(batch, split_size, scheduler)
+		graphed = self.engine.capture(batch, target, loss_fn, self.schedule, mb_sizes, warmup)
+		total = sum(mb_sizes)
+
+		def replay(batch=None, target=None):
+			result, losses = graphed.replay(batch, target)
+			if len(result) == 0:
+				return None, None
+			with torch.no_grad():
+				return result, torch.stack([torch.as_tensor(l, dtype=torch.float32, device="cuda") for l in losses]).sum() / total
+
+		replay.graphed = graphed
+		return replay
 
 	# ------------------------------------------------------------------ parameters
 	def parameters(self):

@@ -77,13 +77,20 @@ class TimerGPU:
 		self.end_event = torch.cuda.Event(enable_timing=True)
 
 	def __enter__(self):
-		self.start_event.record()
+		# timing events cannot be recorded into a stream capture: a step being captured as a graph is
+		# not timed (time() gives 0)
+		self.recorded = not torch.cuda.is_current_stream_capturing()
+		if self.recorded:
+			self.start_event.record()
 		return self
 
 	def __exit__(self, *_):
-		self.end_event.record()
+		if self.recorded:
+			self.end_event.record()
 
 	def time(self):
+		if not self.recorded:
+			return 0.0
 		self.end_event.synchronize()
 		return self.start_event.elapsed_time(self.end_event) / 1000
 

@@ -1,0 +1,141 @@
+"""A stage step captured as a HIP graph (Engine.capture, Pipeline.capture_step) against the same step
+run eagerly: every replay is checked, with eager kernels and device synchronisations between the
+replays and with new input data written into the buffers the graph reads.  Outputs of F are
+bit-identical; gradients agree to 2e-3 (dQ and split-K weight gradients add with fp32 atomics, whose
+order differs from run to run)."""
+
+import pytest
+import torch
+
+from tests.helpers import assert_close, perturb_norms, product_grads
+
+pytestmark = pytest.mark.gpu
+
+
+def _middle_stage(seed=5):
+	from elf_amd import models
+	from elf_amd.execution import HipStageBlock
+	from elf_amd.partitioners.utils import sequential_signatures
+
+	st = models.llama_stage(2, 512, 4, 2, 768, 256, head_dim=128, seed=seed)
+	perturb_norms(st)
+	placement = [0, 1, 2, 3]
+	return st, HipStageBlock(st, 1, placement, sequential_signatures(placement)[1], mb_size=2)
+
+
+def _stream(nmb):
+	from elf_amd.partitioners.utils import sequential_signatures
+	from elf_amd.registry import COMM_SCHEDULERS, SCHEDULERS
+	from elf_amd.scheduling import add_comms
+
+	placement = [0, 1, 2, 3]
+	schedule = COMM_SCHEDULERS["pipelined"](add_comms(SCHEDULERS["zbh1"](placement, nmb), sequential_signatures(placement)))
+	return [op for op in schedule if op.block_id == 1]
+
+
+def test_captured_stage_stream_replays_like_the_eager_one():
+	from elf_amd import kernels as K
+	from elf_amd.execution import Engine
+	from elf_amd.synthetic import make_boundary
+
+	nmb, mb = 4, 2
+	stage, blk = _middle_stage()
+	xs, dys = make_boundary(mb, stage.seq_len, blk.d, nmb, seed=3, device="cuda")
+	blk.set_boundary(inputs=xs, grads=dys, keep_sent=True)
+	stream = _stream(nmb)
+	eng = Engine([blk])
+
+	def eager():
+		blk.zero_grad()
+		blk.set_boundary(inputs=xs, grads=dys, keep_sent=True)
+		eng.train_step(None, None, None, stream, [mb] * nmb)
+		torch.cuda.synchronize()
+		return {m: y.clone() for m, y in blk.sent_forward.items()}, {m: d.clone() for m, d in blk.sent_backward.items()}, {k: v.clone() for k, v in product_grads(stage).items()}
+
+	y0, dx0, g0 = eager()
+	blk.set_boundary(inputs=xs, grads=dys, keep_sent=True)
+	blk.zero_grad()
+	marker = [g.clone().fill_(0.5) for g in blk._fused_g]
+	for g, m in zip(blk._fused_g, marker):
+		g.copy_(m)
+	graphed = eng.capture(None, None, None, stream, [mb] * nmb)
+	assert all(torch.equal(g, m) for g, m in zip(blk._fused_g, marker)), "capturing must not change the gradient accumulators"
+	sent_y, sent_dx = dict(blk.sent_forward), dict(blk.sent_backward)  # tensors the graph writes
+	a = torch.randn(512, 512, device="cuda").to(torch.bfloat16)
+	for rep in range(3):
+		blk.zero_grad()
+		graphed.replay()
+		torch.cuda.synchronize()
+		for m in range(nmb):
+			assert torch.equal(sent_y[m], y0[m]), f"replay {rep}: y[{m}]"
+			assert_close(sent_dx[m], dx0[m], f"replay {rep}: dx[{m}]", rel_max=2e-3, rel_fro=2e-3)
+		got = product_grads(stage)
+		for name in sorted(g0):
+			assert_close(got[name], g0[name], f"replay {rep}: grad {name}", rel_max=2e-3, rel_fro=2e-3)
+		# eager work of the same library and a synchronisation between replays
+		K.gemm(a, a)
+		K.norm_fwd(K.NORM_RMS, a, torch.ones(512, dtype=torch.bfloat16, device="cuda"), None, 1e-5)
+		torch.cuda.synchronize()
+	assert blk.mem_stats()["live_bytes"] == 0
+
+	# new data in the buffers the graph reads: the replay follows it
+	xs2, dys2 = make_boundary(mb, stage.seq_len, blk.d, nmb, seed=4, device="cuda")
+	for dst, src in zip(list(xs) + list(dys), list(xs2) + list(dys2)):
+		dst.copy_(src)
+	blk.zero_grad()
+	graphed.replay()
+	torch.cuda.synchronize()
+	y_rep = {m: t.clone() for m, t in sent_y.items()}
+	g_rep = {k: v.clone() for k, v in product_grads(stage).items()}
+	y1, _, g1 = eager()
+	for m in range(nmb):
+		assert torch.equal(y_rep[m], y1[m]) and not torch.equal(y1[m], y0[m])
+	for name in sorted(g1):
+		assert_close(g_rep[name], g1[name], f"new data: grad {name}", rel_max=2e-3, rel_fro=2e-3)
+
+
+def test_captured_pipeline_step_with_the_one_kernel_loss():
+	"""Two stages (embedding ... head) on one rank, cross-entropy from elf_amd.losses: capture_step's
+	replays on new token ids give the loss and gradients of step() on the same ids."""
+	from elf_amd import losses, models
+	from elf_amd.pipeline import Pipeline
+
+	V, d, S, mb, nmb = 1000, 256, 128, 4, 4
+	first = models.gpt_end_stage(2, d, 4, 1024, S, vocab_in=V, causal=True, seed=41)
+	last = models.gpt_end_stage(2, d, 4, 1024, S, vocab_out=V, causal=True, seed=42)
+	pipe = Pipeline([first, last], torch.zeros(mb, S, dtype=torch.int64), scheduler="afab", partitioner=False, placement=[0, 0])
+	g = torch.Generator().manual_seed(2)
+	draw = lambda: (torch.randint(0, V, (mb * nmb, S), generator=g).cuda(), torch.randint(0, V, (mb * nmb, S), generator=g).cuda())
+	ids, tgt = draw()
+	pipe.zero_grad()
+	replay = pipe.capture_step(ids, tgt, losses.cross_entropy, split_size=mb)
+	for rep in range(3):
+		ids, tgt = draw()
+		pipe.zero_grad()
+		out, loss = replay(ids, tgt)
+		torch.cuda.synchronize()
+		got_loss = float(loss)
+		got_out = [o.clone() for o in out]
+		got = [p.main_grad.clone() for p in pipe.parameters()]  # (names repeat across stages)
+		pipe.zero_grad()
+		want_out, want_loss = pipe(ids, tgt, losses.cross_entropy, split_size=mb)
+		assert got_loss == pytest.approx(float(want_loss), rel=1e-4), f"replay {rep}"
+		for a, b in zip(got_out, want_out):
+			assert torch.equal(a.cpu(), b.cpu())
+		for have, (n, p) in zip(got, pipe.named_parameters()):
+			assert_close(have, p.main_grad, f"replay {rep}: grad {n}", rel_max=2e-3, rel_fro=2e-3)
+
+
+def test_capture_refuses_offload_schedules():
+	from elf_amd.benchmark_utils import get_offloaded_scheduler
+	from elf_amd.execution import Engine
+	from elf_amd.partitioners.utils import sequential_signatures
+	from elf_amd.registry import COMM_SCHEDULERS, SCHEDULERS
+	from elf_amd.scheduling import add_comms
+
+	stage, blk = _middle_stage()
+	placement = [0, 1, 2, 3]
+	sched = get_offloaded_scheduler(SCHEDULERS["1f1b"], 1, 1)
+	schedule = COMM_SCHEDULERS["pipelined"](add_comms(sched(placement, 4), sequential_signatures(placement)))
+	with pytest.raises(NotImplementedError):
+		Engine([blk]).capture(None, None, None, [op for op in schedule if op.block_id == 1], [2] * 4)
