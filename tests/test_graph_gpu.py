@@ -94,13 +94,22 @@ def test_captured_stage_stream_replays_like_the_eager_one():
 		assert_close(g_rep[name], g1[name], f"new data: grad {name}", rel_max=2e-3, rel_fro=2e-3)
 
 
-def test_captured_pipeline_step_with_the_one_kernel_loss():
-	"""Two stages (embedding ... head) on one rank, cross-entropy from elf_amd.losses: capture_step's
-	replays on new token ids give the loss and gradients of step() on the same ids."""
+@pytest.mark.parametrize("loss_kind", ["fused", "torch"])
+def test_captured_pipeline_step(loss_kind):
+	"""Two stages (embedding ... head) on one rank, cross-entropy from elf_amd.losses or torch's under
+	autograd: capture_step's replays on new token ids give the loss and gradients of step() on the
+	same ids."""
+	import torch.nn.functional as F
+
 	from elf_amd import losses, models
 	from elf_amd.pipeline import Pipeline
 
 	V, d, S, mb, nmb = 1000, 256, 128, 4, 4
+
+	def torch_loss(pred, target, *args, **kwargs):
+		return F.cross_entropy(pred.to(torch.float32).view(-1, V), target.view(-1), *args, **kwargs)
+
+	loss_fn = losses.cross_entropy if loss_kind == "fused" else torch_loss
 	first = models.gpt_end_stage(2, d, 4, 1024, S, vocab_in=V, causal=True, seed=41)
 	last = models.gpt_end_stage(2, d, 4, 1024, S, vocab_out=V, causal=True, seed=42)
 	pipe = Pipeline([first, last], torch.zeros(mb, S, dtype=torch.int64), scheduler="afab", partitioner=False, placement=[0, 0])
@@ -108,7 +117,7 @@ def test_captured_pipeline_step_with_the_one_kernel_loss():
 	draw = lambda: (torch.randint(0, V, (mb * nmb, S), generator=g).cuda(), torch.randint(0, V, (mb * nmb, S), generator=g).cuda())
 	ids, tgt = draw()
 	pipe.zero_grad()
-	replay = pipe.capture_step(ids, tgt, losses.cross_entropy, split_size=mb)
+	replay = pipe.capture_step(ids, tgt, loss_fn, split_size=mb)
 	for rep in range(3):
 		ids, tgt = draw()
 		pipe.zero_grad()
@@ -118,7 +127,7 @@ def test_captured_pipeline_step_with_the_one_kernel_loss():
 		got_out = [o.clone() for o in out]
 		got = [p.main_grad.clone() for p in pipe.parameters()]  # (names repeat across stages)
 		pipe.zero_grad()
-		want_out, want_loss = pipe(ids, tgt, losses.cross_entropy, split_size=mb)
+		want_out, want_loss = pipe(ids, tgt, loss_fn, split_size=mb)
 		assert got_loss == pytest.approx(float(want_loss), rel=1e-4), f"replay {rep}"
 		for a, b in zip(got_out, want_out):
 			assert torch.equal(a.cpu(), b.cpu())
