@@ -53,8 +53,11 @@ struct Args {
 // Byte offsets (relative to the tile origin of the current K slice) of the 16-byte chunks this
 // lane fetches for one operand (< 2^31: 256 rows of at most 64 K elements).  "R" tiles are
 // [256 rows][128 B], "T" tiles [64 k][512 B]; LDS chunk slot s of a row holds global chunk
-// s ^ f(row) with f chosen so that 16 consecutive lanes of a fragment read hit 16 distinct
-// 16-byte bank groups.
+// s ^ f(row) with f chosen so that the lanes of a fragment read spread over all banks: an "R"
+// read takes one chunk from each of 32 rows (f = (row / 2) % 8), a "T" transpose read takes 64
+// contiguous bytes from each of four k rows per half-wave (f = 4 * (k % 8): the four rows land in
+// four different 64-byte bank groups; with 2 * (k % 8) pairs of rows shared one and the bank-conflict
+// counter read half of the LDS-active cycles).
 template <bool T, int LPO>
 __device__ __forceinline__ void lane_offsets(int wave, int lane, int64_t ld, uint32_t (&off)[LPO]) {
 #pragma unroll
@@ -65,7 +68,7 @@ __device__ __forceinline__ void lane_offsets(int wave, int lane, int64_t ld, uin
 			off[i] = (uint32_t)((row * ld + ((slot ^ ((row >> 1) & 7)) << 3)) * 2);
 		} else {
 			const int krow = q * 2 + (lane >> 5), slot = lane & 31;
-			off[i] = (uint32_t)((krow * ld + ((slot ^ ((krow & 7) << 1)) << 3)) * 2);
+			off[i] = (uint32_t)((krow * ld + ((slot ^ ((krow & 7) << 2)) << 3)) * 2);
 		}
 	}
 }
@@ -82,8 +85,8 @@ __device__ __forceinline__ bf16x8 frag(const unsigned char* base, int row0, int 
 		const int m = row0 + 16 * ((lane & 31) >> 4) + 4 * (j & 3);
 		const int kk = ks * 16 + 8 * (lane >> 5) + (j >> 2);
 		// rows kk and kk+4 share (kk & 3) but not (kk & 7): compute both swizzles
-		const int c0 = (m >> 3) ^ ((kk & 7) << 1);
-		const int c1 = (m >> 3) ^ (((kk + 4) & 7) << 1);
+		const int c0 = (m >> 3) ^ ((kk & 7) << 2);
+		const int c1 = (m >> 3) ^ (((kk + 4) & 7) << 2);
 		const unsigned char* p0 = base + kk * 512 + c0 * 16 + (j & 1) * 8;
 		const unsigned char* p1 = base + (kk + 4) * 512 + c1 * 16 + (j & 1) * 8;
 		s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 ELF_LDS*)(p0));
