@@ -49,15 +49,18 @@ struct AttnBwdArgs {
 
 // Tiles fetched straight into LDS (lds_dma.h) are unpadded; the 16-byte chunk index of a row is
 // XOR-swizzled with a function of the row chosen so that both access patterns are conflict
-// free: row-wise fragment reads (16 consecutive rows, same chunk) and transpose reads (4
-// consecutive rows x 2 adjacent chunks).
+// free: row-wise fragment reads (16 consecutive rows, same chunk) and transpose reads (a
+// half-wave takes 64 contiguous bytes from each of 4 consecutive rows).
 template <int D>
 struct BwdTile {
 	static constexpr int ROW_BYTES = D * 2;
 	static constexpr int CPR = D / 8;             // 16-byte chunks per row
 	static constexpr int RPI = 1024 / ROW_BYTES;  // rows per DMA wave instruction
 	__device__ static __forceinline__ int swz(int row) {
-		return D == 128 ? (((row & 7) << 1) | ((row >> 3) & 1)) : ((((row >> 1) & 3) << 1) | ((row >> 3) & 1));
+		// D = 128 (16 chunks per row, a row spans all banks): bits [3:2] from row % 4 put four consecutive
+		// rows into four different 64-byte bank groups, bits [1:0] from row / 4 make 16 consecutive rows
+		// distinct.  D = 64 (8 chunks, two rows span all banks): the same for row pairs, bit-reversed.
+		return D == 128 ? (((row & 3) << 2) | ((row >> 2) & 3)) : ((((row >> 1) & 1) << 2) | (((row >> 2) & 1) << 1) | ((row >> 3) & 1));
 	}
 	// row-wise operand: rows row0 + lane%32, 8 consecutive columns from 16*ks + 8*(lane/32)
 	__device__ static __forceinline__ bf16x8 rows(const unsigned char* t, int row0, int ks, int lane) {

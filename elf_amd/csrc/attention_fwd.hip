@@ -9,8 +9,8 @@ namespace attn {
 // ring; tiles are unpadded (a wave instruction fills 1 KiB contiguously), so the 16-byte chunk
 // index of every row is XOR-swizzled: for K (read along d, one row per lane) with a function
 // of the row that spreads 16 consecutive rows over all 16 bank groups, for V (read with the
-// transpose read, 4 rows x 32 B per 16 lanes) with an even value so that chunk pairs stay
-// adjacent.
+// transpose read: a half-wave takes 64 contiguous bytes from each of four consecutive rows) with
+// a multiple of four chunks, so that the four rows land in four different 64-byte bank groups.
 template <int D>
 struct FwdTile {
 	static constexpr int ROW_BYTES = D * 2;
@@ -19,7 +19,7 @@ struct FwdTile {
 	static constexpr int RPI = 1024 / ROW_BYTES;       // rows per DMA wave instruction
 	static constexpr int LOADS = TILE_BYTES / 1024 / 4;  // DMA instructions per wave and operand
 	__device__ static __forceinline__ int k_swz(int row) { return D == 128 ? (row & 15) : ((row >> 1) & 7); }
-	__device__ static __forceinline__ int v_swz(int row) { return D == 128 ? ((row & 7) << 1) : (((row >> 1) & 3) << 1); }
+	__device__ static __forceinline__ int v_swz(int row) { return D == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); }
 };
 
 template <int D, bool CAUSAL>
