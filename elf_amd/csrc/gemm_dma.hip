@@ -17,6 +17,7 @@
 #include "common.h"
 #include "kernels.h"
 #include "lds_dma.h"
+#include <type_traits>
 
 namespace elf {
 
@@ -37,6 +38,15 @@ struct Shape {
 	static constexpr int LOADS_PER_STAGE = LOADS_A + LOADS_B;
 	static_assert(LOADS_PER_STAGE % 2 == 0, "the loads of a slice are issued in two halves");
 };
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>), unrolled at compile time.
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+	if constexpr (N > 0) {
+		static_for<N - 1>(f);
+		f(std::integral_constant<int, N - 1>{});
+	}
+}
 
 struct Args {
 	const bf16_t* A;
@@ -158,23 +168,27 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	const uint32_t lds_a = lds_addr(smem) + wave * (LOADS_A * 1024);
 	const uint32_t lds_b = lds_addr(smem) + A_BYTES + wave * (LOADS_B * 1024);
 
-	// One 1 KiB piece of a slice: the first LOADS_A pieces belong to A, the rest to B.  A piece of a slice past the
-	// end of K is fetched from the last slice into a scratch area behind the ring instead, so that
-	// the main loop needs no branches around its loads (the accumulators stay put in registers).
-	const uint32_t lds_dummy = lds_addr(smem) + NST * STAGE_BYTES + wave * 1024;
-	auto issue_piece = [&](int step, int piece) {
+	// Loads of one K slice: its operand pointers and the LDS addresses of this wave's first piece of
+	// each operand in the slice's stage.  Piece P (compile-time) is one wave instruction filling 1 KiB;
+	// the first LOADS_A pieces belong to A, the rest to B.  A slice past the end of K is fetched from
+	// the last slice into a scratch area behind the ring (shared by all waves: nobody reads it), so
+	// that the main loop needs no branches around its loads and the accumulators stay put in registers.
+	struct SliceLoads {
+		const bf16_t* pa;
+		const bf16_t* pb;
+		uint32_t la, lb;
+	};
+	const uint32_t lds_dummy = lds_addr(smem) + NST * STAGE_BYTES;
+	auto slice_loads = [&](int step) {
 		const bool ok = step < nk;
 		const int sc = ok ? step : nk - 1;
-		const uint32_t st = (uint32_t)(sc % NST) * STAGE_BYTES;
-		if (piece < LOADS_A)
-			dma16(Ap + (int64_t)sc * a_step, aoff[piece], __builtin_amdgcn_readfirstlane(ok ? lds_a + st + piece * 1024 : lds_dummy));
-		else
-			dma16(Bp + (int64_t)sc * b_step, boff[piece - LOADS_A],
-			      __builtin_amdgcn_readfirstlane(ok ? lds_b + st + (piece - LOADS_A) * 1024 : lds_dummy));
+		const uint32_t st = (uint32_t)(sc & 1) * STAGE_BYTES;
+		return SliceLoads{Ap + (int64_t)sc * a_step, Bp + (int64_t)sc * b_step, ok ? lds_a + st : lds_dummy, ok ? lds_b + st : lds_dummy};
 	};
-	auto issue = [&](int step) {
-#pragma unroll
-		for (int i = 0; i < LOADS_PER_STAGE; i++) issue_piece(step, i);
+	auto issue_piece = [&](const SliceLoads& sl, auto pc) {
+		constexpr int P = decltype(pc)::value;
+		if constexpr (P < LOADS_A) dma16_at<P * 1024>(sl.pa, aoff[P], sl.la);
+		else dma16_at<(P - LOADS_A) * 1024>(sl.pb, boff[P - LOADS_A], sl.lb);
 	};
 
 	f32x16 acc[RT][4];
@@ -190,10 +204,13 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	// barrier that publishes slice kt+1 sits before the LAST k16-step of slice kt: by then every
 	// wave has read all of slice kt (its last fragments are in registers), so the same barrier
 	// frees that stage and the fetch of slice kt+2 starts a full slice ahead of its use.
-	issue(0);
-#pragma unroll
-	for (int i = 0; i < LOADS_PER_STAGE / 2; i++) issue_piece(1, i);
-	wait_vmcnt<LOADS_PER_STAGE / 2>();
+	constexpr int HALF = LOADS_PER_STAGE / 2;
+	{
+		const SliceLoads s0 = slice_loads(0), s1 = slice_loads(1);
+		static_for<LOADS_PER_STAGE>([&](auto pc) { issue_piece(s0, pc); });
+		static_for<HALF>([&](auto pc) { issue_piece(s1, pc); });
+		wait_vmcnt<HALF>();
+	}
 	__syncthreads();
 
 	bf16x8 fa[2][RT], fb[2][4];
@@ -213,30 +230,30 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 				acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][i], fb[buf][j], acc[i][j], 0, 0, 0);
 	};
 
-	// The MFMAs of one k16-step with half of this wave's loads of a slice (from `piece0`) dealt between
-	// them: the four waves' loads of a slice are 64 KiB through a 64 B/clk path, and a wave that
+	// The MFMAs of one k16-step with half of this wave's loads of a slice (pieces PIECE0 ...) dealt evenly
+	// between them: the waves' loads of a slice are 64 KiB through a 64 B/clk path, and a wave that
 	// issues them in one burst sits in the queue for ~1000 cycles with its MFMAs behind it.
-	auto mfmas_dma = [&](int buf, int step, int piece0) {
-		constexpr int HALF = LOADS_PER_STAGE / 2, NM = RT * 4;  // HALF loads spread evenly over NM MFMAs
-#pragma unroll
-		for (int i = 0; i < RT; i++)
-#pragma unroll
-			for (int j = 0; j < 4; j++) {
-				acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][i], fb[buf][j], acc[i][j], 0, 0, 0);
-				const int n = i * 4 + j;
-				if ((n + 1) * HALF / NM != n * HALF / NM) {
-					issue_piece(step, piece0 + n * HALF / NM);
-					__builtin_amdgcn_sched_barrier(0);
-				}
+	auto mfmas_dma = [&](int buf, const SliceLoads& sl, auto piece0) {
+		constexpr int PIECE0 = decltype(piece0)::value, NM = RT * 4;
+		static_for<NM>([&](auto nc) {
+			constexpr int n = decltype(nc)::value, i = n / 4, j = n % 4;
+			acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][i], fb[buf][j], acc[i][j], 0, 0, 0);
+			if constexpr ((n + 1) * HALF / NM != n * HALF / NM) {
+				issue_piece(sl, std::integral_constant<int, PIECE0 + n * HALF / NM>{});
+				__builtin_amdgcn_sched_barrier(0);
 			}
+		});
 	};
 
 	load_frags(0, 0, 0);
 	for (int kt = 0; kt < nk; kt++) {
+		// where this iteration's loads go: scalar work, done here so that it overlaps the fragment reads
+		// instead of sitting between two MFMAs
+		const SliceLoads next1 = slice_loads(kt + 1), next2 = slice_loads(kt + 2);
 		// k16-step 0, with the second half of slice kt+1's loads
 		load_frags(1, kt, 1);
 		__builtin_amdgcn_sched_barrier(0);
-		mfmas_dma(0, kt + 1, LOADS_PER_STAGE / 2);
+		mfmas_dma(0, next1, std::integral_constant<int, HALF>{});
 		__builtin_amdgcn_sched_barrier(0);
 #pragma unroll
 		for (int ks = 1; ks < 3; ks++) {
@@ -250,7 +267,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 		load_frags(0, kt + 1, 0);  // past the end this reads a stale stage; the values are unused
 		__builtin_amdgcn_sched_barrier(0);
 		// k16-step 3, with the first half of slice kt+2's loads into the stage the barrier just freed
-		mfmas_dma(1, kt + 2, 0);
+		mfmas_dma(1, next2, std::integral_constant<int, 0>{});
 		__builtin_amdgcn_sched_barrier(0);
 	}
 
@@ -321,9 +338,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 
 template <int NW, int RT, bool AT, bool BT, int EPI>
 static int launch(const Args& a, hipStream_t stream) {
-	// ring + 1 KiB per wave as the target of the loads past the end of K; the epilogue needs a
-	// 32 x 136 fp32 strip per wave
-	constexpr int ring = NST * Shape<NW, RT>::STAGE_BYTES + NW * 1024, epi = NW * 32 * 136 * 4;
+	// the ring + the target of the loads past the end of K (as many KiB as a wave issues loads per
+	// operand); the epilogue needs a 32 x 136 fp32 strip per wave
+	using Sh = Shape<NW, RT>;
+	constexpr int ring = NST * Sh::STAGE_BYTES + (Sh::LOADS_A > Sh::LOADS_B ? Sh::LOADS_A : Sh::LOADS_B) * 1024, epi = NW * 32 * 136 * 4;
 	constexpr int smem = ring > epi ? ring : epi;
 	auto kern = gemm_dma_kernel<NW, RT, AT, BT, EPI>;
 	static bool attr_set = false;

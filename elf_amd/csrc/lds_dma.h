@@ -16,6 +16,13 @@ __device__ __forceinline__ void dma16(const void* base, uint32_t byte_off, uint3
 	asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_byte_addr), "v"(byte_off), "s"(base) : "memory", "m0");
 }
 
+// The same with the LDS address given as a wave-uniform base plus a compile-time byte offset: M0 is
+// written by the add itself.
+template <int IMM>
+__device__ __forceinline__ void dma16_at(const void* base, uint32_t byte_off, uint32_t lds_base) {
+	asm volatile("s_add_u32 m0, %0, %3\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(byte_off), "s"(base), "n"(IMM) : "memory", "m0", "scc");
+}
+
 // s_waitcnt with explicit fields (gfx9 layout: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] at [15:14]).
 template <int VM, int LGKM = 15>
 __device__ __forceinline__ void wait_counters() {
