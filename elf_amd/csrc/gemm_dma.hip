@@ -8,8 +8,8 @@
 //   * a wave instruction fills 1 KiB of LDS contiguously, so tiles cannot be padded; bank
 //     conflicts are avoided by an XOR swizzle of the 16-byte chunk index, applied on the global
 //     side when choosing which chunk a lane fetches and undone when fragments are read;
-//   * 4 waves, one per SIMD, each owning a 128x128 sub-tile (16 accumulator tiles): 8 fragment
-//     reads feed 16 MFMAs, half the LDS traffic per FLOP of the 128x64 arrangement.
+//   * the contraction runs on v_mfma_f32_16x16x32_bf16; 8 waves (two per SIMD) own 64x128 sub-tiles,
+//     or 4 waves (one per SIMD) 128x128 ones.
 // The DMA loads are issued through inline assembly: the compiler cannot see that they write
 // LDS, which is what allows partial vmcnt waits (its own tracking would force vmcnt(0) before
 // every LDS read).  Ordering is explicit: s_waitcnt vmcnt(n) for this wave's slice, then a
@@ -68,6 +68,9 @@ struct Args {
 // contiguous bytes from each of four k rows per half-wave (f = 4 * (k % 8): the four rows land in
 // four different 64-byte bank groups; with 2 * (k % 8) pairs of rows shared one and the bank-conflict
 // counter read half of the LDS-active cycles).
+// chunk swizzle of reduction-major ("T") tiles as a function of the k row
+__device__ __forceinline__ int t_swz(int k) { return ((k & 7) << 2) ^ (((k >> 3) & 1) << 1); }
+
 template <bool T, int LPO>
 __device__ __forceinline__ void lane_offsets(int wave, int lane, int64_t ld, uint32_t (&off)[LPO]) {
 #pragma unroll
@@ -78,25 +81,27 @@ __device__ __forceinline__ void lane_offsets(int wave, int lane, int64_t ld, uin
 			off[i] = (uint32_t)((row * ld + ((slot ^ ((row >> 1) & 7)) << 3)) * 2);
 		} else {
 			const int krow = q * 2 + (lane >> 5), slot = lane & 31;
-			off[i] = (uint32_t)((krow * ld + ((slot ^ ((krow & 7) << 2)) << 3)) * 2);
+			off[i] = (uint32_t)((krow * ld + ((slot ^ t_swz(krow)) << 3)) * 2);
 		}
 	}
 }
 
-// MFMA operand fragment of the 32-row slab at `row0` for k16-step ks of the current stage.
+// Operand fragment of v_mfma_f32_16x16x32_bf16 for the 16-row slab at `row0` and the k32 half `kq`
+// of the current slice: lane l holds row (or column) row0 + l % 16 at k = 32 kq + 8 (l / 16) .. + 7.
+// "R" tiles give it with one 16-byte read; "T" tiles with two transpose reads, each of which hands
+// the 16 lanes of a group the 4 (k) x 16 (rows) block they address row-wise.
 template <bool T>
-__device__ __forceinline__ bf16x8 frag(const unsigned char* base, int row0, int ks, int lane) {
+__device__ __forceinline__ bf16x8 frag(const unsigned char* base, int row0, int kq, int lane) {
 	if constexpr (!T) {
-		const int r = row0 + (lane & 31);
-		const int c = (2 * ks + (lane >> 5)) ^ ((r >> 1) & 7);
+		const int r = row0 + (lane & 15);
+		const int c = (4 * kq + (lane >> 4)) ^ ((r >> 1) & 7);
 		return *reinterpret_cast<const bf16x8*>(base + r * 128 + c * 16);
 	} else {
 		const int j = lane & 15;
-		const int m = row0 + 16 * ((lane & 31) >> 4) + 4 * (j & 3);
-		const int kk = ks * 16 + 8 * (lane >> 5) + (j >> 2);
-		// rows kk and kk+4 share (kk & 3) but not (kk & 7): compute both swizzles
-		const int c0 = (m >> 3) ^ ((kk & 7) << 2);
-		const int c1 = (m >> 3) ^ (((kk + 4) & 7) << 2);
+		const int m = row0 + 4 * (j & 3);
+		const int kk = kq * 32 + 8 * (lane >> 4) + (j >> 2);
+		const int c0 = (m >> 3) ^ t_swz(kk);
+		const int c1 = (m >> 3) ^ t_swz(kk + 4);
 		const unsigned char* p0 = base + kk * 512 + c0 * 16 + (j & 1) * 8;
 		const unsigned char* p1 = base + (kk + 4) * 512 + c1 * 16 + (j & 1) * 8;
 		s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 ELF_LDS*)(p0));
@@ -105,10 +110,10 @@ __device__ __forceinline__ bf16x8 frag(const unsigned char* base, int row0, int 
 	}
 }
 
-// NW = 4, RT = 4: one wave per SIMD, 128x128 wave tiles (16 accumulator tiles, 8 fragment reads per
-// 16 MFMAs).  NW = 8, RT = 2: two waves per SIMD, 64x128 wave tiles (8 accumulator tiles, 6 reads per
-// 8 MFMAs): more LDS traffic per FLOP, but the two waves fill each other's issue gaps (every
-// non-MFMA instruction of a lone wave delays its MFMA stream by a few cycles) and barrier waits.
+// NW = 4, RT = 4: one wave per SIMD, 128x128 wave tiles (16 fragment reads per k32 and 64 MFMAs).
+// NW = 8, RT = 2: two waves per SIMD, 64x128 wave tiles (12 reads per k32 and 32 MFMAs): more LDS
+// traffic per FLOP, but the two waves fill each other's issue gaps (every non-MFMA instruction of a
+// lone wave delays its MFMA stream by a few cycles) and barrier waits.
 // NW = 4, RT = 2: 128x256 workgroup tile for outputs with too few 256x256 tiles to fill the chip
 // (A must be k-contiguous: the reduction-major tile layout below assumes 256 rows).
 template <int NW, int RT, bool AT, bool BT, int EPI>
@@ -191,19 +196,23 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 		else dma16_at<(P - LOADS_A) * 1024>(sl.pb, boff[P - LOADS_A], sl.lb);
 	};
 
-	f32x16 acc[RT][4];
+	// 16x16 accumulator tiles: RT * 2 down, 8 across (the 16x16x32 MFMA moves half as many accumulator
+	// registers per FLOP as the 32x32x16 one, and sustains a higher clock under the power limit)
+	constexpr int RF = RT * 2;
+	f32x4 acc[RF][8];
 #pragma unroll
-	for (int i = 0; i < RT; i++)
+	for (int i = 0; i < RF; i++)
 #pragma unroll
-		for (int j = 0; j < 4; j++)
+		for (int j = 0; j < 8; j++)
 #pragma unroll
-			for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+			for (int r = 0; r < 4; r++) acc[i][j][r] = 0.f;
 
-	// Software pipeline.  While the 16 MFMAs of one k16-step issue, the 8 fragment reads of the
-	// next step are in flight (one wave per SIMD: nothing else would hide the LDS latency).  The
-	// barrier that publishes slice kt+1 sits before the LAST k16-step of slice kt: by then every
-	// wave has read all of slice kt (its last fragments are in registers), so the same barrier
-	// frees that stage and the fetch of slice kt+2 starts a full slice ahead of its use.
+	// Software pipeline.  A slice is four half-steps (k32 half kq = 0, 1 x column half h = 0, 1) of RF * 4
+	// MFMAs; the fragments of a half-step are read during the one before it (B: four 16-column slabs
+	// per half-step, ping-pong; A: RF slabs per k32 half, ping-pong).  The barrier that publishes slice
+	// kt+1 sits before the LAST half-step of slice kt: by then every wave has read all of slice kt (its
+	// last fragments are in registers), so the same barrier frees that stage and the fetch of slice
+	// kt+2 starts a full slice ahead of its use.
 	constexpr int HALF = LOADS_PER_STAGE / 2;
 	{
 		const SliceLoads s0 = slice_loads(0), s1 = slice_loads(1);
@@ -213,31 +222,33 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	}
 	__syncthreads();
 
-	bf16x8 fa[2][RT], fb[2][4];
-	auto load_frags = [&](int buf, int step, int ks) {
+	bf16x8 fa[2][RF], fb[2][4];
+	auto load_a = [&](int buf, int step, int kq) {
 		const unsigned char* sa = smem + (step % NST) * STAGE_BYTES;
-		const unsigned char* sb = sa + A_BYTES;
 #pragma unroll
-		for (int i = 0; i < RT; i++) fa[buf][i] = frag<AT>(sa, wr * (RT * 32) + i * 32, ks, lane);
-#pragma unroll
-		for (int j = 0; j < 4; j++) fb[buf][j] = frag<BT>(sb, wc * 128 + j * 32, ks, lane);
+		for (int i = 0; i < RF; i++) fa[buf][i] = frag<AT>(sa, wr * (RT * 32) + i * 16, kq, lane);
 	};
-	auto mfmas = [&](int buf) {
+	auto load_b = [&](int buf, int step, int kq, int h) {
+		const unsigned char* sb = smem + (step % NST) * STAGE_BYTES + A_BYTES;
 #pragma unroll
-		for (int i = 0; i < RT; i++)
+		for (int j = 0; j < 4; j++) fb[buf][j] = frag<BT>(sb, wc * 128 + (h * 4 + j) * 16, kq, lane);
+	};
+	auto mfmas = [&](int abuf, int bbuf, int h) {
+#pragma unroll
+		for (int i = 0; i < RF; i++)
 #pragma unroll
 			for (int j = 0; j < 4; j++)
-				acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][i], fb[buf][j], acc[i][j], 0, 0, 0);
+				acc[i][h * 4 + j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[abuf][i], fb[bbuf][j], acc[i][h * 4 + j], 0, 0, 0);
 	};
 
-	// The MFMAs of one k16-step with half of this wave's loads of a slice (pieces PIECE0 ...) dealt evenly
+	// The MFMAs of one half-step with half of this wave's loads of a slice (pieces PIECE0 ...) dealt evenly
 	// between them: the waves' loads of a slice are 64 KiB through a 64 B/clk path, and a wave that
 	// issues them in one burst sits in the queue for ~1000 cycles with its MFMAs behind it.
-	auto mfmas_dma = [&](int buf, const SliceLoads& sl, auto piece0) {
-		constexpr int PIECE0 = decltype(piece0)::value, NM = RT * 4;
+	auto mfmas_dma = [&](int abuf, int bbuf, auto hc, const SliceLoads& sl, auto piece0) {
+		constexpr int PIECE0 = decltype(piece0)::value, H = decltype(hc)::value, NM = RF * 4;
 		static_for<NM>([&](auto nc) {
 			constexpr int n = decltype(nc)::value, i = n / 4, j = n % 4;
-			acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][i], fb[buf][j], acc[i][j], 0, 0, 0);
+			acc[i][H * 4 + j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[abuf][i], fb[bbuf][j], acc[i][H * 4 + j], 0, 0, 0);
 			if constexpr ((n + 1) * HALF / NM != n * HALF / NM) {
 				issue_piece(sl, std::integral_constant<int, PIECE0 + n * HALF / NM>{});
 				__builtin_amdgcn_sched_barrier(0);
@@ -245,65 +256,58 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 		});
 	};
 
-	load_frags(0, 0, 0);
+	load_a(0, 0, 0);
+	load_b(0, 0, 0, 0);
 	for (int kt = 0; kt < nk; kt++) {
 		// where this iteration's loads go: scalar work, done here so that it overlaps the fragment reads
 		// instead of sitting between two MFMAs
 		const SliceLoads next1 = slice_loads(kt + 1), next2 = slice_loads(kt + 2);
-		// k16-step 0, with the second half of slice kt+1's loads
-		load_frags(1, kt, 1);
+		// half-step (kq 0, h 0), with the second half of slice kt+1's loads
+		load_b(1, kt, 0, 1);
 		__builtin_amdgcn_sched_barrier(0);
-		mfmas_dma(0, next1, std::integral_constant<int, HALF>{});
+		mfmas_dma(0, 0, std::integral_constant<int, 0>{}, next1, std::integral_constant<int, HALF>{});
 		__builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-		for (int ks = 1; ks < 3; ks++) {
-			load_frags((ks + 1) & 1, kt, ks + 1);
-			__builtin_amdgcn_sched_barrier(0);
-			mfmas(ks & 1);
-			__builtin_amdgcn_sched_barrier(0);
-		}
+		// (kq 0, h 1)
+		load_a(1, kt, 1);
+		load_b(0, kt, 1, 0);
+		__builtin_amdgcn_sched_barrier(0);
+		mfmas(0, 1, 1);
+		__builtin_amdgcn_sched_barrier(0);
+		// (kq 1, h 0)
+		load_b(1, kt, 1, 1);
+		__builtin_amdgcn_sched_barrier(0);
+		mfmas(1, 0, 0);
+		__builtin_amdgcn_sched_barrier(0);
 		wait_counters<0, 0>();  // vmcnt(0): slice kt+1 landed; lgkmcnt(0): slice kt fully read
 		__syncthreads();
-		load_frags(0, kt + 1, 0);  // past the end this reads a stale stage; the values are unused
+		// (kq 1, h 1), with the first half of slice kt+2's loads into the stage the barrier just freed;
+		// past the end the fragment reads hit a stale stage and their values are unused
+		load_a(0, kt + 1, 0);
+		load_b(0, kt + 1, 0, 0);
 		__builtin_amdgcn_sched_barrier(0);
-		// k16-step 3, with the first half of slice kt+2's loads into the stage the barrier just freed
-		mfmas_dma(1, next2, std::integral_constant<int, 0>{});
+		mfmas_dma(1, 1, std::integral_constant<int, 1>{}, next2, std::integral_constant<int, 0>{});
 		__builtin_amdgcn_sched_barrier(0);
 	}
 
-	// Epilogue through LDS (free once every wave has left the main loop).  Register r of a 32x32
-	// accumulator tile holds row (r/4)*8 + (lane/32)*4 + r%4, column lane%32; each wave parks one
-	// 32 x 128 fp32 strip at a time in its own LDS region (row pitch 136 floats: the two half-waves
-	// land on disjoint banks) and reads it back row-wise, so that global accesses are 16 bytes per
-	// lane over 256..512 contiguous bytes per row and accumulators leave the AGPRs only via ds_write.
+	// Epilogue through LDS (free once every wave has left the main loop).  Register r of a 16x16
+	// accumulator tile holds row (lane/16)*4 + r, column lane%16; each wave parks one 32 x 128 fp32 strip
+	// (two rows of accumulator tiles) at a time in its own LDS region (row pitch 136 floats) and reads it
+	// back row-wise, so that global accesses are 16 bytes per lane over 256..512 contiguous bytes per row
+	// and accumulators leave the AGPRs only via ds_write.
 	wait_vmcnt<0>();  // the loads past the end of K issued by the last iterations land in LDS too
 	__syncthreads();
 	constexpr int PITCH = 136;
 	float* ws = reinterpret_cast<float*>(smem) + wave * (32 * PITCH);
-	const int col_l = lane & 31;
-	const int row_l = (lane >> 5) * 4;
-	if constexpr (EPI == EPI_F32_ACC) {
-		if (splits > 1) {
-			// several workgroups add into this tile: fp32 atomics straight from the accumulators, in the
-			// accumulator layout, where a wave instruction covers two full 128-byte rows of 32 columns
-			// (the row-wise 16-byte layout below would touch a quarter of eight lines per instruction)
-			float* cbase = reinterpret_cast<float*>(g.C) + (int64_t)(m0 + wr * (RT * 32) + row_l) * g.ldc + n0 + wc * 128 + col_l;
-#pragma unroll
-			for (int i = 0; i < RT; i++)
-#pragma unroll
-				for (int j = 0; j < 4; j++)
-#pragma unroll
-					for (int r = 0; r < 16; r++)
-						unsafeAtomicAdd(cbase + (int64_t)(i * 32 + (r >> 2) * 8 + (r & 3)) * g.ldc + j * 32, acc[i][j][r]);
-			return;
-		}
-	}
+	const int col_l = lane & 15;
+	const int row_l = (lane >> 4) * 4;
 #pragma unroll
 	for (int i = 0; i < RT; i++) {
 #pragma unroll
-		for (int j = 0; j < 4; j++)
+		for (int ii = 0; ii < 2; ii++)
 #pragma unroll
-			for (int r = 0; r < 16; r++) ws[((r >> 2) * 8 + row_l + (r & 3)) * PITCH + j * 32 + col_l] = acc[i][j][r];
+			for (int j = 0; j < 8; j++)
+#pragma unroll
+				for (int r = 0; r < 4; r++) ws[(ii * 16 + row_l + r) * PITCH + j * 16 + col_l] = acc[i * 2 + ii][j][r];
 		const int grow0 = m0 + wr * (RT * 32) + i * 32;
 		const int gcol0 = n0 + wc * 128;
 		if constexpr (EPI == EPI_BF16 || EPI == EPI_BF16_RESID) {
@@ -324,6 +328,19 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 				*reinterpret_cast<bf16x8*>(reinterpret_cast<bf16_t*>(g.C) + (int64_t)(grow0 + row) * g.ldc + gcol0 + c8) = o;
 			}
 		} else {
+			if (EPI == EPI_F32_ACC && splits > 1) {
+				// several workgroups add into this tile: fp32 atomics, one scalar per lane so that a wave
+				// instruction covers two whole 128-byte rows of 32 columns (16 bytes per lane would touch a
+				// quarter of eight lines per instruction and run at half the speed)
+#pragma unroll
+				for (int it = 0; it < 16; it++) {
+					const int row = it * 2 + (lane >> 5);
+					float* c = reinterpret_cast<float*>(g.C) + (int64_t)(grow0 + row) * g.ldc + gcol0 + (lane & 31);
+#pragma unroll
+					for (int cg = 0; cg < 4; cg++) unsafeAtomicAdd(c + cg * 32, ws[row * PITCH + cg * 32 + (lane & 31)]);
+				}
+				continue;
+			}
 #pragma unroll
 			for (int it = 0; it < 16; it++) {
 				const int row = it * 2 + (lane >> 5), c4 = (lane & 31) * 4;
