@@ -329,7 +329,7 @@ int gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda,
 	}
 	// narrower outputs (e.g. N = 768 at M = 8192): 128x256 tiles of the same kernel fill the chip
 	if (tile_cfg <= 0 && !a_t && M % 128 == 0 && N % 256 == 0 && (int64_t)(M / 128) * (N / 256) >= 128) tile_cfg = 8;
-	if (tile_cfg == 6 || tile_cfg == 7) {
+	if (tile_cfg == 7) {
 		int tail_tiles = -1;  // an explicit k_splits splits every tile
 		if (epi == EPI_F32_ACC && k_splits <= 0) {
 			const int64_t tiles = (int64_t)(M / 256) * (N / 256);
@@ -347,9 +347,9 @@ int gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda,
 				if (nk / k_splits < 16) k_splits = 1;
 			}
 		}
-		return gemm_bf16_dma(a_t, b_t, M, N, K, A, lda, B, ldb, C, ldc, epi, R, ldr, k_splits, tail_tiles, tile_cfg == 7 ? 8 : 4, 256, stream);
+		return gemm_bf16_dma(a_t, b_t, M, N, K, A, lda, B, ldb, C, ldc, epi, R, ldr, k_splits, tail_tiles, 256, stream);
 	}
-	if (tile_cfg == 8) return gemm_bf16_dma(a_t, b_t, M, N, K, A, lda, B, ldb, C, ldc, epi, R, ldr, 1, 0, 4, 128, stream);
+	if (tile_cfg == 8) return gemm_bf16_dma(a_t, b_t, M, N, K, A, lda, B, ldb, C, ldc, epi, R, ldr, 1, 0, 128, stream);
 	if (!a_t && !b_t) return launch_epi<false, false>(g, epi, tile_cfg, stream);
 	if (!a_t && b_t) return launch_epi<false, true>(g, epi, tile_cfg, stream);
 	if (a_t && b_t) return launch_epi<true, true>(g, epi, tile_cfg, stream);

@@ -16,11 +16,11 @@ int gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda,
               void* C, int64_t ldc, int epi, const void* R, int64_t ldr, int tile_cfg, int k_splits,
               hipStream_t stream);
 
-// 256x256 tile (bm = 256; 4 or 8 waves) or 128x256 tile (bm = 128; 4 waves, A k-contiguous) with direct global->LDS
-// loads (gemm_dma.hip); called by gemm_bf16 for tile_cfg 6, 7 and 8.
+// 256x256 tile (bm = 256; 8 waves) or 128x256 tile (bm = 128; 4 waves, A k-contiguous) with direct global->LDS
+// loads (gemm_dma.hip); called by gemm_bf16 for tile_cfg 7 and 8.
 // EPI_F32_ACC only: the last tail_tiles tiles (all of them when tail_tiles < 0) are split k_splits ways along K.
 int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda, const void* B, int64_t ldb, void* C,
-                  int64_t ldc, int epi, const void* R, int64_t ldr, int k_splits, int tail_tiles, int waves, int bm, hipStream_t stream);
+                  int64_t ldc, int epi, const void* R, int64_t ldr, int k_splits, int tail_tiles, int bm, hipStream_t stream);
 
 enum NormKind { NORM_RMS = 0, NORM_LAYER = 1 };
 

@@ -33,7 +33,7 @@ int elf_abi_version(void);
  *   epilogue: 0 C(bf16) = acc; 1 C(bf16) = acc + R(bf16, leading dim ldr);
  *             2 C(fp32) += acc; 3 C(fp32) = acc.
  *   tile_cfg = 0 picks a tile shape from M,N (1: 256x256, 2: 128x128, 3: 64x64, 5: 256x128 register-staged;
- *   6 / 7: 256x256 with direct-to-LDS loads, 4 / 8 waves; 8: 128x256 with direct-to-LDS loads, a_t = 0 only);
+ *   7: 256x256 with direct-to-LDS loads; 8: 128x256 with direct-to-LDS loads, a_t = 0 only);
  *   k_splits = 0 picks a K split (epilogue 2 only).
  * Replaces: F.linear in LinearDX.forward (elf/zb_utils.py:20)            -> a_t=0,b_t=0
  *           torch.mm(grad_output, weight) in LinearDX.backward (:34-37)  -> a_t=0,b_t=1

@@ -40,10 +40,10 @@ def K():
 
 @pytest.mark.parametrize("layout", ["nt", "nn", "tn"])
 @pytest.mark.parametrize("shape", [(256, 256, 64), (512, 768, 256), (1024, 2304, 768), (2048, 1024, 4096)])
-@pytest.mark.parametrize("tile_cfg", [0, 1, 2, 3, 5, 6, 7, 8])
+@pytest.mark.parametrize("tile_cfg", [0, 1, 2, 3, 5, 7, 8])
 def test_gemm_layouts(K, layout, shape, tile_cfg):
 	M, N, Kd = shape
-	if tile_cfg in (1, 5, 6, 7) and (M % 256 or N % 256):
+	if tile_cfg in (1, 5, 7) and (M % 256 or N % 256):
 		pytest.skip("tile does not divide")
 	if tile_cfg == 8 and (layout == "tn" or N % 256):
 		pytest.skip("the 128x256 direct-to-LDS tile needs a k-contiguous A and N % 256 == 0")
@@ -75,10 +75,10 @@ def test_gemm_epilogues(K):
 		_close(acc, 3 * ref + 0.25, rel_fro=1e-5, rel_max=1e-5, what=f"f32 acc ks={ks}")
 
 
-@pytest.mark.parametrize("tile_cfg", [6, 7, 8])
+@pytest.mark.parametrize("tile_cfg", [7, 8])
 @pytest.mark.parametrize("layout", ["nt", "tn", "nn"])
 def test_gemm_direct_to_lds_epilogues_and_k_split(K, tile_cfg, layout):
-	"""The direct-to-LDS kernels (256x256 with 4 and 8 waves, 128x256): every epilogue, short K (1 and
+	"""The direct-to-LDS kernels (256x256 and 128x256 tiles): every epilogue, short K (1 and
 	2 slices: the loop's loads past the end of K), and the K split with fp32 atomics."""
 	if tile_cfg == 8 and layout == "tn":
 		pytest.skip("the 128x256 tile needs a k-contiguous A")
