@@ -83,7 +83,8 @@ def test_fbw_matches_oracle(kind):
 @pytest.mark.parametrize("kind", ["gpt", "llama"])
 def test_short_micro_batches_share_a_stage(kind):
 	"""Micro-batches of 3, 1 and 2 sequences on a stage sized for 3 (an uneven split of the batch,
-	elf/pipeline.py:497-503): each against the oracle, with a recompute of the short one, and the slot
+	elf/pipeline.py:497-503): each against the oracle, with a recompute of the 1-sequence one, an offload
+	round trip of the 2-sequence one, and the slot
 	of the short micro-batch reused by a full one in the next step."""
 	mb, sizes = 3, [3, 1, 2]
 	stage = _stage(kind)
@@ -98,9 +99,14 @@ def test_short_micro_batches_share_a_stage(kind):
 		blk.forward(m, **({"remat_strategy": (lambda name, module: name == "")} if m == 1 else {}))
 		blk.send_forward(m, dst=2)
 		assert_close(blk.sent_forward[m], ref.forward(m, xs[m]), f"{kind} y[{m}] ({n} sequences)")
+	blk.offload(2)  # the 2-sequence micro-batch goes to the pinned arena and comes back before its B
 	for m, n in enumerate(sizes):
 		blk.recv_backward(m, n, src=2)
+		if m == 2:
+			blk.prefetch(2)
 		blk.backward_inputs(m)
+		if m == 2:
+			blk.release(2)
 		blk.send_backward(m, dst=0)
 		assert_close(blk.sent_backward[m], ref.backward_inputs(m, dys[m]), f"{kind} dx[{m}] ({n} sequences)")
 		blk.backward_params(m)
