@@ -15,6 +15,11 @@ int elf_gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t 
 	                      (hipStream_t)stream);
 }
 
+int elf_gemm_act_bf16(int act, int M, int F, int K, const void* A, int64_t lda, const void* W, int64_t ldw,
+                      void* pre, int64_t ldpre, void* out, int64_t ldout, void* stream) {
+	return elf::gemm_act_bf16(act, M, F, K, A, lda, W, ldw, pre, ldpre, out, ldout, (hipStream_t)stream);
+}
+
 #define S_(x) ((hipStream_t)(x))
 int elf_norm_fwd(int kind, const void* x, const void* gamma, const void* beta, void* y, void* stats, int T, int d,
                  float eps, void* stream) {

@@ -340,7 +340,6 @@ int norm_bwd(int kind, const void* dy, const void* x, const void* gamma, const v
 // ------------------------------------------------------------------------------------------
 // Activations.  GELU is the exact (erf) form of nn.GELU():  y = 0.5 x (1 + erf(x / sqrt 2)).
 // SwiGLU: h = silu(g) * u with g = gu[:, :F], u = gu[:, F:].
-__device__ __forceinline__ float gelu_f(float x) { return 0.5f * x * (1.f + erff(x * 0.70710678118654752f)); }
 __device__ __forceinline__ float gelu_grad_f(float x) {
 	const float cdf = 0.5f * (1.f + erff(x * 0.70710678118654752f));
 	const float pdf = 0.3989422804014327f * __expf(-0.5f * x * x);
@@ -373,10 +372,7 @@ __global__ __launch_bounds__(256) void swiglu_fwd_kernel(const bf16_t* __restric
 		const int c8 = (int)(i - row * cpr) * 8;
 		Chunk g = load8(gu + row * 2 * F + c8), u = load8(gu + row * 2 * F + F + c8);
 #pragma unroll
-		for (int j = 0; j < 8; j++) {
-			const float sig = 1.f / (1.f + __expf(-g.v[j]));
-			g.v[j] = g.v[j] * sig * u.v[j];
-		}
+		for (int j = 0; j < 8; j++) g.v[j] = swiglu_f(g.v[j], u.v[j]);
 		store8(h + row * F + c8, g);
 	}
 }

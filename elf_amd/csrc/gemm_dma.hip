@@ -53,7 +53,8 @@ struct Args {
 	const bf16_t* B;
 	void* C;
 	const bf16_t* R;
-	int64_t lda, ldb, ldc, ldr;
+	bf16_t* C2;  // activation epilogues: the activated output
+	int64_t lda, ldb, ldc, ldr, ldc2;
 	int M, N, K;
 	int tiles_m, tiles_n;
 	int k_splits;    // K is split this many ways (fp32 atomics epilogue) for the last tail_tiles tiles
@@ -71,14 +72,18 @@ struct Args {
 // chunk swizzle of reduction-major ("T") tiles as a function of the k row
 __device__ __forceinline__ int t_swz(int k) { return ((k & 7) << 2) ^ (((k >> 3) & 1) << 1); }
 
-template <bool T, int LPO>
-__device__ __forceinline__ void lane_offsets(int wave, int lane, int64_t ld, uint32_t (&off)[LPO]) {
+// PAIRED (k-contiguous operands only): the 256 tile rows are not 256 consecutive operand rows but, for
+// each 128-row half, 64 consecutive rows followed by the 64 rows `pair_rows` further down — the gate and
+// up rows of the same 64 SwiGLU columns, which thereby land in one wave's accumulators.
+template <bool T, int LPO, bool PAIRED = false>
+__device__ __forceinline__ void lane_offsets(int wave, int lane, int64_t ld, uint32_t (&off)[LPO], int64_t pair_rows = 0) {
 #pragma unroll
 	for (int i = 0; i < LPO; i++) {
 		const int q = wave * LPO + i;  // which 1 KiB piece of the operand tile
 		if constexpr (!T) {
 			const int row = q * 8 + (lane >> 3), slot = lane & 7;
-			off[i] = (uint32_t)((row * ld + ((slot ^ ((row >> 1) & 7)) << 3)) * 2);
+			const int64_t grow = PAIRED ? (row >> 7) * 64 + (row & 63) + ((row >> 6) & 1) * pair_rows : row;
+			off[i] = (uint32_t)((grow * ld + ((slot ^ ((row >> 1) & 7)) << 3)) * 2);
 		} else {
 			const int krow = q * 2 + (lane >> 5), slot = lane & 31;
 			off[i] = (uint32_t)((krow * ld + ((slot ^ t_swz(krow)) << 3)) * 2);
@@ -122,6 +127,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	constexpr int BM = Sh::BM, A_BYTES = Sh::A_BYTES, STAGE_BYTES = Sh::STAGE_BYTES;
 	constexpr int LOADS_A = Sh::LOADS_A, LOADS_B = Sh::LOADS_B, LOADS_PER_STAGE = Sh::LOADS_PER_STAGE;
 	static_assert(BM == 256 || !AT, "reduction-major A tiles are laid out for 256 rows");
+	constexpr bool PAIRED = EPI == EPI_BF16_SWIGLU;
+	static_assert(!PAIRED || !BT, "the paired row order is defined for a k-contiguous B");
 	extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 	const int tid = threadIdx.x;
 	const int lane = tid & 63;
@@ -162,12 +169,13 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	if (nk <= 0) return;
 
 	const bf16_t* Ap = AT ? g.A + (int64_t)kt0 * BKS * g.lda + m0 : g.A + (int64_t)m0 * g.lda + (int64_t)kt0 * BKS;
-	const bf16_t* Bp = BT ? g.B + (int64_t)kt0 * BKS * g.ldb + n0 : g.B + (int64_t)n0 * g.ldb + (int64_t)kt0 * BKS;
+	// paired rows: tile column n0 of the (gate | up interleaved) product starts at operand row n0 / 2
+	const bf16_t* Bp = BT ? g.B + (int64_t)kt0 * BKS * g.ldb + n0 : g.B + (int64_t)(PAIRED ? n0 / 2 : n0) * g.ldb + (int64_t)kt0 * BKS;
 	const int64_t a_step = AT ? (int64_t)BKS * g.lda : BKS;
 	const int64_t b_step = BT ? (int64_t)BKS * g.ldb : BKS;
 	uint32_t aoff[LOADS_A], boff[LOADS_B];
 	lane_offsets<AT, LOADS_A>(wave, lane, g.lda, aoff);
-	lane_offsets<BT, LOADS_B>(wave, lane, g.ldb, boff);
+	lane_offsets<BT, LOADS_B, PAIRED>(wave, lane, g.ldb, boff, g.N / 2);
 
 	// this wave's first 1 KiB piece of each operand in stage 0
 	const uint32_t lds_a = lds_addr(smem) + wave * (LOADS_A * 1024);
@@ -310,7 +318,30 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 				for (int r = 0; r < 4; r++) ws[(ii * 16 + row_l + r) * PITCH + j * 16 + col_l] = acc[i * 2 + ii][j][r];
 		const int grow0 = m0 + wr * (RT * 32) + i * 32;
 		const int gcol0 = n0 + wc * 128;
-		if constexpr (EPI == EPI_BF16 || EPI == EPI_BF16_RESID) {
+		if constexpr (EPI == EPI_BF16_SWIGLU) {
+			// the strip's columns are 64 gate columns then the 64 up columns of the same outputs: both go to
+			// their places in C = [gate | up] (kept for the backward) and silu(gate) * up, computed from the
+			// rounded values exactly as a separate pass over C would, to C2
+			const int F = g.N / 2, cg0 = n0 / 2 + wc * 64;
+#pragma unroll
+			for (int it = 0; it < 4; it++) {
+				const int row = it * 8 + (lane >> 3), c8 = (lane & 7) * 8;
+				const float* w = ws + row * PITCH + c8;
+				const f32x4 g0 = *reinterpret_cast<const f32x4*>(w), g1 = *reinterpret_cast<const f32x4*>(w + 4);
+				const f32x4 u0 = *reinterpret_cast<const f32x4*>(w + 64), u1 = *reinterpret_cast<const f32x4*>(w + 68);
+				bf16x8 og, ou, oa;
+#pragma unroll
+				for (int t = 0; t < 8; t++) {
+					og[t] = (bf16_t)(t < 4 ? g0[t] : g1[t - 4]);
+					ou[t] = (bf16_t)(t < 4 ? u0[t] : u1[t - 4]);
+					oa[t] = (bf16_t)swiglu_f((float)og[t], (float)ou[t]);
+				}
+				bf16_t* c = reinterpret_cast<bf16_t*>(g.C) + (int64_t)(grow0 + row) * g.ldc + cg0 + c8;
+				*reinterpret_cast<bf16x8*>(c) = og;
+				*reinterpret_cast<bf16x8*>(c + F) = ou;
+				*reinterpret_cast<bf16x8*>(g.C2 + (int64_t)(grow0 + row) * g.ldc2 + cg0 + c8) = oa;
+			}
+		} else if constexpr (EPI == EPI_BF16 || EPI == EPI_BF16_RESID || EPI == EPI_BF16_GELU) {
 #pragma unroll
 			for (int it = 0; it < 8; it++) {
 				const int row = it * 4 + (lane >> 4), c8 = (lane & 15) * 8;
@@ -326,6 +357,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 #pragma unroll
 				for (int t = 0; t < 8; t++) o[t] = (bf16_t)v[t];
 				*reinterpret_cast<bf16x8*>(reinterpret_cast<bf16_t*>(g.C) + (int64_t)(grow0 + row) * g.ldc + gcol0 + c8) = o;
+				if constexpr (EPI == EPI_BF16_GELU) {
+					bf16x8 o2;
+#pragma unroll
+					for (int t = 0; t < 8; t++) o2[t] = (bf16_t)gelu_f((float)o[t]);
+					*reinterpret_cast<bf16x8*>(g.C2 + (int64_t)(grow0 + row) * g.ldc2 + gcol0 + c8) = o2;
+				}
 			}
 		} else {
 			if (EPI == EPI_F32_ACC && splits > 1) {
@@ -379,6 +416,10 @@ static int launch_epi(const Args& a, int epi, hipStream_t stream) {
 		case EPI_F32_ACC: return launch<NW, RT, AT, BT, EPI_F32_ACC>(a, stream);
 		case EPI_F32_STORE: return launch<NW, RT, AT, BT, EPI_F32_STORE>(a, stream);
 	}
+	if constexpr (!AT && !BT) {
+		if (epi == EPI_BF16_GELU) return launch<NW, RT, AT, BT, EPI_BF16_GELU>(a, stream);
+		if (epi == EPI_BF16_SWIGLU) return launch<NW, RT, AT, BT, EPI_BF16_SWIGLU>(a, stream);
+	}
 	set_error("gemm: unknown epilogue %d", epi);
 	return -1;
 }
@@ -387,12 +428,17 @@ static int launch_epi(const Args& a, int epi, hipStream_t stream) {
 
 // Arguments are validated by gemm_bf16() before it dispatches here.
 int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda, const void* B, int64_t ldb, void* C,
-                  int64_t ldc, int epi, const void* R, int64_t ldr, int k_splits, int tail_tiles, int bm, hipStream_t stream) {
+                  int64_t ldc, int epi, const void* R, int64_t ldr, int k_splits, int tail_tiles, int bm, hipStream_t stream,
+                  void* C2, int64_t ldc2) {
 	ELF_REQUIRE(bm == 256 || bm == 128, "gemm (dma tile): 256- or 128-row tiles");
 	ELF_REQUIRE(M % bm == 0 && N % dma::BN == 0 && K % dma::BKS == 0, "gemm (dma tile): M multiple of %d, N of 256 and K of 64 required", bm);
 	ELF_REQUIRE(bm == 256 || !a_t, "gemm (dma tile): 128-row tiles need a k-contiguous A");
 	const int ntiles = (M / bm) * (N / dma::BN);
-	dma::Args a{(const bf16_t*)A, (const bf16_t*)B, C, (const bf16_t*)R, lda, ldb, ldc, ldr, M, N, K, M / bm, N / dma::BN, k_splits < 1 ? 1 : k_splits,
+	const bool act = epi == EPI_BF16_GELU || epi == EPI_BF16_SWIGLU;
+	ELF_REQUIRE(!act || (C2 && !a_t && !b_t), "gemm (dma tile): activation epilogues need k-contiguous operands and a second output");
+	// the paired rows of the SwiGLU epilogue are addressed with 32-bit byte offsets from the tile's first row
+	ELF_REQUIRE(epi != EPI_BF16_SWIGLU || (int64_t)(N / 2 + 256) * ldb * 2 < (int64_t(1) << 31), "gemm (dma tile): weight too large for the paired-row epilogue");
+	dma::Args a{(const bf16_t*)A, (const bf16_t*)B, C, (const bf16_t*)R, (bf16_t*)C2, lda, ldb, ldc, ldr, ldc2, M, N, K, M / bm, N / dma::BN, k_splits < 1 ? 1 : k_splits,
 	            tail_tiles < 0 || tail_tiles > ntiles ? ntiles : tail_tiles};
 	if (epi != EPI_F32_ACC || a.k_splits == 1) a.k_splits = 1, a.tail_tiles = 0;
 	if (bm == 128) {

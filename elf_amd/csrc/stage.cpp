@@ -212,10 +212,8 @@ static int run_forward(Stage* s, MbState& m, const void* x, void* y, FwdMode mod
 		ELF_TRY(buf_alloc(s, bs, B_H2));
 		ELF_TRY(norm_fwd(norm_kind, bs.b[B_X2].p, p.w[P_NORM2_G], p.w[P_NORM2_B], bs.b[B_H2].p, bs.b[B_ST2].p, T, d, s->cfg.eps, st));
 		ELF_TRY(buf_alloc(s, bs, B_GU));
-		ELF_TRY(gemm_bf16(0, 0, T, s->ffn_in, d, bs.b[B_H2].p, d, p.w[P_W1], d, bs.b[B_GU].p, s->ffn_in, EPI_BF16, nullptr, 0, 0, 0, st));
 		ELF_TRY(buf_alloc(s, bs, B_A));
-		if (s->llama) ELF_TRY(swiglu_fwd(bs.b[B_GU].p, bs.b[B_A].p, T, F, st));
-		else ELF_TRY(gelu_fwd(bs.b[B_GU].p, bs.b[B_A].p, (int64_t)T * F, st));
+		ELF_TRY(gemm_act_bf16(s->llama ? ACT_SWIGLU : ACT_GELU, T, F, d, bs.b[B_H2].p, d, p.w[P_W1], d, bs.b[B_GU].p, s->ffn_in, bs.b[B_A].p, F, st));
 		void* yout;
 		if (i == nb - 1 && s->vocab_out) {
 			const int id = s->final_norm ? B_X : B_H1;

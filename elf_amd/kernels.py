@@ -49,6 +49,25 @@ def gemm(a, b, *, a_t=False, b_t=False, out=None, epilogue=EPI_BF16, residual=No
 	return out
 
 
+ACT_GELU, ACT_SWIGLU = 0, 1
+
+
+def gemm_act(a, w, act):
+	"""(pre, out): pre = a @ w.T; out = gelu(pre) (act 0) or silu(pre[:, :F]) * pre[:, F:] (act 1, w = [gate; up])."""
+	_need(a, torch.bfloat16, "gemm_act.a")
+	_need(w, torch.bfloat16, "gemm_act.w")
+	M, K = a.shape
+	N = w.shape[0]
+	if w.shape[1] != K:
+		raise _lib.ElfStageError(f"gemm_act: reduction sizes differ ({K} vs {w.shape[1]})")
+	F = N // 2 if act == ACT_SWIGLU else N
+	pre = torch.empty((M, N), dtype=torch.bfloat16, device=a.device)
+	out = torch.empty((M, F), dtype=torch.bfloat16, device=a.device)
+	rc = _lib.load().elf_gemm_act_bf16(act, M, F, K, _ptr(a), a.stride(0), _ptr(w), w.stride(0), _ptr(pre), N, _ptr(out), F, _stream())
+	_lib.check(rc, "elf_gemm_act_bf16")
+	return pre, out
+
+
 def norm_fwd(kind, x, gamma, beta=None, eps=1e-5):
 	_need(x, torch.bfloat16, "norm.x")
 	T, d = x.shape

@@ -183,6 +183,49 @@ def test_gelu_swiglu(K):
 	_close(K.swiglu_bwd(dh, gu), gur.grad, what="swiglu bwd")
 
 
+@pytest.mark.parametrize("act", ["gelu", "swiglu"])
+@pytest.mark.parametrize("shape", [(2048, 6144, 128), (1024, 4096, 192), (1536, 8192, 64), (320, 1024, 128)])
+def test_gemm_with_activation_epilogue(K, act, shape):
+	"""Up-projection with GELU / SwiGLU in the GEMM epilogue: against fp32 torch, and bit for bit against the
+	GEMM followed by the activation kernel.  Shapes: 256x256 tiles, 128x256 tiles, a single K slice, and
+	one the fused tiles do not cover (the library then runs the two kernels itself)."""
+	M, N, Kd = shape
+	A = _randn(M, Kd, seed=41)
+	W = _randn(N, Kd, seed=42, scale=0.12)
+	code = K.ACT_GELU if act == "gelu" else K.ACT_SWIGLU
+	pre, out = K.gemm_act(A, W, code)
+	ref_pre = A.float() @ W.float().t()
+	_close(pre, ref_pre, what="pre-activation")
+	p32 = pre.float()
+	if act == "gelu":
+		ref_out = torch.nn.functional.gelu(p32)
+		two = K.gelu_fwd(K.gemm(A, W))
+	else:
+		F = N // 2
+		ref_out = torch.nn.functional.silu(p32[:, :F]) * p32[:, F:]
+		two = K.swiglu_fwd(K.gemm(A, W))
+	_close(out, ref_out, what="activated")
+	assert torch.equal(pre, K.gemm(A, W)), "pre-activation differs from the plain GEMM"
+	assert torch.equal(out, two), "fused activation differs from the separate kernel"
+
+
+def test_gemm_with_activation_strided_outputs(K):
+	# outputs that are column slices of wider buffers, as a caller that packs activations would pass
+	from elf_amd import _lib
+
+	M, F, Kd = 1024, 2048, 128
+	A = _randn(M, Kd, seed=43)
+	W = _randn(2 * F, Kd, seed=44, scale=0.12)
+	pre = torch.zeros(M, 2 * F + 64, dtype=torch.bfloat16, device="cuda")
+	out = torch.zeros(M, F + 64, dtype=torch.bfloat16, device="cuda")
+	rc = _lib.load().elf_gemm_act_bf16(K.ACT_SWIGLU, M, F, Kd, A.data_ptr(), Kd, W.data_ptr(), Kd, pre.data_ptr(), pre.stride(0),
+	                                   out.data_ptr(), out.stride(0), torch.cuda.current_stream().cuda_stream)
+	_lib.check(rc, "elf_gemm_act_bf16")
+	p2, o2 = K.gemm_act(A, W, K.ACT_SWIGLU)
+	assert torch.equal(pre[:, : 2 * F], p2) and torch.equal(out[:, :F], o2)
+	assert pre[:, 2 * F :].abs().max().item() == 0 and out[:, F:].abs().max().item() == 0
+
+
 def _rope_ref(x, S, D, theta):
 	# x: [T, H, D] fp32; half-split rotation, angles in fp64
 	T = x.shape[0]
