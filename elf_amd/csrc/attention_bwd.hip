@@ -1,5 +1,6 @@
 // Attention backward kernels (see attention_common.h for the layout conventions).
 #include "attention_common.h"
+#include <type_traits>
 
 namespace elf {
 namespace attn {
@@ -39,13 +40,27 @@ struct AttnBwdArgs {
 	const bf16_t* dO;
 	const float* nlse2;  // -lse * log2(e)
 	const float* delta;
-	float* dq_acc;  // fp32 [T, Hq*D], zero-initialised by the caller side of the launcher
+	bf16_t* dq_part;  // per key tile partial dQ, see part_row0()
 	bf16_t* dk;
 	bf16_t* dv;
 	int64_t ldq, ldk, ldv, lddo, lddk, lddv;
 	int B, S, Hq, Hkv;
 	float scale;
 };
+
+// dQ partials.  Every 128-key tile contributes a [queries, Hq*D] partial dQ; the partials are written
+// with plain stores, each by exactly one workgroup, rounded to bf16 (like the P and dS operands of the
+// products they come from), and summed in fp32 in a fixed order by dq_reduce_kernel: no atomics, no
+// zero fill, and a result that does not depend on the order in which workgroups run.  (Adding the
+// tiles into one fp32 buffer with atomics costs a read-modify-write of a line that is never cache
+// resident per 32 lanes: 0.3 T lanes/s chip-wide, 0.68 of 1.81 ms at the Llama-3-8B shape.)
+// Layout per batch element: the slices of the key tiles one after the other; with a causal mask
+// slice kt only holds the queries q >= 128 kt, so it starts at row kt S - 128 kt (kt - 1) / 2 and
+// its row index is q - 128 kt.
+__host__ __device__ __forceinline__ int64_t part_row0(int kt, int S, bool causal) {
+	return causal ? (int64_t)kt * S - 64 * (int64_t)kt * (kt - 1) : (int64_t)kt * S;
+}
+__host__ __device__ __forceinline__ int64_t part_rows(int S, bool causal) { return part_row0(S / 128, S, causal); }
 
 // Tiles fetched straight into LDS (lds_dma.h) are unpadded; the 16-byte chunk index of a row is
 // XOR-swizzled with a function of the row chosen so that both access patterns are conflict
@@ -112,11 +127,9 @@ __device__ __forceinline__ bf16x8 ds_t_frag(const unsigned char* t, int k0, int 
 //   dV^T += dO^T P, dK^T += Q^T dS  (A operands: LDS transpose reads; B: P / dS from registers)
 // dS^T goes to LDS; after the next workgroup barrier each wave multiplies the whole 32x128 dS
 // by its slice of K (held in registers as B operands) to get its slice of the dQ tile.  That
-// product runs one tile behind, so a tile costs one barrier, and its atomic adds to the fp32
-// dQ accumulator are issued one more tile later, right after the barrier, because the
-// direct-to-LDS loads can only be awaited together with every other outstanding vector memory
-// operation of the wave.  The softmax scale of dK and dQ is applied by the epilogue / the
-// conversion kernel.  With a causal mask key tile kt meets 1 - kt/nkt of the query tiles, so
+// product runs one tile behind, so a tile costs one barrier; the slice goes to this key tile's
+// partial dQ buffer (bf16).  The softmax scale of dK and dQ is applied by the epilogue / the
+// reduction kernel.  With a causal mask key tile kt meets 1 - kt/nkt of the query tiles, so
 // a workgroup takes the tiles kt and nkt-1-kt one after the other: every workgroup then does
 // the same amount of work.
 template <int D, bool CAUSAL>
@@ -165,13 +178,13 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(AttnBwdArgs a) {
 #pragma unroll
 		for (int i = 0; i < 4; i++) *reinterpret_cast<u32x2*>(t + ds_t_offset(key_l, 8 * i + 4 * g)) = u32x2{0u, 0u};
 	};
-	// registers [r_lo, r_hi) of a dQ accumulator tile -> fp32 atomics (issued a few at a time between
-	// other work: a long burst backs up the memory pipeline and stalls the wave)
-	auto atomics = [&](float* tile, const f32x16& v, int r_lo, int r_hi) {
+	// registers [r_lo, r_hi) of a dQ accumulator tile -> the partial buffer (issued a few at a time
+	// between other work: a long burst backs up the memory pipeline and stalls the wave)
+	auto dq_out = [&](bf16_t* tile, const f32x16& v, int r_lo, int r_hi) {
 		if (!dq_wave) return;
 #pragma unroll
 		for (int r = 0; r < 16; r++)
-			if (r >= r_lo && r < r_hi) unsafeAtomicAdd(tile + ((r >> 2) * 8 + (r & 3)) * HqD + dq_lane, v[r]);
+			if (r >= r_lo && r < r_hi) tile[((r >> 2) * 8 + (r & 3)) * HqD + dq_lane] = (bf16_t)v[r];
 	};
 
 	const int n_pass = (CAUSAL && nkt - 1 - pair != pair) ? 2 : 1;
@@ -256,7 +269,9 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(AttnBwdArgs a) {
 
 		// position of the current tile; dq_prev_tile = where the dQ tile of iteration it-1 goes
 		int cur_h = hk * G, cur_qt = qt_first;
-		float* dq_prev_tile = a.dq_acc + (tok0 + qt_first * BQ) * HqD + cur_h * D;
+		// rows of this key tile's slice: first query of the slice = key0 (causal) or 0
+		bf16_t* const part = a.dq_part + ((int64_t)b * part_rows(a.S, CAUSAL) + part_row0(kt_idx, a.S, CAUSAL) - qt_first * BQ) * HqD;
+		bf16_t* dq_prev_tile = part + (int64_t)(qt_first * BQ) * HqD + cur_h * D;
 
 		for (int it = 0; it < n_iter; it++) {
 			if (it + 1 < n_iter) issue((it + 1) & 1);
@@ -299,7 +314,7 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(AttnBwdArgs a) {
 			__builtin_amdgcn_sched_barrier(0);
 #pragma unroll
 			for (int i = 0; i < NF; i++) bC[i] = TL::rows(sdO, 0, i, lane);
-			atomics(dq_prev_tile, dq, 0, 4);
+			dq_out(dq_prev_tile, dq, 0, 4);
 			__builtin_amdgcn_sched_barrier(0);
 			// dP = dO V^T on the matrix pipe while the vector pipe turns S into P
 #pragma unroll
@@ -312,18 +327,23 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(AttnBwdArgs a) {
 			// wholly after the tile gets P = 0 everywhere)
 			const int kq = wkey0 + kl - q0 - 4 * g;
 			float p[16];
+			auto softmax = [&](auto masked) {
 #pragma unroll
-			for (int r4 = 0; r4 < 4; r4++) {
-				const f32x4 l4 = *reinterpret_cast<const f32x4*>(sLse + r4 * 8 + 4 * g);
+				for (int r4 = 0; r4 < 4; r4++) {
+					const f32x4 l4 = *reinterpret_cast<const f32x4*>(sLse + r4 * 8 + 4 * g);
 #pragma unroll
-				for (int t = 0; t < 4; t++) {
-					float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(s[r4 * 4 + t], sc, l4[t]));
-					if (CAUSAL && r4 * 8 + t < kq) pr = 0.f;
-					p[r4 * 4 + t] = pr;
+					for (int t = 0; t < 4; t++) {
+						float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(s[r4 * 4 + t], sc, l4[t]));
+						if (decltype(masked)::value && r4 * 8 + t < kq) pr = 0.f;
+						p[r4 * 4 + t] = pr;
+					}
 				}
-			}
+			};
+			// only the tiles on the diagonal (the wave's last key lies after the tile's first query) need the mask
+			if (CAUSAL && wkey0 + 31 > q0) softmax(std::true_type{});
+			else softmax(std::false_type{});
 			const bf16x8 pf[2] = {pack8(p), pack8(p + 8)};
-			atomics(dq_prev_tile, dq, 4, 8);
+			dq_out(dq_prev_tile, dq, 4, 8);
 			__builtin_amdgcn_sched_barrier(0);
 			// dV^T[d][key] += dO^T[d][q] P[q][key] while the vector pipe forms dS = P (dP - delta)
 #pragma unroll
@@ -346,22 +366,25 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(AttnBwdArgs a) {
 				*reinterpret_cast<u32x2*>(sdS_cur + ds_t_offset(key_l, 16 * u + 4 * g)) = u32x2{w[0], w[1]};
 				*reinterpret_cast<u32x2*>(sdS_cur + ds_t_offset(key_l, 16 * u + 8 + 4 * g)) = u32x2{w[2], w[3]};
 			}
-			atomics(dq_prev_tile, dq, 8, 12);
+			dq_out(dq_prev_tile, dq, 8, 12);
 			__builtin_amdgcn_sched_barrier(0);
 			// dK^T[d][key] += Q^T[d][q] dS[q][key]
 #pragma unroll
 			for (int i = 0; i < NF; i++)
 				acc_dk[i % DT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bC[i], dsf[i / DT], acc_dk[i % DT], 0, 0, 0);
-			atomics(dq_prev_tile, dq, 12, 16);
-			dq_prev_tile = a.dq_acc + (tok0 + q0) * HqD + cur_h * D;
+			dq_out(dq_prev_tile, dq, 12, 16);
+			dq_prev_tile = part + (int64_t)q0 * HqD + cur_h * D;
 			if (++cur_qt == nqt_all) {
 				cur_qt = qt_first;
 				cur_h++;
 			}
-			wait_vmcnt<0>();
+			// the next tile's loads were issued before this step's 16 partial stores and vector memory
+			// operations complete in order: waiting until 16 are left waits for the loads only
+			if (dq_wave) wait_vmcnt<16>();
+			else wait_vmcnt<0>();
 			__syncthreads();  // the next tile is in LDS, dS^T of this tile is complete, everyone is done with this tile
 		}
-		// drain: dQ product and atomics of the last tile
+		// drain: dQ product and partial of the last tile
 		{
 			const unsigned char* sdS_prev = sdS + ((n_iter + 1) & 1) * DS_BYTES;
 			f32x16 dq;
@@ -370,7 +393,7 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(AttnBwdArgs a) {
 #pragma unroll
 			for (int i = 0; i < NQ; i++)
 				dq = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ds_t_frag(sdS_prev, i * 16, lane), ktf[i], dq, 0, 0, 0);
-			atomics(dq_prev_tile, dq, 0, 16);
+			dq_out(dq_prev_tile, dq, 0, 16);
 		}
 
 		// dK^T / dV^T accumulators: register r <-> d = dt*32 + (r/4)*8 + 4g + r%4, lane <-> key
@@ -393,26 +416,31 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(AttnBwdArgs a) {
 	}
 }
 
-// dq(bf16, row stride ld) = scale * dq_acc(fp32, contiguous [T, cols])
-__global__ __launch_bounds__(256) void cvt_f32_bf16_kernel(const float* __restrict__ src, bf16_t* __restrict__ dst, int64_t T,
-                                                           int cols, int64_t ld, float scale) {
-	const int cpr = cols / 4;
-	const int64_t n = T * cpr;
+// dq[b, q, :] (bf16, row stride ld) = scale * sum over the key tiles that meet q of their partial rows,
+// added in fp32 in ascending tile order; 8 columns (16 bytes) per thread.
+__global__ __launch_bounds__(256) void dq_reduce_kernel(const bf16_t* __restrict__ part, bf16_t* __restrict__ dq, int B, int S, int cols,
+                                                        int64_t ld, float scale, int causal) {
+	const int cpr = cols / 8;
+	const int64_t n = (int64_t)B * S * cpr;
+	const int nkt = S / 128;
+	const int64_t rows_b = part_rows(S, causal);
 	for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
 		const int64_t row = i / cpr;
-		const int c = (int)(i - row * cpr) * 4;
-		const f32x4 v = *reinterpret_cast<const f32x4*>(src + row * cols + c);
-		bf16x4 o;
+		const int c = (int)(i - row * cpr) * 8;
+		const int b = (int)(row / S), q = (int)(row - (int64_t)b * S);
+		const int ns = causal ? q / 128 + 1 : nkt;
+		float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+		const bf16_t* pb = part + (int64_t)b * rows_b * cols + c;
+#pragma unroll 4
+		for (int kt = 0; kt < ns; kt++) {
+			const bf16x8 v = *reinterpret_cast<const bf16x8*>(pb + (part_row0(kt, S, causal) + q - (causal ? 128 * kt : 0)) * cols);
 #pragma unroll
-		for (int t = 0; t < 4; t++) o[t] = (bf16_t)(v[t] * scale);
-		*reinterpret_cast<bf16x4*>(dst + row * ld + c) = o;
-	}
-}
-
-__global__ __launch_bounds__(256) void fill_zero_kernel(f32x4* __restrict__ p, int64_t n4) {
-	for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
-		f32x4 z = {0.f, 0.f, 0.f, 0.f};
-		p[i] = z;
+			for (int t = 0; t < 8; t++) acc[t] += (float)v[t];
+		}
+		bf16x8 o;
+#pragma unroll
+		for (int t = 0; t < 8; t++) o[t] = (bf16_t)(acc[t] * scale);
+		*reinterpret_cast<bf16x8*>(dq + row * ld + c) = o;
 	}
 }
 
@@ -434,9 +462,9 @@ int launch_bwd(const AttnBwdArgs& a, dim3 grid, hipStream_t stream) {
 
 using namespace attn;
 
-int64_t attn_bwd_workspace_bytes(int B, int S, int Hq, int D) {
-	// fp32 dQ accumulator + delta + scaled log-sum-exp
-	return (int64_t)B * S * Hq * D * 4 + 2 * (int64_t)B * S * Hq * 4;
+int64_t attn_bwd_workspace_bytes(int B, int S, int Hq, int D, int causal) {
+	// bf16 dQ partials of every key tile + delta + scaled log-sum-exp
+	return (int64_t)B * part_rows(S, causal != 0) * Hq * D * 2 + 2 * (int64_t)B * S * Hq * 4;
 }
 
 int attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* dO, const void* lse, void* dq,
@@ -454,18 +482,16 @@ int attn_bwd(const void* q, const void* k, const void* v, const void* o, const v
 	ELF_REQUIRE(((uintptr_t)o % 16) == 0 && ((uintptr_t)dO % 16) == 0, "attn_bwd: o and dO must be 16-byte aligned");
 	ProfScope prof(PROF_ATTN_BWD, (causal ? 4.0 : 8.0) * B * Hq * (double)S * S * D, stream);
 	const int64_t T = (int64_t)B * S;
-	float* dq_acc = (float*)workspace;
-	float* delta = dq_acc + T * Hq * D;
+	bf16_t* dq_part = (bf16_t*)workspace;
+	float* delta = (float*)(dq_part + (int64_t)B * part_rows(S, causal != 0) * Hq * D);
 	float* nlse2 = delta + T * Hq;
-	// zero the dQ accumulator with a fill kernel (memset nodes misbehave under graph replay)
-	hipLaunchKernelGGL(fill_zero_kernel, dim3(2048), dim3(256), 0, stream, (f32x4*)dq_acc, T * Hq * D / 4);
 	{
 		const int64_t rows = T * Hq, per_block = 256 / (D / 8);
 		const int64_t want = (rows + per_block - 1) / per_block;
 		hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)(want < 8192 ? want : 8192)), dim3(256), 0, stream, (const bf16_t*)dO,
 	                   (const bf16_t*)o, (const float*)lse, delta, nlse2, lddo, ldo, B, S, Hq, D);
 	}
-	AttnBwdArgs a{(const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, (const bf16_t*)dO, nlse2, delta, dq_acc,
+	AttnBwdArgs a{(const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, (const bf16_t*)dO, nlse2, delta, dq_part,
 	              (bf16_t*)dk, (bf16_t*)dv, ldq, ldk, ldv, lddo, lddk, lddv, B, S, Hq, Hkv, scale};
 	const int nkt = S / 128;
 	const dim3 grid((unsigned)((int64_t)B * Hkv * (causal ? (nkt + 1) / 2 : nkt))), block(256);
@@ -473,10 +499,10 @@ int attn_bwd(const void* q, const void* k, const void* v, const void* o, const v
 	if (D == 128) rc = causal ? launch_bwd<128, true>(a, grid, stream) : launch_bwd<128, false>(a, grid, stream);
 	else rc = causal ? launch_bwd<64, true>(a, grid, stream) : launch_bwd<64, false>(a, grid, stream);
 	if (rc) return rc;
-	const int64_t n4 = T * (Hq * D / 4);
-	const int64_t blocks = (n4 + 255) / 256;
-	hipLaunchKernelGGL(cvt_f32_bf16_kernel, dim3((unsigned)(blocks < 4096 ? blocks : 4096)), dim3(256), 0, stream, dq_acc,
-	                   (bf16_t*)dq, T, Hq * D, lddq, scale);
+	const int64_t n8 = T * (Hq * D / 8);
+	const int64_t blocks = (n8 + 255) / 256;
+	hipLaunchKernelGGL(dq_reduce_kernel, dim3((unsigned)(blocks < 16384 ? blocks : 16384)), dim3(256), 0, stream, dq_part, (bf16_t*)dq, B, S,
+	                   Hq * D, lddq, scale, causal);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
 }

@@ -17,8 +17,8 @@
 // Backward: one workgroup pass = 128 keys of one (batch, kv head); each wave owns 32 keys and
 // keeps their dK^T / dV^T accumulators in registers while the workgroup walks over the
 // query tiles (32 queries at a time) of every query head in the group; dS^T goes through LDS,
-// each wave multiplies it with its slice of K one tile later and adds the dQ tile to an fp32
-// buffer with atomics.
+// each wave multiplies it with its slice of K one tile later and stores its part of the key
+// tile's partial dQ; a second kernel adds the partials of all key tiles in a fixed order.
 #pragma once
 #include "common.h"
 #include "kernels.h"

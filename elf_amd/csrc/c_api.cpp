@@ -69,7 +69,7 @@ int elf_attn_fwd(const void* q, const void* k, const void* v, void* o, void* lse
                  int64_t ldo, int B, int S, int Hq, int Hkv, int D, int causal, float scale, void* stream) {
 	return elf::attn_fwd(q, k, v, o, lse, ldq, ldk, ldv, ldo, B, S, Hq, Hkv, D, causal, scale, S_(stream));
 }
-int64_t elf_attn_bwd_workspace_bytes(int B, int S, int Hq, int D) { return elf::attn_bwd_workspace_bytes(B, S, Hq, D); }
+int64_t elf_attn_bwd_workspace_bytes(int B, int S, int Hq, int D, int causal) { return elf::attn_bwd_workspace_bytes(B, S, Hq, D, causal); }
 int elf_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* dO, const void* lse, void* dq,
                  void* dk, void* dv, void* workspace, int64_t ldq, int64_t ldk, int64_t ldv, int64_t ldo, int64_t lddo,
                  int64_t lddq, int64_t lddk, int64_t lddv, int B, int S, int Hq, int Hkv, int D, int causal, float scale,

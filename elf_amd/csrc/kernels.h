@@ -61,7 +61,7 @@ int cross_entropy_reduce(const void* row_loss, const void* target, int64_t rows,
 // Attention over the packed projection layout; lse is [B, Hq, S] fp32 (natural log).
 int attn_fwd(const void* q, const void* k, const void* v, void* o, void* lse, int64_t ldq, int64_t ldk, int64_t ldv,
              int64_t ldo, int B, int S, int Hq, int Hkv, int D, int causal, float scale, hipStream_t stream);
-int64_t attn_bwd_workspace_bytes(int B, int S, int Hq, int D);
+int64_t attn_bwd_workspace_bytes(int B, int S, int Hq, int D, int causal);
 int attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* dO, const void* lse, void* dq,
              void* dk, void* dv, void* workspace, int64_t ldq, int64_t ldk, int64_t ldv, int64_t ldo, int64_t lddo,
              int64_t lddq, int64_t lddk, int64_t lddv, int B, int S, int Hq, int Hkv, int D, int causal, float scale,

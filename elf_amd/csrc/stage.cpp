@@ -518,7 +518,7 @@ int elf_stage_create(const elf_stage_cfg* cfg, elf_stage_t** out) {
 	if (hipStreamCreateWithFlags(&s->offload_stream, hipStreamNonBlocking) != hipSuccess) return fail("offload stream");
 	if (hipStreamCreateWithFlags(&s->prefetch_stream, hipStreamNonBlocking) != hipSuccess) return fail("prefetch stream");
 	if (hipMalloc((void**)&s->norm_ws, (size_t)norm_bwd_workspace_floats(s->T, s->d) * 4) != hipSuccess) return fail("norm workspace");
-	if (hipMalloc(&s->attn_ws, (size_t)attn_bwd_workspace_bytes(s->B, s->S, s->Hq, s->D)) != hipSuccess) return fail("attention workspace");
+	if (hipMalloc(&s->attn_ws, (size_t)attn_bwd_workspace_bytes(s->B, s->S, s->Hq, s->D, s->cfg.causal)) != hipSuccess) return fail("attention workspace");
 	if (hipMalloc((void**)&s->dummy_grad, (size_t)2 * s->d * 4) != hipSuccess) return fail("gradient sink");
 	if (hipMemset(s->dummy_grad, 0, (size_t)2 * s->d * 4) != hipSuccess) return fail("gradient sink clear");
 	if (s->llama) {

@@ -174,7 +174,7 @@ def attn_bwd(qkv, o, do, lse, B, S, Hq, Hkv, D, causal, scale=None):
 	T, ld = qkv.shape[0], qkv.stride(0)
 	scale = scale if scale is not None else 1.0 / math.sqrt(D)
 	lib = _lib.load()
-	ws = torch.empty(lib.elf_attn_bwd_workspace_bytes(B, S, Hq, D), dtype=torch.uint8, device=qkv.device)
+	ws = torch.empty(lib.elf_attn_bwd_workspace_bytes(B, S, Hq, D, int(causal)), dtype=torch.uint8, device=qkv.device)
 	dqkv = torch.empty_like(qkv)
 	q, k, v = qkv[:, : Hq * D], qkv[:, Hq * D : (Hq + Hkv) * D], qkv[:, (Hq + Hkv) * D :]
 	dq, dk, dv = dqkv[:, : Hq * D], dqkv[:, Hq * D : (Hq + Hkv) * D], dqkv[:, (Hq + Hkv) * D :]

@@ -122,11 +122,14 @@ int elf_cross_entropy_reduce(const void* row_loss, const void* target, int64_t r
  * D in {64, 128}, S % 128 == 0.  lse: fp32 [B, Hq, S] (natural log of the softmax denominator).
  * Replaces SDPA / softmax(QK^T*scale)V forward and its autograd backward
  * (benchmarks/models/simple.py:362-367, 379-386).  The backward needs
- * elf_attn_bwd_workspace_bytes() of 16-byte aligned scratch. */
+ * elf_attn_bwd_workspace_bytes() of 16-byte aligned scratch (the bf16 partial dQ of every 128-key tile,
+ * which a second kernel sums in fp32 in a fixed order — no atomics, run-to-run identical gradients —
+ * plus two fp32 values per query and head): B * S * (S/128 + 1) / 2 * Hq * D * 2 bytes with a causal
+ * mask, B * S * (S/128) * Hq * D * 2 without, + 8 * B * S * Hq. */
 int elf_attn_fwd(const void* q, const void* k, const void* v, void* o, void* lse, int64_t ldq,
                  int64_t ldk, int64_t ldv, int64_t ldo, int B, int S, int Hq, int Hkv, int D,
                  int causal, float scale, void* stream);
-int64_t elf_attn_bwd_workspace_bytes(int B, int S, int Hq, int D);
+int64_t elf_attn_bwd_workspace_bytes(int B, int S, int Hq, int D, int causal);
 int elf_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* dO,
                  const void* lse, void* dq, void* dk, void* dv, void* workspace, int64_t ldq,
                  int64_t ldk, int64_t ldv, int64_t ldo, int64_t lddo, int64_t lddq, int64_t lddk,

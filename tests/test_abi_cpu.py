@@ -56,7 +56,10 @@ def test_argument_errors_without_device(lib):
 	with pytest.raises(_lib.ElfStageError):
 		_lib.check(rc, "elf_norm_fwd")
 	assert lib.elf_norm_bwd_workspace_floats(8192, 4096) == 1024 * 2 * 4096
-	assert lib.elf_attn_bwd_workspace_bytes(2, 4096, 32, 128) == 2 * 4096 * 32 * 128 * 4 + 2 * (2 * 4096 * 32 * 4)
+	# bf16 dQ partials of the 32 key tiles (causal: tile kt only meets the queries from 128 kt on) + two floats per (token, head)
+	stats = 2 * (2 * 4096 * 32 * 4)
+	assert lib.elf_attn_bwd_workspace_bytes(2, 4096, 32, 128, 0) == 2 * (32 * 4096) * 32 * 128 * 2 + stats
+	assert lib.elf_attn_bwd_workspace_bytes(2, 4096, 32, 128, 1) == 2 * sum(4096 - 128 * kt for kt in range(32)) * 32 * 128 * 2 + stats
 
 
 def test_stage_create_rejects_bad_configs(lib):

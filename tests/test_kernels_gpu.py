@@ -304,3 +304,5 @@ def test_attention_fwd_bwd(K, cfg):
 	dqkv = K.attn_bwd(qkv, o, do, lse, B, S, Hq, Hkv, D, causal)
 	for name, sl in (("dq", slice(0, Hq * D)), ("dk", slice(Hq * D, (Hq + Hkv) * D)), ("dv", slice((Hq + Hkv) * D, None))):
 		_close(dqkv[:, sl], dqkv_ref[:, sl], rel_fro=1.5e-2, what=f"attn {name} {cfg}")
+	# no atomics anywhere in the backward: a second run gives the same bits
+	assert torch.equal(dqkv, K.attn_bwd(qkv, o, do, lse, B, S, Hq, Hkv, D, causal))
