@@ -34,10 +34,17 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnArgs a) {
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int g = lane >> 5, ql = lane & 31;
 	const int nqt = a.S / BQ;
-	// heaviest (last) query tiles first when causal
-	const int qt = CAUSAL ? (nqt - 1 - (int)(blockIdx.x % nqt)) : (int)(blockIdx.x % nqt);
-	const int bh = blockIdx.x / nqt;
-	const int h = bh % a.Hq, b = bh / a.Hq;
+	// Workgroup order: query tile by query tile over all (batch, head) pairs; causal: the heaviest (last)
+	// query tiles first, so that the workgroups that start last are the lightest ones (with the tiles
+	// of one head after the other, the last head's heaviest tile started when most of the grid was done
+	// and ran on alone for a third of the kernel's time).  Workgroups go to the 8 XCDs round-robin:
+	// index j within a batch element is mapped to head (j % 8) * (Hq / 8) + j / 8, so that an XCD works
+	// on a contiguous range of heads — the query heads that share a K/V head read it through one L2.
+	const int nbh = a.B * a.Hq;
+	const int qr = (int)(blockIdx.x / nbh), bj = (int)(blockIdx.x % nbh);
+	const int qt = CAUSAL ? nqt - 1 - qr : qr;
+	const int b = bj / a.Hq, j = bj % a.Hq;
+	const int h = a.Hq % 8 == 0 ? (j & 7) * (a.Hq >> 3) + (j >> 3) : j;
 	const int hk = h / (a.Hq / a.Hkv);
 	const int q0 = qt * BQ + wave * 32;  // first query (in sequence) of this wave
 	const int64_t tok0 = (int64_t)b * a.S;
