@@ -162,11 +162,18 @@ def main():
 		from elf_amd.scheduling.ilp import RematScheduler, profile_stage, solve_remat
 
 		stats, _ = profile_stage(block, n_iter=3)
+		# The budget is for everything this process holds on the device.  The ILP's memory model covers weights,
+		# fp32 gradient accumulators, the stage's fixed scratch (2 x Mparams) and the activations; what is resident
+		# beyond that comes off the budget it is given: the boundary tensors of all micro-batches (inputs and
+		# output gradients now, outputs and input gradients as the step produces them; a pipeline would pass them
+		# on one at a time) and the bf16 copies of the gradients that scale_grads leaves behind.
+		unmodelled_mib = max(0.0, torch.cuda.memory_allocated() / 2**20 + stats["Mworkspace"] - 2 * stats["Mparams"])
+		unmodelled_mib += w["n_mb"] * (stats["Minput"] + stats["Moutput"]) + sum(p.numel() * 2 for p in block._fused_w) / 2**20
 		t_ilp = time.perf_counter()
-		solution = solve_remat([stats] * len(placement), placement, SCHEDULERS[w["scheduler"]], w["n_mb"], w["memory_budget_mib"])
+		solution = solve_remat([stats] * len(placement), placement, SCHEDULERS[w["scheduler"]], w["n_mb"], w["memory_budget_mib"] - unmodelled_mib)
 		t_ilp = time.perf_counter() - t_ilp
 		remat = {
-			"memory_budget_mib": w["memory_budget_mib"], "ilp_seconds": t_ilp, "ilp_makespan_ms": solution["objective"],
+			"memory_budget_mib": w["memory_budget_mib"], "unmodelled_resident_mib": unmodelled_mib, "ilp_seconds": t_ilp, "ilp_makespan_ms": solution["objective"],
 			"ilp_peak_mib_rank": solution["peak_mems"][placement[BLOCK_ID]],
 			"decisions_block": {k: int(sum(solution[k][BLOCK_ID])) for k in ("full_fwd", "activations_bwd", "full_bwd")},
 			"profile": {k: stats[k] for k in ("T", "M", "Mpeak", "Mpeak_ckpt", "Mparams", "Mba", "Mbg", "Minput")},
@@ -241,7 +248,8 @@ def main():
 		             "kernel": "elf::dma::gemm_dma_kernel / elf::gemm_kernel (bf16 MFMA GEMM, all layouts)", "launches": g["launches"], "avg_launch_ms": g["avg_ms"]},
 		"stream_mfu": stream_flops(w) / (elapsed / args.steps) / (PEAK_BF16_TFLOPS * 1e12),
 		"kernels": per_kernel,
-		"peak_stage_memory_bytes": mem["peak_bytes"] + torch.cuda.max_memory_allocated(),
+		"peak_stage_memory_bytes": mem["peak_bytes"] + mem["workspace_bytes"] + torch.cuda.max_memory_allocated(),
+		"workspace_bytes": mem["workspace_bytes"],
 		"stash_peak_bytes": mem["peak_bytes"], "offload_d2h_bytes": mem["d2h_bytes"], "offload_h2d_bytes": mem["h2d_bytes"],
 	}
 	if remat is not None:

@@ -48,8 +48,8 @@ __device__ __forceinline__ float bf2f(bf16_t v) { return (float)v; }
 __device__ __forceinline__ bf16_t f2bf(float v) { return (bf16_t)v; }
 
 // 64-lane butterfly reductions (wavefront = 64 on CDNA).
-// MLP activations, shared by the activation kernels and the GEMM epilogues that fuse them so that both
-// give the same bits.  GELU is the exact (erf) form of nn.GELU(): 0.5 x (1 + erf(x / sqrt 2)).
+// MLP activations.  swiglu_f is shared by the activation kernel and the GEMM epilogue that fuses it, so
+// that both give the same bits.  GELU is the exact (erf) form of nn.GELU(): 0.5 x (1 + erf(x / sqrt 2)).
 __device__ __forceinline__ float gelu_f(float x) { return 0.5f * x * (1.f + erff(x * 0.70710678118654752f)); }
 __device__ __forceinline__ float swiglu_f(float g, float u) {
 	// hardware reciprocal (1 ulp): a correctly rounded division is ten more instructions per element, which

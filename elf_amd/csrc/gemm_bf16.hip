@@ -365,14 +365,14 @@ int gemm_act_bf16(int act, int M, int F, int K, const void* A, int64_t lda, cons
 	// the same tile choice as gemm_bf16 makes for this shape; the SwiGLU epilogue pairs 64 gate with 64 up
 	// columns per wave, so a 256-column tile covers 128 outputs
 	int bm = 0;
-	if (K % 64 == 0 && N % 256 == 0 && lda % 8 == 0 && ldw % 8 == 0 && ldpre >= N && ldout >= F && ldpre % 8 == 0 && ldout % 8 == 0 &&
+	if (act == ACT_SWIGLU && K % 64 == 0 && N % 256 == 0 && lda % 8 == 0 && ldw % 8 == 0 && ldpre >= N && ldout >= F && ldpre % 8 == 0 && ldout % 8 == 0 &&
 	    ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0 && ((uintptr_t)pre % 16) == 0 && ((uintptr_t)out % 16) == 0 && lda >= K && ldw >= K) {
 		if (M % 256 == 0 && (int64_t)(M / 256) * (N / 256) >= 192) bm = 256;
 		else if (M % 128 == 0 && (int64_t)(M / 128) * (N / 256) >= 128) bm = 128;
 	}
 	if (bm) {
 		ProfScope prof(PROF_GEMM, 2.0 * M * N * K, stream);
-		return gemm_bf16_dma(0, 0, M, N, K, A, lda, W, ldw, pre, ldpre, act == ACT_SWIGLU ? EPI_BF16_SWIGLU : EPI_BF16_GELU, nullptr, 0, 1, 0,
+		return gemm_bf16_dma(0, 0, M, N, K, A, lda, W, ldw, pre, ldpre, EPI_BF16_SWIGLU, nullptr, 0, 1, 0,
 		                     bm, stream, out, ldout);
 	}
 	ELF_REQUIRE(ldpre == N && ldout == F, "gemm_act: the unfused path needs dense outputs");

@@ -53,7 +53,7 @@ struct Args {
 	const bf16_t* B;
 	void* C;
 	const bf16_t* R;
-	bf16_t* C2;  // activation epilogues: the activated output
+	bf16_t* C2;  // SwiGLU epilogue: the activated output
 	int64_t lda, ldb, ldc, ldr, ldc2;
 	int M, N, K;
 	int tiles_m, tiles_n;
@@ -341,7 +341,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 				*reinterpret_cast<bf16x8*>(c + F) = ou;
 				*reinterpret_cast<bf16x8*>(g.C2 + (int64_t)(grow0 + row) * g.ldc2 + cg0 + c8) = oa;
 			}
-		} else if constexpr (EPI == EPI_BF16 || EPI == EPI_BF16_RESID || EPI == EPI_BF16_GELU) {
+		} else if constexpr (EPI == EPI_BF16 || EPI == EPI_BF16_RESID) {
 #pragma unroll
 			for (int it = 0; it < 8; it++) {
 				const int row = it * 4 + (lane >> 4), c8 = (lane & 15) * 8;
@@ -357,12 +357,6 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 #pragma unroll
 				for (int t = 0; t < 8; t++) o[t] = (bf16_t)v[t];
 				*reinterpret_cast<bf16x8*>(reinterpret_cast<bf16_t*>(g.C) + (int64_t)(grow0 + row) * g.ldc + gcol0 + c8) = o;
-				if constexpr (EPI == EPI_BF16_GELU) {
-					bf16x8 o2;
-#pragma unroll
-					for (int t = 0; t < 8; t++) o2[t] = (bf16_t)gelu_f((float)o[t]);
-					*reinterpret_cast<bf16x8*>(g.C2 + (int64_t)(grow0 + row) * g.ldc2 + gcol0 + c8) = o2;
-				}
 			}
 		} else {
 			if (EPI == EPI_F32_ACC && splits > 1) {
@@ -417,7 +411,6 @@ static int launch_epi(const Args& a, int epi, hipStream_t stream) {
 		case EPI_F32_STORE: return launch<NW, RT, AT, BT, EPI_F32_STORE>(a, stream);
 	}
 	if constexpr (!AT && !BT) {
-		if (epi == EPI_BF16_GELU) return launch<NW, RT, AT, BT, EPI_BF16_GELU>(a, stream);
 		if (epi == EPI_BF16_SWIGLU) return launch<NW, RT, AT, BT, EPI_BF16_SWIGLU>(a, stream);
 	}
 	set_error("gemm: unknown epilogue %d", epi);
@@ -434,8 +427,7 @@ int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t 
 	ELF_REQUIRE(M % bm == 0 && N % dma::BN == 0 && K % dma::BKS == 0, "gemm (dma tile): M multiple of %d, N of 256 and K of 64 required", bm);
 	ELF_REQUIRE(bm == 256 || !a_t, "gemm (dma tile): 128-row tiles need a k-contiguous A");
 	const int ntiles = (M / bm) * (N / dma::BN);
-	const bool act = epi == EPI_BF16_GELU || epi == EPI_BF16_SWIGLU;
-	ELF_REQUIRE(!act || (C2 && !a_t && !b_t), "gemm (dma tile): activation epilogues need k-contiguous operands and a second output");
+	ELF_REQUIRE(epi != EPI_BF16_SWIGLU || (C2 && !a_t && !b_t), "gemm (dma tile): the SwiGLU epilogue needs k-contiguous operands and a second output");
 	// the paired rows of the SwiGLU epilogue are addressed with 32-bit byte offsets from the tile's first row
 	ELF_REQUIRE(epi != EPI_BF16_SWIGLU || (int64_t)(N / 2 + 256) * ldb * 2 < (int64_t(1) << 31), "gemm (dma tile): weight too large for the paired-row epilogue");
 	dma::Args a{(const bf16_t*)A, (const bf16_t*)B, C, (const bf16_t*)R, (bf16_t*)C2, lda, ldb, ldc, ldr, ldc2, M, N, K, M / bm, N / dma::BN, k_splits < 1 ? 1 : k_splits,

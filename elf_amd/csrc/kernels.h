@@ -11,8 +11,7 @@ enum GemmEpilogue {
 	EPI_F32_ACC = 2,     // C(fp32) += acc
 	EPI_F32_STORE = 3,   // C(fp32) = acc
 	// direct-to-LDS tiles with k-contiguous operands only (see gemm_act_bf16):
-	EPI_BF16_GELU = 4,    // C(bf16) = acc, C2(bf16) = gelu(C)
-	EPI_BF16_SWIGLU = 5,  // B = [gate rows; up rows]: C(bf16) = acc = [g | u], C2(bf16) = silu(g) * u
+	EPI_BF16_SWIGLU = 4,  // B = [gate rows; up rows]: C(bf16) = acc = [g | u], C2(bf16) = silu(g) * u
 };
 
 int gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda, const void* B, int64_t ldb,
@@ -28,9 +27,10 @@ int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t 
 
 enum Activation { ACT_GELU = 0, ACT_SWIGLU = 1 };
 // Up-projection of the MLP with its activation: pre = A W^T (A [M, K], W [N, K], N = F for GELU and 2F =
-// [gate rows; up rows] for SwiGLU), out [M, F] = gelu(pre) or silu(pre[:, :F]) * pre[:, F:].  One kernel
-// (activation in the GEMM epilogue) when the shape fits the direct-to-LDS tiles, else the GEMM followed
-// by the activation kernel; both give the same bits.
+// [gate rows; up rows] for SwiGLU), out [M, F] = gelu(pre) or silu(pre[:, :F]) * pre[:, F:].  SwiGLU runs
+// as one kernel (activation in the GEMM epilogue) when the shape fits the direct-to-LDS tiles; otherwise,
+// and for GELU (whose erf costs as much in the epilogue as in a kernel of its own), the GEMM is followed
+// by the activation kernel.  Both ways give the same bits.
 int gemm_act_bf16(int act, int M, int F, int K, const void* A, int64_t lda, const void* W, int64_t ldw, void* pre,
                   int64_t ldpre, void* out, int64_t ldout, hipStream_t stream);
 

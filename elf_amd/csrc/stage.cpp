@@ -104,6 +104,7 @@ struct Stage {
 	void* rope_cs = nullptr;
 	float* norm_ws = nullptr;
 	void* attn_ws = nullptr;
+	int64_t ws_bytes = 0;  // fixed device workspaces of the stage (norm / attention backward scratch, rope table, gradient sink)
 	float* dummy_grad = nullptr;  // sink for norm weight gradients during gradient recompute
 	int64_t d2h_bytes = 0, h2d_bytes = 0;
 
@@ -517,12 +518,16 @@ int elf_stage_create(const elf_stage_cfg* cfg, elf_stage_t** out) {
 	};
 	if (hipStreamCreateWithFlags(&s->offload_stream, hipStreamNonBlocking) != hipSuccess) return fail("offload stream");
 	if (hipStreamCreateWithFlags(&s->prefetch_stream, hipStreamNonBlocking) != hipSuccess) return fail("prefetch stream");
-	if (hipMalloc((void**)&s->norm_ws, (size_t)norm_bwd_workspace_floats(s->T, s->d) * 4) != hipSuccess) return fail("norm workspace");
-	if (hipMalloc(&s->attn_ws, (size_t)attn_bwd_workspace_bytes(s->B, s->S, s->Hq, s->D, s->cfg.causal)) != hipSuccess) return fail("attention workspace");
+	const size_t norm_ws_bytes = (size_t)norm_bwd_workspace_floats(s->T, s->d) * 4;
+	const size_t attn_ws_bytes = (size_t)attn_bwd_workspace_bytes(s->B, s->S, s->Hq, s->D, s->cfg.causal);
+	const size_t rope_bytes = s->llama ? (size_t)s->S * (s->D / 2) * 8 : 0;
+	s->ws_bytes = (int64_t)(norm_ws_bytes + attn_ws_bytes + rope_bytes + (size_t)2 * s->d * 4);
+	if (hipMalloc((void**)&s->norm_ws, norm_ws_bytes) != hipSuccess) return fail("norm workspace");
+	if (hipMalloc(&s->attn_ws, attn_ws_bytes) != hipSuccess) return fail("attention workspace");
 	if (hipMalloc((void**)&s->dummy_grad, (size_t)2 * s->d * 4) != hipSuccess) return fail("gradient sink");
 	if (hipMemset(s->dummy_grad, 0, (size_t)2 * s->d * 4) != hipSuccess) return fail("gradient sink clear");
 	if (s->llama) {
-		if (hipMalloc(&s->rope_cs, (size_t)s->S * (s->D / 2) * 8) != hipSuccess) return fail("rope table");
+		if (hipMalloc(&s->rope_cs, rope_bytes) != hipSuccess) return fail("rope table");
 		if (rope_table(s->rope_cs, s->S, s->D, cfg->rope_theta, nullptr) != 0) return fail("rope table fill");
 		if (hipStreamSynchronize(nullptr) != hipSuccess) return fail("rope table sync");
 	}
@@ -739,6 +744,7 @@ int elf_stage_mem_stats(elf_stage_t* h, elf_mem_stats* out) {
 	out->pinned_bytes = s->pinned->size_bytes();
 	out->d2h_bytes = s->d2h_bytes;
 	out->h2d_bytes = s->h2d_bytes;
+	out->workspace_bytes = s->ws_bytes;
 	return 0;
 }
 

@@ -85,7 +85,7 @@ class StageConfig(ctypes.Structure):
 class MemStats(ctypes.Structure):
 	"""elf_mem_stats of include/elf_stage.h."""
 
-	_fields_ = [(n, ctypes.c_int64) for n in ("live_bytes", "peak_bytes", "reserved_bytes", "pinned_bytes", "d2h_bytes", "h2d_bytes")]
+	_fields_ = [(n, ctypes.c_int64) for n in ("live_bytes", "peak_bytes", "reserved_bytes", "pinned_bytes", "d2h_bytes", "h2d_bytes", "workspace_bytes")]
 
 
 _P = ctypes.c_void_p

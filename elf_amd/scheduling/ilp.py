@@ -51,8 +51,11 @@ def profile_stage(stage, sample_metadata=None, n_iter=10):
 	Mpeak_ckpt    the same for a forward that keeps nothing (whole-stage checkpoint)
 	Mba / Mbg     the two halves of the W stash after B: layer inputs / output gradients
 	Minput, Moutput  boundary tensor sizes;  Tcomm 0 (no transfers on one GPU)
-	Mparams       MiB of the bf16 weights x 1.5: the ILP charges 2 x Mparams per stage for weights +
-	              gradients, and this executor keeps bf16 weights plus fp32 accumulators (6 B/param)
+	Mparams       MiB of the bf16 weights x 1.5, plus half of Mworkspace: the ILP charges 2 x Mparams per
+	              stage for weights + gradients, this executor keeps bf16 weights plus fp32 accumulators
+	              (6 B/param), and the stage's fixed scratch is resident like they are
+	Mworkspace    MiB of fixed device scratch the stage allocated at creation (attention backward
+	              partials, norm backward partials, rope table)
 
 	Memory = bytes held by the stage library (stash + temporaries) + torch's allocator (boundary
 	tensors).  Returns ``(stats, next_stage_input)`` like the reference (warm-up output on the CPU).
@@ -165,7 +168,8 @@ def profile_stage(stage, sample_metadata=None, n_iter=10):
 
 	stats = {
 		"T": T, "M": M, "Mpeak": Mpeak, "Mpeak_ckpt": peak_ckpt,
-		"Mparams": 1.5 * sum(w.numel() * 2 for w in block._fused_w) / MiB,
+		"Mparams": 1.5 * sum(w.numel() * 2 for w in block._fused_w) / MiB + 0.5 * block.mem_stats()["workspace_bytes"] / MiB,
+		"Mworkspace": block.mem_stats()["workspace_bytes"] / MiB,
 		"Mba": mba, "Mbg": M["b"] - mba, "Minput": x.numel() * x.element_size() / MiB, "Moutput": dy.numel() * 2 / MiB, "Tcomm": 0.0,
 		"forward_remat_options": [], "backward_remat_options": [],
 	}

@@ -43,12 +43,12 @@ int elf_gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t 
                   int64_t ldb, void* C, int64_t ldc, int epilogue, const void* R, int64_t ldr,
                   int tile_cfg, int k_splits, void* stream);
 
-/* The MLP's up-projection with its activation in the GEMM epilogue (one kernel, the pre-activation never
- * re-read): pre = A W^T with A [M, K] and W [N, K], both k contiguous; act 0 (GELU): N = F,
- * out[M, F] = gelu(pre); act 1 (SwiGLU): N = 2F, W = [gate rows; up rows], pre[M, 2F] = [g | u],
- * out[M, F] = silu(g) * u.  pre is kept because the backward needs it.  Same bits as elf_gemm_bf16
- * (epilogue 0) followed by elf_gelu_fwd / elf_swiglu_fwd, which is also what runs for shapes the fused
- * tiles do not cover (M not a multiple of 128, N not of 256, or too few tiles to fill the chip).
+/* The MLP's up-projection with its activation: pre = A W^T with A [M, K] and W [N, K], both k contiguous;
+ * act 0 (GELU): N = F, out[M, F] = gelu(pre); act 1 (SwiGLU): N = 2F, W = [gate rows; up rows],
+ * pre[M, 2F] = [g | u], out[M, F] = silu(g) * u.  pre is kept because the backward needs it.  SwiGLU is
+ * computed in the GEMM epilogue (one kernel, the pre-activation never re-read); GELU, and shapes the
+ * fused tiles do not cover (M not a multiple of 128, N not of 256, or too few tiles to fill the chip),
+ * run elf_gemm_bf16 (epilogue 0) followed by elf_gelu_fwd / elf_swiglu_fwd.  Same bits either way.
  * Replaces: fc1 + nn.GELU() of the GPT block's MLP (benchmarks/models/simple.py:44-52) run through
  *           LinearDX.forward (elf/zb_utils.py:20); no reference module for SwiGLU. */
 int elf_gemm_act_bf16(int act, int M, int F, int K, const void* A, int64_t lda, const void* W, int64_t ldw,
@@ -195,6 +195,7 @@ typedef struct elf_mem_stats {
 	int64_t pinned_bytes;    /* size of the pinned-host arena */
 	int64_t d2h_bytes;       /* total bytes offloaded */
 	int64_t h2d_bytes;       /* total bytes brought back */
+	int64_t workspace_bytes; /* fixed device scratch allocated at create (attention / norm backward, rope table) */
 } elf_mem_stats;
 
 int elf_stage_create(const elf_stage_cfg* cfg, elf_stage_t** out);

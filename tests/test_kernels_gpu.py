@@ -186,9 +186,10 @@ def test_gelu_swiglu(K):
 @pytest.mark.parametrize("act", ["gelu", "swiglu"])
 @pytest.mark.parametrize("shape", [(2048, 6144, 128), (1024, 4096, 192), (1536, 8192, 64), (320, 1024, 128)])
 def test_gemm_with_activation_epilogue(K, act, shape):
-	"""Up-projection with GELU / SwiGLU in the GEMM epilogue: against fp32 torch, and bit for bit against the
-	GEMM followed by the activation kernel.  Shapes: 256x256 tiles, 128x256 tiles, a single K slice, and
-	one the fused tiles do not cover (the library then runs the two kernels itself)."""
+	"""Up-projection with its activation (SwiGLU: in the GEMM epilogue; GELU: GEMM + activation kernel
+	behind the same entry point): against fp32 torch, and bit for bit against the GEMM followed by the
+	activation kernel.  Shapes: 256x256 tiles, 128x256 tiles, a single K slice, and one the fused tiles
+	do not cover (the library then runs the two kernels itself)."""
 	M, N, Kd = shape
 	A = _randn(M, Kd, seed=41)
 	W = _randn(N, Kd, seed=42, scale=0.12)

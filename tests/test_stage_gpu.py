@@ -78,6 +78,12 @@ def test_fbw_matches_oracle(kind):
 	st = blk.mem_stats()
 	assert st["live_bytes"] == 0, "every stash must be gone after W"
 	assert st["peak_bytes"] > 0
+	# fixed scratch allocated at creation: at least the attention backward's workspace
+	from elf_amd import _lib
+
+	c = blk.cfg
+	attn_ws = _lib.load().elf_attn_bwd_workspace_bytes(c.mb, c.seq, c.n_heads, c.head_dim, int(c.causal))
+	assert attn_ws <= st["workspace_bytes"] <= attn_ws + (64 << 20)
 
 
 @pytest.mark.parametrize("kind", ["gpt", "llama"])
