@@ -214,6 +214,10 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(AttnBwdArgs a) {
 			for (int ks = 0; ks < NF; ks++) {
 				kf[ks] = *reinterpret_cast<const bf16x8*>(kp + ks * 16);
 				vf[ks] = *reinterpret_cast<const bf16x8*>(vp + ks * 16);
+				// the pass-long B operands live in the accumulator half of the register file (the matrix
+				// pipe reads them there directly): pinning them at their definition keeps the allocator from
+				// copying them into the vector half before every product
+				asm volatile("" : "+a"(kf[ks]), "+a"(vf[ks]));
 			}
 		}
 		f32x16 acc_dk[DT], acc_dv[DT];
