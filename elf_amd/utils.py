@@ -8,7 +8,13 @@ import torch.distributed as dist
 
 logger = logging.getLogger("utils")
 
-__all__ = ["Placement", "Timer", "TimerCPU", "TimerGPU"]
+__all__ = ["Placement", "TensorMetadata", "Timer", "TimerCPU", "TimerGPU", "WIRE_DTYPES"]
+
+# Position in this table = the dtype code on the wire (order of the reference's elf/utils.py:19-31).
+WIRE_DTYPES = (
+	torch.float16, torch.bfloat16, torch.float32, torch.float64, torch.int16, torch.int32, torch.int64,
+	torch.complex32, torch.complex64, torch.complex128, torch.bool,
+)
 
 
 class Placement(list):
@@ -50,6 +56,49 @@ class Placement(list):
 
 	def is_tail(self, rank):
 		return rank == self[-1]
+
+
+class TensorMetadata:
+	"""What a stage tells its neighbour about a boundary tensor before the first payload: a header of
+	MAX_SIZE fp32 values [dtype code, dim 0, dim 1, ..., 0 padding], the wire format of the reference's
+	elf/utils.py:150-220 (sent by block.py:552-568, received by :536-548).  The shape is that of one
+	sample (the sender describes ``value[0]``, block.py:577-584); ``get_buffer`` puts the batch
+	dimension back.  As in the reference a zero ends the shape when the header is decoded, so a
+	dimension of extent 0 (and everything after it) does not survive the round trip, and extents are
+	carried as fp32 (exact up to 2**24).  On one GPU no header travels: the boundary buffers are local;
+	the class is here so that a stage pair on two devices can speak the reference's format."""
+
+	MAX_SIZE = 16
+
+	def __init__(self, t):
+		self.shape = list(t.shape)
+		self.dtype = t.dtype
+		self.device = torch.cuda.current_device() if torch.cuda.is_available() else "cpu"
+
+	@staticmethod
+	def from_tensor(t):
+		"""Decode a received header."""
+		assert t.dim() == 1, "Metadata should only have one dimension"
+		fields = [int(v) for v in t.tolist()]
+		meta = TensorMetadata(torch.empty(0, dtype=WIRE_DTYPES[fields[0]]))
+		extents = fields[1:]
+		meta.shape = extents[: extents.index(0)] if 0 in extents else extents
+		return meta
+
+	def to_tensor(self):
+		"""Encode for sending.  More than MAX_SIZE - 1 dimensions do not fit (IndexError, as in the reference)."""
+		if len(self.shape) > self.MAX_SIZE - 1:
+			raise IndexError(f"TensorMetadata: {len(self.shape)} dimensions do not fit a header of {self.MAX_SIZE} values")
+		header = [float(WIRE_DTYPES.index(self.dtype))] + [float(e) for e in self.shape]
+		header += [0.0] * (self.MAX_SIZE - len(header))
+		return torch.tensor(header, dtype=torch.float32, device=self.device)
+
+	def get_buffer(self, batch_size):
+		"""An uninitialised tensor for ``batch_size`` samples of this description."""
+		return torch.empty((batch_size, *self.shape), dtype=self.dtype, device=self.device)
+
+	def __repr__(self):
+		return f"TensorMetadata({self.shape})"
 
 
 class TimerCPU:
