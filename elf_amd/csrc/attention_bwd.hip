@@ -164,7 +164,7 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(AttnBwdArgs a) {
 	const int dq_dt = wave % DT;
 	const int key_l = wave * 32 + kl;                        // this lane's key within the tile
 	const int nqt_all = a.S / BQ;
-	const int dq_lane = (4 * g) * (int)HqD + dq_dt * 32 + kl;  // lane part of a dQ tile address (elements)
+	const int dq_lane = kl * (int)HqD + dq_dt * 32 + 4 * g;  // lane part of a dQ tile address (elements): query kl, first of 4 columns
 
 	// DMA plan for one (Q, dO) tile pair: wave w moves rows [w*8, w*8+8) of each
 	uint32_t qoff[Q_LOADS], dooff[Q_LOADS];
@@ -178,13 +178,19 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(AttnBwdArgs a) {
 #pragma unroll
 		for (int i = 0; i < 4; i++) *reinterpret_cast<u32x2*>(t + ds_t_offset(key_l, 8 * i + 4 * g)) = u32x2{0u, 0u};
 	};
-	// registers [r_lo, r_hi) of a dQ accumulator tile -> the partial buffer (issued a few at a time
-	// between other work: a long burst backs up the memory pipeline and stalls the wave)
+	// registers [r_lo, r_hi) of a dQ^T accumulator tile -> the partial buffer.  The dQ product is computed
+	// transposed (rows d, columns q) so that a lane holds 4 consecutive columns of one query's row:
+	// four 8-byte stores per tile and lane (2-byte stores, one per register, cost 500 cycles more per tile)
 	auto dq_out = [&](bf16_t* tile, const f32x16& v, int r_lo, int r_hi) {
 		if (!dq_wave) return;
 #pragma unroll
-		for (int r = 0; r < 16; r++)
-			if (r >= r_lo && r < r_hi) tile[((r >> 2) * 8 + (r & 3)) * HqD + dq_lane] = (bf16_t)v[r];
+		for (int j = 0; j < 4; j++)
+			if (4 * j >= r_lo && 4 * j < r_hi) {
+				bf16x4 o;
+#pragma unroll
+				for (int t = 0; t < 4; t++) o[t] = (bf16_t)v[4 * j + t];
+				*reinterpret_cast<bf16x4*>(tile + dq_lane + 8 * j) = o;
+			}
 	};
 
 	const int n_pass = (CAUSAL && nkt - 1 - pair != pair) ? 2 : 1;
@@ -266,7 +272,7 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(AttnBwdArgs a) {
 		zero_ds(sdS + DS_BYTES);  // the "previous tile" of the first iteration
 		wait_vmcnt<0>();
 		__syncthreads();
-		// this wave's slice of K as B operands of the dQ product (n = d column, k = key)
+		// this wave's slice of K^T as A operands of the dQ^T product (rows d, k = key)
 		bf16x8 ktf[NQ];
 #pragma unroll
 		for (int i = 0; i < NQ; i++) ktf[i] = TL::template cols<false>(sKt, i * 16, dq_dt * 32, lane);
@@ -299,7 +305,7 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(AttnBwdArgs a) {
 				// dQ product of the previous tile, interleaved with S of this one
 #pragma unroll
 				for (int i = 0; i < NF; i++) {
-					dq = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bC[i], ktf[i], dq, 0, 0, 0);
+					dq = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktf[i], bC[i], dq, 0, 0, 0);
 					s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bA[i], kf[i], s, 0, 0, 0);
 				}
 			} else {
@@ -310,7 +316,7 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(AttnBwdArgs a) {
 #pragma unroll
 					for (int i = 0; i < NQ; i++) bD[i] = ds_t_frag(sdS_prev, i * 16, lane);
 #pragma unroll
-					for (int i = 0; i < NQ; i++) dq = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bD[i], ktf[i], dq, 0, 0, 0);
+					for (int i = 0; i < NQ; i++) dq = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktf[i], bD[i], dq, 0, 0, 0);
 				}
 #pragma unroll
 				for (int i = 0; i < NF; i++) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bA[i], kf[i], s, 0, 0, 0);
@@ -382,9 +388,9 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(AttnBwdArgs a) {
 				cur_qt = qt_first;
 				cur_h++;
 			}
-			// the next tile's loads were issued before this step's 16 partial stores and vector memory
-			// operations complete in order: waiting until 16 are left waits for the loads only
-			if (dq_wave) wait_vmcnt<16>();
+			// the next tile's loads were issued before this step's 4 partial stores and vector memory
+			// operations complete in order: waiting until 4 are left waits for the loads only
+			if (dq_wave) wait_vmcnt<4>();
 			else wait_vmcnt<0>();
 			__syncthreads();  // the next tile is in LDS, dS^T of this tile is complete, everyone is done with this tile
 		}
@@ -396,7 +402,7 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(AttnBwdArgs a) {
 			for (int r = 0; r < 16; r++) dq[r] = 0.f;
 #pragma unroll
 			for (int i = 0; i < NQ; i++)
-				dq = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ds_t_frag(sdS_prev, i * 16, lane), ktf[i], dq, 0, 0, 0);
+				dq = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktf[i], ds_t_frag(sdS_prev, i * 16, lane), dq, 0, 0, 0);
 			dq_out(dq_prev_tile, dq, 0, 16);
 		}
 
