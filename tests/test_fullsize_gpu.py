@@ -103,6 +103,37 @@ def test_attention_properties_at_full_size(K):
 	assert gh[:, p + 1:].abs().max().item() == 0.0
 
 
+def test_attention_one_kv_group_at_full_sequence_length(K):
+	"""One grouped-query group (4 query heads on 1 kv head) at the full sequence length, against fp32
+	torch: 32 key tiles per query row, so the backward sums the deepest stack of per-tile dQ partials
+	the benchmark shape has.  Tolerances of the small-shape kernel tests."""
+	import math
+
+	B, Hq, Hkv = 1, 4, 1
+	qkv = _randn(B * SEQ, (Hq + 2 * Hkv) * HD, seed=11)
+	do = _randn(B * SEQ, Hq * HD, seed=12)
+	x = qkv.float().requires_grad_(True)
+	q = x[:, : Hq * HD].reshape(SEQ, Hq, HD).transpose(0, 1)
+	k = x[:, Hq * HD : (Hq + 1) * HD].reshape(SEQ, 1, HD).transpose(0, 1)
+	v = x[:, (Hq + 1) * HD :].reshape(SEQ, 1, HD).transpose(0, 1)
+	s = (q @ k.transpose(-1, -2)) / math.sqrt(HD)
+	s = s.masked_fill(~torch.ones(SEQ, SEQ, dtype=torch.bool, device="cuda").tril(), float("-inf"))
+	o_ref = (torch.softmax(s, dim=-1) @ v).transpose(0, 1).reshape(SEQ, Hq * HD)
+	o_ref.backward(do.float())
+	o, lse = K.attn_fwd(qkv, B, SEQ, Hq, Hkv, HD, True)
+	g = K.attn_bwd(qkv, o, do, lse, B, SEQ, Hq, Hkv, HD, True).float()
+
+	def close(got, ref, what):
+		scale = ref.abs().max().item()
+		assert (got - ref).abs().max().item() <= 2e-2 * scale, what
+		assert ((got - ref).norm() / ref.norm()).item() <= 1.5e-2, what
+
+	close(o.float(), o_ref.detach(), "o")
+	close(g[:, : Hq * HD], x.grad[:, : Hq * HD], "dq")
+	close(g[:, Hq * HD : (Hq + 1) * HD], x.grad[:, Hq * HD : (Hq + 1) * HD], "dk")
+	close(g[:, (Hq + 1) * HD :], x.grad[:, (Hq + 1) * HD :], "dv")
+
+
 def test_bandwidth_kernels_at_full_size(K):
 	"""RMSNorm output has unit RMS under gamma = 1; SwiGLU of (g, u) with u = 1 is silu(g); RoPE
 	keeps the norm of every (x_i, x_{i+D/2}) pair and its backward undoes its forward; the gradient
