@@ -241,12 +241,16 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 #pragma unroll
 		for (int j = 0; j < 4; j++) fb[buf][j] = frag<BT>(sb, wc * 128 + (h * 4 + j) * 16, kq, lane);
 	};
+	// The wave raises its issue priority for the length of an MFMA cluster: of the two waves on a SIMD the one
+	// feeding the matrix pipe goes first and the other's fragment reads fill the gaps (+1 % on the stream).
 	auto mfmas = [&](int abuf, int bbuf, int h) {
+		__builtin_amdgcn_s_setprio(1);
 #pragma unroll
 		for (int i = 0; i < RF; i++)
 #pragma unroll
 			for (int j = 0; j < 4; j++)
 				acc[i][h * 4 + j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[abuf][i], fb[bbuf][j], acc[i][h * 4 + j], 0, 0, 0);
+		__builtin_amdgcn_s_setprio(0);
 	};
 
 	// The MFMAs of one half-step with half of this wave's loads of a slice (pieces PIECE0 ...) dealt evenly
@@ -254,6 +258,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	// issues them in one burst sits in the queue for ~1000 cycles with its MFMAs behind it.
 	auto mfmas_dma = [&](int abuf, int bbuf, auto hc, const SliceLoads& sl, auto piece0) {
 		constexpr int PIECE0 = decltype(piece0)::value, H = decltype(hc)::value, NM = RF * 4;
+		__builtin_amdgcn_s_setprio(1);
 		static_for<NM>([&](auto nc) {
 			constexpr int n = decltype(nc)::value, i = n / 4, j = n % 4;
 			acc[i][H * 4 + j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[abuf][i], fb[bbuf][j], acc[i][H * 4 + j], 0, 0, 0);
@@ -262,6 +267,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 				__builtin_amdgcn_sched_barrier(0);
 			}
 		});
+		__builtin_amdgcn_s_setprio(0);
 	};
 
 	load_a(0, 0, 0);
