@@ -8,8 +8,9 @@
 //   * a wave instruction fills 1 KiB of LDS contiguously, so tiles cannot be padded; bank
 //     conflicts are avoided by an XOR swizzle of the 16-byte chunk index, applied on the global
 //     side when choosing which chunk a lane fetches and undone when fragments are read;
-//   * the contraction runs on v_mfma_f32_16x16x32_bf16; each wave owns a 64x128 sub-tile (8 waves, two
-//     per SIMD, for the 256x256 tile; 4 waves for the 128x256 one).
+//   * the contraction runs on v_mfma_f32_16x16x32_bf16; the 256x256 tile is worked by four waves with
+//     128x128 sub-tiles (one per SIMD; k-contiguous A) or by eight with 64x128 sub-tiles (two per SIMD;
+//     both operands reduction-major), the 128x256 tile by four with 64x128 sub-tiles.
 // The DMA loads are issued through inline assembly: the compiler cannot see that they write
 // LDS, which is what allows partial vmcnt waits (its own tracking would force vmcnt(0) before
 // every LDS read).  Ordering is explicit: s_waitcnt vmcnt(n) for this wave's slice, then a
@@ -115,12 +116,27 @@ __device__ __forceinline__ bf16x8 frag(const unsigned char* base, int row0, int 
 	}
 }
 
+// NW = 4, RT = 4: 256x256 workgroup tile, one wave per SIMD with a 128x128 wave tile: 16 fragment reads per
+// k32 for 64 MFMAs, a third less LDS traffic per FLOP than the eight-wave shape, which on this power-limited
+// part is worth 2-4 % (forward and dX GEMMs).  It needs two things a lone wave does not forgive: all 256
+// accumulator registers are live, so the MFMAs are tied in place by hand (mfma_acc), and nothing else
+// fills issue gaps, so the next half-step's fragment reads and the slice's loads are dealt between the
+// MFMAs one at a time (half_step).  Left to the builtin and to bursts of reads it ran 12 % slower than
+// the eight-wave shape.
 // NW = 8, RT = 2: 256x256 workgroup tile, two waves per SIMD with 64x128 wave tiles (12 fragment reads per
-// k32 and 32 MFMAs); the two waves fill each other's issue gaps (every non-MFMA instruction of a lone
-// wave delays its MFMA stream by a few cycles) and barrier waits — a variant with one wave per SIMD and
-// 128x128 wave tiles reads a third less from LDS per FLOP and was 10-15 % slower.
+// k32 and 32 MFMAs); the two waves fill each other's issue gaps and barrier waits.  Used when both
+// operands are reduction-major (dW): each of their fragments costs two transpose reads and an address.
 // NW = 4, RT = 2: 128x256 workgroup tile for outputs with too few 256x256 tiles to fill the chip
 // (A must be k-contiguous: the reduction-major tile layout below assumes 256 rows).
+// acc += a b.  ASM: as one in-place instruction on accumulator registers — the builtin leaves source and
+// destination accumulators untied, and when all 256 accumulator registers are live (128x128 wave tiles) the
+// allocator then copies accumulator tiles around inside the loop (192 copies per K slice).
+template <bool ASM>
+__device__ __forceinline__ void mfma_acc(f32x4& acc, const bf16x8& a, const bf16x8& b) {
+	if constexpr (ASM) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+	else acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+}
+
 template <int NW, int RT, bool AT, bool BT, int EPI>
 __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	using Sh = Shape<NW, RT>;
@@ -270,12 +286,47 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 		__builtin_amdgcn_s_setprio(0);
 	};
 
+	// One wave per SIMD (NW = 4): nothing else fills the gaps, so the fragment reads of the next half-step
+	// are dealt between the MFMAs as well (one read per two MFMAs, B slabs first: they are needed first).
+	constexpr bool ONE_WAVE = NW == 4 && RT == 4;
+	auto half_step = [&](int abuf, int bbuf, auto hc, int pb_buf, int pb_step, int pb_kq, int pb_h, bool pa, int pa_buf, int pa_step, int pa_kq,
+	                     const SliceLoads& sl, auto piece0) {
+		constexpr int PIECE0 = decltype(piece0)::value, H = decltype(hc)::value, NM = RF * 4;
+		const unsigned char* sa = smem + (pa_step % NST) * STAGE_BYTES;
+		const unsigned char* sb = smem + (pb_step % NST) * STAGE_BYTES + A_BYTES;
+		static_for<NM>([&](auto nc) {
+			constexpr int n = decltype(nc)::value, i = n / 4, j = n % 4;
+			mfma_acc<true>(acc[i][H * 4 + j], fa[abuf][i], fb[bbuf][j]);
+			if constexpr (n % 2 == 1) {
+				constexpr int r = n / 2;
+				if constexpr (r < 4) fb[pb_buf][r] = frag<BT>(sb, wc * 128 + (pb_h * 4 + r) * 16, pb_kq, lane);
+				else if constexpr (r - 4 < RF) {
+					if (pa) fa[pa_buf][r - 4] = frag<AT>(sa, wr * (RT * 32) + (r - 4) * 16, pa_kq, lane);
+				}
+			}
+			if constexpr (PIECE0 >= 0 && (n + 1) * HALF / NM != n * HALF / NM) issue_piece(sl, std::integral_constant<int, (PIECE0 < 0 ? 0 : PIECE0) + n * HALF / NM>{});
+			__builtin_amdgcn_sched_barrier(0);
+		});
+	};
+
 	load_a(0, 0, 0);
 	load_b(0, 0, 0, 0);
 	for (int kt = 0; kt < nk; kt++) {
 		// where this iteration's loads go: scalar work, done here so that it overlaps the fragment reads
 		// instead of sitting between two MFMAs
 		const SliceLoads next1 = slice_loads(kt + 1), next2 = slice_loads(kt + 2);
+		if constexpr (ONE_WAVE) {
+			constexpr std::integral_constant<int, 0> H0{};
+			constexpr std::integral_constant<int, 1> H1{};
+			constexpr std::integral_constant<int, -1> NO_DMA{};
+			half_step(0, 0, H0, 1, kt, 0, 1, false, 0, kt, 0, next1, std::integral_constant<int, HALF>{});
+			half_step(0, 1, H1, 0, kt, 1, 0, true, 1, kt, 1, next1, NO_DMA);
+			half_step(1, 0, H0, 1, kt, 1, 1, false, 0, kt, 0, next1, NO_DMA);
+			wait_counters<0, 0>();  // vmcnt(0): slice kt+1 landed; lgkmcnt(0): slice kt fully read
+			__syncthreads();
+			half_step(1, 1, H1, 0, kt + 1, 0, 0, true, 0, kt + 1, 0, next2, std::integral_constant<int, 0>{});
+			continue;
+		}
 		// half-step (kq 0, h 0), with the second half of slice kt+1's loads
 		load_b(1, kt, 0, 1);
 		__builtin_amdgcn_sched_barrier(0);
@@ -443,8 +494,11 @@ int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t 
 		if (!b_t) return dma::launch_epi<4, 2, false, false>(a, epi, stream);
 		return dma::launch_epi<4, 2, false, true>(a, epi, stream);
 	}
-	if (!a_t && !b_t) return dma::launch_epi<8, 2, false, false>(a, epi, stream);
-	if (!a_t && b_t) return dma::launch_epi<8, 2, false, true>(a, epi, stream);
+	// k-contiguous A (forward, dX): four waves with 128x128 wave tiles; both operands reduction-major (dW): eight
+	// waves with 64x128 wave tiles (its transpose reads cost two LDS instructions and an address each, which a
+	// lone wave per SIMD does not hide: 3-7 % slower there)
+	if (!a_t && !b_t) return dma::launch_epi<4, 4, false, false>(a, epi, stream);
+	if (!a_t && b_t) return dma::launch_epi<4, 4, false, true>(a, epi, stream);
 	if (a_t && b_t) return dma::launch_epi<8, 2, true, true>(a, epi, stream);
 	set_error("gemm: layout A=T,B=R is not used by any stage contraction");
 	return -1;
