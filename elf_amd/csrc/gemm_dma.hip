@@ -127,7 +127,8 @@ __device__ __forceinline__ bf16x8 frag(const unsigned char* base, int row0, int 
 // k32 and 32 MFMAs); the two waves fill each other's issue gaps and barrier waits.  Used when both
 // operands are reduction-major (dW): each of their fragments costs two transpose reads and an address.
 // NW = 4, RT = 2: 128x256 workgroup tile for outputs with too few 256x256 tiles to fill the chip
-// (A must be k-contiguous: the reduction-major tile layout below assumes 256 rows).
+// (A must be k-contiguous: the reduction-major tile layout below assumes 256 rows).  One wave per SIMD
+// as well, so it runs the same interleaved loop (+35-40 % on the GPT-2-small shapes over read bursts).
 // acc += a b.  ASM: as one in-place instruction on accumulator registers — the builtin leaves source and
 // destination accumulators untied, and when all 256 accumulator registers are live (128x128 wave tiles) the
 // allocator then copies accumulator tiles around inside the loop (192 copies per K slice).
@@ -288,7 +289,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 
 	// One wave per SIMD (NW = 4): nothing else fills the gaps, so the fragment reads of the next half-step
 	// are dealt between the MFMAs as well (one read per two MFMAs, B slabs first: they are needed first).
-	constexpr bool ONE_WAVE = NW == 4 && RT == 4;
+	constexpr bool ONE_WAVE = NW == 4;
 	auto half_step = [&](int abuf, int bbuf, auto hc, int pb_buf, int pb_step, int pb_kq, int pb_h, bool pa, int pa_buf, int pa_step, int pa_kq,
 	                     const SliceLoads& sl, auto piece0) {
 		constexpr int PIECE0 = decltype(piece0)::value, H = decltype(hc)::value, NM = RF * 4;
