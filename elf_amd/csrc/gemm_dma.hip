@@ -116,6 +116,24 @@ __device__ __forceinline__ bf16x8 frag(const unsigned char* base, int row0, int 
 	}
 }
 
+// The two byte offsets (within the operand tile of stage 0, k32 half 0) that frag<true> reads for the
+// 16-row slab at row0, and the fragment read from them for k32 half kq of the tile at `base`.
+__device__ __forceinline__ void frag_t_offsets(int row0, int lane, uint32_t (&o)[2]) {
+	const int j = lane & 15;
+	const int m = row0 + 4 * (j & 3);
+	const int kk = 8 * (lane >> 4) + (j >> 2);
+	o[0] = (uint32_t)(kk * 512 + (((m >> 3) ^ t_swz(kk)) << 4) + (j & 1) * 8);
+	o[1] = (uint32_t)((kk + 4) * 512 + (((m >> 3) ^ t_swz(kk + 4)) << 4) + (j & 1) * 8);
+}
+// o: LDS byte addresses; imm: a compile-time byte offset (stage and k32 half) that ends up in the
+// instructions' offset fields.  t_swz only looks at k % 16, so the second k32 half of a tile lies 32 rows
+// of 512 bytes further on.
+__device__ __forceinline__ bf16x8 frag_t_at(const uint32_t (&o)[2], uint32_t imm) {
+	s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 ELF_LDS*)(uintptr_t)(o[0] + imm));
+	s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 ELF_LDS*)(uintptr_t)(o[1] + imm));
+	return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+}
+
 // NW = 4, RT = 4: 256x256 workgroup tile, one wave per SIMD with a 128x128 wave tile: 16 fragment reads per
 // k32 for 64 MFMAs, a third less LDS traffic per FLOP than the eight-wave shape, which on this power-limited
 // part is worth 2-4 % (forward and dX GEMMs).  It needs two things a lone wave does not forgive: all 256
@@ -196,7 +214,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 
 	// this wave's first 1 KiB piece of each operand in stage 0
 	const uint32_t lds_a = lds_addr(smem) + wave * (LOADS_A * 1024);
-	const uint32_t lds_b = lds_addr(smem) + A_BYTES + wave * (LOADS_B * 1024);
+	const uint32_t lds_b = lds_addr(smem) + NST * A_BYTES + wave * (LOADS_B * 1024);
 
 	// Loads of one K slice: its operand pointers and the LDS addresses of this wave's first piece of
 	// each operand in the slice's stage.  Piece P (compile-time) is one wave instruction filling 1 KiB;
@@ -212,8 +230,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	auto slice_loads = [&](int step) {
 		const bool ok = step < nk;
 		const int sc = ok ? step : nk - 1;
-		const uint32_t st = (uint32_t)(sc & 1) * STAGE_BYTES;
-		return SliceLoads{Ap + (int64_t)sc * a_step, Bp + (int64_t)sc * b_step, ok ? lds_a + st : lds_dummy, ok ? lds_b + st : lds_dummy};
+		const uint32_t st = (uint32_t)(sc & 1);
+		return SliceLoads{Ap + (int64_t)sc * a_step, Bp + (int64_t)sc * b_step, ok ? lds_a + st * A_BYTES : lds_dummy, ok ? lds_b + st * B_BYTES : lds_dummy};
 	};
 	auto issue_piece = [&](const SliceLoads& sl, auto pc) {
 		constexpr int P = decltype(pc)::value;
@@ -249,12 +267,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 
 	bf16x8 fa[2][RF], fb[2][4];
 	auto load_a = [&](int buf, int step, int kq) {
-		const unsigned char* sa = smem + (step % NST) * STAGE_BYTES;
+		const unsigned char* sa = smem + (step % NST) * A_BYTES;
 #pragma unroll
 		for (int i = 0; i < RF; i++) fa[buf][i] = frag<AT>(sa, wr * (RT * 32) + i * 16, kq, lane);
 	};
 	auto load_b = [&](int buf, int step, int kq, int h) {
-		const unsigned char* sb = smem + (step % NST) * STAGE_BYTES + A_BYTES;
+		const unsigned char* sb = smem + NST * A_BYTES + (step % NST) * B_BYTES;
 #pragma unroll
 		for (int j = 0; j < 4; j++) fb[buf][j] = frag<BT>(sb, wc * 128 + (h * 4 + j) * 16, kq, lane);
 	};
@@ -290,69 +308,110 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	// One wave per SIMD (NW = 4): nothing else fills the gaps, so the fragment reads of the next half-step
 	// are dealt between the MFMAs as well (one read per two MFMAs, B slabs first: they are needed first).
 	constexpr bool ONE_WAVE = NW == 4;
-	auto half_step = [&](int abuf, int bbuf, auto hc, int pb_buf, int pb_step, int pb_kq, int pb_h, bool pa, int pa_buf, int pa_step, int pa_kq,
+	// Reduction-major operands in this loop: the two transpose-read addresses of every fragment are computed
+	// once (k32 half 0 of stage 0); the k32 half and the stage are compile-time here (the loop is unrolled
+	// by two slices) and go into the instructions' offset fields, so the loop has no address arithmetic.
+	uint32_t ta[AT && ONE_WAVE ? RF : 1][2], tb[BT && ONE_WAVE ? 8 : 1][2];
+	if constexpr (ONE_WAVE) {
+		if constexpr (AT)
+#pragma unroll
+			for (int i = 0; i < RF; i++) {
+				frag_t_offsets(wr * (RT * 32) + i * 16, lane, ta[i]);
+				ta[i][0] += lds_addr(smem), ta[i][1] += lds_addr(smem);
+				// opaque from here on: folded into these, the tile's base would push the loop's offsets past 16 bits
+				asm volatile("" : "+v"(ta[i][0]), "+v"(ta[i][1]));
+			}
+		if constexpr (BT)
+#pragma unroll
+			for (int i = 0; i < 8; i++) {
+				frag_t_offsets(wc * 128 + i * 16, lane, tb[i]);
+				tb[i][0] += lds_addr(smem) + NST * A_BYTES, tb[i][1] += lds_addr(smem) + NST * A_BYTES;
+				asm volatile("" : "+v"(tb[i][0]), "+v"(tb[i][1]));
+			}
+	}
+	auto half_step = [&](int abuf, int bbuf, auto hc, int pb_buf, auto pb_stage, int pb_kq, int pb_h, bool pa, int pa_buf, auto pa_stage, int pa_kq,
 	                     const SliceLoads& sl, auto piece0) {
 		constexpr int PIECE0 = decltype(piece0)::value, H = decltype(hc)::value, NM = RF * 4;
-		const unsigned char* sa = smem + (pa_step % NST) * STAGE_BYTES;
-		const unsigned char* sb = smem + (pb_step % NST) * STAGE_BYTES + A_BYTES;
+		constexpr int SA = decltype(pa_stage)::value, SB = decltype(pb_stage)::value;
+		const unsigned char* sa = smem + SA * A_BYTES;
+		const unsigned char* sb = smem + NST * A_BYTES + SB * B_BYTES;
 		static_for<NM>([&](auto nc) {
 			constexpr int n = decltype(nc)::value, i = n / 4, j = n % 4;
 			mfma_acc<true>(acc[i][H * 4 + j], fa[abuf][i], fb[bbuf][j]);
 			if constexpr (n % 2 == 1) {
 				constexpr int r = n / 2;
-				if constexpr (r < 4) fb[pb_buf][r] = frag<BT>(sb, wc * 128 + (pb_h * 4 + r) * 16, pb_kq, lane);
-				else if constexpr (r - 4 < RF) {
-					if (pa) fa[pa_buf][r - 4] = frag<AT>(sa, wr * (RT * 32) + (r - 4) * 16, pa_kq, lane);
+				if constexpr (r < 4) {
+					if constexpr (BT) fb[pb_buf][r] = frag_t_at(tb[pb_h * 4 + r], (uint32_t)(SB * B_BYTES + pb_kq * (32 * 512)));
+					else fb[pb_buf][r] = frag<BT>(sb, wc * 128 + (pb_h * 4 + r) * 16, pb_kq, lane);
+				} else if constexpr (r - 4 < RF) {
+					if (pa) {
+						if constexpr (AT) fa[pa_buf][r - 4] = frag_t_at(ta[r - 4], (uint32_t)(SA * A_BYTES + pa_kq * (32 * 512)));
+						else fa[pa_buf][r - 4] = frag<AT>(sa, wr * (RT * 32) + (r - 4) * 16, pa_kq, lane);
+					}
 				}
 			}
 			if constexpr (PIECE0 >= 0 && (n + 1) * HALF / NM != n * HALF / NM) issue_piece(sl, std::integral_constant<int, (PIECE0 < 0 ? 0 : PIECE0) + n * HALF / NM>{});
 			__builtin_amdgcn_sched_barrier(0);
 		});
 	};
+	// one K slice held in stage S; the next one's fragments come from stage 1 - S
+	auto slice_one_wave = [&](auto sc, int kt) {
+		constexpr int S = decltype(sc)::value;
+		constexpr std::integral_constant<int, S> CUR{};
+		constexpr std::integral_constant<int, 1 - S> NXT{};
+		constexpr std::integral_constant<int, 0> H0{};
+		constexpr std::integral_constant<int, 1> H1{};
+		constexpr std::integral_constant<int, -1> NO_DMA{};
+		// where this slice's loads go: scalar work
+		const SliceLoads next1 = slice_loads(kt + 1), next2 = slice_loads(kt + 2);
+		half_step(0, 0, H0, 1, CUR, 0, 1, false, 0, CUR, 0, next1, std::integral_constant<int, HALF>{});
+		half_step(0, 1, H1, 0, CUR, 1, 0, true, 1, CUR, 1, next1, NO_DMA);
+		half_step(1, 0, H0, 1, CUR, 1, 1, false, 0, CUR, 0, next1, NO_DMA);
+		wait_counters<0, 0>();  // vmcnt(0): slice kt+1 landed; lgkmcnt(0): slice kt fully read
+		__syncthreads();
+		// with the first half of slice kt+2's loads into the stage the barrier just freed; past the end the
+		// fragment reads hit a stale stage and their values are unused
+		half_step(1, 1, H1, 0, NXT, 0, 0, true, 0, NXT, 0, next2, std::integral_constant<int, 0>{});
+	};
 
 	load_a(0, 0, 0);
 	load_b(0, 0, 0, 0);
-	for (int kt = 0; kt < nk; kt++) {
-		// where this iteration's loads go: scalar work, done here so that it overlaps the fragment reads
-		// instead of sitting between two MFMAs
-		const SliceLoads next1 = slice_loads(kt + 1), next2 = slice_loads(kt + 2);
-		if constexpr (ONE_WAVE) {
-			constexpr std::integral_constant<int, 0> H0{};
-			constexpr std::integral_constant<int, 1> H1{};
-			constexpr std::integral_constant<int, -1> NO_DMA{};
-			half_step(0, 0, H0, 1, kt, 0, 1, false, 0, kt, 0, next1, std::integral_constant<int, HALF>{});
-			half_step(0, 1, H1, 0, kt, 1, 0, true, 1, kt, 1, next1, NO_DMA);
-			half_step(1, 0, H0, 1, kt, 1, 1, false, 0, kt, 0, next1, NO_DMA);
+	if constexpr (ONE_WAVE) {
+		for (int kt = 0; kt < nk; kt += 2) {
+			slice_one_wave(std::integral_constant<int, 0>{}, kt);
+			if (kt + 1 < nk) slice_one_wave(std::integral_constant<int, 1>{}, kt + 1);
+		}
+	} else {
+		for (int kt = 0; kt < nk; kt++) {
+			// where this iteration's loads go: scalar work, done here so that it overlaps the fragment reads
+			// instead of sitting between two MFMAs
+			const SliceLoads next1 = slice_loads(kt + 1), next2 = slice_loads(kt + 2);
+			// half-step (kq 0, h 0), with the second half of slice kt+1's loads
+			load_b(1, kt, 0, 1);
+			__builtin_amdgcn_sched_barrier(0);
+			mfmas_dma(0, 0, std::integral_constant<int, 0>{}, next1, std::integral_constant<int, HALF>{});
+			__builtin_amdgcn_sched_barrier(0);
+			// (kq 0, h 1)
+			load_a(1, kt, 1);
+			load_b(0, kt, 1, 0);
+			__builtin_amdgcn_sched_barrier(0);
+			mfmas(0, 1, 1);
+			__builtin_amdgcn_sched_barrier(0);
+			// (kq 1, h 0)
+			load_b(1, kt, 1, 1);
+			__builtin_amdgcn_sched_barrier(0);
+			mfmas(1, 0, 0);
+			__builtin_amdgcn_sched_barrier(0);
 			wait_counters<0, 0>();  // vmcnt(0): slice kt+1 landed; lgkmcnt(0): slice kt fully read
 			__syncthreads();
-			half_step(1, 1, H1, 0, kt + 1, 0, 0, true, 0, kt + 1, 0, next2, std::integral_constant<int, 0>{});
-			continue;
+			// (kq 1, h 1), with the first half of slice kt+2's loads into the stage the barrier just freed;
+			// past the end the fragment reads hit a stale stage and their values are unused
+			load_a(0, kt + 1, 0);
+			load_b(0, kt + 1, 0, 0);
+			__builtin_amdgcn_sched_barrier(0);
+			mfmas_dma(1, 1, std::integral_constant<int, 1>{}, next2, std::integral_constant<int, 0>{});
+			__builtin_amdgcn_sched_barrier(0);
 		}
-		// half-step (kq 0, h 0), with the second half of slice kt+1's loads
-		load_b(1, kt, 0, 1);
-		__builtin_amdgcn_sched_barrier(0);
-		mfmas_dma(0, 0, std::integral_constant<int, 0>{}, next1, std::integral_constant<int, HALF>{});
-		__builtin_amdgcn_sched_barrier(0);
-		// (kq 0, h 1)
-		load_a(1, kt, 1);
-		load_b(0, kt, 1, 0);
-		__builtin_amdgcn_sched_barrier(0);
-		mfmas(0, 1, 1);
-		__builtin_amdgcn_sched_barrier(0);
-		// (kq 1, h 0)
-		load_b(1, kt, 1, 1);
-		__builtin_amdgcn_sched_barrier(0);
-		mfmas(1, 0, 0);
-		__builtin_amdgcn_sched_barrier(0);
-		wait_counters<0, 0>();  // vmcnt(0): slice kt+1 landed; lgkmcnt(0): slice kt fully read
-		__syncthreads();
-		// (kq 1, h 1), with the first half of slice kt+2's loads into the stage the barrier just freed;
-		// past the end the fragment reads hit a stale stage and their values are unused
-		load_a(0, kt + 1, 0);
-		load_b(0, kt + 1, 0, 0);
-		__builtin_amdgcn_sched_barrier(0);
-		mfmas_dma(1, 1, std::integral_constant<int, 1>{}, next2, std::integral_constant<int, 0>{});
-		__builtin_amdgcn_sched_barrier(0);
 	}
 
 	// Epilogue through LDS (free once every wave has left the main loop).  Register r of a 16x16
@@ -496,8 +555,8 @@ int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t 
 		return dma::launch_epi<4, 2, false, true>(a, epi, stream);
 	}
 	// k-contiguous A (forward, dX): four waves with 128x128 wave tiles; both operands reduction-major (dW): eight
-	// waves with 64x128 wave tiles (its transpose reads cost two LDS instructions and an address each, which a
-	// lone wave per SIMD does not hide: 3-7 % slower there)
+	// waves with 64x128 wave tiles (with two transpose reads per fragment on both operands the lone wave wins on
+	// some shapes by 2-3 % and loses on most by 1-10 %)
 	if (!a_t && !b_t) return dma::launch_epi<4, 4, false, false>(a, epi, stream);
 	if (!a_t && b_t) return dma::launch_epi<4, 4, false, true>(a, epi, stream);
 	if (a_t && b_t) return dma::launch_epi<8, 2, true, true>(a, epi, stream);
