@@ -147,13 +147,13 @@ __device__ __forceinline__ bf16x8 frag_t_at(const uint32_t (&o)[2], uint32_t imm
 // NW = 4, RT = 2: 128x256 workgroup tile for outputs with too few 256x256 tiles to fill the chip
 // (A must be k-contiguous: the reduction-major tile layout below assumes 256 rows).  One wave per SIMD
 // as well, so it runs the same interleaved loop (+35-40 % on the GPT-2-small shapes over read bursts).
-// acc += a b.  ASM: as one in-place instruction on accumulator registers — the builtin leaves source and
+// acc += a b as one in-place instruction on accumulator registers — the builtin leaves source and
 // destination accumulators untied, and when all 256 accumulator registers are live (128x128 wave tiles) the
-// allocator then copies accumulator tiles around inside the loop (192 copies per K slice).
-template <bool ASM>
+// allocator then copies accumulator tiles around inside the loop (192 copies per K slice).  Every
+// accumulator tile is touched once per half-step, so consecutive MFMAs never depend on each other, and the
+// epilogue reads the accumulators only after a wait and a workgroup barrier.
 __device__ __forceinline__ void mfma_acc(f32x4& acc, const bf16x8& a, const bf16x8& b) {
-	if constexpr (ASM) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
-	else acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+	asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
 }
 
 template <int NW, int RT, bool AT, bool BT, int EPI>
@@ -276,43 +276,17 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 #pragma unroll
 		for (int j = 0; j < 4; j++) fb[buf][j] = frag<BT>(sb, wc * 128 + (h * 4 + j) * 16, kq, lane);
 	};
-	// The wave raises its issue priority for the length of an MFMA cluster: of the two waves on a SIMD the one
-	// feeding the matrix pipe goes first and the other's fragment reads fill the gaps (+1 % on the stream).
-	auto mfmas = [&](int abuf, int bbuf, int h) {
-		__builtin_amdgcn_s_setprio(1);
-#pragma unroll
-		for (int i = 0; i < RF; i++)
-#pragma unroll
-			for (int j = 0; j < 4; j++)
-				acc[i][h * 4 + j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[abuf][i], fb[bbuf][j], acc[i][h * 4 + j], 0, 0, 0);
-		__builtin_amdgcn_s_setprio(0);
-	};
-
-	// The MFMAs of one half-step with half of this wave's loads of a slice (pieces PIECE0 ...) dealt evenly
-	// between them: the waves' loads of a slice are 64 KiB through a 64 B/clk path, and a wave that
-	// issues them in one burst sits in the queue for ~1000 cycles with its MFMAs behind it.
-	auto mfmas_dma = [&](int abuf, int bbuf, auto hc, const SliceLoads& sl, auto piece0) {
-		constexpr int PIECE0 = decltype(piece0)::value, H = decltype(hc)::value, NM = RF * 4;
-		__builtin_amdgcn_s_setprio(1);
-		static_for<NM>([&](auto nc) {
-			constexpr int n = decltype(nc)::value, i = n / 4, j = n % 4;
-			acc[i][H * 4 + j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[abuf][i], fb[bbuf][j], acc[i][H * 4 + j], 0, 0, 0);
-			if constexpr ((n + 1) * HALF / NM != n * HALF / NM) {
-				issue_piece(sl, std::integral_constant<int, PIECE0 + n * HALF / NM>{});
-				__builtin_amdgcn_sched_barrier(0);
-			}
-		});
-		__builtin_amdgcn_s_setprio(0);
-	};
-
-	// One wave per SIMD (NW = 4): nothing else fills the gaps, so the fragment reads of the next half-step
-	// are dealt between the MFMAs as well (one read per two MFMAs, B slabs first: they are needed first).
-	constexpr bool ONE_WAVE = NW == 4;
+	// One half-step: RF * 4 MFMAs with the fragment reads of the next half-step (one read per two MFMAs, B
+	// slabs first: they are needed first) and, in two of the four half-steps, half of this wave's loads of a
+	// slice dealt between them one at a time.  A lone wave per SIMD has nothing else to fill its issue
+	// gaps, and a wave that issues its loads in one burst (64 KiB per slice through a 64 B/clk path) sits in
+	// the queue for ~1000 cycles with its MFMAs behind it.  With two waves per SIMD the wave also raises
+	// its issue priority for the length of the half-step: the one feeding the matrix pipe goes first.
 	// Reduction-major operands in this loop: the two transpose-read addresses of every fragment are computed
 	// once (k32 half 0 of stage 0); the k32 half and the stage are compile-time here (the loop is unrolled
 	// by two slices) and go into the instructions' offset fields, so the loop has no address arithmetic.
-	uint32_t ta[AT && ONE_WAVE ? RF : 1][2], tb[BT && ONE_WAVE ? 8 : 1][2];
-	if constexpr (ONE_WAVE) {
+	uint32_t ta[AT ? RF : 1][2], tb[BT ? 8 : 1][2];
+	{
 		if constexpr (AT)
 #pragma unroll
 			for (int i = 0; i < RF; i++) {
@@ -335,9 +309,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 		constexpr int SA = decltype(pa_stage)::value, SB = decltype(pb_stage)::value;
 		const unsigned char* sa = smem + SA * A_BYTES;
 		const unsigned char* sb = smem + NST * A_BYTES + SB * B_BYTES;
+		if constexpr (NW == 8) __builtin_amdgcn_s_setprio(1);
 		static_for<NM>([&](auto nc) {
 			constexpr int n = decltype(nc)::value, i = n / 4, j = n % 4;
-			mfma_acc<true>(acc[i][H * 4 + j], fa[abuf][i], fb[bbuf][j]);
+			mfma_acc(acc[i][H * 4 + j], fa[abuf][i], fb[bbuf][j]);
 			if constexpr (n % 2 == 1) {
 				constexpr int r = n / 2;
 				if constexpr (r < 4) {
@@ -353,9 +328,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 			if constexpr (PIECE0 >= 0 && (n + 1) * HALF / NM != n * HALF / NM) issue_piece(sl, std::integral_constant<int, (PIECE0 < 0 ? 0 : PIECE0) + n * HALF / NM>{});
 			__builtin_amdgcn_sched_barrier(0);
 		});
+		if constexpr (NW == 8) __builtin_amdgcn_s_setprio(0);
 	};
 	// one K slice held in stage S; the next one's fragments come from stage 1 - S
-	auto slice_one_wave = [&](auto sc, int kt) {
+	auto slice = [&](auto sc, int kt) {
 		constexpr int S = decltype(sc)::value;
 		constexpr std::integral_constant<int, S> CUR{};
 		constexpr std::integral_constant<int, 1 - S> NXT{};
@@ -376,42 +352,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 
 	load_a(0, 0, 0);
 	load_b(0, 0, 0, 0);
-	if constexpr (ONE_WAVE) {
-		for (int kt = 0; kt < nk; kt += 2) {
-			slice_one_wave(std::integral_constant<int, 0>{}, kt);
-			if (kt + 1 < nk) slice_one_wave(std::integral_constant<int, 1>{}, kt + 1);
-		}
-	} else {
-		for (int kt = 0; kt < nk; kt++) {
-			// where this iteration's loads go: scalar work, done here so that it overlaps the fragment reads
-			// instead of sitting between two MFMAs
-			const SliceLoads next1 = slice_loads(kt + 1), next2 = slice_loads(kt + 2);
-			// half-step (kq 0, h 0), with the second half of slice kt+1's loads
-			load_b(1, kt, 0, 1);
-			__builtin_amdgcn_sched_barrier(0);
-			mfmas_dma(0, 0, std::integral_constant<int, 0>{}, next1, std::integral_constant<int, HALF>{});
-			__builtin_amdgcn_sched_barrier(0);
-			// (kq 0, h 1)
-			load_a(1, kt, 1);
-			load_b(0, kt, 1, 0);
-			__builtin_amdgcn_sched_barrier(0);
-			mfmas(0, 1, 1);
-			__builtin_amdgcn_sched_barrier(0);
-			// (kq 1, h 0)
-			load_b(1, kt, 1, 1);
-			__builtin_amdgcn_sched_barrier(0);
-			mfmas(1, 0, 0);
-			__builtin_amdgcn_sched_barrier(0);
-			wait_counters<0, 0>();  // vmcnt(0): slice kt+1 landed; lgkmcnt(0): slice kt fully read
-			__syncthreads();
-			// (kq 1, h 1), with the first half of slice kt+2's loads into the stage the barrier just freed;
-			// past the end the fragment reads hit a stale stage and their values are unused
-			load_a(0, kt + 1, 0);
-			load_b(0, kt + 1, 0, 0);
-			__builtin_amdgcn_sched_barrier(0);
-			mfmas_dma(1, 1, std::integral_constant<int, 1>{}, next2, std::integral_constant<int, 0>{});
-			__builtin_amdgcn_sched_barrier(0);
-		}
+	for (int kt = 0; kt < nk; kt += 2) {
+		slice(std::integral_constant<int, 0>{}, kt);
+		if (kt + 1 < nk) slice(std::integral_constant<int, 1>{}, kt + 1);
 	}
 
 	// Epilogue through LDS (free once every wave has left the main loop).  Register r of a 16x16
