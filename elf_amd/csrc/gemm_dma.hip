@@ -402,6 +402,14 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 				*reinterpret_cast<bf16x8*>(g.C2 + (int64_t)(grow0 + row) * g.ldc2 + cg0 + c8) = oa;
 			}
 		} else if constexpr (EPI == EPI_BF16 || EPI == EPI_BF16_RESID) {
+			// the strip's residual values first, all loads in flight together: read inside the loop below each
+			// one would be awaited (a full trip to HBM) before the store that follows it in program order
+			bf16x8 rs[EPI == EPI_BF16_RESID ? 8 : 1];
+			if constexpr (EPI == EPI_BF16_RESID) {
+#pragma unroll
+				for (int it = 0; it < 8; it++)
+					rs[it] = *reinterpret_cast<const bf16x8*>(g.R + (int64_t)(grow0 + it * 4 + (lane >> 4)) * g.ldr + gcol0 + (lane & 15) * 8);
+			}
 #pragma unroll
 			for (int it = 0; it < 8; it++) {
 				const int row = it * 4 + (lane >> 4), c8 = (lane & 15) * 8;
@@ -409,9 +417,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 				const f32x4 hi = *reinterpret_cast<const f32x4*>(ws + row * PITCH + c8 + 4);
 				float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
 				if constexpr (EPI == EPI_BF16_RESID) {
-					const bf16x8 rs = *reinterpret_cast<const bf16x8*>(g.R + (int64_t)(grow0 + row) * g.ldr + gcol0 + c8);
 #pragma unroll
-					for (int t = 0; t < 8; t++) v[t] += (float)rs[t];
+					for (int t = 0; t < 8; t++) v[t] += (float)rs[it][t];
 				}
 				bf16x8 o;
 #pragma unroll
@@ -432,12 +439,21 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 				}
 				continue;
 			}
+			// fp32 accumulate: the strip's 16 loads of C all in flight before the first store (left inside the
+			// loop each load is awaited on its own, 16 trips to HBM in a row per strip: 43 k cycles of a
+			// 360 k-cycle dW tile)
+			f32x4 cv[EPI == EPI_F32_ACC ? 16 : 1];
+			if constexpr (EPI == EPI_F32_ACC) {
+#pragma unroll
+				for (int it = 0; it < 16; it++)
+					cv[it] = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(g.C) + (int64_t)(grow0 + it * 2 + (lane >> 5)) * g.ldc + gcol0 + (lane & 31) * 4);
+			}
 #pragma unroll
 			for (int it = 0; it < 16; it++) {
 				const int row = it * 2 + (lane >> 5), c4 = (lane & 31) * 4;
 				f32x4 v = *reinterpret_cast<const f32x4*>(ws + row * PITCH + c4);
 				float* c = reinterpret_cast<float*>(g.C) + (int64_t)(grow0 + row) * g.ldc + gcol0 + c4;
-				if constexpr (EPI == EPI_F32_ACC) v += *reinterpret_cast<const f32x4*>(c);
+				if constexpr (EPI == EPI_F32_ACC) v += cv[it];
 				*reinterpret_cast<f32x4*>(c) = v;
 			}
 		}
