@@ -426,6 +426,323 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(AttnBwdArgs a) {
 	}
 }
 
+// The same pass for a wave that has its SIMD to itself (head_dim 128: K / V rows and accumulators fill the
+// register file).  Nothing else fills its issue gaps, so the schedule is explicit: Q / dO tiles in a three-stage
+// ring fetched two steps ahead, every fragment read issued one product ahead of its use into two buffers
+// that alternate roles, and every MFMA pinned between its share of the reads and of the vector work.
+// 2690 against 3650 cycles per tile; in the stream (between GEMMs) the call takes 1.04 against 1.13 ms.  At
+// head_dim 64 the plain kernel above keeps two waves per SIMD, which this schedule's live ranges would cost.
+template <int D, bool CAUSAL>
+__global__ __launch_bounds__(256) void attn_bwd_kernel_lone(AttnBwdArgs a) {
+	using TL = BwdTile<D>;
+	constexpr int BKV = 128, BQ = 32;
+	constexpr int NF = D / 16;  // fragments per operand tile
+	constexpr int DT = D / 32;
+	constexpr int NQ = BKV / 16;  // fragments of the dQ product (all 128 keys); waves 0..DT-1 own one 32-column slice each
+	constexpr int K_BYTES = BKV * TL::ROW_BYTES, Q_BYTES = BQ * TL::ROW_BYTES;
+	constexpr int STAGE = 2 * Q_BYTES + 256;  // Q tile, dO tile, 32 nlse2 + 32 delta floats
+	constexpr int NSTAGE = 3;                 // tiles are fetched two steps ahead
+	constexpr int DS_BYTES = BKV * BQ * 2;
+	constexpr int Q_LOADS = 8 / TL::RPI;  // DMA instructions per wave and tile (8 rows per wave)
+	extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
+	unsigned char* const sKt = smem_raw;            // K tile, [key][d]
+	unsigned char* const sStage = sKt + K_BYTES;       // NSTAGE x {Q [q][d], dO [q][d], nlse2, delta}
+	unsigned char* const sdS = sStage + NSTAGE * STAGE;  // 2 x dS^T [key][q]
+
+	const int tid = threadIdx.x, lane = tid & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+	const int g = lane >> 5, kl = lane & 31;
+	const int nkt = a.S / BKV;
+	const int npair = CAUSAL ? (nkt + 1) / 2 : nkt;
+	const int pair = blockIdx.x % npair;
+	const int bh = blockIdx.x / npair;
+	const int hk = bh % a.Hkv, b = bh / a.Hkv;
+	const int G = a.Hq / a.Hkv;
+	const int64_t tok0 = (int64_t)b * a.S;
+	const int64_t HqD = (int64_t)a.Hq * D;
+	const float sc = a.scale * LOG2E;
+	const bool dq_wave = DT == 4 || wave < DT;  // head_dim 64: two slices, waves 2 and 3 have no dQ share
+	const int dq_dt = wave % DT;
+	const int key_l = wave * 32 + kl;                        // this lane's key within the tile
+	const int nqt_all = a.S / BQ;
+	const int dq_lane = kl * (int)HqD + dq_dt * 32 + 4 * g;  // lane part of a dQ tile address (elements): query kl, first of 4 columns
+
+	// DMA plan for one (Q, dO) tile pair: wave w moves rows [w*8, w*8+8) of each
+	uint32_t qoff[Q_LOADS], dooff[Q_LOADS];
+#pragma unroll
+	for (int i = 0; i < Q_LOADS; i++) {
+		const int row = wave * 8 + i * TL::RPI + lane / TL::CPR, slot = lane % TL::CPR;
+		qoff[i] = (uint32_t)((row * a.ldq + ((slot ^ TL::swz(row)) << 3)) * 2);
+		dooff[i] = (uint32_t)((row * a.lddo + ((slot ^ TL::swz(row)) << 3)) * 2);
+	}
+	auto zero_ds = [&](unsigned char* t) {
+#pragma unroll
+		for (int i = 0; i < 4; i++) *reinterpret_cast<u32x2*>(t + ds_t_offset(key_l, 8 * i + 4 * g)) = u32x2{0u, 0u};
+	};
+	// registers [r_lo, r_hi) of a dQ accumulator tile -> the partial buffer (issued a few at a time
+	// between other work: a long burst backs up the memory pipeline and stalls the wave)
+	auto dq_out = [&](bf16_t* tile, const f32x16& v, int r_lo, int r_hi) {
+		if (!dq_wave) return;
+#pragma unroll
+		for (int j = 0; j < 4; j++)
+			if (4 * j >= r_lo && 4 * j < r_hi) {
+				bf16x4 o;
+#pragma unroll
+				for (int t = 0; t < 4; t++) o[t] = (bf16_t)v[4 * j + t];
+				*reinterpret_cast<bf16x4*>(tile + dq_lane + 8 * j) = o;
+			}
+	};
+
+	const int n_pass = (CAUSAL && nkt - 1 - pair != pair) ? 2 : 1;
+#pragma unroll 1
+	for (int pass = 0; pass < n_pass; pass++) {
+		const int kt_idx = pass == 0 ? pair : nkt - 1 - pair;
+		const int key0 = kt_idx * BKV;       // first key of the pass
+		const int wkey0 = key0 + wave * 32;  // first key of this wave
+		if (pass > 0) __syncthreads();       // every wave is done with the LDS of the previous pass
+
+		// K tile -> LDS; this wave moves rows [wave*32, wave*32+32)
+		{
+			const bf16_t* kb = a.k + (tok0 + key0) * a.ldk + hk * D;
+#pragma unroll
+			for (int i = 0; i < 32 / TL::RPI; i++) {
+				const int row = wave * 32 + i * TL::RPI + lane / TL::CPR, slot = lane % TL::CPR;
+				dma16(kb, (uint32_t)((row * a.ldk + ((slot ^ TL::swz(row)) << 3)) * 2),
+				      __builtin_amdgcn_readfirstlane(lds_addr(sKt) + (wave * 32 + i * TL::RPI) * TL::ROW_BYTES));
+			}
+		}
+		// own K and V rows as B operands (n = key, 8 consecutive d) in registers
+		bf16x8 kf[NF], vf[NF];
+		{
+			const bf16_t* kp = a.k + (tok0 + wkey0 + kl) * a.ldk + hk * D + 8 * g;
+			const bf16_t* vp = a.v + (tok0 + wkey0 + kl) * a.ldv + hk * D + 8 * g;
+#pragma unroll
+			for (int ks = 0; ks < NF; ks++) {
+				kf[ks] = *reinterpret_cast<const bf16x8*>(kp + ks * 16);
+				vf[ks] = *reinterpret_cast<const bf16x8*>(vp + ks * 16);
+				asm volatile("" : "+a"(kf[ks]), "+a"(vf[ks]));
+			}
+		}
+		f32x16 acc_dk[DT], acc_dv[DT];
+#pragma unroll
+		for (int i = 0; i < DT; i++)
+#pragma unroll
+			for (int r = 0; r < 16; r++) acc_dk[i][r] = acc_dv[i][r] = 0.f;
+
+		// Walk over (query head in group, query tile); causal: only tiles that reach key0.
+		const int qt_first = CAUSAL ? key0 / BQ : 0;
+		const int n_iter = G * (nqt_all - qt_first);
+
+		// tile whose loads are issued next: running pointers, recomputed when the walk moves to the next head
+		int ld_h = hk * G, ld_qt = qt_first;
+		const bf16_t* ld_q;
+		const bf16_t* ld_do;
+		const float* ld_stat;  // lanes 0..31: nlse2 of the tile's queries, lanes 32..63: delta
+		auto seek = [&]() {
+			const int64_t row = tok0 + ld_qt * BQ;
+			ld_q = a.q + row * a.ldq + ld_h * D;
+			ld_do = a.dO + row * a.lddo + ld_h * D;
+			ld_stat = (lane < 32 ? a.nlse2 : a.delta) + ((int64_t)b * a.Hq + ld_h) * a.S + ld_qt * BQ + (lane & 31);
+		};
+		seek();
+		const uint32_t lds_stage = lds_addr(sStage) + wave * 8 * TL::ROW_BYTES;
+		auto issue = [&](int stage) {
+			const uint32_t st = lds_stage + (uint32_t)stage * STAGE;
+#pragma unroll
+			for (int i = 0; i < Q_LOADS; i++) {
+				dma16(ld_q, qoff[i], __builtin_amdgcn_readfirstlane(st + i * TL::RPI * TL::ROW_BYTES));
+				dma16(ld_do, dooff[i], __builtin_amdgcn_readfirstlane(st + Q_BYTES + i * TL::RPI * TL::ROW_BYTES));
+			}
+			if (wave == 0) dma4(ld_stat, __builtin_amdgcn_readfirstlane(st + 2 * Q_BYTES));
+			if (++ld_qt == nqt_all) {
+				ld_qt = qt_first;
+				ld_h++;
+				seek();
+			} else {
+				ld_q += BQ * a.ldq;
+				ld_do += BQ * a.lddo;
+				ld_stat += BQ;
+			}
+		};
+
+		issue(0);
+		if (n_iter > 1) issue(1);
+		zero_ds(sdS + DS_BYTES);  // the "previous tile" of the first iteration
+		wait_vmcnt<0>();
+		__syncthreads();
+		// this wave's slice of K as B operands of the dQ product (n = d column, k = key)
+		bf16x8 ktf[NQ];
+#pragma unroll
+		for (int i = 0; i < NQ; i++) ktf[i] = TL::template cols<false>(sKt, i * 16, dq_dt * 32, lane);
+
+		// position of the current tile; dq_prev_tile = where the dQ tile of iteration it-1 goes
+		int cur_h = hk * G, cur_qt = qt_first;
+		// rows of this key tile's slice: first query of the slice = key0 (causal) or 0
+		bf16_t* const part = a.dq_part + ((int64_t)b * part_rows(a.S, CAUSAL) + part_row0(kt_idx, a.S, CAUSAL) - qt_first * BQ) * HqD;
+		bf16_t* dq_prev_tile = part + (int64_t)(qt_first * BQ) * HqD + cur_h * D;
+
+		// One step = one (head, 32-query tile).  Two fragment buffers alternate roles so that every LDS
+		// read is issued one product ahead of the MFMAs that consume it (one wave per SIMD: nothing else
+		// hides the latency): X enters holding the Q rows of this tile, read during the previous step
+		// (the tile has been in LDS since the barrier before that step), and leaves free; Y leaves
+		// holding the Q rows of the next tile, so the caller swaps the two for the next step.
+		//   Y <- dS^T(prev)     | S  = X(Q) K^T
+		//   X <- dO rows        | dQ(prev) = Y K            softmax on the vector pipe
+		//   Y <- dO^T           | dP = X(dO) V^T
+		//   X <- Q^T            | dV^T += Y(dO^T) P         dS on the vector pipe, dS^T -> LDS
+		//   Y <- Q rows (next)  | dK^T += X(Q^T) dS
+		int stage = 0;  // it % NSTAGE
+		auto step = [&](bf16x8(&X)[NQ], bf16x8(&Y)[NQ], int it) {
+			const int load_stage = stage == 0 ? 2 : stage - 1;  // (it + 2) % 3
+			const unsigned char* sQ = sStage + stage * STAGE;
+			const unsigned char* sdO = sQ + Q_BYTES;
+			const float* sLse = reinterpret_cast<const float*>(sdO + Q_BYTES);
+			stage = stage == NSTAGE - 1 ? 0 : stage + 1;
+			const unsigned char* sQ_next = sStage + stage * STAGE;
+			const unsigned char* sdS_prev = sdS + ((it + 1) & 1) * DS_BYTES;
+			unsigned char* sdS_cur = sdS + (it & 1) * DS_BYTES;
+			const int q0 = cur_qt * BQ;
+
+			f32x16 dq, s, dp;
+#pragma unroll
+			for (int r = 0; r < 16; r++) dq[r] = s[r] = dp[r] = 0.f;
+			// A single wave per SIMD issues in order, so matrix and vector work only overlap where the
+			// program interleaves them: every product below is a loop of "one MFMA + its share of the
+			// LDS reads and vector work that ride along", pinned by scheduling barriers.
+			// causal mask: key > query  <=>  row index of the accumulator register < key - q0
+			// (never true for a tile that lies wholly after the wave's keys; a wave whose keys lie
+			// wholly after the tile gets P = 0 everywhere)
+			const int kq = wkey0 + kl - q0 - 4 * g;
+			f32x4 l4[4];
+			// S = Q K^T, with the dS^T fragments of the previous tile on their way; the loads of the tile after
+			// next and the reads of this tile's statistics go between the MFMAs too
+#pragma unroll
+			for (int i = 0; i < NF; i++) {
+				if (dq_wave) {
+#pragma unroll
+					for (int j = i * (NQ / NF); j < (i + 1) * (NQ / NF); j++) Y[j] = ds_t_frag(sdS_prev, j * 16, lane);
+				}
+				s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(X[i], kf[i], s, 0, 0, 0);
+				if (i == 0 && it + 2 < n_iter) issue(load_stage);
+				if (i == NF / 2) {
+#pragma unroll
+					for (int r4 = 0; r4 < 4; r4++) l4[r4] = *reinterpret_cast<const f32x4*>(sLse + r4 * 8 + 4 * g);
+				}
+				__builtin_amdgcn_sched_barrier(0);
+			}
+			// dQ of the previous tile = dS K, with the dO rows on their way and P = exp2(S sc - lse) on the vector pipe
+			float p[16];
+			auto dq_and_softmax = [&](auto masked) {
+#pragma unroll
+				for (int i = 0; i < NQ; i++) {
+					if (i < NF) X[i] = TL::rows(sdO, 0, i, lane);
+					if (dq_wave) dq = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktf[i], Y[i], dq, 0, 0, 0);
+#pragma unroll
+					for (int r = i * (16 / NQ); r < (i + 1) * (16 / NQ); r++) {
+						float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(s[r], sc, l4[r >> 2][r & 3]));
+						if (decltype(masked)::value && (r >> 2) * 8 + (r & 3) < kq) pr = 0.f;
+						p[r] = pr;
+					}
+					__builtin_amdgcn_sched_barrier(0);
+				}
+			};
+			// only the tiles on the diagonal (the wave's last key lies after the tile's first query) need the mask
+			if (CAUSAL && wkey0 + 31 > q0) dq_and_softmax(std::true_type{});
+			else dq_and_softmax(std::false_type{});
+			const bf16x8 pf[2] = {pack8(p), pack8(p + 8)};
+			f32x4 d4[4];
+#pragma unroll
+			for (int r4 = 0; r4 < 4; r4++) d4[r4] = *reinterpret_cast<const f32x4*>(sLse + 32 + r4 * 8 + 4 * g);
+			// dP = dO V^T, with the dO^T fragments (rows d, k = queries in accumulator order) on their way and the
+			// previous tile's dQ partial going out
+#pragma unroll
+			for (int i = 0; i < NF; i++) {
+				Y[i] = TL::template cols<true>(sdO, (i / DT) * 16, (i % DT) * 32, lane);
+				dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(X[i], vf[i], dp, 0, 0, 0);
+				if ((i * 4) % NF == 0) dq_out(dq_prev_tile, dq, (i * 4 / NF) * 4, (i * 4 / NF) * 4 + 4);
+				__builtin_amdgcn_sched_barrier(0);
+			}
+			// dV^T[d][key] += dO^T[d][q] P[q][key], with the Q^T fragments on their way and dS = P (dP - delta) on
+			// the vector pipe
+			// (dS in the first half of the slots, its packing and the dS^T writes in the next two)
+			float ds[16];
+			bf16x8 dsf[2];
+#pragma unroll
+			for (int i = 0; i < NF; i++) {
+				X[i] = TL::template cols<true>(sQ, (i / DT) * 16, (i % DT) * 32, lane);
+				acc_dv[i % DT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(Y[i], pf[i / DT], acc_dv[i % DT], 0, 0, 0);
+				if (i < NF / 2) {
+#pragma unroll
+					for (int r = i * (32 / NF); r < (i + 1) * (32 / NF); r++) ds[r] = p[r] * (dp[r] - d4[r >> 2][r & 3]);
+				} else if (i < NF / 2 + 2) {
+					// accumulator rows of register r: q = (r/4)*8 + 4g + r%4 -> four 8-byte groups per lane
+					const int u = i - NF / 2;
+					dsf[u] = pack8(ds + 8 * u);
+					const u32x4 w = __builtin_bit_cast(u32x4, dsf[u]);
+					*reinterpret_cast<u32x2*>(sdS_cur + ds_t_offset(key_l, 16 * u + 4 * g)) = u32x2{w[0], w[1]};
+					*reinterpret_cast<u32x2*>(sdS_cur + ds_t_offset(key_l, 16 * u + 8 + 4 * g)) = u32x2{w[2], w[3]};
+				}
+				__builtin_amdgcn_sched_barrier(0);
+			}
+			// dK^T[d][key] += Q^T[d][q] dS[q][key], with the Q rows of the next tile on their way (past the last
+			// tile: a stale stage, values unused)
+#pragma unroll
+			for (int i = 0; i < NF; i++) {
+				Y[i] = TL::rows(sQ_next, 0, i, lane);
+				acc_dk[i % DT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(X[i], dsf[i / DT], acc_dk[i % DT], 0, 0, 0);
+				__builtin_amdgcn_sched_barrier(0);
+			}
+			dq_prev_tile = part + (int64_t)q0 * HqD + cur_h * D;
+			if (++cur_qt == nqt_all) {
+				cur_qt = qt_first;
+				cur_h++;
+			}
+			// the loads of the tile after next were issued before this step's 4 partial stores and vector
+			// memory operations complete in order: waiting until 4 are left waits for the loads only
+			if (dq_wave) wait_counters<4, 0>();
+			else wait_counters<0, 0>();
+			__syncthreads();  // the tile after next is in LDS, dS^T of this tile is complete, everyone is done with this tile
+		};
+
+		bf16x8 fragA[NQ], fragB[NQ];
+#pragma unroll
+		for (int i = 0; i < NF; i++) fragA[i] = TL::rows(sStage, 0, i, lane);
+		for (int it = 0; it < n_iter; it += 2) {
+			step(fragA, fragB, it);
+			if (it + 1 < n_iter) step(fragB, fragA, it + 1);
+		}
+		// drain: dQ product and partial of the last tile
+		{
+			const unsigned char* sdS_prev = sdS + ((n_iter + 1) & 1) * DS_BYTES;
+			f32x16 dq;
+#pragma unroll
+			for (int r = 0; r < 16; r++) dq[r] = 0.f;
+#pragma unroll
+			for (int i = 0; i < NQ; i++)
+				dq = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktf[i], ds_t_frag(sdS_prev, i * 16, lane), dq, 0, 0, 0);
+			dq_out(dq_prev_tile, dq, 0, 16);
+		}
+
+		// dK^T / dV^T accumulators: register r <-> d = dt*32 + (r/4)*8 + 4g + r%4, lane <-> key
+		bf16_t* dkp = a.dk + (tok0 + wkey0 + kl) * a.lddk + hk * D;
+		bf16_t* dvp = a.dv + (tok0 + wkey0 + kl) * a.lddv + hk * D;
+#pragma unroll
+		for (int dt = 0; dt < DT; dt++) {
+#pragma unroll
+			for (int r4 = 0; r4 < 4; r4++) {
+				bf16x4 k4, v4;
+#pragma unroll
+				for (int u = 0; u < 4; u++) {
+					k4[u] = (bf16_t)(acc_dk[dt][r4 * 4 + u] * a.scale);
+					v4[u] = (bf16_t)acc_dv[dt][r4 * 4 + u];
+				}
+				*reinterpret_cast<bf16x4*>(dkp + dt * 32 + r4 * 8 + 4 * g) = k4;
+				*reinterpret_cast<bf16x4*>(dvp + dt * 32 + r4 * 8 + 4 * g) = v4;
+			}
+		}
+	}
+}
+
 // dq[b, q, :] (bf16, row stride ld) = scale * sum over the key tiles that meet q of their partial rows,
 // added in fp32 in ascending tile order; 8 columns (16 bytes) per thread.
 __global__ __launch_bounds__(256) void dq_reduce_kernel(const bf16_t* __restrict__ part, bf16_t* __restrict__ dq, int B, int S, int cols,
@@ -456,8 +773,10 @@ __global__ __launch_bounds__(256) void dq_reduce_kernel(const bf16_t* __restrict
 
 template <int D, bool CAUSAL>
 int launch_bwd(const AttnBwdArgs& a, dim3 grid, hipStream_t stream) {
-	constexpr int smem = 128 * D * 2 + 2 * (2 * 32 * D * 2 + 256) + 2 * 128 * 32 * 2;
-	auto kern = attn_bwd_kernel<D, CAUSAL>;
+	// K tile + the Q / dO ring (two stages, three for the lone-wave schedule) + two dS^T tiles
+	constexpr bool LONE = D == 128;
+	constexpr int smem = 128 * D * 2 + (LONE ? 3 : 2) * (2 * 32 * D * 2 + 256) + 2 * 128 * 32 * 2;
+	auto kern = LONE ? attn_bwd_kernel_lone<D, CAUSAL> : attn_bwd_kernel<D, CAUSAL>;
 	static bool attr_set = false;
 	if (!attr_set) {
 		ELF_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
