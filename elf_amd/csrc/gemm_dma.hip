@@ -60,6 +60,7 @@ struct Args {
 	int tiles_m, tiles_n;
 	int k_splits;    // K is split this many ways (fp32 atomics epilogue) for the last tail_tiles tiles
 	int tail_tiles;  // tiles_m * tiles_n for a uniform split, 0 when nothing is split
+	int walk;        // 1: all XCDs share one band of 16 tile rows at a time (see the tile assignment)
 };
 
 // Byte offsets (relative to the tile origin of the current K slice) of the 16-byte chunks this
@@ -170,7 +171,18 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int wr = wave >> 1, wc = wave & 1;
 
-	// Tile assignment (XCD-contiguous, grouped by 8 tile rows).  The first ntiles - tail_tiles tiles
+	// Tile assignment.  Workgroup w runs on XCD w % 8, whose 32 CUs hold 32 tiles at a time (a round);
+	// both walks give an XCD 8 tile rows x 4 tile columns per round (12 operand slabs through its L2 for
+	// 32 tiles) and differ in where the 8 XCDs are relative to each other:
+	//  * default: each XCD owns a contiguous run of tiles (8 tile rows at a time, along the columns).  The
+	//    XCDs work on different row groups; a row slab of A is needed in as many rounds as the row has
+	//    column groups, so A has to stay in the memory-side cache between them;
+	//  * walk = 1 (A larger than that cache holds next to B): the 8 XCDs share a 16 x 16 block of tiles per
+	//    round, bands of 16 tile rows walked along the columns; a row slab of A is live for one band only
+	//    (weight gradient of the gate/up projection, 28672 x 4096 at K = 8192: +7 %; the down projection's
+	//    forward at K = 14336: +7 %; smaller A operands lose up to 3 % to it).  A last, partly filled
+	//    round shares each 8 x 4 block between several XCDs.
+	// The first ntiles - tail_tiles tiles
 	// are computed whole, one workgroup each; each of the last tail_tiles is shared by k_splits
 	// workgroups that take a K range each and add their part with atomics.  Splitting only the tail
 	// turns the last, partly filled round of workgroups of a launch into a full round of shorter ones.
@@ -189,13 +201,36 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 			pid = full + q / splits;
 		}
 	}
-	if ((ntiles & 7) == 0) pid = (pid & 7) * (ntiles >> 3) + (pid >> 3);
-	constexpr int GROUP_M = 8;
-	const int per_group = GROUP_M * g.tiles_n;
-	const int first_m = (pid / per_group) * GROUP_M;
-	const int gsz = min(g.tiles_m - first_m, GROUP_M);
-	const int m0 = (first_m + (pid % per_group) % gsz) * BM;
-	const int n0 = ((pid % per_group) / gsz) * BN;
+	int m0, n0;
+	const int nsb = ntiles >> 5, nrem = nsb & 7;
+	if (g.walk && (g.tiles_m & 7) == 0 && (g.tiles_n & 3) == 0 && (nrem == 0 || nrem == 1 || nrem == 2 || nrem == 4)) {
+		const int x = pid & 7, i = pid >> 3, nfull = nsb >> 3;
+		int sb, jj;
+		if (i < nfull * 32) {
+			sb = (i >> 5) * 8 + x;
+			jj = i & 31;
+		} else {
+			const int k = 8 / nrem;
+			sb = nfull * 8 + x / k;
+			jj = (x % k) * (32 / k) + (i - nfull * 32);
+		}
+		const int nsb_n = g.tiles_n >> 2, nsb_m = g.tiles_m >> 3;
+		const int band = sb / (2 * nsb_n), within = sb - band * 2 * nsb_n;
+		const bool pair = 2 * band + 1 < nsb_m;
+		const int sbm = 2 * band + (pair ? within & 1 : 0), sbn = pair ? within >> 1 : within;
+		m0 = (sbm * 8 + (jj & 7)) * BM;
+		n0 = (sbn * 4 + (jj >> 3)) * BN;
+	} else {
+		if ((ntiles & 7) == 0) pid = (pid & 7) * (ntiles >> 3) + (pid >> 3);
+		constexpr int GROUP_M = 8;
+		const int per_group = GROUP_M * g.tiles_n;
+		const int first_m = (pid / per_group) * GROUP_M;
+		const int gsz = min(g.tiles_m - first_m, GROUP_M);
+		m0 = (first_m + (pid % per_group) % gsz) * BM;
+		n0 = ((pid % per_group) / gsz) * BN;
+	}
+	m0 = __builtin_amdgcn_readfirstlane(m0);
+	n0 = __builtin_amdgcn_readfirstlane(n0);
 
 	const int nk_total = g.K / BKS;
 	const int nk_per = (nk_total + splits - 1) / splits;
@@ -507,7 +542,10 @@ int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t 
 	// the paired rows of the SwiGLU epilogue are addressed with 32-bit byte offsets from the tile's first row
 	ELF_REQUIRE(epi != EPI_BF16_SWIGLU || (int64_t)(N / 2 + 256) * ldb * 2 < (int64_t(1) << 31), "gemm (dma tile): weight too large for the paired-row epilogue");
 	dma::Args a{(const bf16_t*)A, (const bf16_t*)B, C, (const bf16_t*)R, (bf16_t*)C2, lda, ldb, ldc, ldr, ldc2, M, N, K, M / bm, N / dma::BN, k_splits < 1 ? 1 : k_splits,
-	            tail_tiles < 0 || tail_tiles > ntiles ? ntiles : tail_tiles};
+	            tail_tiles < 0 || tail_tiles > ntiles ? ntiles : tail_tiles, 0};
+	// An A operand too large to stay in the 256 MB memory-side cache next to B: walk the output in bands so
+	// that every row slab of A is fetched from HBM in one round only
+	a.walk = (int64_t)M * K * 2 >= (int64_t(160) << 20);
 	if (epi != EPI_F32_ACC || a.k_splits == 1) a.k_splits = 1, a.tail_tiles = 0;
 	if (bm == 128) {
 		if (!b_t) return dma::launch_epi<4, 2, false, false>(a, epi, stream);

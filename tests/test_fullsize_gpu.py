@@ -23,9 +23,11 @@ def K():
 	return kernels
 
 
-# the Llama-3-8B FFN shapes (256x256 tiles; for tn the dW shape whose 896 tiles get a K-split tail) and
-# the GPT-2-small ones (N = 768: 128x256 tiles; dW with 36 tiles: K split over all of them)
-@pytest.mark.parametrize("dims", [(T, FFN, D_MODEL), (T, 768, 3072)])
+# the Llama-3-8B FFN shapes (256x256 tiles; for tn the dW shape whose 896 tiles get a K-split tail), the
+# down projection's (an A operand of 235 MB: the tile walk in bands of 16 tile rows; for tn the 14336 x 4096
+# weight gradient, whose split tail is the walk's partly filled last round) and the GPT-2-small ones
+# (N = 768: 128x256 tiles; dW with 36 tiles: K split over all of them)
+@pytest.mark.parametrize("dims", [(T, FFN, D_MODEL), (T, D_MODEL, FFN), (T, 768, 3072)])
 @pytest.mark.parametrize("layout", ["nt", "nn", "tn"])
 def test_gemm_row_and_column_probes_at_full_size(K, layout, dims):
 	"""C = A B^T (for tn the matching dW shape, K = tokens): 64 sampled rows and columns of the result
@@ -50,6 +52,21 @@ def test_gemm_row_and_column_probes_at_full_size(K, layout, dims):
 	for got, ref in ((C[rows].float(), ref_r), (C[:, cols].float(), ref_c)):
 		assert (got - ref).abs().max().item() <= 2e-2 * ref.abs().max().item()
 		assert ((got - ref).norm() / ref.norm()).item() <= 5e-3
+
+
+@pytest.mark.parametrize("dims", [(6144, 3072, 14336), (10240, 2048, 8192), (8192, 3072, 14336)])
+def test_gemm_band_walk_with_a_partly_filled_last_round(K, dims):
+	"""A operands of 160 MB and more take the tile walk in bands of 16 tile rows; 288, 320 and 384 tiles
+	leave 1, 2 and 4 blocks of 8 x 4 tiles for the last round, which the 8 XCDs then share.  Every
+	element against an fp32 product of the same bf16 operands."""
+	M, N, Kd = dims
+	A = _randn(M, Kd, seed=11)
+	B = _randn(N, Kd, seed=12, scale=0.05)
+	ref = A.float() @ B.float().t()
+	for C in (K.gemm(A, B), K.gemm(A, B.t().contiguous(), b_t=True)):
+		err = (C.float() - ref).abs()
+		assert err.max().item() <= 2e-2 * ref.abs().max().item()
+		assert (err.norm() / ref.norm()).item() <= 5e-3
 
 
 def test_gemm_fp32_accumulation_is_additive_at_full_size(K):
