@@ -43,6 +43,11 @@ enum BufId {
 static const unsigned ACT_MASK = (1u << B_X) | (1u << B_ST1) | (1u << B_H1) | (1u << B_QKV) | (1u << B_O) | (1u << B_LSE) |
                                  (1u << B_X2) | (1u << B_ST2) | (1u << B_H2) | (1u << B_GU) | (1u << B_A);
 static const unsigned WIN_MASK = (1u << B_H1) | (1u << B_O) | (1u << B_H2) | (1u << B_A);
+// Outputs of one bandwidth-bound kernel over a buffer that is kept anyway (norm of the block input, norm of
+// the attention residual, activation of the gate/up product) and read by W only: an offloaded micro-batch
+// drops them after F and B forms them again from the restored inputs instead of moving them over the host
+// link twice (a third of the stash bytes; the same kernels on the same inputs: bit-identical)
+static const unsigned REFORM_MASK = (1u << B_H1) | (1u << B_H2) | (1u << B_A);
 static const unsigned WGRAD_MASK = (1u << B_DY) | (1u << B_DGU) | (1u << B_DX2) | (1u << B_DQKV);
 
 enum ParamId { P_NORM1_G = 0, P_NORM1_B, P_WQKV, P_WO, P_NORM2_G, P_NORM2_B, P_W1, P_W2, P_COUNT };
@@ -55,13 +60,15 @@ struct Buf {
 	bool owned = false;
 	PinnedPool::Block host;  // valid while offloaded
 	bool offloaded = false;
+	bool dropped = false;  // REFORM_MASK buffer of an offloaded micro-batch: B forms it again
 };
 
 struct BlockState {
 	Buf b[B_COUNT];
 	// offload copies run block by block: this block's device->host copies are done at off_ev,
-	// its host->device copies at pre_ev
-	hipEvent_t off_ev = nullptr, pre_ev = nullptr;
+	// its host->device copies, which come in the order B needs them, at pre_ffn (gate/up product), pre_x2
+	// (+ the FFN norm's input) and pre_ev (everything)
+	hipEvent_t off_ev = nullptr, pre_ev = nullptr, pre_ffn = nullptr, pre_x2 = nullptr;
 };
 
 struct MbState {
@@ -131,6 +138,7 @@ struct Stage {
 static int buf_alloc(Stage* s, BlockState& bs, int id) {
 	Buf& b = bs.b[id];
 	if (b.p && b.owned) return 0;
+	b.dropped = false;
 	b.bytes = s->buf_bytes(id);
 	b.p = s->pool.alloc(b.bytes);
 	if (!b.p) return -3;
@@ -167,7 +175,9 @@ static void destroy_events(MbState& m) {
 	for (auto& bs : m.blk) {
 		if (bs.off_ev) (void)hipEventDestroy(bs.off_ev);
 		if (bs.pre_ev) (void)hipEventDestroy(bs.pre_ev);
-		bs.off_ev = bs.pre_ev = nullptr;
+		if (bs.pre_ffn) (void)hipEventDestroy(bs.pre_ffn);
+		if (bs.pre_x2) (void)hipEventDestroy(bs.pre_x2);
+		bs.off_ev = bs.pre_ev = bs.pre_ffn = bs.pre_x2 = nullptr;
 	}
 }
 
@@ -299,19 +309,32 @@ static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool gra
 			bs.b[B_DY].bytes = s->buf_bytes(B_DY);
 		}
 		const void* dyin = bs.b[B_DY].p;
-		if (m.offloaded && m.prefetched && bs.pre_ev) ELF_CHECK_HIP(hipStreamWaitEvent(st, bs.pre_ev, 0));
+		// a prefetched micro-batch: B waits for each group of buffers where it first reads one, and forms what the
+		// offload dropped again from them (norm_fwd rewrites the statistics with the same values)
+		const bool pre = m.offloaded && m.prefetched && bs.pre_ev;
 		// FFN
 		void* d_a = s->pool.alloc((size_t)T * F * 2);
 		if (!d_a) return -3;
 		ELF_TRY(gemm_bf16(0, 1, T, F, d, dyin, d, p.w[P_W2], F, d_a, F, EPI_BF16, nullptr, 0, 0, 0, st));
 		ELF_TRY(buf_alloc(s, bs, B_DGU));
+		if (pre) ELF_CHECK_HIP(hipStreamWaitEvent(st, bs.pre_ffn, 0));
 		if (s->llama) ELF_TRY(swiglu_bwd(d_a, bs.b[B_GU].p, bs.b[B_DGU].p, T, F, st));
 		else ELF_TRY(gelu_bwd(d_a, bs.b[B_GU].p, bs.b[B_DGU].p, (int64_t)T * F, st));
 		s->pool.free(d_a);
+		if (bs.b[B_A].dropped) {
+			ELF_TRY(buf_alloc(s, bs, B_A));
+			if (s->llama) ELF_TRY(swiglu_fwd(bs.b[B_GU].p, bs.b[B_A].p, T, F, st));
+			else ELF_TRY(gelu_fwd(bs.b[B_GU].p, bs.b[B_A].p, (int64_t)T * F, st));
+		}
 		void* d_h = s->pool.alloc((size_t)T * d * 2);
 		if (!d_h) return -3;
 		ELF_TRY(gemm_bf16(0, 1, T, d, s->ffn_in, bs.b[B_DGU].p, s->ffn_in, p.w[P_W1], d, d_h, d, EPI_BF16, nullptr, 0, 0, 0, st));
 		ELF_TRY(buf_alloc(s, bs, B_DX2));
+		if (pre) ELF_CHECK_HIP(hipStreamWaitEvent(st, bs.pre_x2, 0));
+		if (bs.b[B_H2].dropped) {
+			ELF_TRY(buf_alloc(s, bs, B_H2));
+			ELF_TRY(norm_fwd(norm_kind, bs.b[B_X2].p, p.w[P_NORM2_G], p.w[P_NORM2_B], bs.b[B_H2].p, bs.b[B_ST2].p, T, d, s->cfg.eps, st));
+		}
 		ELF_TRY(norm_bwd(norm_kind, d_h, bs.b[B_X2].p, p.w[P_NORM2_G], bs.b[B_ST2].p, dyin, bs.b[B_DX2].p,
 		                 grads_only ? s->dummy_grad : p.g[P_NORM2_G], grads_only ? s->dummy_grad + d : p.g[P_NORM2_B], s->norm_ws, T, d, st));
 		// attention
@@ -319,6 +342,11 @@ static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool gra
 		if (!d_o) return -3;
 		ELF_TRY(gemm_bf16(0, 1, T, s->Hq * s->D, d, bs.b[B_DX2].p, d, p.w[P_WO], s->Hq * s->D, d_o, s->Hq * s->D, EPI_BF16, nullptr, 0, 0, 0, st));
 		ELF_TRY(buf_alloc(s, bs, B_DQKV));
+		if (pre) ELF_CHECK_HIP(hipStreamWaitEvent(st, bs.pre_ev, 0));
+		if (bs.b[B_H1].dropped) {
+			ELF_TRY(buf_alloc(s, bs, B_H1));
+			ELF_TRY(norm_fwd(norm_kind, bs.b[B_X].p, p.w[P_NORM1_G], p.w[P_NORM1_B], bs.b[B_H1].p, bs.b[B_ST1].p, T, d, s->cfg.eps, st));
+		}
 		{
 			const bf16_t* q = (const bf16_t*)bs.b[B_QKV].p;
 			bf16_t* dq = (bf16_t*)bs.b[B_DQKV].p;
@@ -384,7 +412,8 @@ static int run_backward_params(Stage* s, MbState& m, hipStream_t st) {
 // ---------------------------------------------------------------------------------------------
 // Offload (elf/execution/offload.py:228-268, 330-390): every stage-owned activation buffer of
 // more than 1 MiB goes to the pinned arena on the offload stream; the device copy returns to the
-// pool once that copy has finished.
+// pool once that copy has finished.  The REFORM_MASK buffers are not copied: they go back to the pool at
+// once and run_backward forms them again.
 static int do_offload_block(Stage* s, BlockState& bs, hipStream_t st) {
 	hipEvent_t ready;
 	ELF_CHECK_HIP(hipEventCreateWithFlags(&ready, hipEventDisableTiming));
@@ -396,6 +425,13 @@ static int do_offload_block(Stage* s, BlockState& bs, hipStream_t st) {
 	for (int id = 0; id < B_COUNT; id++) {
 		Buf& b = bs.b[id];
 		if (!(ACT_MASK & (1u << id)) || !b.p || !b.owned || b.bytes <= (size_t(1) << 20)) continue;
+		if (REFORM_MASK & (1u << id)) {
+			s->pool.free(b.p);  // F's kernels are queued: the pool hands it out again in stream order
+			b.p = nullptr;
+			b.owned = false;
+			b.dropped = true;
+			continue;
+		}
 		if (!s->pinned->allocate((int64_t)(b.bytes / 2), 2, /*bf16*/ 1, &b.host)) return -3;
 		ELF_CHECK_HIP(hipMemcpyAsync(b.host.ptr, b.p, b.bytes, hipMemcpyDeviceToHost, s->offload_stream));
 		s->d2h_bytes += (int64_t)b.bytes;
@@ -443,11 +479,21 @@ static int do_restore(Stage* s, MbState& m, bool async, hipStream_t st) {
 	for (int i = (int)m.blk.size() - 1; i >= 0; i--) {
 		BlockState& bs = m.blk[i];
 		if (bs.off_ev) ELF_CHECK_HIP(hipStreamWaitEvent(cs, bs.off_ev, 0));
-		for (int id = 0; id < B_COUNT; id++) {
+		// in the order B reads them: the gate/up product (activation backward, after one GEMM), the FFN norm's
+		// input and statistics, then the attention's and the first norm's buffers
+		static const int order[] = {B_GU, B_X2, B_ST2, B_O, B_LSE, B_QKV, B_X, B_ST1};
+		static_assert(sizeof(order) / sizeof(order[0]) == 8, "every ACT_MASK buffer outside REFORM_MASK is listed");
+		for (int id : order) {
 			Buf& b = bs.b[id];
-			if (!b.offloaded) continue;
-			ELF_CHECK_HIP(hipMemcpyAsync(b.p, b.host.ptr, b.bytes, hipMemcpyHostToDevice, cs));
-			s->h2d_bytes += (int64_t)b.bytes;
+			if (b.offloaded) {
+				ELF_CHECK_HIP(hipMemcpyAsync(b.p, b.host.ptr, b.bytes, hipMemcpyHostToDevice, cs));
+				s->h2d_bytes += (int64_t)b.bytes;
+			}
+			if (async && (id == B_GU || id == B_ST2)) {
+				hipEvent_t& ev = id == B_GU ? bs.pre_ffn : bs.pre_x2;
+				if (!ev) ELF_CHECK_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+				ELF_CHECK_HIP(hipEventRecord(ev, cs));
+			}
 		}
 		if (async) {
 			if (!bs.pre_ev) ELF_CHECK_HIP(hipEventCreateWithFlags(&bs.pre_ev, hipEventDisableTiming));
