@@ -153,7 +153,8 @@ def main():
 	if not args.no_cpu_baseline:
 		cpu_stats = cpu_baseline(w, stage)
 	placement = w.get("placement", PLACEMENT)
-	block = HipStageBlock(stage, BLOCK_ID, placement, sequential_signatures(placement)[BLOCK_ID], mb_size=w["mb"])
+	# as Pipeline does: a stage that runs under a memory budget holds the lean stash
+	block = HipStageBlock(stage, BLOCK_ID, placement, sequential_signatures(placement)[BLOCK_ID], mb_size=w["mb"], lean_stash=bool(w.get("memory_budget_mib")))
 	xs, dys = make_boundary(w["mb"], w["seq"], w["d"], w["n_mb"], seed=1, device="cuda")
 	block.set_boundary(inputs=xs, grads=dys)
 	remat = None

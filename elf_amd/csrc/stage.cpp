@@ -46,7 +46,8 @@ static const unsigned WIN_MASK = (1u << B_H1) | (1u << B_O) | (1u << B_H2) | (1u
 // Outputs of one bandwidth-bound kernel over a buffer that is kept anyway (norm of the block input, norm of
 // the attention residual, activation of the gate/up product) and read by W only: an offloaded micro-batch
 // drops them after F and B forms them again from the restored inputs instead of moving them over the host
-// link twice (a third of the stash bytes; the same kernels on the same inputs: bit-identical)
+// link twice (a third of the stash bytes; the same kernels on the same inputs: bit-identical).  A stage with a
+// lean stash (elf_stage_set_lean_stash) does the same for every micro-batch, to hold less between F and B.
 static const unsigned REFORM_MASK = (1u << B_H1) | (1u << B_H2) | (1u << B_A);
 static const unsigned WGRAD_MASK = (1u << B_DY) | (1u << B_DGU) | (1u << B_DX2) | (1u << B_DQKV);
 
@@ -99,6 +100,7 @@ struct Stage {
 	// optional final norm + output head behind the last block (logits [T, vld], vld >= vocab_out)
 	int vocab_in = 0, vocab_out = 0, vld = 0;
 	bool final_norm = false;
+	bool lean = false;  // elf_stage_set_lean_stash: F keeps no REFORM_MASK buffer, B forms them again
 	void* xw[XP_COUNT] = {};
 	float* xg[XP_COUNT] = {};
 	std::map<int, MbState> mbs;
@@ -246,6 +248,13 @@ static int run_forward(Stage* s, MbState& m, const void* x, void* y, FwdMode mod
 		}
 		// the block's stash starts its way to the host while the next block computes
 		if (offload && mode == SAVE_ALL) ELF_TRY(do_offload_block(s, bs, st));
+		else if (s->lean && mode == SAVE_ALL) {
+			for (int id = 0; id < B_COUNT; id++)
+				if ((REFORM_MASK & (1u << id)) && bs.b[id].p && bs.b[id].owned) {
+					buf_free(s, bs, id);
+					bs.b[id].dropped = true;
+				}
+		}
 	}
 	if (s->vocab_out) {
 		// last stage: (final norm,) logits = h W_head^T   (benchmarks/models/simple.py:497, 508)
@@ -642,6 +651,13 @@ int elf_stage_set_ends(elf_stage_t* h, int vocab_in, int vocab_out, int vocab_ou
 	s->vocab_out = vocab_out;
 	s->vld = vocab_out ? vocab_out_ld : 0;
 	s->final_norm = final_norm != 0;
+	return 0;
+}
+
+int elf_stage_set_lean_stash(elf_stage_t* h, int on) {
+	Stage* s = (Stage*)h;
+	ELF_REQUIRE(s, "elf_stage_set_lean_stash: null stage");
+	s->lean = on != 0;
 	return 0;
 }
 

@@ -96,6 +96,7 @@ for _name, _ret, _args in [
 	("elf_stage_bind_param", _I, [_P, _I, _I, _P, _P]),
 	("elf_stage_set_ends", _I, [_P, _I, _I, _I, _I]),
 	("elf_stage_set_mb_samples", _I, [_P, _I, _I]),
+	("elf_stage_set_lean_stash", _I, [_P, _I]),
 	("elf_stage_forward", _I, [_P, _I, _P, _P, ctypes.c_uint32, _P]),
 	("elf_stage_backward_inputs", _I, [_P, _I, _P, _P, _P, ctypes.c_uint32, _P]),
 	("elf_stage_backward_params", _I, [_P, _I, _P]),
@@ -131,9 +132,12 @@ class HipStageBlock:
 	Weight gradients accumulate in fp32 (``param.main_grad`` views of fused fp32 buffers) across
 	the W passes of a step; ``scale_grads`` divides by the batch size and writes the bf16
 	``param.grad`` the reference exposes.
+
+	``lean_stash=True``: forwards keep neither the norm outputs nor the FFN activation and B forms them
+	again (a third less held between F and B, same results); ``Pipeline`` sets it under a memory budget.
 	"""
 
-	def __init__(self, model, id_, placement, signature, pp_group=None, dp_group=None, recv_pgs=None, send_pgs=None, *, mb_size, seq_len=None):
+	def __init__(self, model, id_, placement, signature, pp_group=None, dp_group=None, recv_pgs=None, send_pgs=None, *, mb_size, seq_len=None, lean_stash=False):
 		if not torch.cuda.is_available():
 			raise _lib.ElfStageError("HipStageBlock needs an MI355X: there is no CPU path for the stage kernels")
 		self.lib = _lib.load()
@@ -155,6 +159,7 @@ class HipStageBlock:
 		self._handle = None
 		self._samples = {}  # mb -> sequences in it, where fewer than mb_size
 		self._kept = {}  # mb -> external tensors the library still points at (x until B/recompute, dy until W)
+		self.lean_stash = bool(lean_stash)
 		self._build(mb_size, seq_len)
 
 	# ------------------------------------------------------------------ set-up
@@ -183,6 +188,8 @@ class HipStageBlock:
 		handle = ctypes.c_void_p()
 		_lib.check(self.lib.elf_stage_create(ctypes.byref(cfg), ctypes.byref(handle)), "elf_stage_create")
 		self._handle = handle
+		if self.lean_stash:
+			_lib.check(self.lib.elf_stage_set_lean_stash(self._handle, 1), "elf_stage_set_lean_stash")
 
 		def fuse(params, pad_rows=0):
 			"""Move `params` (row blocks of one matrix) into one bf16 buffer + one fp32 grad buffer

@@ -306,4 +306,6 @@ class Pipeline:
 	def _create_pipeline(self, parts, signatures):
 		ids = self.placement.get_ids(self.rank)
 		assert len(parts) == len(ids), f"rank {self.rank} owns blocks {ids} of placement {list(self.placement)} but got {len(parts)} stage module(s)"
-		return [HipStageBlock(part, i, self.placement, signatures[i], mb_size=self.mb_size) for part, i in zip(parts, ids)]
+		# under a memory budget the stages hold the lean stash: the remat ILP then starts from a third less per micro-batch
+		lean = self.cfg.memory_budget is not None
+		return [HipStageBlock(part, i, self.placement, signatures[i], mb_size=self.mb_size, lean_stash=lean) for part, i in zip(parts, ids)]

@@ -26,12 +26,12 @@ def _stage(kind):
 	return st
 
 
-def _block(stage, mb):
+def _block(stage, mb, **kw):
 	from elf_amd.execution import HipStageBlock
 	from elf_amd.partitioners.utils import sequential_signatures
 
 	placement = [0, 1, 2, 3]
-	return HipStageBlock(stage, 1, placement, sequential_signatures(placement)[1], mb_size=mb)
+	return HipStageBlock(stage, 1, placement, sequential_signatures(placement)[1], mb_size=mb, **kw)
 
 
 def _oracle(stage, mb, **kw):
@@ -132,7 +132,7 @@ def test_short_micro_batches_share_a_stage(kind):
 
 
 @pytest.mark.parametrize("kind", ["gpt", "llama"])
-@pytest.mark.parametrize("variant", ["full_fwd", "activations_bwd", "full_bwd", "offload", "offload_no_prefetch"])
+@pytest.mark.parametrize("variant", ["full_fwd", "activations_bwd", "full_bwd", "offload", "offload_no_prefetch", "lean_stash"])
 def test_remat_and_offload_variants_equal_plain(kind, variant):
 	"""Every remat / offload variant must give the results of the plain F-B-W sequence (same
 	kernels on the same data; only dQ and split-K accumulate with atomics, hence a tolerance)."""
@@ -144,8 +144,10 @@ def test_remat_and_offload_variants_equal_plain(kind, variant):
 	xs, dys = R.make_boundary(cfg, 2, seed=21)
 	xs, dys = [x.cuda() for x in xs], [d.cuda() for d in dys]
 
+	held_after_f = {}
+
 	def run(variant):
-		blk = _block(stage, mb)
+		blk = _block(stage, mb, lean_stash=variant == "lean_stash")
 		blk.zero_grad()
 		blk.set_boundary(inputs=xs, grads=dys, keep_sent=True)
 		root = lambda name, module: name == ""
@@ -160,6 +162,7 @@ def test_remat_and_offload_variants_equal_plain(kind, variant):
 			else:
 				blk.forward(m)
 			blk.send_forward(m, dst=2)
+		held_after_f[variant] = blk.mem_stats()["live_bytes"]
 		if variant.startswith("offload"):
 			torch.cuda.synchronize()
 			st = blk.mem_stats()
@@ -202,6 +205,10 @@ def test_remat_and_offload_variants_equal_plain(kind, variant):
 
 	y0, dx0, g0 = run("plain")
 	y1, dx1, g1 = run(variant)
+	if variant == "lean_stash":
+		# two micro-batches after F: per block the two norm outputs and the FFN activation less
+		T = mb * cfg["seq"]
+		assert held_after_f["plain"] - held_after_f["lean_stash"] == 2 * cfg["n_blocks"] * (2 * T * cfg["d_model"] + T * cfg["ffn"]) * 2
 	for m in range(2):
 		assert torch.equal(y0[m], y1[m]), "forward outputs must be bit-identical"
 		assert_close(dx1[m], dx0[m], f"{variant} dx[{m}]", rel_max=2e-3, rel_fro=1e-3)
