@@ -283,7 +283,7 @@ static int run_forward(Stage* s, MbState& m, const void* x, void* y, FwdMode mod
 // grads_only: recompute of the W stash gradients (RECOMPUTE_BACKWARD_INPUTS): no norm weight
 // gradients, and the chain stops once the first block's QKV output gradient is known
 // (elf/zb_utils.py:584-604, elf/execution/block.py:340-374).
-static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool grads_only, hipStream_t st) {
+static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool grads_only, hipStream_t st, bool reform = true) {
 	const int nb = s->cfg.n_blocks;
 	const int T = s->T, d = s->d, F = s->F;
 	const int norm_kind = s->llama ? NORM_RMS : NORM_LAYER;
@@ -330,7 +330,7 @@ static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool gra
 		if (s->llama) ELF_TRY(swiglu_bwd(d_a, bs.b[B_GU].p, bs.b[B_DGU].p, T, F, st));
 		else ELF_TRY(gelu_bwd(d_a, bs.b[B_GU].p, bs.b[B_DGU].p, (int64_t)T * F, st));
 		s->pool.free(d_a);
-		if (bs.b[B_A].dropped) {
+		if (reform && bs.b[B_A].dropped) {
 			ELF_TRY(buf_alloc(s, bs, B_A));
 			if (s->llama) ELF_TRY(swiglu_fwd(bs.b[B_GU].p, bs.b[B_A].p, T, F, st));
 			else ELF_TRY(gelu_fwd(bs.b[B_GU].p, bs.b[B_A].p, (int64_t)T * F, st));
@@ -340,7 +340,7 @@ static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool gra
 		ELF_TRY(gemm_bf16(0, 1, T, d, s->ffn_in, bs.b[B_DGU].p, s->ffn_in, p.w[P_W1], d, d_h, d, EPI_BF16, nullptr, 0, 0, 0, st));
 		ELF_TRY(buf_alloc(s, bs, B_DX2));
 		if (pre) ELF_CHECK_HIP(hipStreamWaitEvent(st, bs.pre_x2, 0));
-		if (bs.b[B_H2].dropped) {
+		if (reform && bs.b[B_H2].dropped) {
 			ELF_TRY(buf_alloc(s, bs, B_H2));
 			ELF_TRY(norm_fwd(norm_kind, bs.b[B_X2].p, p.w[P_NORM2_G], p.w[P_NORM2_B], bs.b[B_H2].p, bs.b[B_ST2].p, T, d, s->cfg.eps, st));
 		}
@@ -352,7 +352,7 @@ static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool gra
 		ELF_TRY(gemm_bf16(0, 1, T, s->Hq * s->D, d, bs.b[B_DX2].p, d, p.w[P_WO], s->Hq * s->D, d_o, s->Hq * s->D, EPI_BF16, nullptr, 0, 0, 0, st));
 		ELF_TRY(buf_alloc(s, bs, B_DQKV));
 		if (pre) ELF_CHECK_HIP(hipStreamWaitEvent(st, bs.pre_ev, 0));
-		if (bs.b[B_H1].dropped) {
+		if (reform && bs.b[B_H1].dropped) {
 			ELF_TRY(buf_alloc(s, bs, B_H1));
 			ELF_TRY(norm_fwd(norm_kind, bs.b[B_X].p, p.w[P_NORM1_G], p.w[P_NORM1_B], bs.b[B_H1].p, bs.b[B_ST1].p, T, d, s->cfg.eps, st));
 		}
@@ -713,7 +713,8 @@ int elf_stage_backward_inputs(elf_stage_t* h, int mb, const void* x, const void*
 	}
 	if (x && s->vocab_in) m.ids = x;
 	else if (x) m.blk[0].b[B_X].p = const_cast<void*>(x);
-	ELF_TRY(run_backward(s, m, dy, dx, false, st));
+	// the W-stash inputs are dropped below: no point in forming the ones F or the offload left out
+	ELF_TRY(run_backward(s, m, dy, dx, false, st, !(flags & ELF_BWD_RECOMPUTE_ACTIVATIONS)));
 	if (flags & ELF_BWD_RECOMPUTE_GRADIENTS) free_mask(s, m, WGRAD_MASK), m.has_wgrad = false;
 	if (flags & ELF_BWD_RECOMPUTE_ACTIVATIONS) free_mask(s, m, WIN_MASK), m.has_win = false;
 	return 0;

@@ -132,12 +132,15 @@ def test_short_micro_batches_share_a_stage(kind):
 
 
 @pytest.mark.parametrize("kind", ["gpt", "llama"])
+@pytest.mark.parametrize("lean", [False, True])
 @pytest.mark.parametrize("variant", ["full_fwd", "activations_bwd", "full_bwd", "offload", "offload_no_prefetch", "lean_stash"])
-def test_remat_and_offload_variants_equal_plain(kind, variant):
+def test_remat_and_offload_variants_equal_plain(kind, variant, lean):
 	"""Every remat / offload variant must give the results of the plain F-B-W sequence (same
 	kernels on the same data; only dQ and split-K accumulate with atomics, hence a tolerance)."""
 	from elf_amd.scheduling import OpOptions
 
+	if lean and variant == "lean_stash":
+		pytest.skip("the lean stash alone is the lean = False case of this variant")
 	mb = 16 if variant.startswith("offload") else 2  # only buffers above 1 MiB are offloaded
 	stage = _stage(kind)
 	R, cfg, _ = _oracle(stage, mb)
@@ -147,7 +150,7 @@ def test_remat_and_offload_variants_equal_plain(kind, variant):
 	held_after_f = {}
 
 	def run(variant):
-		blk = _block(stage, mb, lean_stash=variant == "lean_stash")
+		blk = _block(stage, mb, lean_stash=variant == "lean_stash" or (lean and variant != "plain"))
 		blk.zero_grad()
 		blk.set_boundary(inputs=xs, grads=dys, keep_sent=True)
 		root = lambda name, module: name == ""
