@@ -177,10 +177,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	//  * default: each XCD owns a contiguous run of tiles (8 tile rows at a time, along the columns).  The
 	//    XCDs work on different row groups; a row slab of A is needed in as many rounds as the row has
 	//    column groups, so A has to stay in the memory-side cache between them;
-	//  * walk = 1 (A larger than that cache holds next to B): the 8 XCDs share a 16 x 16 block of tiles per
-	//    round, bands of 16 tile rows walked along the columns; a row slab of A is live for one band only
-	//    (weight gradient of the gate/up projection, 28672 x 4096 at K = 8192: +7 %; the down projection's
-	//    forward at K = 14336: +7 %; smaller A operands lose up to 3 % to it).  A last, partly filled
+	//  * walk = 1: the 8 XCDs share a 16 x 16 block of tiles per round, bands of 16 tile rows walked along the
+	//    columns; a row slab of A is live for one band only, B is fetched once per band (weight gradient of
+	//    the gate/up projection, 28672 x 4096 at K = 8192, A = 470 MB: 5-7 % faster).  A last, partly filled
 	//    round shares each 8 x 4 block between several XCDs.
 	// The first ntiles - tail_tiles tiles
 	// are computed whole, one workgroup each; each of the last tail_tiles is shared by k_splits
@@ -543,9 +542,13 @@ int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t 
 	ELF_REQUIRE(epi != EPI_BF16_SWIGLU || (int64_t)(N / 2 + 256) * ldb * 2 < (int64_t(1) << 31), "gemm (dma tile): weight too large for the paired-row epilogue");
 	dma::Args a{(const bf16_t*)A, (const bf16_t*)B, C, (const bf16_t*)R, (bf16_t*)C2, lda, ldb, ldc, ldr, ldc2, M, N, K, M / bm, N / dma::BN, k_splits < 1 ? 1 : k_splits,
 	            tail_tiles < 0 || tail_tiles > ntiles ? ntiles : tail_tiles, 0};
-	// An A operand too large to stay in the 256 MB memory-side cache next to B: walk the output in bands so
-	// that every row slab of A is fetched from HBM in one round only
-	a.walk = (int64_t)M * K * 2 >= (int64_t(160) << 20);
+	// The band walk fetches every row slab of A from HBM in one round only and B once per band; the default
+	// walk wants A in the 256 MB memory-side cache for the whole launch and streams B once.  Inside the stage's
+	// stream (operands cold, per-shape times from a kernel trace) the bands are 0-5 % faster on every shape but
+	// the one with a small A and a B beyond that cache (gate/up projection forward, 67 MB against 235 MB: 2 %
+	// slower), which keeps the default.
+	const int64_t big = int64_t(160) << 20;
+	a.walk = !((int64_t)M * K * 2 < big && (int64_t)N * K * 2 >= big);
 	if (epi != EPI_F32_ACC || a.k_splits == 1) a.k_splits = 1, a.tail_tiles = 0;
 	if (bm == 128) {
 		if (!b_t) return dma::launch_epi<4, 2, false, false>(a, epi, stream);
