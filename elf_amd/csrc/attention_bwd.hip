@@ -751,14 +751,16 @@ __global__ __launch_bounds__(256) void dq_reduce_kernel(const bf16_t* __restrict
 	const int64_t n = (int64_t)B * S * cpr;
 	const int nkt = S / 128;
 	const int64_t rows_b = part_rows(S, causal);
-	for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+	for (int64_t j = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; j < n; j += (int64_t)gridDim.x * blockDim.x) {
+		// last rows first: under a causal mask they sum the most partials, and the launch then ends on the short ones
+		const int64_t i = n - 1 - j;
 		const int64_t row = i / cpr;
 		const int c = (int)(i - row * cpr) * 8;
 		const int b = (int)(row / S), q = (int)(row - (int64_t)b * S);
 		const int ns = causal ? q / 128 + 1 : nkt;
 		float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 		const bf16_t* pb = part + (int64_t)b * rows_b * cols + c;
-#pragma unroll 4
+#pragma unroll 8
 		for (int kt = 0; kt < ns; kt++) {
 			const bf16x8 v = *reinterpret_cast<const bf16x8*>(pb + (part_row0(kt, S, causal) + q - (causal ? 128 * kt : 0)) * cols);
 #pragma unroll
