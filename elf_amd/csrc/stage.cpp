@@ -49,6 +49,9 @@ static const unsigned WIN_MASK = (1u << B_H1) | (1u << B_O) | (1u << B_H2) | (1u
 // link twice (a third of the stash bytes; the same kernels on the same inputs: bit-identical).  A stage with a
 // lean stash (elf_stage_set_lean_stash) does the same for every micro-batch, to hold less between F and B.
 static const unsigned REFORM_MASK = (1u << B_H1) | (1u << B_H2) | (1u << B_A);
+// An offloaded micro-batch also leaves out the QKV projection's output: one GEMM over the re-formed norm
+// output (plus RoPE) costs a third of the link time its 2 x 168 MB would take at the 70B shape.
+static const unsigned OFFLOAD_REFORM_MASK = REFORM_MASK | (1u << B_QKV);
 static const unsigned WGRAD_MASK = (1u << B_DY) | (1u << B_DGU) | (1u << B_DX2) | (1u << B_DQKV);
 
 enum ParamId { P_NORM1_G = 0, P_NORM1_B, P_WQKV, P_WO, P_NORM2_G, P_NORM2_B, P_W1, P_W2, P_COUNT };
@@ -352,9 +355,14 @@ static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool gra
 		ELF_TRY(gemm_bf16(0, 1, T, s->Hq * s->D, d, bs.b[B_DX2].p, d, p.w[P_WO], s->Hq * s->D, d_o, s->Hq * s->D, EPI_BF16, nullptr, 0, 0, 0, st));
 		ELF_TRY(buf_alloc(s, bs, B_DQKV));
 		if (pre) ELF_CHECK_HIP(hipStreamWaitEvent(st, bs.pre_ev, 0));
-		if (reform && bs.b[B_H1].dropped) {
+		if (bs.b[B_H1].dropped && (reform || bs.b[B_QKV].dropped)) {
 			ELF_TRY(buf_alloc(s, bs, B_H1));
 			ELF_TRY(norm_fwd(norm_kind, bs.b[B_X].p, p.w[P_NORM1_G], p.w[P_NORM1_B], bs.b[B_H1].p, bs.b[B_ST1].p, T, d, s->cfg.eps, st));
+		}
+		if (bs.b[B_QKV].dropped) {
+			ELF_TRY(buf_alloc(s, bs, B_QKV));
+			ELF_TRY(gemm_bf16(0, 0, T, s->nqkv, d, bs.b[B_H1].p, d, p.w[P_WQKV], d, bs.b[B_QKV].p, s->nqkv, EPI_BF16, nullptr, 0, 0, 0, st));
+			if (s->llama) ELF_TRY(rope_apply(bs.b[B_QKV].p, s->rope_cs, T, s->S, s->nqkv, s->Hq + s->Hkv, s->D, 0, st));
 		}
 		{
 			const bf16_t* q = (const bf16_t*)bs.b[B_QKV].p;
@@ -421,7 +429,7 @@ static int run_backward_params(Stage* s, MbState& m, hipStream_t st) {
 // ---------------------------------------------------------------------------------------------
 // Offload (elf/execution/offload.py:228-268, 330-390): every stage-owned activation buffer of
 // more than 1 MiB goes to the pinned arena on the offload stream; the device copy returns to the
-// pool once that copy has finished.  The REFORM_MASK buffers are not copied: they go back to the pool at
+// pool once that copy has finished.  The OFFLOAD_REFORM_MASK buffers are not copied: they go back to the pool at
 // once and run_backward forms them again.
 static int do_offload_block(Stage* s, BlockState& bs, hipStream_t st) {
 	hipEvent_t ready;
@@ -434,7 +442,7 @@ static int do_offload_block(Stage* s, BlockState& bs, hipStream_t st) {
 	for (int id = 0; id < B_COUNT; id++) {
 		Buf& b = bs.b[id];
 		if (!(ACT_MASK & (1u << id)) || !b.p || !b.owned || b.bytes <= (size_t(1) << 20)) continue;
-		if (REFORM_MASK & (1u << id)) {
+		if (OFFLOAD_REFORM_MASK & (1u << id)) {
 			s->pool.free(b.p);  // F's kernels are queued: the pool hands it out again in stream order
 			b.p = nullptr;
 			b.owned = false;

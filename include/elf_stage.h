@@ -237,8 +237,9 @@ int elf_stage_recompute_forward(elf_stage_t* s, int mb, const void* x, int save,
 int elf_stage_recompute_backward_inputs(elf_stage_t* s, int mb, const void* dy, void* stream);
 /* Offload life cycle (OffloadToCPU, offload.py:166-411): offload is also implied by
  * ELF_FWD_OFFLOAD; prefetch = PREFETCH_ACTIVATIONS; release returns the pinned blocks.  Of the
- * stash, the two norm outputs and the FFN activation are not copied: backward_inputs forms them
- * again from the restored buffers with the forward's kernels (bit-identical). */
+ * stash, the two norm outputs, the FFN activation and the QKV projection's output are not copied:
+ * backward_inputs forms them again from the restored buffers with the forward's kernels
+ * (bit-identical). */
 int elf_stage_offload(elf_stage_t* s, int mb, void* stream);
 int elf_stage_prefetch(elf_stage_t* s, int mb, void* stream);
 int elf_stage_release(elf_stage_t* s, int mb);

@@ -170,11 +170,11 @@ def test_remat_and_offload_variants_equal_plain(kind, variant, lean):
 			torch.cuda.synchronize()
 			st = blk.mem_stats()
 			assert st["d2h_bytes"] > 0 and st["pinned_bytes"] >= st["d2h_bytes"]
-			# what crosses the link: the stage-owned buffers above 1 MiB minus the two norm outputs and the
-			# FFN activation, which B forms again from the restored buffers
+			# what crosses the link: the stage-owned buffers above 1 MiB minus the two norm outputs, the FFN
+			# activation and the QKV projection's output, which B forms again from the restored buffers
 			T, d, hq, hkv, hd = mb * cfg["seq"], cfg["d_model"], cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
 			ffn_in = cfg["ffn"] * (2 if kind == "llama" else 1)
-			per_block = [T * (hq + 2 * hkv) * hd * 2, T * hq * hd * 2, mb * hq * cfg["seq"] * 4, T * d * 2, T * ffn_in * 2]
+			per_block = [T * hq * hd * 2, mb * hq * cfg["seq"] * 4, T * d * 2, T * ffn_in * 2]
 			moved = sum(b for b in per_block if b > 1 << 20) * cfg["n_blocks"] + (T * d * 2 if T * d * 2 > 1 << 20 else 0) * (cfg["n_blocks"] - 1)
 			assert st["d2h_bytes"] == 2 * moved
 		for m in range(2):
