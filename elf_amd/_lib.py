@@ -26,6 +26,7 @@ _SIGNATURES = {
 	"elf_gelu_fwd": (c_int, [_P, _P, c_int64, _P]),
 	"elf_gelu_bwd": (c_int, [_P, _P, _P, c_int64, _P]),
 	"elf_gemm_act_bf16": (c_int, [c_int, c_int, c_int, c_int, _P, c_int64, _P, c_int64, _P, c_int64, _P, c_int64, _P]),
+	"elf_gemm_swiglu_bwd_bf16": (c_int, [c_int, c_int, c_int, _P, c_int64, _P, c_int64, _P, c_int64, _P, c_int64, _P, _P]),
 	"elf_swiglu_fwd": (c_int, [_P, _P, c_int64, c_int, _P]),
 	"elf_swiglu_bwd": (c_int, [_P, _P, _P, c_int64, c_int, _P]),
 	"elf_rope_table": (c_int, [_P, c_int, c_int, c_double, _P]),

@@ -20,6 +20,11 @@ int elf_gemm_act_bf16(int act, int M, int F, int K, const void* A, int64_t lda, 
 	return elf::gemm_act_bf16(act, M, F, K, A, lda, W, ldw, pre, ldpre, out, ldout, (hipStream_t)stream);
 }
 
+int elf_gemm_swiglu_bwd_bf16(int M, int F, int K, const void* dY, int64_t lddy, const void* W, int64_t ldw,
+                             const void* gu, int64_t ldgu, void* dgu, int64_t lddgu, void* scratch, void* stream) {
+	return elf::gemm_swiglu_bwd_bf16(M, F, K, dY, lddy, W, ldw, gu, ldgu, dgu, lddgu, scratch, (hipStream_t)stream);
+}
+
 #define S_(x) ((hipStream_t)(x))
 int elf_norm_fwd(int kind, const void* x, const void* gamma, const void* beta, void* y, void* stats, int T, int d,
                  float eps, void* stream) {

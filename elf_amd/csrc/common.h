@@ -58,6 +58,14 @@ __device__ __forceinline__ float swiglu_f(float g, float u) {
 	return g * sig * u;
 }
 
+// Gradient of silu(g) * u with respect to g and u for the incoming gradient d; shared by the activation
+// backward kernel and the GEMM epilogue that fuses it, so that both give the same bits.
+__device__ __forceinline__ void swiglu_bwd_f(float d, float g, float u, float& dg, float& du) {
+	const float sig = 1.f / (1.f + __expf(-g));
+	dg = d * u * sig * (1.f + g * (1.f - sig));
+	du = d * g * sig;
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
 	for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);

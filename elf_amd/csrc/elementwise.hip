@@ -387,11 +387,7 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const bf16_t* __restric
 		Chunk g = load8(gu + row * 2 * F + c8), u = load8(gu + row * 2 * F + F + c8), d = load8(dh + row * F + c8);
 		Chunk dg, du;
 #pragma unroll
-		for (int j = 0; j < 8; j++) {
-			const float sig = 1.f / (1.f + __expf(-g.v[j]));
-			dg.v[j] = d.v[j] * u.v[j] * sig * (1.f + g.v[j] * (1.f - sig));
-			du.v[j] = d.v[j] * g.v[j] * sig;
-		}
+		for (int j = 0; j < 8; j++) swiglu_bwd_f(d.v[j], g.v[j], u.v[j], dg.v[j], du.v[j]);
 		store8(dgu + row * 2 * F + c8, dg);
 		store8(dgu + row * 2 * F + F + c8, du);
 	}

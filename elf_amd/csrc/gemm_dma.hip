@@ -435,6 +435,36 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 				*reinterpret_cast<bf16x8*>(c + F) = ou;
 				*reinterpret_cast<bf16x8*>(g.C2 + (int64_t)(grow0 + row) * g.ldc2 + cg0 + c8) = oa;
 			}
+		} else if constexpr (EPI == EPI_BF16_SWIGLU_BWD) {
+			// the tile is d = dY W over F columns; g and u of the same rows and columns lie F columns apart in R,
+			// their gradients likewise in C.  All loads of the strip first (see the residual epilogue below); d is
+			// rounded to bf16 before it is used, as a separate pass over a stored d would read it
+			const int F = g.N;
+			bf16x8 gs[8], us[8];
+#pragma unroll
+			for (int it = 0; it < 8; it++) {
+				const bf16_t* r = g.R + (int64_t)(grow0 + it * 4 + (lane >> 4)) * g.ldr + gcol0 + (lane & 15) * 8;
+				gs[it] = *reinterpret_cast<const bf16x8*>(r);
+				us[it] = *reinterpret_cast<const bf16x8*>(r + F);
+			}
+#pragma unroll
+			for (int it = 0; it < 8; it++) {
+				const int row = it * 4 + (lane >> 4), c8 = (lane & 15) * 8;
+				const f32x4 lo = *reinterpret_cast<const f32x4*>(ws + row * PITCH + c8);
+				const f32x4 hi = *reinterpret_cast<const f32x4*>(ws + row * PITCH + c8 + 4);
+				bf16x8 og, ou;
+#pragma unroll
+				for (int t = 0; t < 8; t++) {
+					const float d = (float)(bf16_t)(t < 4 ? lo[t] : hi[t - 4]);
+					float dg, du;
+					swiglu_bwd_f(d, (float)gs[it][t], (float)us[it][t], dg, du);
+					og[t] = (bf16_t)dg;
+					ou[t] = (bf16_t)du;
+				}
+				bf16_t* c = reinterpret_cast<bf16_t*>(g.C) + (int64_t)(grow0 + row) * g.ldc + gcol0 + c8;
+				*reinterpret_cast<bf16x8*>(c) = og;
+				*reinterpret_cast<bf16x8*>(c + F) = ou;
+			}
 		} else if constexpr (EPI == EPI_BF16 || EPI == EPI_BF16_RESID) {
 			// the strip's residual values first, all loads in flight together: read inside the loop below each
 			// one would be awaited (a full trip to HBM) before the store that follows it in program order
@@ -522,6 +552,9 @@ static int launch_epi(const Args& a, int epi, hipStream_t stream) {
 	}
 	if constexpr (!AT && !BT) {
 		if (epi == EPI_BF16_SWIGLU) return launch<NW, RT, AT, BT, EPI_BF16_SWIGLU>(a, stream);
+	}
+	if constexpr (NW == 4 && RT == 4 && !AT && BT) {
+		if (epi == EPI_BF16_SWIGLU_BWD) return launch<NW, RT, AT, BT, EPI_BF16_SWIGLU_BWD>(a, stream);
 	}
 	set_error("gemm: unknown epilogue %d", epi);
 	return -1;

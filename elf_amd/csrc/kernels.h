@@ -12,6 +12,8 @@ enum GemmEpilogue {
 	EPI_F32_STORE = 3,   // C(fp32) = acc
 	// direct-to-LDS tiles with k-contiguous operands only (see gemm_act_bf16):
 	EPI_BF16_SWIGLU = 4,  // B = [gate rows; up rows]: C(bf16) = acc = [g | u], C2(bf16) = silu(g) * u
+	// k-contiguous A only (see gemm_swiglu_bwd_bf16): R = [g | u] (bf16, N columns each), acc rounded to bf16 = d:
+	EPI_BF16_SWIGLU_BWD = 5,  // C(bf16) = [d silu'(g) u | d silu(g)]
 };
 
 int gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda, const void* B, int64_t ldb,
@@ -33,6 +35,15 @@ enum Activation { ACT_GELU = 0, ACT_SWIGLU = 1 };
 // by the activation kernel.  Both ways give the same bits.
 int gemm_act_bf16(int act, int M, int F, int K, const void* A, int64_t lda, const void* W, int64_t ldw, void* pre,
                   int64_t ldpre, void* out, int64_t ldout, hipStream_t stream);
+
+// Backward of the MLP's down projection into its SwiGLU: dgu [M, 2F] = the gradient of [g | u] for
+// d = dY W (dY [M, K], W [K, F] = the down projection's weight as it lies in memory), with gu [M, 2F] the saved
+// gate/up product.  One kernel (activation backward in the GEMM epilogue, d never reaches memory) when the shape
+// fits the direct-to-LDS tiles; otherwise the GEMM writes d into `scratch` [M, F] and the activation backward
+// kernel follows.  Both ways give the same bits.  `scratch` may be null when gemm_swiglu_bwd_fused(M, F, K).
+bool gemm_swiglu_bwd_fused(int M, int F, int K);
+int gemm_swiglu_bwd_bf16(int M, int F, int K, const void* dY, int64_t lddy, const void* W, int64_t ldw, const void* gu,
+                         int64_t ldgu, void* dgu, int64_t lddgu, void* scratch, hipStream_t stream);
 
 enum NormKind { NORM_RMS = 0, NORM_LAYER = 1 };
 

@@ -324,15 +324,20 @@ static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool gra
 		// a prefetched micro-batch: B waits for each group of buffers where it first reads one, and forms what the
 		// offload dropped again from them (norm_fwd rewrites the statistics with the same values)
 		const bool pre = m.offloaded && m.prefetched && bs.pre_ev;
-		// FFN
-		void* d_a = s->pool.alloc((size_t)T * F * 2);
-		if (!d_a) return -3;
-		ELF_TRY(gemm_bf16(0, 1, T, F, d, dyin, d, p.w[P_W2], F, d_a, F, EPI_BF16, nullptr, 0, 0, 0, st));
+		// FFN: dY W2 and the activation's backward, in one kernel for SwiGLU where the shape allows (a prefetched
+		// micro-batch keeps them apart: the GEMM then runs while the gate/up product is still on the link)
 		ELF_TRY(buf_alloc(s, bs, B_DGU));
-		if (pre) ELF_CHECK_HIP(hipStreamWaitEvent(st, bs.pre_ffn, 0));
-		if (s->llama) ELF_TRY(swiglu_bwd(d_a, bs.b[B_GU].p, bs.b[B_DGU].p, T, F, st));
-		else ELF_TRY(gelu_bwd(d_a, bs.b[B_GU].p, bs.b[B_DGU].p, (int64_t)T * F, st));
-		s->pool.free(d_a);
+		if (s->llama && !pre && gemm_swiglu_bwd_fused(T, F, d)) {
+			ELF_TRY(gemm_swiglu_bwd_bf16(T, F, d, dyin, d, p.w[P_W2], F, bs.b[B_GU].p, s->ffn_in, bs.b[B_DGU].p, s->ffn_in, nullptr, st));
+		} else {
+			void* d_a = s->pool.alloc((size_t)T * F * 2);
+			if (!d_a) return -3;
+			ELF_TRY(gemm_bf16(0, 1, T, F, d, dyin, d, p.w[P_W2], F, d_a, F, EPI_BF16, nullptr, 0, 0, 0, st));
+			if (pre) ELF_CHECK_HIP(hipStreamWaitEvent(st, bs.pre_ffn, 0));
+			if (s->llama) ELF_TRY(swiglu_bwd(d_a, bs.b[B_GU].p, bs.b[B_DGU].p, T, F, st));
+			else ELF_TRY(gelu_bwd(d_a, bs.b[B_GU].p, bs.b[B_DGU].p, (int64_t)T * F, st));
+			s->pool.free(d_a);
+		}
 		if (reform && bs.b[B_A].dropped) {
 			ELF_TRY(buf_alloc(s, bs, B_A));
 			if (s->llama) ELF_TRY(swiglu_fwd(bs.b[B_GU].p, bs.b[B_A].p, T, F, st));

@@ -68,6 +68,25 @@ def gemm_act(a, w, act):
 	return pre, out
 
 
+def gemm_swiglu_bwd(dy, w2, gu, fused=True):
+	"""dgu [M, 2F]: gradient of gu = [g | u] for d = dy @ w2 (dy [M, K], w2 [K, F]); ``fused=False`` forces the
+	GEMM + activation-backward pair (same bits)."""
+	for t, n in ((dy, "dy"), (w2, "w2"), (gu, "gu")):
+		_need(t, torch.bfloat16, "gemm_swiglu_bwd." + n)
+	M, K = dy.shape
+	F = w2.shape[1]
+	if w2.shape[0] != K or tuple(gu.shape) != (M, 2 * F):
+		raise _lib.ElfStageError(f"gemm_swiglu_bwd: shapes {tuple(dy.shape)}, {tuple(w2.shape)}, {tuple(gu.shape)} do not fit")
+	dgu = torch.empty_like(gu)
+	if not fused:
+		d = gemm(dy, w2, b_t=True)
+		return swiglu_bwd(d, gu)
+	scratch = torch.empty((M, F), dtype=torch.bfloat16, device=dy.device)
+	rc = _lib.load().elf_gemm_swiglu_bwd_bf16(M, F, K, _ptr(dy), dy.stride(0), _ptr(w2), w2.stride(0), _ptr(gu), 2 * F, _ptr(dgu), 2 * F, _ptr(scratch), _stream())
+	_lib.check(rc, "elf_gemm_swiglu_bwd_bf16")
+	return dgu
+
+
 def norm_fwd(kind, x, gamma, beta=None, eps=1e-5):
 	_need(x, torch.bfloat16, "norm.x")
 	T, d = x.shape

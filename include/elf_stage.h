@@ -53,6 +53,16 @@ int elf_gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t 
  *           LinearDX.forward (elf/zb_utils.py:20); no reference module for SwiGLU. */
 int elf_gemm_act_bf16(int act, int M, int F, int K, const void* A, int64_t lda, const void* W, int64_t ldw,
                       void* pre, int64_t ldpre, void* out, int64_t ldout, void* stream);
+/* Backward of the down-projection into the SwiGLU: d = dY W with dY [M, K] and W [K, F] (the down
+ * projection's weight [d_model, F] as it lies in memory), then dgu[M, 2F] = [d silu'(g) u | d silu(g)]
+ * from the saved gu[M, 2F] = [g | u].  One kernel (activation backward in the GEMM epilogue, d never
+ * reaches memory) when M and F are multiples of 256, K of 64 and the tiles fill the chip; otherwise
+ * elf_gemm_bf16(0, 1, ...) into scratch [M, F] followed by elf_swiglu_bwd (scratch may be null only for
+ * the fused shapes).  Same bits either way.
+ * Replaces: LinearDX.backward of fc2 (elf/zb_utils.py:29-41) followed by autograd's backward of
+ *           silu(gate) * up; no reference module for SwiGLU. */
+int elf_gemm_swiglu_bwd_bf16(int M, int F, int K, const void* dY, int64_t lddy, const void* W, int64_t ldw,
+                             const void* gu, int64_t ldgu, void* dgu, int64_t lddgu, void* scratch, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Bandwidth-bound stage ops.  bf16 row-major tensors, fp32 math, one rounding on store.

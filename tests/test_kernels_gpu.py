@@ -210,6 +210,24 @@ def test_gemm_with_activation_epilogue(K, act, shape):
 	assert torch.equal(out, two), "fused activation differs from the separate kernel"
 
 
+@pytest.mark.parametrize("shape", [(8192, 2048, 256), (4096, 3072, 64), (512, 1024, 128)])
+def test_gemm_with_swiglu_backward_epilogue(K, shape):
+	"""dX of the down projection with the SwiGLU's backward in the GEMM epilogue: against fp32 torch autograd
+	of silu(g) * u, and bit for bit against the GEMM followed by the activation-backward kernel.  Shapes: two the
+	fused tiles cover (one with a single K slice) and one they do not (the library runs the two kernels itself)."""
+	M, F, Kd = shape
+	dY = _randn(M, Kd, seed=51)
+	W2 = _randn(Kd, F, seed=52, scale=0.1)
+	gu = _randn(M, 2 * F, seed=53)
+	dgu = K.gemm_swiglu_bwd(dY, W2, gu)
+	two = K.gemm_swiglu_bwd(dY, W2, gu, fused=False)
+	assert torch.equal(dgu, two), "fused activation backward differs from the separate kernels"
+	d = (dY.float() @ W2.float()).to(torch.bfloat16).float()
+	g32 = gu.float().requires_grad_(True)
+	(torch.nn.functional.silu(g32[:, :F]) * g32[:, F:]).backward(d)
+	_close(dgu, g32.grad, what="gradient of [g | u]")
+
+
 def test_gemm_with_activation_strided_outputs(K):
 	# outputs that are column slices of wider buffers, as a caller that packs activations would pass
 	from elf_amd import _lib
