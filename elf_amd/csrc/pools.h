@@ -19,7 +19,10 @@ class DevicePool {
 	~DevicePool();
 	void* alloc(size_t bytes);  // nullptr on failure (message in get_error())
 	void free(void* p);
-	void free_after(void* p, hipEvent_t ev);  // event ownership stays with the caller
+	// event ownership stays with the caller, who must call drain() before destroying the event
+	void free_after(void* p, hipEvent_t ev);
+	void poll() { if (!pending_.empty()) poll_pending(false); }  // return blocks whose event has fired
+	void drain() { poll_pending(true); }                         // wait for every pending event
 	void trim();                              // release every cached block to the driver
 	size_t live_bytes() const { return live_; }
 	size_t peak_bytes() const { return peak_; }

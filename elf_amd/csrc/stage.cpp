@@ -140,6 +140,20 @@ struct Stage {
 		if (_rc) return _rc;     \
 	} while (0)
 
+// A pool temporary of one function: returned on every path out of it (release() hands it back early).
+struct PoolTmp {
+	DevicePool& pool;
+	void* p;
+	PoolTmp(DevicePool& pl, size_t bytes) : pool(pl), p(bytes ? pl.alloc(bytes) : nullptr) {}
+	~PoolTmp() { pool.free(p); }
+	PoolTmp(const PoolTmp&) = delete;
+	PoolTmp& operator=(const PoolTmp&) = delete;
+	void release() {
+		pool.free(p);
+		p = nullptr;
+	}
+};
+
 static int buf_alloc(Stage* s, BlockState& bs, int id) {
 	Buf& b = bs.b[id];
 	if (b.p && b.owned) return 0;
@@ -189,7 +203,19 @@ static void destroy_events(MbState& m) {
 static int do_offload_block(Stage* s, BlockState& bs, hipStream_t st);
 
 // ---------------------------------------------------------------------------------------------
-static int run_forward(Stage* s, MbState& m, const void* x, void* y, FwdMode mode, hipStream_t st, bool offload = false) {
+// remat: ELF_FWD_REMAT_ATTN / ELF_FWD_REMAT_NORM of a forward that keeps its stash: the buffers those module
+// checkpoints stand for are dropped block by block and run_backward forms them again.
+static int run_forward(Stage* s, MbState& m, const void* x, void* y, FwdMode mode, hipStream_t st, bool offload = false, unsigned remat = 0) {
+	unsigned remat_drop = 0;
+	if (mode == SAVE_ALL && (remat & ELF_FWD_REMAT_ATTN)) remat_drop |= (1u << B_O) | (1u << B_LSE);
+	if (mode == SAVE_ALL && (remat & ELF_FWD_REMAT_NORM)) remat_drop |= (1u << B_ST1) | (1u << B_ST2);
+	auto drop = [&](BlockState& bs, unsigned mask) {
+		for (int id = 0; id < B_COUNT; id++)
+			if ((mask & (1u << id)) && bs.b[id].p && bs.b[id].owned) {
+				buf_free(s, bs, id);
+				bs.b[id].dropped = true;
+			}
+	};
 	const int nb = s->cfg.n_blocks;
 	const int T = s->T, d = s->d, F = s->F;
 	const int norm_kind = s->llama ? NORM_RMS : NORM_LAYER;
@@ -249,15 +275,10 @@ static int run_forward(Stage* s, MbState& m, const void* x, void* y, FwdMode mod
 			for (int id = 0; id < B_COUNT; id++)
 				if ((ACT_MASK & (1u << id)) && !(keep & (1u << id))) buf_free(s, bs, id);
 		}
+		if (remat_drop) drop(bs, remat_drop);
 		// the block's stash starts its way to the host while the next block computes
 		if (offload && mode == SAVE_ALL) ELF_TRY(do_offload_block(s, bs, st));
-		else if (s->lean && mode == SAVE_ALL) {
-			for (int id = 0; id < B_COUNT; id++)
-				if ((REFORM_MASK & (1u << id)) && bs.b[id].p && bs.b[id].owned) {
-					buf_free(s, bs, id);
-					bs.b[id].dropped = true;
-				}
-		}
+		else if (s->lean && mode == SAVE_ALL) drop(bs, REFORM_MASK);
 	}
 	if (s->vocab_out) {
 		// last stage: (final norm,) logits = h W_head^T   (benchmarks/models/simple.py:497, 508)
@@ -268,6 +289,7 @@ static int run_forward(Stage* s, MbState& m, const void* x, void* y, FwdMode mod
 			ELF_TRY(norm_fwd(norm_kind, hd.b[B_X].p, s->xw[XP_FNORM_G], s->xw[XP_FNORM_B], hd.b[B_H1].p, hd.b[B_ST1].p, T, d, s->cfg.eps, st));
 		}
 		ELF_TRY(gemm_bf16(0, 0, T, s->vld, d, hd.b[B_H1].p, d, s->xw[XP_HEAD], d, y, s->vld, EPI_BF16, nullptr, 0, 0, 0, st));
+		if (remat_drop) drop(hd, remat_drop & (1u << B_ST1));
 		if (mode != SAVE_ALL) {
 			const unsigned keep = mode == SAVE_WIN ? WIN_MASK : 0u;
 			for (int id = 0; id < B_COUNT; id++)
@@ -300,12 +322,15 @@ static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool gra
 		BlockState& last = m.blk[nb - 1];
 		ELF_TRY(buf_alloc(s, last, B_DY));
 		if (s->final_norm) {
-			void* d_hn = s->pool.alloc((size_t)T * d * 2);
-			if (!d_hn) return -3;
-			ELF_TRY(gemm_bf16(0, 1, T, d, s->vld, dy, s->vld, s->xw[XP_HEAD], d, d_hn, d, EPI_BF16, nullptr, 0, 0, 0, st));
-			ELF_TRY(norm_bwd(norm_kind, d_hn, hd.b[B_X].p, s->xw[XP_FNORM_G], hd.b[B_ST1].p, nullptr, last.b[B_DY].p,
+			if (hd.b[B_ST1].dropped) {  // the final norm was checkpointed: run it again for its statistics
+				ELF_TRY(buf_alloc(s, hd, B_ST1));
+				ELF_TRY(norm_fwd(norm_kind, hd.b[B_X].p, s->xw[XP_FNORM_G], s->xw[XP_FNORM_B], hd.b[B_H1].p, hd.b[B_ST1].p, T, d, s->cfg.eps, st));
+			}
+			PoolTmp d_hn(s->pool, (size_t)T * d * 2);
+			if (!d_hn.p) return -3;
+			ELF_TRY(gemm_bf16(0, 1, T, d, s->vld, dy, s->vld, s->xw[XP_HEAD], d, d_hn.p, d, EPI_BF16, nullptr, 0, 0, 0, st));
+			ELF_TRY(norm_bwd(norm_kind, d_hn.p, hd.b[B_X].p, s->xw[XP_FNORM_G], hd.b[B_ST1].p, nullptr, last.b[B_DY].p,
 			                 grads_only ? s->dummy_grad : s->xg[XP_FNORM_G], grads_only ? s->dummy_grad + d : s->xg[XP_FNORM_B], s->norm_ws, T, d, st));
-			s->pool.free(d_hn);
 		} else {
 			ELF_TRY(gemm_bf16(0, 1, T, d, s->vld, dy, s->vld, s->xw[XP_HEAD], d, last.b[B_DY].p, d, EPI_BF16, nullptr, 0, 0, 0, st));
 		}
@@ -330,38 +355,39 @@ static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool gra
 		if (s->llama && !pre && gemm_swiglu_bwd_fused(T, F, d)) {
 			ELF_TRY(gemm_swiglu_bwd_bf16(T, F, d, dyin, d, p.w[P_W2], F, bs.b[B_GU].p, s->ffn_in, bs.b[B_DGU].p, s->ffn_in, nullptr, st));
 		} else {
-			void* d_a = s->pool.alloc((size_t)T * F * 2);
-			if (!d_a) return -3;
-			ELF_TRY(gemm_bf16(0, 1, T, F, d, dyin, d, p.w[P_W2], F, d_a, F, EPI_BF16, nullptr, 0, 0, 0, st));
+			PoolTmp d_a(s->pool, (size_t)T * F * 2);
+			if (!d_a.p) return -3;
+			ELF_TRY(gemm_bf16(0, 1, T, F, d, dyin, d, p.w[P_W2], F, d_a.p, F, EPI_BF16, nullptr, 0, 0, 0, st));
 			if (pre) ELF_CHECK_HIP(hipStreamWaitEvent(st, bs.pre_ffn, 0));
-			if (s->llama) ELF_TRY(swiglu_bwd(d_a, bs.b[B_GU].p, bs.b[B_DGU].p, T, F, st));
-			else ELF_TRY(gelu_bwd(d_a, bs.b[B_GU].p, bs.b[B_DGU].p, (int64_t)T * F, st));
-			s->pool.free(d_a);
+			if (s->llama) ELF_TRY(swiglu_bwd(d_a.p, bs.b[B_GU].p, bs.b[B_DGU].p, T, F, st));
+			else ELF_TRY(gelu_bwd(d_a.p, bs.b[B_GU].p, bs.b[B_DGU].p, (int64_t)T * F, st));
 		}
 		if (reform && bs.b[B_A].dropped) {
 			ELF_TRY(buf_alloc(s, bs, B_A));
 			if (s->llama) ELF_TRY(swiglu_fwd(bs.b[B_GU].p, bs.b[B_A].p, T, F, st));
 			else ELF_TRY(gelu_fwd(bs.b[B_GU].p, bs.b[B_A].p, (int64_t)T * F, st));
 		}
-		void* d_h = s->pool.alloc((size_t)T * d * 2);
-		if (!d_h) return -3;
-		ELF_TRY(gemm_bf16(0, 1, T, d, s->ffn_in, bs.b[B_DGU].p, s->ffn_in, p.w[P_W1], d, d_h, d, EPI_BF16, nullptr, 0, 0, 0, st));
+		PoolTmp d_h(s->pool, (size_t)T * d * 2);
+		if (!d_h.p) return -3;
+		ELF_TRY(gemm_bf16(0, 1, T, d, s->ffn_in, bs.b[B_DGU].p, s->ffn_in, p.w[P_W1], d, d_h.p, d, EPI_BF16, nullptr, 0, 0, 0, st));
 		ELF_TRY(buf_alloc(s, bs, B_DX2));
 		if (pre) ELF_CHECK_HIP(hipStreamWaitEvent(st, bs.pre_x2, 0));
-		if (reform && bs.b[B_H2].dropped) {
+		if ((reform && bs.b[B_H2].dropped) || bs.b[B_ST2].dropped) {  // dropped by the lean stash / offload, or a checkpointed norm
 			ELF_TRY(buf_alloc(s, bs, B_H2));
+			ELF_TRY(buf_alloc(s, bs, B_ST2));
 			ELF_TRY(norm_fwd(norm_kind, bs.b[B_X2].p, p.w[P_NORM2_G], p.w[P_NORM2_B], bs.b[B_H2].p, bs.b[B_ST2].p, T, d, s->cfg.eps, st));
 		}
-		ELF_TRY(norm_bwd(norm_kind, d_h, bs.b[B_X2].p, p.w[P_NORM2_G], bs.b[B_ST2].p, dyin, bs.b[B_DX2].p,
+		ELF_TRY(norm_bwd(norm_kind, d_h.p, bs.b[B_X2].p, p.w[P_NORM2_G], bs.b[B_ST2].p, dyin, bs.b[B_DX2].p,
 		                 grads_only ? s->dummy_grad : p.g[P_NORM2_G], grads_only ? s->dummy_grad + d : p.g[P_NORM2_B], s->norm_ws, T, d, st));
 		// attention
-		void* d_o = s->pool.alloc((size_t)T * s->Hq * s->D * 2);
-		if (!d_o) return -3;
-		ELF_TRY(gemm_bf16(0, 1, T, s->Hq * s->D, d, bs.b[B_DX2].p, d, p.w[P_WO], s->Hq * s->D, d_o, s->Hq * s->D, EPI_BF16, nullptr, 0, 0, 0, st));
+		PoolTmp d_o(s->pool, (size_t)T * s->Hq * s->D * 2);
+		if (!d_o.p) return -3;
+		ELF_TRY(gemm_bf16(0, 1, T, s->Hq * s->D, d, bs.b[B_DX2].p, d, p.w[P_WO], s->Hq * s->D, d_o.p, s->Hq * s->D, EPI_BF16, nullptr, 0, 0, 0, st));
 		ELF_TRY(buf_alloc(s, bs, B_DQKV));
 		if (pre) ELF_CHECK_HIP(hipStreamWaitEvent(st, bs.pre_ev, 0));
-		if (bs.b[B_H1].dropped && (reform || bs.b[B_QKV].dropped)) {
+		if ((bs.b[B_H1].dropped && (reform || bs.b[B_QKV].dropped)) || bs.b[B_ST1].dropped) {
 			ELF_TRY(buf_alloc(s, bs, B_H1));
+			ELF_TRY(buf_alloc(s, bs, B_ST1));
 			ELF_TRY(norm_fwd(norm_kind, bs.b[B_X].p, p.w[P_NORM1_G], p.w[P_NORM1_B], bs.b[B_H1].p, bs.b[B_ST1].p, T, d, s->cfg.eps, st));
 		}
 		if (bs.b[B_QKV].dropped) {
@@ -369,23 +395,29 @@ static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool gra
 			ELF_TRY(gemm_bf16(0, 0, T, s->nqkv, d, bs.b[B_H1].p, d, p.w[P_WQKV], d, bs.b[B_QKV].p, s->nqkv, EPI_BF16, nullptr, 0, 0, 0, st));
 			if (s->llama) ELF_TRY(rope_apply(bs.b[B_QKV].p, s->rope_cs, T, s->S, s->nqkv, s->Hq + s->Hkv, s->D, 0, st));
 		}
+		if (bs.b[B_LSE].dropped) {  // checkpointed attention core: its output and log-sum-exp are formed again
+			ELF_TRY(buf_alloc(s, bs, B_O));
+			ELF_TRY(buf_alloc(s, bs, B_LSE));
+			const bf16_t* q = (const bf16_t*)bs.b[B_QKV].p;
+			ELF_TRY(attn_fwd(q, q + s->Hq * s->D, q + (s->Hq + s->Hkv) * s->D, bs.b[B_O].p, bs.b[B_LSE].p, s->nqkv, s->nqkv, s->nqkv,
+			                 s->Hq * s->D, s->B, s->S, s->Hq, s->Hkv, s->D, s->cfg.causal, scale, st));
+		}
 		{
 			const bf16_t* q = (const bf16_t*)bs.b[B_QKV].p;
 			bf16_t* dq = (bf16_t*)bs.b[B_DQKV].p;
 			const int ko = s->Hq * s->D, vo = (s->Hq + s->Hkv) * s->D;
-			ELF_TRY(attn_bwd(q, q + ko, q + vo, bs.b[B_O].p, d_o, bs.b[B_LSE].p, dq, dq + ko, dq + vo, s->attn_ws, s->nqkv, s->nqkv, s->nqkv,
+			ELF_TRY(attn_bwd(q, q + ko, q + vo, bs.b[B_O].p, d_o.p, bs.b[B_LSE].p, dq, dq + ko, dq + vo, s->attn_ws, s->nqkv, s->nqkv, s->nqkv,
 			                 s->Hq * s->D, s->Hq * s->D, s->nqkv, s->nqkv, s->nqkv, s->B, s->S, s->Hq, s->Hkv, s->D, s->cfg.causal, scale, st));
 		}
-		s->pool.free(d_o);
+		d_o.release();
 		if (s->llama) ELF_TRY(rope_apply(bs.b[B_DQKV].p, s->rope_cs, T, s->S, s->nqkv, s->Hq + s->Hkv, s->D, 1, st));
 		if (!(grads_only && i == 0)) {
-			ELF_TRY(gemm_bf16(0, 1, T, d, s->nqkv, bs.b[B_DQKV].p, s->nqkv, p.w[P_WQKV], d, d_h, d, EPI_BF16, nullptr, 0, 0, 0, st));
+			ELF_TRY(gemm_bf16(0, 1, T, d, s->nqkv, bs.b[B_DQKV].p, s->nqkv, p.w[P_WQKV], d, d_h.p, d, EPI_BF16, nullptr, 0, 0, 0, st));
 			void* dxout;
-			void* d_emb = nullptr;
+			PoolTmp d_emb(s->pool, i == 0 && s->vocab_in ? (size_t)T * d * 2 : 0);
 			if (i == 0 && s->vocab_in) {
-				d_emb = s->pool.alloc((size_t)T * d * 2);
-				if (!d_emb) return -3;
-				dxout = d_emb;
+				if (!d_emb.p) return -3;
+				dxout = d_emb.p;
 			} else if (i == 0) {
 				dxout = dx;
 			} else {
@@ -393,15 +425,13 @@ static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool gra
 				ELF_TRY(buf_alloc(s, pv, B_DY));
 				dxout = pv.b[B_DY].p;
 			}
-			ELF_TRY(norm_bwd(norm_kind, d_h, bs.b[B_X].p, p.w[P_NORM1_G], bs.b[B_ST1].p, bs.b[B_DX2].p, dxout,
+			ELF_TRY(norm_bwd(norm_kind, d_h.p, bs.b[B_X].p, p.w[P_NORM1_G], bs.b[B_ST1].p, bs.b[B_DX2].p, dxout,
 			                 grads_only ? s->dummy_grad : p.g[P_NORM1_G], grads_only ? s->dummy_grad + d : p.g[P_NORM1_B], s->norm_ws, T, d, st));
-			if (d_emb) {
+			if (i == 0 && s->vocab_in) {
 				// first stage: the embedding is not a split layer, its gradient accumulates inside B
-				if (!grads_only) ELF_TRY(embedding_bwd(m.ids, d_emb, s->xg[XP_EMBED], T, d, s->vocab_in, st));
-				s->pool.free(d_emb);
+				if (!grads_only) ELF_TRY(embedding_bwd(m.ids, d_emb.p, s->xg[XP_EMBED], T, d, s->vocab_in, st));
 			}
 		}
-		s->pool.free(d_h);
 		// B consumed the activation stash; what is left is the W stash
 		for (int id = 0; id < B_COUNT; id++)
 			if ((ACT_MASK & (1u << id)) && !(WIN_MASK & (1u << id))) buf_free(s, bs, id);
@@ -607,6 +637,7 @@ void elf_stage_destroy(elf_stage_t* h) {
 	if (!h) return;
 	Stage* s = (Stage*)h;
 	(void)hipDeviceSynchronize();
+	s->pool.drain();  // blocks waiting on per-block copy events go back before those events are destroyed
 	for (auto& kv : s->mbs) {
 		do_release(s, kv.second);
 		free_mask(s, kv.second, ~0u);
@@ -695,8 +726,9 @@ int elf_stage_forward(elf_stage_t* h, int mb, const void* x, void* y, uint32_t f
 	MbState& m = mb_state(s, mb);
 	ELF_REQUIRE(!m.has_acts && !m.has_win && !m.has_wgrad && !m.remat_root, "elf_stage_forward: micro-batch %d is already in flight", mb);
 	use_mb(s, mb);
+	ELF_REQUIRE(!(flags & ~(ELF_FWD_REMAT_ROOT | ELF_FWD_REMAT_ATTN | ELF_FWD_OFFLOAD | ELF_FWD_REMAT_NORM)), "elf_stage_forward: unknown flag bits 0x%x", flags);
 	const bool root = flags & ELF_FWD_REMAT_ROOT;
-	ELF_TRY(run_forward(s, m, x, y, root ? SAVE_NONE : SAVE_ALL, (hipStream_t)stream, (flags & ELF_FWD_OFFLOAD) && !root));
+	ELF_TRY(run_forward(s, m, x, y, root ? SAVE_NONE : SAVE_ALL, (hipStream_t)stream, (flags & ELF_FWD_OFFLOAD) && !root, root ? 0u : flags));
 	m.remat_root = root;
 	if (root) m.has_win = false;
 	return 0;
@@ -727,7 +759,11 @@ int elf_stage_backward_inputs(elf_stage_t* h, int mb, const void* x, const void*
 	if (x && s->vocab_in) m.ids = x;
 	else if (x) m.blk[0].b[B_X].p = const_cast<void*>(x);
 	// the W-stash inputs are dropped below: no point in forming the ones F or the offload left out
-	ELF_TRY(run_backward(s, m, dy, dx, false, st, !(flags & ELF_BWD_RECOMPUTE_ACTIVATIONS)));
+	if (int rc = run_backward(s, m, dy, dx, false, st, !(flags & ELF_BWD_RECOMPUTE_ACTIVATIONS))) {
+		free_mask(s, m, WGRAD_MASK);  // half-written output gradients are of no use to W
+		m.has_wgrad = false;
+		return rc;
+	}
 	if (flags & ELF_BWD_RECOMPUTE_GRADIENTS) free_mask(s, m, WGRAD_MASK), m.has_wgrad = false;
 	if (flags & ELF_BWD_RECOMPUTE_ACTIVATIONS) free_mask(s, m, WIN_MASK), m.has_win = false;
 	return 0;
@@ -801,6 +837,7 @@ int elf_stage_clear(elf_stage_t* h) {
 	Stage* s = (Stage*)h;
 	ELF_REQUIRE(s, "elf_stage_clear: null stage");
 	ELF_CHECK_HIP(hipDeviceSynchronize());
+	s->pool.drain();  // blocks waiting on per-block copy events go back before those events are destroyed
 	for (auto& kv : s->mbs) {
 		ELF_TRY(do_release(s, kv.second));
 		free_mask(s, kv.second, ~0u);
@@ -814,6 +851,7 @@ int elf_stage_clear(elf_stage_t* h) {
 int elf_stage_mem_stats(elf_stage_t* h, elf_mem_stats* out) {
 	Stage* s = (Stage*)h;
 	ELF_REQUIRE(s && out, "elf_stage_mem_stats: null argument");
+	s->pool.poll();  // buffers whose copy to the host has finished no longer count as live
 	out->live_bytes = (int64_t)s->pool.live_bytes();
 	out->peak_bytes = (int64_t)s->pool.peak_bytes();
 	out->reserved_bytes = (int64_t)s->pool.reserved_bytes();

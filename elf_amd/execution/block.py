@@ -112,7 +112,7 @@ for _name, _ret, _args in [
 	_lib.register(_name, _ret, _args)
 
 ARCH_GPT, ARCH_LLAMA = 0, 1
-FWD_REMAT_ROOT, FWD_OFFLOAD = 1, 4
+FWD_REMAT_ROOT, FWD_REMAT_ATTN, FWD_OFFLOAD, FWD_REMAT_NORM = 1, 2, 4, 8
 BWD_RECOMPUTE_ACTIVATIONS, BWD_RECOMPUTE_GRADIENTS = 1, 2
 # parameter ids of elf_stage_bind_param
 P_NORM1_G, P_NORM1_B, P_WQKV, P_WO, P_NORM2_G, P_NORM2_B, P_W1, P_W2 = range(8)
@@ -159,6 +159,7 @@ class HipStageBlock:
 		self._handle = None
 		self._samples = {}  # mb -> sequences in it, where fewer than mb_size
 		self._kept = {}  # mb -> external tensors the library still points at (x until B/recompute, dy until W)
+		self._remat_cache = {}  # id(strategy) -> (strategy, forward flags)
 		self.lean_stash = bool(lean_stash)
 		self._build(mb_size, seq_len)
 
@@ -338,6 +339,48 @@ class HipStageBlock:
 		room = dy.untyped_storage().nbytes() // dy.element_size() - dy.storage_offset()
 		return room >= rows * self.vld
 
+	def _remat_flags(self, strategy):
+		"""Forward flags for a ``remat_strategy`` (elf/execution/remat.py:26-74: every module the strategy
+		selects runs under ``checkpoint``).  What this executor can express: the stage root (whole-stage
+		checkpoint), all attention cores, all norm modules; an activation module (``nn.GELU``) may be
+		selected too and changes nothing, because the only tensor it would keep is its own input, which the
+		stash holds as the FFN pre-activation either way; ``nn.Dropout`` modules do not occur in these
+		blocks.  A strategy that selects nothing runs a plain forward, as in the reference.  Anything else
+		(single blocks, linears, some but not all modules of a kind) raises: a remat decision is never
+		dropped silently."""
+		if strategy is None:
+			return 0
+		key = id(strategy)
+		cached = self._remat_cache.get(key)
+		if cached is not None and cached[0] is strategy:
+			return cached[1]
+		named = list(self.model.named_modules())
+		selected = [(n, m) for n, m in named if strategy(n, m)]
+		if any(n == "" for n, _ in selected):
+			flags = FWD_REMAT_ROOT
+		else:
+			norms, cores, acts = set(), set(), set()
+			for b in self.blocks:
+				norms.update((id(b.norm1), id(b.norm2)))
+				cores.add(id(b.attn.attn))
+				if hasattr(b.mlp, "activation"):
+					acts.add(id(b.mlp.activation))
+			if self.ends is not None and self.ends.norm_f is not None:
+				norms.add(id(self.ends.norm_f))
+			chosen = {id(m) for _, m in selected}
+			flags = 0
+			for group, flag in ((norms, FWD_REMAT_NORM), (cores, FWD_REMAT_ATTN), (acts, 0)):
+				hit = chosen & group
+				if hit and hit != group:
+					raise _lib.ElfStageError(f"{self}: remat_strategy selects some but not all modules of one kind; this executor checkpoints a kind of module for the whole stage")
+				if hit:
+					flags |= flag
+			other = [n for n, m in selected if id(m) not in norms | cores | acts]
+			if other:
+				raise _lib.ElfStageError(f"{self}: remat_strategy selects {other[:4]}; this executor can checkpoint the stage root, the attention cores and the norm modules")
+		self._remat_cache[key] = (strategy, flags)
+		return flags
+
 	def _timed(self, name):
 		t = Timer(name=name)
 		self.compute_time.append(t)
@@ -345,15 +388,13 @@ class HipStageBlock:
 
 	# ------------------------------------------------------------------ compute ops
 	def forward(self, mb_id, **options):
-		"""F.  Options: ``remat_strategy`` (only a strategy that selects the stage root changes what
-		is kept: whole-stage checkpoint) and ``activation_offload`` (handled by the offloader the
-		engine wraps around this call)."""
+		"""F.  Options: ``remat_strategy`` (see ``_remat_flags``) and ``activation_offload`` (handled by
+		the offloader the engine wraps around this call)."""
 		var = self.input_variables[0]
 		x = var.wait_and_pop(mb_id)
 		self._set_samples(mb_id, x, self.seq if self.vocab_in else self.seq * self.d)
 		x = self._check_ids(x, mb_id) if self.vocab_in else self._check_io(x, "stage input", mb_id)
-		strategy = options.get(OpOptions.REMAT_STRATEGY)
-		flags = FWD_REMAT_ROOT if (strategy is not None and strategy("", self.model)) else 0
+		flags = self._remat_flags(options.get(OpOptions.REMAT_STRATEGY))
 		ybuf, y = self._new_output(x, mb_id)
 		with self._timed(f"forward({self.id}:{mb_id})"):
 			_lib.check(self.lib.elf_stage_forward(self._handle, mb_id, x.data_ptr(), ybuf.data_ptr(), flags, _stream()), "elf_stage_forward")
@@ -457,7 +498,7 @@ class HipStageBlock:
 		self.sent_forward, self.sent_backward = {}, {}
 
 	def _remote(self, peer):
-		return peer is not None and self.placement[peer] != self.rank
+		return peer is not None and self.placement[peer] != self.rank and peer not in getattr(self, "local_ids", ())
 
 	def _need_feed(self, feed, what):
 		if feed is None:

@@ -52,11 +52,13 @@ class Engine:
 	"""Runs a list of operations on the blocks of one rank; feeds the pipeline input to the first
 	block and computes the loss on the last one."""
 
-	def __init__(self, blocks):
+	def __init__(self, blocks, all_ranks=False):
+		"""``all_ranks``: the blocks belong to several ranks of the placement that this one process plays
+		(``Pipeline(all_ranks=True)``); the schedule must then come in an order one process can run."""
 		self.blocks = blocks
 		self.rank = blocks[0].rank if blocks else None
 		for b in blocks:
-			assert b.rank == self.rank, "All blocks in a stage should be on the same rank"
+			assert all_ranks or b.rank == self.rank, "All blocks in a stage should be on the same rank"
 		self.id_to_block = {b.id: b for b in blocks}
 		self.offload_stream = torch.cuda.Stream() if _GPU() else None
 		self.pool = None  # the pinned arena lives in the stage library

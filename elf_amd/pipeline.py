@@ -13,6 +13,10 @@ What differs, because this build runs one process on one GPU: the stages this pr
 arrive already partitioned (``partitioner=False``: tracing and graph partitioning are not part of
 this path), every stage of the placement must live on this process' rank (stages on the same rank
 hand tensors over locally, as in the reference engine), and no process groups are created.
+``all_ranks=True`` lets the one process play every rank of a placement such as ``[0, 1]``: it owns
+all stages, hands boundary tensors over locally and interprets the ops of all ranks in an order in
+which every rank keeps its own op order and no compute op runs before the data it consumes was sent
+(``sequential_order``), so that a schedule written for several devices runs on one.
 """
 
 import logging
@@ -26,13 +30,52 @@ import torch.distributed as dist
 from .execution import Engine, HipStageBlock
 from .partitioners.utils import Signature, sequential_signatures
 from .registry import COMM_SCHEDULERS, PARTITIONERS, SCHEDULERS, TRACERS, resolve
-from .scheduling import add_comms, check_schedule_validity, schedule_to_str
+from .scheduling import OperationType, add_comms, check_schedule_validity, schedule_to_str
 from .scheduling.ilp import AutoScheduler, profile_stage, stagerematify
 from .utils import Placement
 
 logger = logging.getLogger("pipeline")
 
-__all__ = ["Pipeline", "PipelineConfig"]
+__all__ = ["Pipeline", "PipelineConfig", "sequential_order"]
+
+
+def sequential_order(schedule, signatures):
+	"""One order in which a single process can run the ops of every rank of ``schedule``.
+
+	Each rank's ops keep their relative order.  Receives are posts (``irecv`` in the reference,
+	block.py:420-446) and never block; a FORWARD waits until every producer of the block's inputs has
+	emitted its SEND_FORWARD for that micro-batch, a BACKWARD_INPUTS until every consumer of its
+	outputs has emitted its SEND_BACKWARD: what ``Variable.wait_and_pop`` waits for.  Ranks are served
+	round-robin, each running until its next op has to wait.  Raises if the schedule deadlocks."""
+	T = OperationType
+	ranks = sorted({op.rank for op in schedule})
+	queues = {r: [op for op in schedule if op.rank == r] for r in ranks}
+	heads = {r: 0 for r in ranks}
+	sent = set()  # (kind, producing block, consuming block, micro-batch)
+
+	def ready(op):
+		sig = signatures[op.block_id]
+		if op.op == T.FORWARD:
+			return all((T.SEND_FORWARD, src, op.block_id, op.mb_id) in sent for src in sig.get_all_sources() if src is not None)
+		if op.op == T.BACKWARD_INPUTS:
+			return all((T.SEND_BACKWARD, dst, op.block_id, op.mb_id) in sent for dst in sig.get_all_targets() if dst is not None)
+		return True
+
+	out = []
+	while any(heads[r] < len(queues[r]) for r in ranks):
+		progressed = False
+		for r in ranks:
+			while heads[r] < len(queues[r]) and ready(queues[r][heads[r]]):
+				op = queues[r][heads[r]]
+				heads[r] += 1
+				if op.op in (T.SEND_FORWARD, T.SEND_BACKWARD):
+					sent.add((op.op, op.block_id, op.options.get("dst"), op.mb_id))
+				out.append(op)
+				progressed = True
+		if not progressed:
+			stuck = {r: str(queues[r][heads[r]]) for r in ranks if heads[r] < len(queues[r])}
+			raise RuntimeError(f"sequential_order: the schedule deadlocks, every rank waits: {stuck}")
+	return out
 
 
 @dataclass
@@ -77,16 +120,23 @@ class Pipeline:
 	``StageModule``) or the list of stage modules this rank owns, in block-id order.  ``sample`` has
 	the shape of one micro-batch ``[mb, seq, d_model]`` (or pass ``mb_size=``)."""
 
-	def __init__(self, model, sample=None, *, config=None, mb_size=None, **kwargs):
+	def __init__(self, model, sample=None, *, config=None, mb_size=None, all_ranks=False, **kwargs):
 		ws, rank = _world()
 		if ws == 1 and not (dist.is_available() and dist.is_initialized()):
 			logger.warning("Trying to create a pipeline but no multi-gpu distributed setup has been found.")
 		self.cfg = (config or PipelineConfig(**kwargs)).resolve()
-		self.pp = self.cfg.pp or ws // self.cfg.dp
-		self.dp = self.cfg.dp
-		assert self.pp * self.dp == ws, f"Requested PP = {self.pp}, DP = {self.dp} need {self.pp * self.dp} processes, but {ws} were spawned"
+		self.all_ranks = bool(all_ranks)
 		if ws != 1:
 			raise NotImplementedError("this build runs the stages of one process on one GPU: start it with a world size of 1")
+		if self.all_ranks:
+			if self.cfg.placement == "auto" and not self.cfg.pp:
+				raise ValueError("Pipeline(all_ranks=True) needs an explicit placement or pp")
+			self.pp = self.cfg.pp or len(set(self.cfg.placement))
+			self.dp = 1
+		else:
+			self.pp = self.cfg.pp or ws // self.cfg.dp
+			self.dp = self.cfg.dp
+			assert self.pp * self.dp == ws, f"Requested PP = {self.pp}, DP = {self.dp} need {self.pp * self.dp} processes, but {ws} were spawned"
 		self.rank = rank
 		if self.cfg.placement == "auto":
 			try:
@@ -112,7 +162,7 @@ class Pipeline:
 			mb_size = (sample[0] if isinstance(sample, (list, tuple)) else sample).size(0)
 		self.mb_size = int(mb_size)
 		self.blocks = self._create_pipeline(parts, signatures)
-		self.engine = Engine(self.blocks)
+		self.engine = Engine(self.blocks, all_ranks=self.all_ranks)
 		self.schedule = []
 		self.last_nmb = 0
 		self.stats, self.detailed_stats = None, None
@@ -253,10 +303,10 @@ class Pipeline:
 			logger.info(f"Saved model to {path}")
 
 	def is_first(self):
-		return self.placement.is_head(self.rank)
+		return self.all_ranks or self.placement.is_head(self.rank)
 
 	def is_last(self):
-		return self.placement.is_tail(self.rank)
+		return self.all_ranks or self.placement.is_tail(self.rank)
 
 	def get_profiling_statistics(self):
 		if not self._remat_stats:
@@ -288,6 +338,8 @@ class Pipeline:
 		check_schedule_validity(schedule)
 		if self.rank == 0:
 			logger.debug(f"Schedule:\n{schedule_to_str(schedule)}")
+		if self.all_ranks:
+			schedule = sequential_order(schedule, self.signatures)
 		ids = [b.id for b in self.blocks]
 		self.schedule = [op for op in schedule if op.block_id in ids]
 
@@ -304,8 +356,12 @@ class Pipeline:
 		return parts, signatures
 
 	def _create_pipeline(self, parts, signatures):
-		ids = self.placement.get_ids(self.rank)
+		ids = list(range(len(self.placement))) if self.all_ranks else self.placement.get_ids(self.rank)
 		assert len(parts) == len(ids), f"rank {self.rank} owns blocks {ids} of placement {list(self.placement)} but got {len(parts)} stage module(s)"
 		# under a memory budget the stages hold the lean stash: the remat ILP then starts from a third less per micro-batch
 		lean = self.cfg.memory_budget is not None
-		return [HipStageBlock(part, i, self.placement, signatures[i], mb_size=self.mb_size, lean_stash=lean) for part, i in zip(parts, ids)]
+		blocks = [HipStageBlock(part, i, self.placement, signatures[i], mb_size=self.mb_size, lean_stash=lean) for part, i in zip(parts, ids)]
+		if self.all_ranks:
+			for b in blocks:
+				b.local_ids = set(ids)  # peers on other ranks of the placement are in this process too
+		return blocks

@@ -188,12 +188,22 @@ enum { ELF_P_NORM1_G = 0, ELF_P_NORM1_B, ELF_P_WQKV, ELF_P_WO, ELF_P_NORM2_G, EL
  *  11 output head [vocab_out_ld, d] (rows >= vocab_out are padding and must be zero) */
 enum { ELF_P_EMBED = 8, ELF_P_FNORM_G, ELF_P_FNORM_B, ELF_P_HEAD };
 
-/* Forward flags (FORWARD options, elf/scheduling/scheduling.py:58-86):
- *  REMAT_ROOT: remat_strategy selects the whole stage (name == ""), i.e. full checkpointing: only
- *              the stage input is kept and B re-runs the forward (elf/execution/remat.py:26-74);
+/* Forward flags (FORWARD options, elf/scheduling/scheduling.py:58-86).  remat_strategy selects modules
+ * whose forward runs under checkpoint(): what they keep for the backward is not kept, and the backward
+ * runs them again (elf/execution/remat.py:26-74).  The strategies the benchmarks build
+ * (benchmarks/benchmark_utils.py:295-335) map onto:
+ *  REMAT_ROOT: the whole stage (name == "", "full"): only the stage input is kept and B re-runs the
+ *              forward;
+ *  REMAT_ATTN: the attention cores ("selective"): the attention output and log-sum-exp of every block
+ *              are dropped after F and B runs the attention forward again from the kept q, k, v (same
+ *              kernel on the same inputs: bit-identical);
+ *  REMAT_NORM: the norm modules ("simple": LayerNorm; a GELU module keeps nothing but its own input, which
+ *              the FFN pre-activation stash holds either way): the per-row statistics of every norm are
+ *              dropped after F and B runs the norm forward again;
  *  OFFLOAD:    activation_offload: the stash goes to pinned host memory on a side stream
- *              (elf/execution/offload.py:228-268, 330-352). */
-enum { ELF_FWD_REMAT_ROOT = 1u, ELF_FWD_OFFLOAD = 4u };
+ *              (elf/execution/offload.py:228-268, 330-352).
+ * REMAT_ROOT overrides the other two. */
+enum { ELF_FWD_REMAT_ROOT = 1u, ELF_FWD_REMAT_ATTN = 2u, ELF_FWD_OFFLOAD = 4u, ELF_FWD_REMAT_NORM = 8u };
 /* BACKWARD_INPUTS flags: recompute_activations drops the W-stash inputs after B,
  * recompute_gradients drops the W-stash output gradients (elf/execution/block.py:659-694). */
 enum { ELF_BWD_RECOMPUTE_ACTIVATIONS = 1u, ELF_BWD_RECOMPUTE_GRADIENTS = 2u };

@@ -143,30 +143,39 @@ def attention(q, k, v, causal, use_sdpa=False):
 
 # --------------------------------------------------------------------------------------------
 # blocks.  `p` is a dict: norm weights are plain leaf tensors, linears are SplitLinear objects.
+# cfg["_ckpt"] (set per forward by RefStage) names the kinds of sub-module whose forward runs under
+# checkpoint(use_reentrant=False), as RematManager.apply_selective_remat wraps the modules a
+# remat_strategy selects (elf/execution/remat.py:42-58): "norm", "attn", "act".
+def _sub(cfg, kind, fn, *args):
+	if kind in cfg.get("_ckpt", ()):
+		return checkpoint(fn, *args, use_reentrant=False)
+	return fn(*args)
+
+
 def gpt_block(x, p, cfg, use_sdpa=False):
 	B, S, d = x.shape
 	H, D = cfg["n_heads"], cfg["head_dim"]
-	y = layer_norm(x, p["norm1_g"], p["norm1_b"], cfg["eps"])
+	y = _sub(cfg, "norm", layer_norm, x, p["norm1_g"], p["norm1_b"], cfg["eps"])
 	qkv = p["wqkv"](y)
 	q, k, v = qkv.split([H * D, H * D, H * D], dim=-1)
-	o = attention(q.reshape(B, S, H, D), k.reshape(B, S, H, D), v.reshape(B, S, H, D), cfg["causal"], use_sdpa)
+	o = _sub(cfg, "attn", attention, q.reshape(B, S, H, D), k.reshape(B, S, H, D), v.reshape(B, S, H, D), cfg["causal"], use_sdpa)
 	x2 = x + p["wo"](o.reshape(B, S, H * D))
-	y = layer_norm(x2, p["norm2_g"], p["norm2_b"], cfg["eps"])
-	return x2 + p["w2"](F.gelu(p["w1"](y)))
+	y = _sub(cfg, "norm", layer_norm, x2, p["norm2_g"], p["norm2_b"], cfg["eps"])
+	return x2 + p["w2"](_sub(cfg, "act", F.gelu, p["w1"](y)))
 
 
 def llama_block(x, p, cfg, use_sdpa=False):
 	B, S, d = x.shape
 	Hq, Hkv, D, Fh = cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"], cfg["ffn"]
 	cos, sin = cfg["_rope"]
-	y = rms_norm(x, p["norm1_g"], cfg["eps"])
+	y = _sub(cfg, "norm", rms_norm, x, p["norm1_g"], cfg["eps"])
 	qkv = p["wqkv"](y)
 	q, k, v = qkv.split([Hq * D, Hkv * D, Hkv * D], dim=-1)
 	q = rope(q.reshape(B, S, Hq, D), cos, sin)
 	k = rope(k.reshape(B, S, Hkv, D), cos, sin)
-	o = attention(q, k, v.reshape(B, S, Hkv, D), cfg["causal"], use_sdpa)
+	o = _sub(cfg, "attn", attention, q, k, v.reshape(B, S, Hkv, D), cfg["causal"], use_sdpa)
 	x2 = x + p["wo"](o.reshape(B, S, Hq * D))
-	y = rms_norm(x2, p["norm2_g"], cfg["eps"])
+	y = _sub(cfg, "norm", rms_norm, x2, p["norm2_g"], cfg["eps"])
 	gu = p["w1"](y)
 	return x2 + p["w2"](F.silu(gu[..., :Fh]) * gu[..., Fh:])
 
@@ -256,7 +265,10 @@ class RefStage:
 			x = self.block_fn(x, b, self.cfg, self.use_sdpa)
 		if "normf_g" in self.ends:
 			e = self.ends
-			x = rms_norm(x, e["normf_g"], self.cfg["eps"]) if self.cfg["arch"] == ARCH_LLAMA else layer_norm(x, e["normf_g"], e["normf_b"], self.cfg["eps"])
+			if self.cfg["arch"] == ARCH_LLAMA:
+				x = _sub(self.cfg, "norm", rms_norm, x, e["normf_g"], self.cfg["eps"])
+			else:
+				x = _sub(self.cfg, "norm", layer_norm, x, e["normf_g"], e["normf_b"], self.cfg["eps"])
 		if "head" in self.ends:
 			x = self.ends["head"](x)
 		return x
@@ -267,9 +279,12 @@ class RefStage:
 		return x.to(device=self.device, dtype=self.compute_dtype).detach().requires_grad_(True)
 
 	# F (block.py:210-263)
-	def forward(self, mb, x, remat_root=False):
+	def forward(self, mb, x, remat_root=False, remat=()):
+		"""``remat``: kinds of sub-module ("norm", "attn", "act") checkpointed in this forward."""
 		x = self._as_input(x)
+		self.cfg["_ckpt"] = tuple(remat)
 		y = checkpoint(self._model, x, use_reentrant=False) if remat_root else self._model(x)
+		self.cfg["_ckpt"] = ()
 		for lin in self._linears():
 			lin.move_last("input", mb)
 			if remat_root:

@@ -36,14 +36,33 @@ from elf.scheduling.ilp import RematScheduler  # noqa: E402
 from elf.partitioners.utils import sequential_signatures  # noqa: E402
 
 
+def probes():
+	"""(label, module name, module) triples a remat strategy is evaluated on: the stage root, a
+	sub-module name without a module, and one instance of each module class the benchmark's
+	strategies look at (plus a Linear, which none of them selects)."""
+	import torch.nn as nn
+	from models.simple import Attention, FastAttention
+
+	return [
+		("root", "", None), ("x", "x", None), ("gelu", "mlp.activation", nn.GELU()), ("layernorm", "norm1", nn.LayerNorm(4)),
+		("dropout", "dropout", nn.Dropout()), ("linear", "proj", nn.Linear(2, 2)), ("attention", "attn.attn", Attention(8)),
+		("fastattention", "attn.attn", FastAttention(8)),
+	]
+
+
+PROBES = None
+
+
 def enc(op):
-	"""[OperationType value, block, mb, rank(, {option: value})]; a callable option value is
-	replaced by "fn:" + the names it selects among ("", "x") - "fn:" + "" means root only."""
+	"""[OperationType value, block, mb, rank(, {option: value})]; a callable option value (a remat
+	strategy) is replaced by "fn:" + the labels of the probes it selects, e.g. "fn:root"."""
+	global PROBES
 	opts = {}
 	for k, v in op.options.items():
 		k = str(k.value) if hasattr(k, "value") else str(k)
 		if callable(v):
-			v = "fn:" + ",".join(n for n in ("", "x") if v(n, None))
+			PROBES = PROBES or probes()
+			v = "fn:" + ",".join(label for label, name, module in PROBES if v(name, module))
 		opts[k] = v
 	rec = [op.op.value, op.block_id, op.mb_id, op.rank]
 	return rec + [opts] if opts else rec
@@ -92,7 +111,8 @@ for sched, placement, nmb, ratio, pt in [("1f1b", [0, 1, 2, 3], 8, 1, 1), ("1f1b
 	add(f"offload:{sched}", get_offloaded_scheduler(sched, ratio, pt)(placement, nmb), scheduler=sched, placement=placement, nmb=nmb, ratio=ratio, prefetching_time=pt)
 s = add_comms(get_offloaded_scheduler("1f1b", 1, 1)([0, 1, 2, 3], 8), sequential_signatures([0, 1, 2, 3]))
 add("offload+comm:1f1b", COMM_SCHEDULERS["pipelined"](s), scheduler="1f1b", placement=[0, 1, 2, 3], nmb=8, ratio=1, prefetching_time=1, comm="pipelined")
-add("ckpt:full", get_checkpointed_scheduler("1f1b", "full")([0, 1], 2), scheduler="1f1b", placement=[0, 1], nmb=2, type="full")
+for kind in ("full", "simple", "selective"):
+	add(f"ckpt:{kind}", get_checkpointed_scheduler("1f1b", kind)([0, 1], 2), scheduler="1f1b", placement=[0, 1], nmb=2, type=kind)
 
 out = os.path.join(os.path.dirname(os.path.abspath(__file__)), "schedule_vectors.json")
 with open(out, "w") as f:

@@ -73,3 +73,16 @@ def assert_close(got, ref, what, rel_max=2e-2, rel_fro=1e-2):
 	assert err <= rel_max * scale, f"{what}: max abs err {err:.4g} > {rel_max} * {scale:.4g}"
 	assert fro <= rel_fro, f"{what}: relative Frobenius error {fro:.4g} > {rel_fro}"
 	return err / scale, fro
+
+
+def assert_close_dev(got, ref, what, rel_max=2e-2, rel_fro=1e-2):
+	"""``assert_close`` without leaving the device (for tensors of hundreds of MB)."""
+	assert got.shape == ref.shape, f"{what}: shape {tuple(got.shape)} vs {tuple(ref.shape)}"
+	diff = got.float() - ref.float()
+	assert torch.isfinite(diff).all().item(), f"{what}: non-finite values"
+	scale = ref.abs().max().item() + 1e-12
+	err = diff.abs().max().item()
+	fro = (diff.double().norm() / (ref.double().norm() + 1e-12)).item()
+	assert err <= rel_max * scale, f"{what}: max abs err {err:.4g} > {rel_max} * {scale:.4g}"
+	assert fro <= rel_fro, f"{what}: relative Frobenius error {fro:.4g} > {rel_fro}"
+	return err / scale, fro

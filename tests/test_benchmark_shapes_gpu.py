@@ -1,0 +1,175 @@
+"""Whole stages at the shapes the benchmark workloads run, through the C ABI (HipStageBlock), against the
+oracle stage (oracle/stage_ref.py) in fp32 on the GPU from the same bf16-rounded weights and boundary
+tensors: one block, one micro-batch, F -> B -> W, every output compared (y, dX, every fp32 dW / dgamma).
+
+  llama3_8b   4096 wide, 32 query / 8 kv heads of 128, FFN 14336, 2 sequences of 4096
+  llama3_8b_long   the same block on 1 sequence of 8192 (64 key tiles per query row in the attention)
+  llama3_70b  8192 wide, 64 query / 8 kv heads of 128, FFN 28672, 1 sequence of 8192 (the GEMMs with
+              N = 57344 and K = 28672, a 1.9 GB fp32 weight gradient), once more through an
+              offload -> prefetch -> B -> release round trip
+  gpt2_small  3 blocks, 768 wide, 12 heads of 64, FFN 3072 GELU, LayerNorm, 8 sequences of 1024
+
+Tolerance: rel 2e-2 of the tensor's largest magnitude (the path's stated bf16 bar) and a relative
+Frobenius bound of 1e-2 - or, where bf16 arithmetic itself is further than half of that from the fp32
+truth, 1.25 times the error of the same oracle stage run in bf16 by PyTorch (the reference's own arithmetic):
+at 8192 x 28672 with N(0, 0.02) weights the activations grow to a few units and ten roundings to bf16 along
+a block add up to about 1 % in PyTorch as well.
+The kernel-level probes at the 70B shapes sit next to the 8B ones in tests/test_fullsize_gpu.py."""
+
+import gc
+
+import pytest
+import torch
+
+from tests.helpers import assert_close_dev, cfg_from_stage, oracle_params_from_stage, perturb_norms, product_grads
+
+pytestmark = pytest.mark.gpu
+
+LLAMA_SHAPES = {
+	"llama3_8b": dict(d=4096, hq=32, hkv=8, hd=128, ffn=14336, seq=4096, mb=2),
+	"llama3_8b_long": dict(d=4096, hq=32, hkv=8, hd=128, ffn=14336, seq=8192, mb=1),
+	"llama3_70b": dict(d=8192, hq=64, hkv=8, hd=128, ffn=28672, seq=8192, mb=1),
+}
+
+
+def _block(stage, mb, **kw):
+	from elf_amd.execution import HipStageBlock
+	from elf_amd.partitioners.utils import sequential_signatures
+
+	placement = [0, 1, 2, 3]
+	return HipStageBlock(stage, 1, placement, sequential_signatures(placement)[1], mb_size=mb, **kw)
+
+
+def _fbw(blk, m, mb):
+	blk.recv_forward(m, mb, src=0)
+	blk.forward(m)
+	blk.send_forward(m, dst=2)
+	blk.recv_backward(m, mb, src=2)
+	blk.backward_inputs(m)
+	blk.send_backward(m, dst=0)
+	blk.backward_params(m)
+	return blk.sent_forward[m], blk.sent_backward[m]
+
+
+def _fro(got, ref):
+	return ((got.double() - ref.double()).norm() / ref.double().norm()).item()
+
+
+def _free():
+	gc.collect()
+	torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("name", list(LLAMA_SHAPES))
+def test_one_block_stage_matches_oracle_at_benchmark_shape(name):
+	from elf_amd import models
+	from elf_amd.synthetic import make_boundary
+	from oracle import stage_ref as R
+
+	s = LLAMA_SHAPES[name]
+	mb = s["mb"]
+	print(f"[case] one-block stage {name}: {s}", flush=True)
+	stage = models.llama_stage(1, s["d"], s["hq"], s["hkv"], s["ffn"], s["seq"], head_dim=s["hd"], seed=21)
+	perturb_norms(stage)
+	cfg = cfg_from_stage(stage, mb)
+	xs, dys = make_boundary(mb, s["seq"], s["d"], 1, seed=22, device="cuda")
+
+	# oracle first, its results kept as fp32 tensors, then its graph and weights are dropped
+	ref = R.RefStage(cfg, oracle_params_from_stage(stage), device="cuda")
+	want_y = ref.forward(0, xs[0])
+	want_dx = ref.backward_inputs(0, dys[0])
+	ref.backward_params(0)
+	want_g = {k: v.detach().clone() for k, v in ref.grads().items()}
+	del ref
+	_free()
+	# the same oracle stage in the reference's own arithmetic (bf16 tensors, PyTorch kernels): how far bf16
+	# itself is from the fp32 truth at this shape
+	ref16 = R.RefStage(cfg, oracle_params_from_stage(stage), compute_dtype=torch.bfloat16, device="cuda")
+	y16 = ref16.forward(0, xs[0])
+	dx16 = ref16.backward_inputs(0, dys[0])
+	fro16 = {"y": _fro(y16, want_y), "dx": _fro(dx16, want_dx)}
+	del ref16, y16, dx16
+	_free()
+	bound = {k: max(1e-2, 1.25 * v) for k, v in fro16.items()}
+	print(f"[bf16 torch vs fp32] {name}: y {fro16['y']:.4g}, dx {fro16['dx']:.4g}", flush=True)
+
+	blk = _block(stage, mb)
+	blk.set_boundary(inputs=xs, grads=dys, keep_sent=True)
+	y, dx = _fbw(blk, 0, mb)
+	torch.cuda.synchronize()
+	print(f"[hip vs fp32] {name}: y {_fro(y, want_y):.4g}, dx {_fro(dx, want_dx):.4g}", flush=True)
+	assert_close_dev(y, want_y, f"{name} y", rel_fro=bound["y"])
+	assert_close_dev(dx, want_dx, f"{name} dx", rel_fro=bound["dx"])
+	got_g = product_grads(stage)
+	assert set(got_g) == set(want_g)
+	for k in sorted(want_g):
+		print(f"[hip vs fp32] {name}: grad {k} {_fro(got_g[k], want_g[k]):.4g}", flush=True)
+		assert_close_dev(got_g[k], want_g[k], f"{name} grad {k}", rel_fro=max(bound.values()))
+	assert blk.mem_stats()["live_bytes"] == 0
+	if name != "llama3_70b":
+		return
+
+	# the same micro-batch again as slot 1 through the offload life cycle: outputs bit for bit, and the
+	# gradient accumulators now hold twice the first pass
+	del want_y, want_dx, want_g
+	first_g = {k: v.clone() for k, v in got_g.items()}
+	del got_g
+	blk.set_boundary(inputs={1: xs[0]}.__getitem__, grads={1: dys[0]}.__getitem__, keep_sent=True)
+	before = blk.mem_stats()
+	blk.recv_forward(1, mb, src=0)
+	blk.forward(1)
+	blk.offload(1)
+	blk.send_forward(1, dst=2)
+	torch.cuda.synchronize()  # the copies to the host have finished: the stash is off the device
+	held = blk.mem_stats()
+	assert held["d2h_bytes"] - before["d2h_bytes"] > (1 << 30), "a 70B-shaped block moves more than a GiB per micro-batch"
+	assert held["live_bytes"] < (64 << 20), "only the small statistics stay on the device"
+	blk.recv_backward(1, mb, src=2)
+	blk.prefetch(1)
+	blk.backward_inputs(1)
+	blk.release(1)
+	blk.send_backward(1, dst=0)
+	blk.backward_params(1)
+	torch.cuda.synchronize()
+	after = blk.mem_stats()
+	assert after["h2d_bytes"] - before["h2d_bytes"] == held["d2h_bytes"] - before["d2h_bytes"]
+	assert torch.equal(blk.sent_forward[1], y) and torch.equal(blk.sent_backward[1], dx)
+	now_g = product_grads(stage)
+	for k in sorted(first_g):
+		assert_close_dev(now_g[k], 2 * first_g[k], f"{name} grad {k} after the offloaded pass", rel_max=2e-3, rel_fro=1e-4)
+	assert after["live_bytes"] == 0
+
+
+def test_gpt2_small_stage_matches_oracle():
+	"""The GPT-2-small-shaped stage of the 1F1B workload: 3 blocks of LayerNorm / 12-head attention /
+	GELU FFN, 8 sequences of 1024 tokens per micro-batch, two micro-batches in flight."""
+	from elf_amd import models
+	from elf_amd.synthetic import make_boundary
+	from oracle import stage_ref as R
+
+	mb, seq, d, n_mb = 8, 1024, 768, 2
+	print("[case] gpt2-small stage: 3 blocks, d 768, 12 heads, ffn 3072, 8 x 1024 tokens", flush=True)
+	stage = models.gpt_stage(3, d, 12, 3072, seq, causal=False, seed=31)
+	perturb_norms(stage)
+	cfg = cfg_from_stage(stage, mb)
+	ref = R.RefStage(cfg, oracle_params_from_stage(stage), device="cuda")
+	xs, dys = make_boundary(mb, seq, d, n_mb, seed=32, device="cuda")
+	blk = _block(stage, mb)
+	blk.set_boundary(inputs=xs, grads=dys, keep_sent=True)
+	for m in range(n_mb):
+		blk.recv_forward(m, mb, src=0)
+		blk.forward(m)
+		blk.send_forward(m, dst=2)
+		assert_close_dev(blk.sent_forward[m], ref.forward(m, xs[m]), f"gpt2s y[{m}]")
+	for m in range(n_mb):
+		blk.recv_backward(m, mb, src=2)
+		blk.backward_inputs(m)
+		blk.send_backward(m, dst=0)
+		assert_close_dev(blk.sent_backward[m], ref.backward_inputs(m, dys[m]), f"gpt2s dx[{m}]")
+		blk.backward_params(m)
+		ref.backward_params(m)
+	got, want = product_grads(stage), ref.grads()
+	assert set(got) == set(want)
+	for k in sorted(want):
+		assert_close_dev(got[k], want[k], f"gpt2s grad {k}")
+	assert blk.mem_stats()["live_bytes"] == 0

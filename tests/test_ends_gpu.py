@@ -134,11 +134,15 @@ def test_first_and_last_stage_match_oracle(case, variant):
 
 
 @pytest.mark.parametrize("loss_kind", ["torch", "fused"])
-def test_reference_small_configuration_through_pipeline(loss_kind):
+@pytest.mark.parametrize("scheduler,placement", [("afab", [0, 0]), ("1f1b", [0, 1]), ("zbh1", [0, 1])])
+def test_reference_small_configuration_through_pipeline(loss_kind, scheduler, placement):
 	"""4-layer GPT-style decoder, d 256, 4 heads, FFN 1024 GELU, LayerNorm, seq 128, vocabulary 1000,
 	micro-batch 4 x 8 micro-batches, cross-entropy on fp32 logits flattened over the sequence
-	(FullTransformer.loss_fn, benchmarks/models/simple.py:519-523), as two stages on one rank; once with
-	that torch loss under autograd and once with the library's one-kernel cross-entropy."""
+	(FullTransformer.loss_fn, benchmarks/models/simple.py:519-523), as two stages: on one rank under
+	AFAB, and as the two ranks of a pp = 2 pipeline under 1F1B and ZB-H1 (the reference's small
+	configuration: its op streams for both ranks, comm ops included, interpreted by one process);
+	once with that torch loss under autograd and once with the library's one-kernel cross-entropy.
+	Loss and every gradient against the un-pipelined model in fp32."""
 	from elf_amd import models
 	from elf_amd.pipeline import Pipeline
 
@@ -165,9 +169,21 @@ def test_reference_small_configuration_through_pipeline(loss_kind):
 	want_loss = F.cross_entropy(logits.view(-1, V), tgt.view(-1), reduction="sum") / (S * mb * nmb)
 	want_loss.backward()
 
-	pipe = Pipeline([first, last], ids[:mb], scheduler="afab", partitioner=False, placement=[0, 0])
+	pipe = Pipeline([first, last], ids[:mb], scheduler=scheduler, partitioner=False, placement=placement, all_ranks=len(set(placement)) > 1)
 	pipe.zero_grad()
 	result, loss = pipe(ids, tgt, loss_fn, split_size=mb)
+	if len(set(placement)) > 1:
+		from elf_amd.scheduling import OperationType as T
+
+		kinds = [(op.op, op.rank) for op in pipe.schedule]
+		for r in (0, 1):  # both ranks' streams ran, with their comm ops
+			assert sum(k == (T.FORWARD, r) for k in kinds) == nmb and sum(k == (T.BACKWARD_INPUTS, r) for k in kinds) == nmb
+		sends = [op for op in pipe.schedule if op.op == T.SEND_FORWARD and op.options.get("dst") is not None]
+		recvs = [op for op in pipe.schedule if op.op == T.RECV_BACKWARD and op.options.get("src") is not None]
+		assert len(sends) == nmb and all(op.rank == 0 for op in sends) and len(recvs) == nmb and all(op.rank == 0 for op in recvs)
+		# 1F1B on the first of two ranks: two forwards in flight before the first backward
+		first_b = next(i for i, k in enumerate(kinds) if k == (T.BACKWARD_INPUTS, 0))
+		assert sum(k == (T.FORWARD, 0) for k in kinds[:first_b]) == 2
 	assert len(result) == nmb and tuple(result[0].shape) == (mb, S, V)
 	assert_close(torch.cat([r.float() for r in result]), logits.detach(), "logits")
 	assert abs(float(loss) - float(want_loss.detach())) <= 1e-2 * float(want_loss.detach())

@@ -1,7 +1,9 @@
 """Properties that do not depend on size, checked at the benchmark's full shapes (Llama-3-8B-shaped
-stage: 8192 tokens per micro-batch, d_model 4096, 32 query / 8 kv heads of 128, FFN 14336), where
-an oracle run would take minutes.  Each property is one a wrong tile index, a dropped K slice, a
-mis-masked attention tile or a lost accumulation would break."""
+stage: 8192 tokens per micro-batch, d_model 4096, 32 query / 8 kv heads of 128, FFN 14336; and the
+Llama-3-70B-shaped one: d_model 8192, 64 query / 8 kv heads, FFN 28672, one sequence of 8192).  Each
+property is one a wrong tile index, a dropped K slice, a mis-masked attention tile or a lost
+accumulation would break.  Whole stages at these shapes against the oracle are in
+tests/test_benchmark_shapes_gpu.py."""
 
 import pytest
 import torch
@@ -27,7 +29,8 @@ def K():
 # down projection's (an A operand of 235 MB: the tile walk in bands of 16 tile rows; for tn the 14336 x 4096
 # weight gradient, whose split tail is the walk's partly filled last round) and the GPT-2-small ones
 # (N = 768: 128x256 tiles; dW with 36 tiles: K split over all of them)
-@pytest.mark.parametrize("dims", [(T, FFN, D_MODEL), (T, D_MODEL, FFN), (T, 768, 3072)])
+# and the Llama-3-70B FFN shapes (N = 57344: 7168 tiles, a 940 MB weight; K = 28672; for tn a 1.9 GB fp32 result)
+@pytest.mark.parametrize("dims", [(T, FFN, D_MODEL), (T, D_MODEL, FFN), (T, 768, 3072), (T, 57344, 8192), (T, 8192, 28672)])
 @pytest.mark.parametrize("layout", ["nt", "nn", "tn"])
 def test_gemm_row_and_column_probes_at_full_size(K, layout, dims):
 	"""C = A B^T (for tn the matching dW shape, K = tokens): 64 sampled rows and columns of the result
@@ -85,11 +88,14 @@ def test_gemm_fp32_accumulation_is_additive_at_full_size(K):
 	assert ((split - one).norm() / one.norm()).item() <= 1e-5
 
 
-def test_attention_properties_at_full_size(K):
-	"""Causal GQA attention at batch 2 x seq 4096: (1) with V = 1 every output is 1 (rows of P sum
+@pytest.mark.parametrize("shape", [(2, 4096, 32, 8), (1, 8192, 32, 8), (1, 8192, 64, 8)])
+def test_attention_properties_at_full_size(K, shape):
+	"""Causal GQA attention at batch 2 x seq 4096 (Llama-3-8B-shaped stage), 1 x 8192 (its long-sequence
+	variant) and 1 x 8192 with 64 query heads (70B-shaped): (1) with V = 1 every output is 1 (rows of P sum
 	to one); (2) changing keys / values / queries after position p leaves outputs up to p unchanged
 	bit for bit; (3) dQ, dK, dV are linear in dO; (4) with dO = 0 all gradients vanish."""
-	B = 2
+	B, SEQ, HQ, HKV = shape
+	print(f"[case] attention properties B={B} S={SEQ} Hq={HQ} Hkv={HKV}", flush=True)
 	nq, nkv = HQ * HD, HKV * HD
 	qkv = _randn(B * SEQ, nq + 2 * nkv, seed=7, scale=0.5)
 	ones = qkv.clone()
@@ -120,13 +126,15 @@ def test_attention_properties_at_full_size(K):
 	assert gh[:, p + 1:].abs().max().item() == 0.0
 
 
-def test_attention_one_kv_group_at_full_sequence_length(K):
-	"""One grouped-query group (4 query heads on 1 kv head) at the full sequence length, against fp32
-	torch: 32 key tiles per query row, so the backward sums the deepest stack of per-tile dQ partials
-	the benchmark shape has.  Tolerances of the small-shape kernel tests."""
+@pytest.mark.parametrize("SEQ,Hq", [(4096, 4), (8192, 4), (8192, 8)])
+def test_attention_one_kv_group_at_full_sequence_length(K, SEQ, Hq):
+	"""One grouped-query group (4 or 8 query heads on 1 kv head) at the full sequence length, against fp32
+	torch: 32 or 64 key tiles per query row, so the backward sums the deepest stack of per-tile dQ
+	partials the benchmark shapes have.  Tolerances of the small-shape kernel tests."""
 	import math
 
-	B, Hq, Hkv = 1, 4, 1
+	print(f"[case] attention one kv group S={SEQ} Hq={Hq}", flush=True)
+	B, Hkv = 1, 1
 	qkv = _randn(B * SEQ, (Hq + 2 * Hkv) * HD, seed=11)
 	do = _randn(B * SEQ, Hq * HD, seed=12)
 	x = qkv.float().requires_grad_(True)

@@ -185,7 +185,7 @@ def test_remat_variants_give_the_same_gradients(kind):
 
 	def run(variant):
 		ref = R.RefStage(cfg, params, compute_dtype=torch.float64, acc_dtype=torch.float64)
-		y = ref.forward(0, xs[0], remat_root=variant == "full_fwd")
+		y = ref.forward(0, xs[0], remat_root=variant == "full_fwd", remat={"simple": ("norm", "act"), "selective": ("attn",)}.get(variant, ()))
 		if variant == "activations_bwd":
 			dx = ref.backward_inputs(0, dys[0], recompute_activations=True)
 			assert all(not lin.inputs and lin.grad_outputs for lin in ref._linears())
@@ -201,7 +201,7 @@ def test_remat_variants_give_the_same_gradients(kind):
 		return y, dx, ref.grads()
 
 	y0, dx0, g0 = run("plain")
-	for variant in ("full_fwd", "activations_bwd", "full_bwd"):
+	for variant in ("full_fwd", "activations_bwd", "full_bwd", "simple", "selective"):
 		y, dx, g = run(variant)
 		assert torch.allclose(y, y0, atol=1e-10) and torch.allclose(dx, dx0, atol=1e-10)
 		for name in g0:

@@ -219,6 +219,105 @@ def test_remat_and_offload_variants_equal_plain(kind, variant, lean):
 		assert_close(g1[name], g0[name], f"{variant} grad {name}", rel_max=2e-3, rel_fro=1e-3)
 
 
+def _pool_round(nbytes):
+	"""Size the stage's device pool charges for a buffer (2 MiB steps from 1 MiB up, 512 B below)."""
+	gran = (2 << 20) if nbytes >= (1 << 20) else 512
+	return -(-nbytes // gran) * gran
+
+
+@pytest.mark.parametrize("kind", ["gpt", "llama"])
+@pytest.mark.parametrize("strategy_kind", ["simple", "selective", "norms_and_cores"])
+@pytest.mark.parametrize("offload", [False, True])
+def test_module_remat_strategies_match_the_oracle(kind, strategy_kind, offload):
+	"""remat_strategy functions that select sub-modules (benchmarks/benchmark_utils.py:311-321: "simple" =
+	GELU / LayerNorm / Dropout modules, "selective" = attention cores; plus one that picks every norm of
+	either kind and the cores): the forward drops what those modules would have kept (asserted on the
+	library's live bytes), B forms it again, and y, dX and every gradient match the oracle run with
+	checkpoint() around the same sub-modules, and the plain run of this library."""
+	from elf_amd.benchmark_utils import _strategy
+	from elf_amd.scheduling import OpOptions
+
+	mb = 16 if offload else 2  # only buffers above 1 MiB are offloaded
+	stage = _stage(kind)
+	R, cfg, ref = _oracle(stage, mb)
+	if strategy_kind == "norms_and_cores":
+		strategy = lambda name, module: type(module).__name__ in ("LayerNorm", "RMSNorm", "Attention")
+	else:
+		strategy = _strategy(strategy_kind)
+	# what the strategy selects in this stage, in the oracle's terms
+	picked = {type(m).__name__ for n, m in stage.named_modules() if strategy(n, m)}
+	kinds = tuple(k for k, names in (("norm", {"LayerNorm", "RMSNorm"}), ("attn", {"Attention"}), ("act", {"GELU"})) if picked & names)
+	if strategy_kind == "simple":
+		assert kinds == (("norm", "act") if kind == "gpt" else ()), "the llama block has no LayerNorm / GELU module: nothing is selected"
+	xs, dys = R.make_boundary(cfg, 1, seed=23)
+	x, dy = xs[0].cuda(), dys[0].cuda()
+
+	def run(strategy):
+		blk = _block(stage, mb)
+		blk.zero_grad()
+		blk.set_boundary(inputs=[x], grads=[dy], keep_sent=True)
+		blk.recv_forward(0, mb, src=0)
+		blk.forward(0, **({OpOptions.REMAT_STRATEGY: strategy} if strategy else {}))
+		held = blk.mem_stats()["live_bytes"]
+		if offload:
+			blk.offload(0)
+		blk.send_forward(0, dst=2)
+		blk.recv_backward(0, mb, src=2)
+		if offload:
+			blk.prefetch(0)
+		blk.backward_inputs(0)
+		if offload:
+			blk.release(0)
+		blk.send_backward(0, dst=0)
+		blk.backward_params(0)
+		torch.cuda.synchronize()
+		assert blk.mem_stats()["live_bytes"] == 0
+		return blk.sent_forward[0], blk.sent_backward[0], {k: v.clone() for k, v in product_grads(stage).items()}, held
+
+	y0, dx0, g0, held0 = run(None)
+	y1, dx1, g1, held1 = run(strategy)
+	T = mb * cfg["seq"]
+	saved = 0
+	if "norm" in kinds:
+		saved += 2 * _pool_round(T * 2 * 4)
+	if "attn" in kinds:
+		saved += _pool_round(T * cfg["n_heads"] * cfg["head_dim"] * 2) + _pool_round(mb * cfg["n_heads"] * cfg["seq"] * 4)
+	assert held0 - held1 == cfg["n_blocks"] * saved
+	assert torch.equal(y1, y0) and torch.equal(dx1, dx0), "the re-formed buffers are bit-identical, so are y and dX"
+	want_y = ref.forward(0, xs[0], remat=kinds)
+	want_dx = ref.backward_inputs(0, dys[0])
+	ref.backward_params(0)
+	assert_close(y1, want_y, f"{kind} {strategy_kind} y")
+	assert_close(dx1, want_dx, f"{kind} {strategy_kind} dx")
+	want = ref.grads()
+	for name in sorted(want):
+		assert_close(g1[name], want[name], f"{kind} {strategy_kind} grad {name}")
+		assert_close(g1[name], g0[name], f"{kind} {strategy_kind} grad {name} vs plain", rel_max=2e-3, rel_fro=1e-3)
+
+
+def test_remat_strategies_this_executor_cannot_express_raise():
+	from elf_amd._lib import ElfStageError
+	from elf_amd.scheduling import OpOptions
+
+	stage = _stage("gpt")
+	blk = _block(stage, 2)
+	x = torch.zeros(2, 128, 256, dtype=torch.bfloat16, device="cuda")
+	for m, strategy in enumerate([
+		lambda name, module: type(module).__name__ == "Linear",  # linears are not checkpointable units here
+		lambda name, module: name == "0",  # one block of the stage
+		lambda name, module: name == "0.norm1",  # one norm of many
+	]):
+		blk.set_boundary(inputs={m: x}.__getitem__)
+		blk.recv_forward(m, 2, src=0)
+		with pytest.raises(ElfStageError):
+			blk.forward(m, **{OpOptions.REMAT_STRATEGY: strategy})
+	# a strategy that selects nothing is a plain forward, as in the reference
+	blk.set_boundary(inputs={5: x}.__getitem__)
+	blk.recv_forward(5, 2, src=0)
+	blk.forward(5, **{OpOptions.REMAT_STRATEGY: lambda name, module: False})
+	blk.clear()
+
+
 def test_engine_runs_1f1b_and_zbh1_streams():
 	"""The Engine interprets the filtered op stream of a middle stage (block 1 of pp = 4) and gives
 	the same gradients as the oracle stage driven by the same stream."""
