@@ -35,6 +35,10 @@ int elf_norm_bwd(int kind, const void* dy, const void* x, const void* gamma, con
                  void* dx, float* dgamma, float* dbeta, float* workspace, int T, int d, void* stream) {
 	return elf::norm_bwd(kind, dy, x, gamma, stats, dres, dx, dgamma, dbeta, workspace, T, d, S_(stream));
 }
+int elf_norm_bwd_noalloc(int kind, const void* dy, const void* x, const void* gamma, const void* stats, const void* dres,
+                         void* dx, float* dgamma, float* dbeta, int T, int d, void* stream) {
+	return elf::norm_bwd_noalloc(kind, dy, x, gamma, stats, dres, dx, dgamma, dbeta, T, d, S_(stream));
+}
 int elf_gelu_fwd(const void* x, void* y, int64_t n, void* stream) { return elf::gelu_fwd(x, y, n, S_(stream)); }
 int elf_gelu_bwd(const void* dy, const void* x, void* dx, int64_t n, void* stream) {
 	return elf::gelu_bwd(dy, x, dx, n, S_(stream));

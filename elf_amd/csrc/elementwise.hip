@@ -8,6 +8,8 @@
 // (benchmarks/models/simple.py:44-52 GELU FFN, :444-445 LayerNorm, :460/:466 residual adds;
 // elf/execution/block.py:518-527 scale_grads).  RMSNorm, RoPE and SwiGLU have no reference
 // module; their definitions are the textbook ones stated next to each kernel.
+#include <mutex>
+
 #include "common.h"
 #include "kernels.h"
 
@@ -313,11 +315,8 @@ static int norm_bwd_dispatch(const void* dy, const void* x, const void* gamma, c
 	return 0;
 }
 
-int norm_bwd(int kind, const void* dy, const void* x, const void* gamma, const void* stats, const void* dres,
-             void* dx, float* dgamma, float* dbeta, float* workspace, int T, int d, hipStream_t s) {
-	ELF_REQUIRE(T > 0 && d > 0 && d % 8 == 0 && d <= 8192, "norm_bwd: d must be a multiple of 8 and <= 8192 (d=%d)", d);
-	ELF_REQUIRE(dy && x && gamma && stats && dx && dgamma && workspace, "norm_bwd: null pointer");
-	ProfScope prof(PROF_NORM_BWD, (dres ? 8.0 : 6.0) * T * d, s);
+static int norm_bwd_launch(int kind, const void* dy, const void* x, const void* gamma, const void* stats, const void* dres,
+                           void* dx, float* dgamma, float* dbeta, float* workspace, int T, int d, hipStream_t s) {
 	int rc;
 	if (kind == NORM_LAYER) {
 		ELF_REQUIRE(dbeta != nullptr, "norm_bwd: LayerNorm needs dbeta");
@@ -335,6 +334,56 @@ int norm_bwd(int kind, const void* dy, const void* x, const void* gamma, const v
 	                   kind == NORM_LAYER ? dbeta : nullptr);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
+}
+
+int norm_bwd(int kind, const void* dy, const void* x, const void* gamma, const void* stats, const void* dres,
+             void* dx, float* dgamma, float* dbeta, float* workspace, int T, int d, hipStream_t s) {
+	ELF_REQUIRE(T > 0 && d > 0 && d % 8 == 0 && d <= 8192, "norm_bwd: d must be a multiple of 8 and <= 8192 (d=%d)", d);
+	ELF_REQUIRE(dy && x && gamma && stats && dx && dgamma && workspace, "norm_bwd: null pointer");
+	ProfScope prof(PROF_NORM_BWD, (dres ? 8.0 : 6.0) * T * d, s);
+	return norm_bwd_launch(kind, dy, x, gamma, stats, dres, dx, dgamma, dbeta, workspace, T, d, s);
+}
+
+// Norm backward for callers that cannot allocate (code under HIP graph capture, tight serving loops): the
+// per-workgroup partial sums of dgamma / dbeta go to an array that is part of the library's device image
+// instead of a workspace argument.  Its size covers every shape norm_bwd accepts: at most 1024 partial rows
+// of 2 x 8192 floats = 64 MiB, which every GPU the library runs on holds until the process ends.  The host
+// sees `scratch` as a stand-in symbol only; its device address is looked up once per device.
+constexpr int64_t NORM_BWD_SCRATCH_FLOATS = (int64_t)1024 * 2 * 8192;
+static __device__ __align__(256) float scratch[NORM_BWD_SCRATCH_FLOATS];
+constexpr int MAX_DEVICES = 64;
+static float* scratch_ptr[MAX_DEVICES] = {};
+static std::mutex scratch_mutex;
+
+int norm_bwd_scratch_prepare() {
+	int dev = -1;
+	ELF_CHECK_HIP(hipGetDevice(&dev));
+	ELF_REQUIRE(dev >= 0 && dev < MAX_DEVICES, "norm_bwd_noalloc: device index %d out of range", dev);
+	std::lock_guard<std::mutex> lock(scratch_mutex);
+	if (!scratch_ptr[dev]) {
+		float* p = nullptr;
+		ELF_CHECK_HIP(hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch)));
+		ELF_REQUIRE(p != nullptr, "norm_bwd_noalloc: no device address for the scratch array");
+		scratch_ptr[dev] = p;
+	}
+	return 0;
+}
+
+int norm_bwd_noalloc(int kind, const void* dy, const void* x, const void* gamma, const void* stats, const void* dres,
+                     void* dx, float* dgamma, float* dbeta, int T, int d, hipStream_t s) {
+	ELF_REQUIRE(T > 0 && d > 0 && d % 8 == 0 && d <= 8192, "norm_bwd_noalloc: d must be a multiple of 8 and <= 8192 (d=%d)", d);
+	ELF_REQUIRE(dy && x && gamma && stats && dx && dgamma, "norm_bwd_noalloc: null pointer");
+	ELF_REQUIRE(norm_bwd_workspace_floats(T, d) <= NORM_BWD_SCRATCH_FLOATS,
+	            "norm_bwd_noalloc: T = %d, d = %d needs %lld floats of scratch, the built-in array holds %lld", T, d,
+	            (long long)norm_bwd_workspace_floats(T, d), (long long)NORM_BWD_SCRATCH_FLOATS);
+	int dev = -1;
+	ELF_CHECK_HIP(hipGetDevice(&dev));
+	ELF_REQUIRE(dev >= 0 && dev < MAX_DEVICES, "norm_bwd_noalloc: device index %d out of range", dev);
+	if (!scratch_ptr[dev]) {
+		if (int rc = norm_bwd_scratch_prepare()) return rc;
+	}
+	// every workgroup writes its whole partial row before the fold reads it: nothing has to start at zero
+	return norm_bwd_launch(kind, dy, x, gamma, stats, dres, dx, dgamma, dbeta, scratch_ptr[dev], T, d, s);
 }
 
 // ------------------------------------------------------------------------------------------

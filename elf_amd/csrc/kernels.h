@@ -53,6 +53,12 @@ int norm_fwd(int kind, const void* x, const void* gamma, const void* beta, void*
 int64_t norm_bwd_workspace_floats(int T, int d);
 int norm_bwd(int kind, const void* dy, const void* x, const void* gamma, const void* stats, const void* dres,
              void* dx, float* dgamma, float* dbeta, float* workspace, int T, int d, hipStream_t s);
+// The same with the partial sums in an array of the library's device image instead of a workspace argument
+// (no allocation anywhere on the path); norm_bwd_scratch_prepare looks the array's address up for the
+// current device (done by the first call on a device otherwise).
+int norm_bwd_scratch_prepare();
+int norm_bwd_noalloc(int kind, const void* dy, const void* x, const void* gamma, const void* stats, const void* dres,
+                     void* dx, float* dgamma, float* dbeta, int T, int d, hipStream_t s);
 int gelu_fwd(const void* x, void* y, int64_t n, hipStream_t s);
 int gelu_bwd(const void* dy, const void* x, void* dx, int64_t n, hipStream_t s);
 int swiglu_fwd(const void* gu, void* h, int64_t T, int F, hipStream_t s);

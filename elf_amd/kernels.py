@@ -107,6 +107,14 @@ def norm_bwd(kind, dy, x, gamma, stats, dgamma, dbeta=None, dres=None):
 	return dx
 
 
+def norm_bwd_noalloc(kind, dy, x, gamma, stats, dgamma, dx, dbeta=None, dres=None):
+	"""``norm_bwd`` through the entry point that allocates nothing: the caller brings ``dx`` too."""
+	T, d = x.shape
+	rc = _lib.load().elf_norm_bwd_noalloc(kind, _ptr(dy), _ptr(x), _ptr(gamma), _ptr(stats), _ptr(dres), _ptr(dx), _ptr(dgamma), _ptr(dbeta), T, d, _stream())
+	_lib.check(rc, "elf_norm_bwd_noalloc")
+	return dx
+
+
 def gelu_fwd(x):
 	y = torch.empty_like(x)
 	_lib.check(_lib.load().elf_gelu_fwd(_ptr(x), _ptr(y), x.numel(), _stream()), "elf_gelu_fwd")

@@ -80,6 +80,19 @@ int elf_norm_bwd(int kind, const void* dy, const void* x, const void* gamma, con
                  const void* dres, void* dx, float* dgamma, float* dbeta, float* workspace, int T,
                  int d, void* stream);
 
+/* elf_norm_bwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results
+ * as elf_norm_bwd without the workspace: the per-workgroup partial sums of dgamma / dbeta go to a 64 MiB
+ * array that is part of the library's device image (1024 partial rows of 2 x 8192 floats: enough for every
+ * T and every d <= 8192 that elf_norm_bwd accepts; a shape that needs more is refused with an error), held
+ * by every GPU the library runs on until the process ends.  The call allocates nothing on the host or the
+ * device (kernel timing through elf_prof_enable does not cover it).  All calls on one GPU share the array:
+ * calls that overlap in time on one GPU (different streams or host threads) race and must be serialised by
+ * the caller.  Nothing in the array has to be cleared between calls (every partial row is written in full
+ * before it is read). */
+int elf_norm_bwd_noalloc(int kind, const void* dy, const void* x, const void* gamma, const void* stats,
+                         const void* dres, void* dx, float* dgamma, float* dbeta, int T, int d, void* stream);
+
 /* Exact (erf) GELU of nn.GELU() (benchmarks/models/simple.py:44-52) over n elements. */
 int elf_gelu_fwd(const void* x, void* y, int64_t n, void* stream);
 int elf_gelu_bwd(const void* dy, const void* x, void* dx, int64_t n, void* stream);
