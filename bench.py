@@ -9,10 +9,12 @@ activations and boundary gradients already resident in HBM.  ``roofline`` is for
 kernel family (the bf16 MFMA GEMM): algorithmic FLOPs (2MNK per launch) divided by the launch
 durations measured live with HIP events on the launch stream, against the published dense bf16
 peak.  ``cpu_baseline`` times the plain-PyTorch CPU restatement of the reference stage (oracle/)
-on a bounded sample (one micro-batch of F, B and W through ONE block, fp32) on the host cores.
+on a bounded sample (one micro-batch of F, B and W through ONE block, fp32; one warm-up pass, median of
+three) on the host cores.
 """
 
 import argparse
+import contextlib
 import ctypes
 import json
 import os
@@ -87,8 +89,11 @@ def op_stream(w, sched=None):
 	return [op for op in schedule if op.block_id == BLOCK_ID]
 
 
-def cpu_baseline(w, stage_module):
-	"""Oracle stage on the host cores: F, B, W of ONE micro-batch through ONE block, fp32."""
+def cpu_baseline(w, stage_module, repeats=3):
+	"""Oracle stage on the host cores: F, B, W of ONE micro-batch through ONE block, fp32; one untimed
+	warm-up pass, then the median of ``repeats`` timed passes."""
+	import statistics
+
 	import torch
 	from oracle import stage_ref as R
 	from tests.helpers import cfg_from_stage, oracle_params_from_stage
@@ -100,20 +105,107 @@ def cpu_baseline(w, stage_module):
 	params = [{k: v.cpu() for k, v in oracle_params_from_stage(stage_module)[0].items()}]
 	ref = R.RefStage(cfg, params, compute_dtype=torch.float32, device="cpu", use_sdpa=True)
 	xs, dys = R.make_boundary(cfg, 1, seed=1)
-	t0 = time.perf_counter()
-	ref.forward(0, xs[0])
-	t1 = time.perf_counter()
-	ref.backward_inputs(0, dys[0])
-	t2 = time.perf_counter()
-	ref.backward_params(0)
-	t3 = time.perf_counter()
+
+	def one_pass():
+		t0 = time.perf_counter()
+		ref.forward(0, xs[0])
+		t1 = time.perf_counter()
+		ref.backward_inputs(0, dys[0])
+		t2 = time.perf_counter()
+		ref.backward_params(0)
+		t3 = time.perf_counter()
+		ref.zero_grad()
+		return t1 - t0, t2 - t1, t3 - t2
+
+	one_pass()  # warm-up: thread pool, allocator, first-touch of the weights
+	runs = [one_pass() for _ in range(repeats)]
+	f, b, wt = (statistics.median(r[i] for r in runs) for i in range(3))
 	T = w["mb"] * w["seq"]
-	per_block = t3 - t0
+	per_block = statistics.median(sum(r) for r in runs)
 	return {
 		"value": T / (per_block * w["n_blocks"]), "unit": "tokens/s", "cores": cores, "kind": "port",
-		"sample": f"oracle/stage_ref.py RefStage on CPU, fp32, SDPA attention: 1 micro-batch ({T} tokens) of F+B+W through 1 of {w['n_blocks']} blocks "
-		          f"(F {t1 - t0:.2f}s, B {t2 - t1:.2f}s, W {t3 - t2:.2f}s), extrapolated to the {w['n_blocks']}-block stage; no warm-up",
+		"sample": f"oracle/stage_ref.py RefStage on CPU, fp32, SDPA attention: 1 micro-batch ({T} tokens) of F+B+W through 1 of {w['n_blocks']} blocks, "
+		          f"1 warm-up pass then the median of {repeats} (F {f:.2f}s, B {b:.2f}s, W {wt:.2f}s), extrapolated to the {w['n_blocks']}-block stage",
 	}
+
+
+class Telemetry:
+	"""Socket power and shader clock sampled on a host thread while the timed steps run (``--telemetry``):
+	amdsmi's gpu_metrics (per-XCD ``current_gfxclks``, ``average_socket_power`` / ``current_socket_power``)
+	where the module is importable, else the hwmon ``power1_input`` file alone."""
+
+	def __init__(self, period=0.05):
+		import threading
+
+		self.period, self.samples, self._stop = period, [], threading.Event()
+		self._thread = threading.Thread(target=self._run, daemon=True)
+		self._smi = None
+		try:
+			import amdsmi
+
+			amdsmi.amdsmi_init()
+			self._smi, self._dev = amdsmi, amdsmi.amdsmi_get_processor_handles()[0]
+		except Exception:
+			self._smi = None
+
+	def _sample(self):
+		rec = {}
+		if self._smi is not None:
+			try:
+				m = self._smi.amdsmi_get_gpu_metrics_info(self._dev)
+				clks = [c for c in (m.get("current_gfxclks") or []) if isinstance(c, (int, float)) and 0 < c < 60000]
+				if clks:
+					rec["sclk_mhz"] = sum(clks) / len(clks)
+				for key in ("current_socket_power", "average_socket_power"):
+					v = m.get(key)
+					if isinstance(v, (int, float)) and 0 < v < 60000:
+						rec["power_w"] = float(v)
+						break
+			except Exception:
+				pass
+		if "power_w" not in rec:
+			import glob
+
+			for f in glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input"):
+				try:
+					rec["power_w"] = int(open(f).read()) / 1e6
+					break
+				except Exception:
+					pass
+		return rec
+
+	def _run(self):
+		while not self._stop.is_set():
+			rec = self._sample()
+			if rec:
+				rec["t"] = time.perf_counter()
+				self.samples.append(rec)
+			self._stop.wait(self.period)
+
+	def __enter__(self):
+		self._thread.start()
+		return self
+
+	def __exit__(self, *_):
+		self._stop.set()
+		self._thread.join()
+
+	def summary(self, t0, t1):
+		"""Over the samples taken in [t0 + 20 % , t1] (the first fifth is left to the governor to settle)."""
+		lo = t0 + 0.2 * (t1 - t0)
+		out = {"samples": 0, "period_s": self.period, "power_cap_w": None}
+		try:
+			import glob
+
+			out["power_cap_w"] = int(open(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_cap")[0]).read()) / 1e6
+		except Exception:
+			pass
+		for key in ("sclk_mhz", "power_w"):
+			vals = [r[key] for r in self.samples if key in r and lo <= r["t"] <= t1]
+			if vals:
+				out["samples"] = max(out["samples"], len(vals))
+				out[key] = {"mean": sum(vals) / len(vals), "min": min(vals), "max": max(vals)}
+		return out
 
 
 def main():
@@ -128,6 +220,8 @@ def main():
 	ap.add_argument("--graph", action="store_true",
 	                help="time replays of the step captured as one HIP graph (Engine.capture) instead of eager steps; the per-kernel figures "
 	                     "then come from one extra eager step after the timed region (a replay runs no host code that could bracket launches)")
+	ap.add_argument("--telemetry", action="store_true",
+	                help="sample socket power and shader clock on a host thread during the timed steps and report them under \"telemetry\"")
 	ap.add_argument("--calibration-copy", action="store_true",
 	                help="also launch one elf::add_kernel over 2 x 128 MiB in, 128 MiB out: a kernel of known HBM traffic to scale profiler byte counters with")
 	args = ap.parse_args()
@@ -213,11 +307,13 @@ def main():
 	else:
 		lib.elf_prof_enable(1)
 	mem_before = block.mem_stats()
-	t0 = time.perf_counter()
-	for _ in range(args.steps):
-		step()
-	torch.cuda.synchronize()
-	elapsed = time.perf_counter() - t0
+	telemetry = Telemetry() if args.telemetry else contextlib.nullcontext()
+	with telemetry:
+		t0 = time.perf_counter()
+		for _ in range(args.steps):
+			step()
+		torch.cuda.synchronize()
+		elapsed = time.perf_counter() - t0
 	if args.graph:
 		lib.elf_prof_enable(1)
 		eager_step()
@@ -262,6 +358,8 @@ def main():
 		h2d = mem["h2d_bytes"] - mem_before["h2d_bytes"]
 		out["host_link"] = {"d2h_gbs": d2h / elapsed / 1e9, "h2d_gbs": h2d / elapsed / 1e9, "d2h_bytes_per_step": d2h / args.steps,
 		                    "h2d_bytes_per_step": h2d / args.steps, "prefetching_time": w.get("prefetching_time", 1)}
+	if args.telemetry:
+		out["telemetry"] = telemetry.summary(t0, t0 + elapsed)
 	if cpu_stats is not None:
 		out["cpu_baseline"] = cpu_stats
 	print(json.dumps(out))

@@ -590,6 +590,45 @@ int add_bf16(const void* a, const void* b, void* out, int64_t n, hipStream_t s) 
 }
 
 // ------------------------------------------------------------------------------------------
+// Bias gradient of a split linear layer (elf/zb_utils.py:247-252: go.sum(0) added to bias.grad in
+// LinearDW.backward): out[c] += sum_t x[t, c] in fp32.  A workgroup owns 256 columns and one of gridDim.y
+// slices of the rows; its 8 row groups are folded through LDS and the slices meet in the accumulator
+// through fp32 atomics.
+__global__ __launch_bounds__(256) void colsum_kernel(const bf16_t* __restrict__ x, int64_t ld, float* __restrict__ out, int64_t T, int N) {
+	__shared__ float red[8][256];
+	const int cl = threadIdx.x & 31, rg = threadIdx.x >> 5;
+	const int c0 = (blockIdx.x * 32 + cl) * 8;
+	float s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+	if (c0 < N) {
+		for (int64_t t = (int64_t)blockIdx.y * 8 + rg; t < T; t += 8 * (int64_t)gridDim.y) {
+			const Chunk c = load8(x + t * ld + c0);
+#pragma unroll
+			for (int j = 0; j < 8; j++) s[j] += c.v[j];
+		}
+	}
+#pragma unroll
+	for (int j = 0; j < 8; j++) red[rg][cl * 8 + j] = s[j];
+	__syncthreads();
+	const int c = blockIdx.x * 256 + threadIdx.x;
+	if (c < N) {
+		float t = 0.f;
+#pragma unroll
+		for (int r = 0; r < 8; r++) t += red[r][threadIdx.x];
+		unsafeAtomicAdd(out + c, t);
+	}
+}
+int colsum_bf16(const void* x, int64_t ld, void* out_f32, int64_t T, int N, hipStream_t s) {
+	ELF_REQUIRE(x && out_f32 && T > 0 && N > 0 && N % 8 == 0 && ld % 8 == 0 && ld >= N, "colsum: N and the row stride must be multiples of 8 (T=%lld N=%d ld=%lld)",
+	            (long long)T, N, (long long)ld);
+	const int col_blocks = (N + 255) / 256;
+	int64_t slices = (2048 + col_blocks - 1) / col_blocks;  // about eight workgroups per CU
+	if (slices > (T + 7) / 8) slices = (T + 7) / 8;
+	hipLaunchKernelGGL(colsum_kernel, dim3(col_blocks, (unsigned)slices), dim3(256), 0, s, (const bf16_t*)x, ld, (float*)out_f32, T, N);
+	ELF_CHECK_HIP(hipGetLastError());
+	return 0;
+}
+
+// ------------------------------------------------------------------------------------------
 // Token embedding of a pipeline's first stage (benchmarks/models/simple.py:496, 502):
 // out[t, :] = table[ids[t], :].  One 16-byte chunk per lane; rows of ids outside [0, V) give a
 // zero row (the host cannot check ids without a device round trip).

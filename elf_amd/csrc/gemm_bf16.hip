@@ -304,7 +304,8 @@ int gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda,
 	ELF_REQUIRE(lda % 8 == 0 && ldb % 8 == 0, "gemm: leading dimensions must be multiples of 8 elements");
 	ELF_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)B % 16) == 0, "gemm: operands must be 16-byte aligned");
 	ELF_REQUIRE(lda >= (a_t ? M : K) && ldb >= (b_t ? N : K) && ldc >= N, "gemm: leading dimension too small");
-	ELF_REQUIRE(epi != EPI_BF16_RESID || (R != nullptr && ldr >= N), "gemm: residual epilogue needs R");
+	// ldr == 0: R is one row of N values added to every row of C (the bias of a linear layer)
+	ELF_REQUIRE(epi != EPI_BF16_RESID || (R != nullptr && (ldr >= N || ldr == 0)), "gemm: residual epilogue needs R");
 	ProfScope prof(PROF_GEMM, 2.0 * M * N * K, stream);
 	GemmArgs g;
 	g.A = (const bf16_t*)A;

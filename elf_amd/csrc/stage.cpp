@@ -833,6 +833,12 @@ int elf_stage_release(elf_stage_t* h, int mb) {
 	return do_release(s, it->second);
 }
 
+int elf_stage_reserve_pinned(elf_stage_t* h, int64_t bytes) {
+	Stage* s = (Stage*)h;
+	ELF_REQUIRE(s && bytes > 0, "elf_stage_reserve_pinned: bad argument");
+	return s->pinned->reserve(bytes, 2, /*bf16*/ 1) ? 0 : -3;
+}
+
 int elf_stage_clear(elf_stage_t* h) {
 	Stage* s = (Stage*)h;
 	ELF_REQUIRE(s, "elf_stage_clear: null stage");

@@ -20,7 +20,7 @@ from ..utils import Timer
 
 logger = logging.getLogger("block")
 
-__all__ = ["Variable", "HipStageBlock", "StageConfig", "MemStats"]
+__all__ = ["Variable", "StageBlockBase", "HipStageBlock", "StageConfig", "MemStats"]
 
 
 class Variable:
@@ -105,6 +105,7 @@ for _name, _ret, _args in [
 	("elf_stage_offload", _I, [_P, _I, _P]),
 	("elf_stage_prefetch", _I, [_P, _I, _P]),
 	("elf_stage_release", _I, [_P, _I]),
+	("elf_stage_reserve_pinned", _I, [_P, ctypes.c_int64]),
 	("elf_stage_clear", _I, [_P]),
 	("elf_stage_mem_stats", _I, [_P, ctypes.POINTER(MemStats)]),
 	("elf_stage_reset_peak", _I, [_P]),
@@ -123,7 +124,107 @@ def _stream():
 	return torch.cuda.current_stream().cuda_stream
 
 
-class HipStageBlock:
+class StageBlockBase:
+	"""What every stage executor of this build shares: identity, the ``Variable`` slots of the stage's
+	signature, and the transfer ops (on one GPU a peer is either in this process or stands for another
+	rank and is fed from local buffers, ``set_boundary``).  Sub-classes add the compute ops of the
+	PipelineBlock duck type (elf/execution/block.py:134-694)."""
+
+	def _init_common(self, model, id_, placement, signature, pp_group, dp_group, recv_pgs, send_pgs):
+		self.id = id_
+		self.placement = placement
+		self.rank = placement[id_]
+		self.is_first = id_ == 0
+		self.is_last = id_ == len(placement) - 1
+		self.signature = signature
+		self.pp_group, self.dp_group = pp_group, dp_group
+		self.recv_pgs, self.send_pgs = recv_pgs, send_pgs
+		self.model = model.cuda()
+		self.device = torch.cuda.current_device()
+		self.input_variables = [Variable(n, s, pp_group) for n, s in zip(signature.inputs, signature.sources)]
+		self.output_variables = [[Variable(n, d, pp_group) for d in dsts] for n, dsts in zip(signature.outputs, signature.targets)]
+		self.compute_time = []
+		self.send_ops = []
+
+	def __str__(self):
+		return f"Rank {self.rank} - Layer {self.id}"
+
+	def _timed(self, name):
+		t = Timer(name=name)
+		self.compute_time.append(t)
+		return t
+
+	# ------------------------------------------------------------------ transfers (single GPU: peers are local or absent)
+	def set_boundary(self, inputs=None, grads=None, keep_sent=False):
+		"""Stand-ins for the stage's remote peers: ``inputs(mb)`` / ``grads(mb)`` (callables or
+		sequences of tensors) supply what RECV_FORWARD / RECV_BACKWARD would receive from another
+		rank; what SEND_FORWARD / SEND_BACKWARD would ship is dropped, or collected in
+		``sent_forward`` / ``sent_backward`` when ``keep_sent`` is set."""
+		self._feed_x = (lambda mb: inputs[mb]) if inputs is not None and not callable(inputs) else inputs
+		self._feed_dy = (lambda mb: grads[mb]) if grads is not None and not callable(grads) else grads
+		self._keep_sent = keep_sent
+		self.sent_forward, self.sent_backward = {}, {}
+
+	def _remote(self, peer):
+		return peer is not None and self.placement[peer] != self.rank and peer not in getattr(self, "local_ids", ())
+
+	def _need_feed(self, feed, what):
+		if feed is None:
+			raise NotImplementedError(f"{self}: {what} from another rank needs set_boundary(): this build feeds stage boundaries from local buffers")
+		return feed
+
+	def _sends_input_grads(self):
+		return True
+
+	def send_forward(self, mb_id, **options):
+		dst = options.get("dst")
+		if self._remote(dst):
+			for targets in self.output_variables:
+				for target in targets:
+					if target.peer == dst:
+						y = target.get(target.to_send, mb_id)
+						if getattr(self, "_keep_sent", False):
+							self.sent_forward[mb_id] = y
+
+	def send_backward(self, mb_id, **options):
+		dst = options.get("dst")
+		if self._remote(dst) and self._sends_input_grads():
+			for var in self.input_variables:
+				if var.peer == dst:
+					dx = var.get(var.to_send, mb_id)
+					if getattr(self, "_keep_sent", False):
+						self.sent_backward[mb_id] = dx
+
+	def recv_forward(self, mb_id, mb_size, **options):
+		src = options.get("src")
+		if self._remote(src):
+			for var in self.input_variables:
+				if var.peer == src:
+					x = self._need_feed(getattr(self, "_feed_x", None), "recv_forward")(mb_id)
+					var.set(var.to_process, mb_id, (None, x))
+
+	def recv_backward(self, mb_id, mb_size, **options):
+		src = options.get("src")
+		if self._remote(src):
+			for targets in self.output_variables:
+				for target in targets:
+					if target.peer == src:
+						dy = self._need_feed(getattr(self, "_feed_dy", None), "recv_backward")(mb_id)
+						target.set(target.to_process, mb_id, (None, dy))
+
+	def _wait_for_send_ops(self):
+		self.send_ops.clear()
+
+	def all_reduce_param_grads(self, **options):
+		if self.dp_group is None:
+			return
+		import torch.distributed as dist
+
+		for g in self._grad_buffers():
+			dist.all_reduce(g, group=self.dp_group, op=dist.ReduceOp.AVG, async_op=True)
+
+
+class HipStageBlock(StageBlockBase):
 	"""One pipeline stage (a chain of TransformerBlock or LlamaBlock modules) executed by
 	libelf_stage.so.
 
@@ -141,22 +242,10 @@ class HipStageBlock:
 		if not torch.cuda.is_available():
 			raise _lib.ElfStageError("HipStageBlock needs an MI355X: there is no CPU path for the stage kernels")
 		self.lib = _lib.load()
-		self.id = id_
-		self.placement = placement
-		self.rank = placement[id_]
-		self.is_first = id_ == 0
-		self.is_last = id_ == len(placement) - 1
-		self.signature = signature
-		self.pp_group, self.dp_group = pp_group, dp_group
-		self.recv_pgs, self.send_pgs = recv_pgs, send_pgs
-		self.model = model.cuda()
-		self.device = torch.cuda.current_device()
-		self.input_variables = [Variable(n, s, pp_group) for n, s in zip(signature.inputs, signature.sources)]
-		self.output_variables = [[Variable(n, d, pp_group) for d in dsts] for n, dsts in zip(signature.outputs, signature.targets)]
-		assert len(self.input_variables) == 1 and len(self.output_variables) == 1, "a transformer-block stage has one input and one output"
-		self.compute_time = []
-		self.send_ops = []
 		self._handle = None
+		self._init_common(model, id_, placement, signature, pp_group, dp_group, recv_pgs, send_pgs)
+		if len(self.input_variables) != 1 or len(self.output_variables) != 1:
+			raise _lib.ElfStageError("HipStageBlock: a chain of transformer blocks has one input and one output (AutogradStageBlock runs stages with other signatures)")
 		self._samples = {}  # mb -> sequences in it, where fewer than mb_size
 		self._kept = {}  # mb -> external tensors the library still points at (x until B/recompute, dy until W)
 		self._remat_cache = {}  # id(strategy) -> (strategy, forward flags)
@@ -261,9 +350,6 @@ class HipStageBlock:
 				self._handle = None
 		except Exception:
 			pass
-
-	def __str__(self):
-		return f"Rank {self.rank} - Layer {self.id}"
 
 	def _rows(self, mb_id):
 		"""Tokens in micro-batch ``mb_id`` (fewer than ``T`` for a short last micro-batch)."""
@@ -381,11 +467,6 @@ class HipStageBlock:
 		self._remat_cache[key] = (strategy, flags)
 		return flags
 
-	def _timed(self, name):
-		t = Timer(name=name)
-		self.compute_time.append(t)
-		return t
-
 	# ------------------------------------------------------------------ compute ops
 	def forward(self, mb_id, **options):
 		"""F.  Options: ``remat_strategy`` (see ``_remat_flags``) and ``activation_offload`` (handled by
@@ -478,69 +559,11 @@ class HipStageBlock:
 		for p in self.main_grads:
 			p.grad = None
 
-	def all_reduce_param_grads(self, **options):
-		if self.dp_group is None:
-			return
-		import torch.distributed as dist
+	def _grad_buffers(self):
+		return self._fused_g
 
-		for g in self._fused_g:
-			dist.all_reduce(g, group=self.dp_group, op=dist.ReduceOp.AVG, async_op=True)
-
-	# ------------------------------------------------------------------ transfers (single GPU: peers are local or absent)
-	def set_boundary(self, inputs=None, grads=None, keep_sent=False):
-		"""Stand-ins for the stage's remote peers: ``inputs(mb)`` / ``grads(mb)`` (callables or
-		sequences of tensors) supply what RECV_FORWARD / RECV_BACKWARD would receive from another
-		rank; what SEND_FORWARD / SEND_BACKWARD would ship is dropped, or collected in
-		``sent_forward`` / ``sent_backward`` when ``keep_sent`` is set."""
-		self._feed_x = (lambda mb: inputs[mb]) if inputs is not None and not callable(inputs) else inputs
-		self._feed_dy = (lambda mb: grads[mb]) if grads is not None and not callable(grads) else grads
-		self._keep_sent = keep_sent
-		self.sent_forward, self.sent_backward = {}, {}
-
-	def _remote(self, peer):
-		return peer is not None and self.placement[peer] != self.rank and peer not in getattr(self, "local_ids", ())
-
-	def _need_feed(self, feed, what):
-		if feed is None:
-			raise NotImplementedError(f"{self}: {what} from another rank needs set_boundary(): this build feeds stage boundaries from local buffers")
-		return feed
-
-	def send_forward(self, mb_id, **options):
-		dst = options.get("dst")
-		if self._remote(dst):
-			for target in self.output_variables[0]:
-				if target.peer == dst:
-					y = target.get(target.to_send, mb_id)
-					if getattr(self, "_keep_sent", False):
-						self.sent_forward[mb_id] = y
-
-	def send_backward(self, mb_id, **options):
-		dst = options.get("dst")
-		if self._remote(dst) and not self.vocab_in:  # token ids have no gradient to send
-			var = self.input_variables[0]
-			if var.peer == dst:
-				dx = var.get(var.to_send, mb_id)
-				if getattr(self, "_keep_sent", False):
-					self.sent_backward[mb_id] = dx
-
-	def recv_forward(self, mb_id, mb_size, **options):
-		src = options.get("src")
-		if self._remote(src):
-			var = self.input_variables[0]
-			if var.peer == src:
-				x = self._need_feed(getattr(self, "_feed_x", None), "recv_forward")(mb_id)
-				var.set(var.to_process, mb_id, (None, x))
-
-	def recv_backward(self, mb_id, mb_size, **options):
-		src = options.get("src")
-		if self._remote(src):
-			for target in self.output_variables[0]:
-				if target.peer == src:
-					dy = self._need_feed(getattr(self, "_feed_dy", None), "recv_backward")(mb_id)
-					target.set(target.to_process, mb_id, (None, dy))
-
-	def _wait_for_send_ops(self):
-		self.send_ops.clear()
+	def _sends_input_grads(self):
+		return not self.vocab_in  # token ids have no gradient to send
 
 	# ------------------------------------------------------------------ offload hooks used by StageOffloader
 	def offload(self, mb_id):
@@ -552,11 +575,24 @@ class HipStageBlock:
 	def release(self, mb_id):
 		_lib.check(self.lib.elf_stage_release(self._handle, mb_id), "elf_stage_release")
 
+	def reserve_pinned(self, nbytes):
+		"""Grow the pinned-host arena of activation offload by ``nbytes`` ahead of the first step."""
+		_lib.check(self.lib.elf_stage_reserve_pinned(self._handle, int(nbytes)), "elf_stage_reserve_pinned")
+
 	def clear(self):
 		"""Drop every micro-batch state held by the library and the tensors pinned for it."""
 		_lib.check(self.lib.elf_stage_clear(self._handle), "elf_stage_clear")
 		self._kept.clear()
 		self._samples.clear()
+
+	def end_step(self):
+		"""After a step whose every micro-batch went through W the library holds nothing: only the
+		references kept for it are dropped, without the device synchronisation of ``clear``.  A step
+		that left state behind (a forward-only schedule) is cleared in full."""
+		if self.mem_stats()["live_bytes"] == 0 and not any("x" in k for k in self._kept.values()):
+			self._kept.clear()
+		else:
+			self.clear()
 
 	def mem_stats(self):
 		st = MemStats()

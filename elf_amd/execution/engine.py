@@ -25,7 +25,7 @@ logger = logging.getLogger("engine")
 precise_timings = os.environ.get("ELF_TIMINGS", False)
 precise_memory = os.environ.get("ELF_MEMORY", False)
 
-__all__ = ["Engine", "GraphedStep", "compute_loss"]
+__all__ = ["Engine", "GraphedStep", "compute_loss", "preallocate_pool"]
 
 _GPU = torch.cuda.is_available
 
@@ -48,6 +48,31 @@ def _mem():
 	return (torch.cuda.memory_allocated(), torch.cuda.max_memory_allocated()) if _GPU() else (0, 0)
 
 
+def preallocate_pool(blocks):
+	"""``ELF_PREALLOCATE_POOL="bf16:8,f32:1"`` (GiB per dtype, elf/execution/engine.py:71-93) grows the
+	pinned-host memory of activation offload before the first step.  The reference has one pool per
+	process keyed by dtype; here every stage owns one arena that holds its stash as raw bf16-sized
+	elements, so the sizes of all dtypes are added up and shared evenly among the blocks that can offload.
+	Returns the bytes reserved per block (0 when the variable is not set)."""
+	val = os.environ.get("ELF_PREALLOCATE_POOL")
+	if not val:
+		return 0
+	known = {"f16", "f32", "f64", "bf16", "i8", "i16", "i32", "c64"}
+	total = 0
+	for part in val.split(","):
+		dtype, size = part.split(":")
+		if dtype not in known:
+			raise KeyError(dtype)
+		total += int(size) * 1024**3
+	able = [b for b in blocks if hasattr(b, "reserve_pinned")]
+	if not able or total <= 0:
+		return 0
+	share = total // len(able)
+	for b in able:
+		b.reserve_pinned(share)
+	return share
+
+
 class Engine:
 	"""Runs a list of operations on the blocks of one rank; feeds the pipeline input to the first
 	block and computes the loss on the last one."""
@@ -62,6 +87,7 @@ class Engine:
 		self.id_to_block = {b.id: b for b in blocks}
 		self.offload_stream = torch.cuda.Stream() if _GPU() else None
 		self.pool = None  # the pinned arena lives in the stage library
+		preallocate_pool(blocks)
 
 	def _offloader(self, block, mb):
 		if hasattr(block, "offload"):

@@ -31,8 +31,9 @@ def _need(t, dtype, name):
 		raise _lib.ElfStageError(f"{name}: innermost dimension must be contiguous")
 
 
-def gemm(a, b, *, a_t=False, b_t=False, out=None, epilogue=EPI_BF16, residual=None, tile_cfg=0, k_splits=0):
-	"""C[M,N] (+)= sum_k A(m,k) B(n,k).  a: [M,K] (or [K,M] if a_t); b: [N,K] (or [K,N] if b_t)."""
+def gemm(a, b, *, a_t=False, b_t=False, out=None, epilogue=EPI_BF16, residual=None, residual_ld=None, tile_cfg=0, k_splits=0):
+	"""C[M,N] (+)= sum_k A(m,k) B(n,k).  a: [M,K] (or [K,M] if a_t); b: [N,K] (or [K,N] if b_t).
+	``residual_ld=0``: ``residual`` is one row of N values added to every row (a bias)."""
 	_need(a, torch.bfloat16, "gemm.a")
 	_need(b, torch.bfloat16, "gemm.b")
 	K, M = (a.shape[0], a.shape[1]) if a_t else (a.shape[1], a.shape[0])
@@ -44,7 +45,7 @@ def gemm(a, b, *, a_t=False, b_t=False, out=None, epilogue=EPI_BF16, residual=No
 		out = (torch.zeros if epilogue == EPI_F32_ACC else torch.empty)((M, N), dtype=dt, device=a.device)
 	lib = _lib.load()
 	rc = lib.elf_gemm_bf16(int(a_t), int(b_t), M, N, K, _ptr(a), a.stride(0), _ptr(b), b.stride(0), _ptr(out), out.stride(0),
-	                       epilogue, _ptr(residual), residual.stride(0) if residual is not None else 0, tile_cfg, k_splits, _stream())
+	                       epilogue, _ptr(residual), (residual.stride(0) if residual_ld is None else residual_ld) if residual is not None else 0, tile_cfg, k_splits, _stream())
 	_lib.check(rc, "elf_gemm_bf16")
 	return out
 
@@ -161,6 +162,14 @@ def add(a, b):
 	out = torch.empty_like(a)
 	_lib.check(_lib.load().elf_add_bf16(_ptr(a), _ptr(b), _ptr(out), a.numel(), _stream()), "elf_add_bf16")
 	return out
+
+
+def colsum_(x, out_f32):
+	"""out_f32 [N] += x.sum(0) for x: bf16 [T, N]."""
+	_need(x, torch.bfloat16, "colsum.x")
+	_need(out_f32, torch.float32, "colsum.out")
+	_lib.check(_lib.load().elf_colsum_bf16(_ptr(x), x.stride(0), _ptr(out_f32), x.shape[0], x.shape[1], _stream()), "elf_colsum_bf16")
+	return out_f32
 
 
 def embedding_fwd(ids, table):

@@ -27,7 +27,8 @@ from typing import Any, List
 import torch
 import torch.distributed as dist
 
-from .execution import Engine, HipStageBlock
+from .execution import AutogradStageBlock, Engine, HipStageBlock
+from .models import EndStage, LlamaBlock, TransformerBlock
 from .partitioners.utils import Signature, sequential_signatures
 from .registry import COMM_SCHEDULERS, PARTITIONERS, SCHEDULERS, TRACERS, resolve
 from .scheduling import OperationType, add_comms, check_schedule_validity, schedule_to_str
@@ -107,6 +108,15 @@ class PipelineConfig:
 		return {k: v for k, v in asdict(self).items() if v is not None}
 
 
+def _is_transformer_chain(module):
+	"""Whether ``module`` is what ``HipStageBlock`` runs inside the library: a chain of ``TransformerBlock``
+	or of ``LlamaBlock`` modules, bare or inside an ``EndStage``.  Any other stage module runs through
+	``AutogradStageBlock`` (PyTorch autograd with the linear layers on the HIP GEMM)."""
+	core = module.blocks if isinstance(module, EndStage) else module
+	blocks = [core] if isinstance(core, (TransformerBlock, LlamaBlock)) else list(core.children())
+	return bool(blocks) and all(isinstance(b, (TransformerBlock, LlamaBlock)) for b in blocks) and len({type(b) for b in blocks}) == 1 and getattr(core, "seq_len", None) is not None
+
+
 def _world():
 	if dist.is_available() and dist.is_initialized():
 		return dist.get_world_size(), dist.get_rank()
@@ -170,6 +180,8 @@ class Pipeline:
 		# ILP remat: profile now, solve lazily at the first step() (elf/pipeline.py:186-207)
 		self._remat_stats = None
 		if self.cfg.memory_budget is not None:
+			if any(not isinstance(b, HipStageBlock) for b in self.blocks):
+				raise NotImplementedError("Pipeline: memory_budget profiles stages on the native executor; a stage that is not a chain of transformer blocks cannot be profiled")
 			own = {b.id: profile_stage(b)[0] for b in self.blocks}
 			assert len(own) == len(self.placement), "memory_budget needs the statistics of every stage of the placement"
 			self._remat_stats = [own[i] for i in range(len(self.placement))]
@@ -194,7 +206,7 @@ class Pipeline:
 			for var in block.output_variables:
 				for dst in var:
 					dst.clear()
-			block.clear()
+			(getattr(block, "end_step", None) or block.clear)()
 		self.stats, self.detailed_stats = stats, detailed_stats
 		if len(result) != 0:
 			with torch.no_grad():
@@ -360,7 +372,7 @@ class Pipeline:
 		assert len(parts) == len(ids), f"rank {self.rank} owns blocks {ids} of placement {list(self.placement)} but got {len(parts)} stage module(s)"
 		# under a memory budget the stages hold the lean stash: the remat ILP then starts from a third less per micro-batch
 		lean = self.cfg.memory_budget is not None
-		blocks = [HipStageBlock(part, i, self.placement, signatures[i], mb_size=self.mb_size, lean_stash=lean) for part, i in zip(parts, ids)]
+		blocks = [(HipStageBlock if _is_transformer_chain(part) else AutogradStageBlock)(part, i, self.placement, signatures[i], mb_size=self.mb_size, lean_stash=lean) for part, i in zip(parts, ids)]
 		if self.all_ranks:
 			for b in blocks:
 				b.local_ids = set(ids)  # peers on other ranks of the placement are in this process too

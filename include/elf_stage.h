@@ -30,7 +30,8 @@ int elf_abi_version(void);
  *   C[M,N] (+)= sum_k A(m,k) * B(n,k), bf16 inputs, fp32 accumulation on MFMA.
  *   a_t = 0: A is [M,K] (k contiguous, leading dim lda); a_t = 1: A is [K,M] (m contiguous).
  *   b_t = 0: B is [N,K] (k contiguous, leading dim ldb); b_t = 1: B is [K,N] (n contiguous).
- *   epilogue: 0 C(bf16) = acc; 1 C(bf16) = acc + R(bf16, leading dim ldr);
+ *   epilogue: 0 C(bf16) = acc; 1 C(bf16) = acc + R(bf16, leading dim ldr; ldr = 0: R is one row of N values
+ *             added to every row of C, the bias of nn.Linear);
  *             2 C(fp32) += acc; 3 C(fp32) = acc.
  *   tile_cfg = 0 picks a tile shape from M,N (1: 256x256, 2: 128x128, 3: 64x64, 5: 256x128 register-staged;
  *   7: 256x256 with direct-to-LDS loads; 8: 128x256 with direct-to-LDS loads, a_t = 0 only);
@@ -114,6 +115,11 @@ int elf_scale_grads(void* acc_f32, void* out_bf16, int64_t n, float scale, void*
 /* out = a + b over n bf16 elements: gradient fan-in of an output with several targets
  * (elf/execution/block.py:651-655) and residual adds (simple.py:460,466). */
 int elf_add_bf16(const void* a, const void* b, void* out, int64_t n, void* stream);
+
+/* out_f32[c] += sum over the T rows of x[t, c] (x: bf16 [T, N], row stride ld; N and ld multiples of 8).
+ * Replaces the bias gradient of LinearDW.backward, go.sum(0) added to bias.grad (elf/zb_utils.py:247-252),
+ * with fp32 accumulation. */
+int elf_colsum_bf16(const void* x, int64_t ld, void* out_f32, int64_t T, int N, void* stream);
 
 /* Token embedding of a first pipeline stage: out[t, :] = table[ids[t], :] (ids: int64 [T], table: bf16
  * [V, d], d % 8 == 0; an id outside [0, V) gives a zero row) and its weight gradient dtable[ids[t], :] +=
@@ -276,6 +282,11 @@ int elf_stage_recompute_backward_inputs(elf_stage_t* s, int mb, const void* dy, 
 int elf_stage_offload(elf_stage_t* s, int mb, void* stream);
 int elf_stage_prefetch(elf_stage_t* s, int mb, void* stream);
 int elf_stage_release(elf_stage_t* s, int mb);
+/* Grow the stage's pinned-host arena by one chunk of `bytes` now, so that the first offloaded micro-batches
+ * do not pay for hipHostMalloc inside the step: what ELF_PREALLOCATE_POOL asks of the reference's pool
+ * (preallocate_pool, elf/execution/engine.py:71-93; PinnedHostTensorPool.reserve, offload.py:45-70: the
+ * chunk has exactly the requested size, not the next power of two). */
+int elf_stage_reserve_pinned(elf_stage_t* s, int64_t bytes);
 /* Drop every micro-batch state (Pipeline.step clears all slots after a step, pipeline.py:265-275). */
 int elf_stage_clear(elf_stage_t* s);
 int elf_stage_mem_stats(elf_stage_t* s, elf_mem_stats* out);

@@ -85,3 +85,42 @@ def test_monotone_in_budget():
 	objs = [solve_remat(st, [0, 1], SCHEDULERS["1f1b"], 4, b)["objective"] for b in (330, 345, 360, 450, 1000)]
 	assert all(a >= b - 1e-6 - 0.03 * b for a, b in zip(objs, objs[1:]))
 	assert objs[-1] == pytest.approx(min(objs), rel=0.03)
+
+
+def test_auto_scheduler_picks_the_best_base_scheduler_and_stagerematify_applies_its_plan():
+	"""``AutoScheduler`` (elf/scheduling/ilp.py:828-853 of the reference: solve the ILP for every registered
+	base scheduler, keep the smallest makespan) and ``stagerematify`` (the lazy per-call wrapper
+	``Pipeline(memory_budget=)`` builds): the chosen plan is the best of the per-scheduler solutions, the op
+	list is that scheduler's list rewritten by ``RematScheduler``, and a tight budget shows up as remat ops."""
+	from elf_amd.scheduling import OperationType as T, OpOptions, check_schedule_validity
+	from elf_amd.scheduling.ilp import AutoScheduler, RematScheduler, stagerematify
+
+	st, placement, nmb = [_stats(), _stats()], [0, 1], 4
+	loose, tight = 10_000, 400  # the no-remat peak of rank 0 under 1F1B is 410 (see the first test); nothing fits below 330
+	auto = AutoScheduler(st, loose)
+	assert "auto" not in auto.schedulers and "fixed" not in auto.schedulers and "1f1b" in auto.schedulers and "zbh1" in auto.schedulers
+	objectives = {}
+	for name in auto.schedulers:
+		try:
+			objectives[name] = solve_remat(st, placement, SCHEDULERS[name], nmb, loose)["objective"]
+		except Exception:
+			pass
+	best = min(objectives, key=objectives.get)
+	got = auto(placement, nmb)
+	check_schedule_validity(got)
+	want = RematScheduler(SCHEDULERS[best], solve_remat(st, placement, SCHEDULERS[best], nmb, loose))(placement, nmb)
+	assert [(o.op, o.block_id, o.mb_id, o.rank) for o in got] == [(o.op, o.block_id, o.mb_id, o.rank) for o in want]
+	assert not any(o.op in (T.RECOMPUTE_FORWARD, T.RECOMPUTE_BACKWARD_INPUTS) or o.options.get(OpOptions.REMAT_STRATEGY) for o in got)
+
+	def remat_ops(schedule):
+		return [o for o in schedule if o.op in (T.RECOMPUTE_FORWARD, T.RECOMPUTE_BACKWARD_INPUTS) or o.options.get(OpOptions.REMAT_STRATEGY) is not None]
+
+	constrained = AutoScheduler(st, tight)(placement, nmb)
+	check_schedule_validity(constrained)
+	assert remat_ops(constrained), "a budget below the no-remat peak must force rematerialisation"
+	wrapped = stagerematify(SCHEDULERS["1f1b"], st, tight)
+	s1 = wrapped(placement, nmb)
+	s2 = RematScheduler(SCHEDULERS["1f1b"], solve_remat(st, placement, SCHEDULERS["1f1b"], nmb, tight))(placement, nmb)
+	assert [(o.op, o.block_id, o.mb_id, o.rank) for o in s1] == [(o.op, o.block_id, o.mb_id, o.rank) for o in s2] and remat_ops(s1)
+	with pytest.raises(RuntimeError):
+		AutoScheduler(st, 1.0)(placement, nmb)  # no scheduler fits 1 MiB

@@ -37,3 +37,23 @@ def test_partial_overrides_keep_the_other_defaults(override):
 	cfg = PipelineConfig(**override)
 	for name, want in {**REFERENCE_DEFAULTS, **override}.items():
 		assert getattr(cfg, name) == want, name
+
+
+def test_reference_package_name_resolves_to_this_build():
+	"""``from elf import Pipeline`` (the reference's top-level names, elf/__init__.py:1-13) and its
+	sub-module paths reach the elf_amd modules, not copies of them."""
+	import elf
+	import elf.scheduling
+	import elf_amd.scheduling
+	from elf import Pipeline, PipelineConfig, Placement, replace_layer_with_layer_dw, sequential_signatures
+	from elf.registry import SCHEDULERS
+	from elf.zb_utils import LinearDW
+
+	import elf_amd.pipeline
+	import elf_amd.registry
+	import elf_amd.zb_utils
+
+	assert Pipeline is elf_amd.pipeline.Pipeline and PipelineConfig is elf_amd.pipeline.PipelineConfig
+	assert elf.scheduling is elf_amd.scheduling and SCHEDULERS is elf_amd.registry.SCHEDULERS and LinearDW is elf_amd.zb_utils.LinearDW
+	assert Placement([0, 1]).get_ids(1) == [1] and len(sequential_signatures([0, 1])) == 2 and callable(replace_layer_with_layer_dw)
+	assert set(elf.__all__) >= {"Pipeline", "PipelineConfig", "Placement", "sequential_signatures", "replace_layer_with_layer_dw"}

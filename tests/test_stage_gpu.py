@@ -430,3 +430,31 @@ def test_error_paths():
 	blk.recv_forward(2, 3, src=0)
 	with pytest.raises(ElfStageError):
 		blk.forward(2)  # more sequences than the stage was sized for
+
+
+def test_preallocate_pool_reserves_the_pinned_arena_before_the_first_step(monkeypatch):
+	"""ELF_PREALLOCATE_POOL (elf/execution/engine.py:71-93): the Engine grows the stage's pinned arena by the
+	requested size when it is built, so an offloaded micro-batch that fits finds its host blocks there and
+	the arena does not grow inside the step."""
+	from elf_amd.execution import Engine
+
+	monkeypatch.setenv("ELF_PREALLOCATE_POOL", "bf16:1")
+	mb = 16
+	stage = _stage("llama")
+	blk = _block(stage, mb)
+	assert blk.mem_stats()["pinned_bytes"] == 0
+	Engine([blk])
+	assert blk.mem_stats()["pinned_bytes"] == 1 << 30, "one chunk of exactly the requested size (reserve does not round to a power of two)"
+	R, cfg, _ = _oracle(stage, mb)
+	xs, dys = R.make_boundary(cfg, 1, seed=3)
+	blk.set_boundary(inputs=[xs[0].cuda()], grads=[dys[0].cuda()])
+	blk.recv_forward(0, mb, src=0)
+	blk.forward(0)
+	blk.offload(0)
+	torch.cuda.synchronize()
+	st = blk.mem_stats()
+	assert 0 < st["d2h_bytes"] < (1 << 30) and st["pinned_bytes"] == 1 << 30
+	blk.clear()
+	monkeypatch.setenv("ELF_PREALLOCATE_POOL", "q4:1")
+	with pytest.raises(KeyError):
+		Engine([blk])
