@@ -216,11 +216,11 @@ def test_autograd_stage_block_on_a_generic_module(variant):
 			targets[0].set(targets[0].to_process, m, (None, gr))
 		if variant == "activations_bwd":
 			blk.backward_inputs(m, **{OpOptions.RECOMPUTE_ACTIVATIONS: True})
-			assert all(l.is_empty("input") and not l.is_empty("grad_output") for l in blk._layers_dw())
+			assert all(l.ctx["input"][m] is None and l.ctx["grad_output"][m] is not None for l in blk._layers_dw())
 			blk.recompute_forward(m)
 		elif variant == "full_bwd":
 			blk.backward_inputs(m, **{OpOptions.RECOMPUTE_ACTIVATIONS: True, OpOptions.RECOMPUTE_GRADIENTS: True})
-			assert all(l.is_empty("input") and l.is_empty("grad_output") for l in blk._layers_dw())
+			assert all(l.ctx["input"][m] is None and l.ctx["grad_output"][m] is None for l in blk._layers_dw())
 			norm_grad = blk.model.norm.weight.grad.clone()
 			blk.recompute_forward(m, **{OpOptions.SAVE: True})
 			blk.recompute_backward_inputs(m)
@@ -230,7 +230,7 @@ def test_autograd_stage_block_on_a_generic_module(variant):
 		for var, want in zip(blk.input_variables, want_dx[m]):
 			assert_close(var.get(var.to_send, m), want, f"{variant} dx[{m}]")
 		blk.backward_params(m)
-		assert all(l.is_empty("input") and l.is_empty("grad_output") for l in blk._layers_dw())
+		assert all(l.ctx["input"][m] is None and l.ctx["grad_output"][m] is None for l in blk._layers_dw())
 	ref_params = dict(ref.named_parameters())
 	for name, p in blk.model.named_parameters():
 		got = p.main_grad if getattr(p, "main_grad", None) is not None else p.grad
@@ -277,7 +277,7 @@ def test_pipeline_builds_generic_stages_for_other_modules(scheduler, placement):
 	want_loss = F.mse_loss(out, tgt.float(), reduction="sum") / (128 * mb * n_mb)
 	want_loss.backward()
 	assert_close(torch.cat([r.float() for r in result]), out.detach(), "pipeline output")
-	assert abs(float(loss) - float(want_loss)) <= 2e-2 * float(want_loss)
+	assert abs(float(loss) - float(want_loss.detach())) <= 2e-2 * float(want_loss.detach())
 	for stage, ref in zip(stages, refs):
 		ref_params = dict(ref.named_parameters())
 		for name, p in stage.named_parameters():
