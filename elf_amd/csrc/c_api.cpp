@@ -26,6 +26,10 @@ int elf_gemm_swiglu_bwd_bf16(int M, int F, int K, const void* dY, int64_t lddy, 
 }
 
 #define S_(x) ((hipStream_t)(x))
+int elf_gemm_rope_bf16(int M, int N, int K, const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, const void* cs, int S,
+                       int n_rot_heads, int D, void* stream) {
+	return elf::gemm_rope_bf16(M, N, K, A, lda, W, ldw, C, ldc, cs, S, n_rot_heads, D, S_(stream));
+}
 int elf_norm_fwd(int kind, const void* x, const void* gamma, const void* beta, void* y, void* stats, int T, int d,
                  float eps, void* stream) {
 	return elf::norm_fwd(kind, x, gamma, beta, y, stats, T, d, eps, S_(stream));

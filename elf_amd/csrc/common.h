@@ -66,6 +66,14 @@ __device__ __forceinline__ void swiglu_bwd_f(float d, float g, float u, float& d
 	du = d * g * sig;
 }
 
+// Half-split rotary rotation of one (x_i, x_{i+D/2}) pair by the angle whose (cos, sin) is (c, s); the backward
+// passes -s.  Shared by the RoPE kernel and by the GEMM / attention epilogues that fuse it, so that all of them
+// give the same bits: one rounded product and one fused multiply-add per output.
+__device__ __forceinline__ void rope_rot(float lo, float hi, float c, float s, float& out_lo, float& out_hi) {
+	out_lo = __builtin_fmaf(lo, c, -(hi * s));
+	out_hi = __builtin_fmaf(hi, c, lo * s);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
 	for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);

@@ -518,9 +518,7 @@ __global__ __launch_bounds__(256) void rope_kernel(bf16_t* __restrict__ buf, con
 #pragma unroll
 		for (int j = 0; j < 8; j++) {
 			const float2 t2 = tab[j];
-			const float sn = t2.y * sign;
-			oa.v[j] = a.v[j] * t2.x - b.v[j] * sn;
-			ob.v[j] = b.v[j] * t2.x + a.v[j] * sn;
+			rope_rot(a.v[j], b.v[j], t2.x, t2.y * sign, oa.v[j], ob.v[j]);
 		}
 		store8(p, oa);
 		store8(p + D / 2, ob);

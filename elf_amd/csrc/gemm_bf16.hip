@@ -381,6 +381,27 @@ int gemm_act_bf16(int act, int M, int F, int K, const void* A, int64_t lda, cons
 	return act == ACT_SWIGLU ? swiglu_fwd(pre, out, M, F, stream) : gelu_fwd(pre, out, (int64_t)M * F, stream);
 }
 
+bool gemm_rope_fused(int M, int N, int K, int D) {
+	if (!(M > 0 && N > 0 && K > 0 && K % 64 == 0 && N % 256 == 0 && (D == 64 || D == 128))) return false;
+	// the tile choice gemm_bf16 makes for this shape
+	return (M % 256 == 0 && (int64_t)(M / 256) * (N / 256) >= 192) || (M % 128 == 0 && (int64_t)(M / 128) * (N / 256) >= 128);
+}
+
+int gemm_rope_bf16(int M, int N, int K, const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, const void* cs,
+                   int S, int n_rot_heads, int D, hipStream_t stream) {
+	ELF_REQUIRE(M > 0 && N > 0 && K > 0 && A && W && C && cs, "gemm_rope: empty problem or null operand");
+	ELF_REQUIRE(S > 0 && M % S == 0 && n_rot_heads >= 0 && (int64_t)n_rot_heads * D <= N, "gemm_rope: bad head layout (S=%d, heads=%d, D=%d, N=%d)", S, n_rot_heads, D, N);
+	if (gemm_rope_fused(M, N, K, D) && lda % 8 == 0 && ldw % 8 == 0 && ldc % 8 == 0 && lda >= K && ldw >= K && ldc >= N && ((uintptr_t)A % 16) == 0 &&
+	    ((uintptr_t)W % 16) == 0 && ((uintptr_t)C % 16) == 0 && ((uintptr_t)cs % 16) == 0) {
+		// the rotation's arithmetic is not counted: the figure stays the GEMM's
+		ProfScope prof(PROF_GEMM, 2.0 * M * N * K, stream);
+		const int bm = (M % 256 == 0 && (int64_t)(M / 256) * (N / 256) >= 192) ? 256 : 128;
+		return gemm_bf16_dma(0, 0, M, N, K, A, lda, W, ldw, C, ldc, EPI_BF16_ROPE, nullptr, 0, 1, 0, bm, stream, nullptr, 0, cs, S, n_rot_heads * D, D);
+	}
+	if (int rc = gemm_bf16(0, 0, M, N, K, A, lda, W, ldw, C, ldc, EPI_BF16, nullptr, 0, 0, 0, stream)) return rc;
+	return n_rot_heads ? rope_apply(C, cs, M, S, (int)ldc, n_rot_heads, D, 0, stream) : 0;
+}
+
 bool gemm_swiglu_bwd_fused(int M, int F, int K) {
 	return M > 0 && F > 0 && K > 0 && M % 256 == 0 && F % 256 == 0 && K % 64 == 0 && (int64_t)(M / 256) * (F / 256) >= 192;
 }

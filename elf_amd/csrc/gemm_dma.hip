@@ -61,6 +61,9 @@ struct Args {
 	int k_splits;    // K is split this many ways (fp32 atomics epilogue) for the last tail_tiles tiles
 	int tail_tiles;  // tiles_m * tiles_n for a uniform split, 0 when nothing is split
 	int walk;        // 1: all XCDs share one band of 16 tile rows at a time (see the tile assignment)
+	// EPI_BF16_ROPE: (cos, sin) table [rope_S, rope_D / 2], columns below rope_cols are rotated, heads are rope_D wide
+	const float2* rope_cs;
+	int rope_S, rope_cols, rope_D;
 };
 
 // Byte offsets (relative to the tile origin of the current K slice) of the 16-byte chunks this
@@ -465,6 +468,44 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 				*reinterpret_cast<bf16x8*>(c) = og;
 				*reinterpret_cast<bf16x8*>(c + F) = ou;
 			}
+		} else if constexpr (EPI == EPI_BF16_ROPE) {
+			// A 128-column strip holds whole heads (rope_D = 64 or 128).  A lane takes, for one row, 8 columns of a
+			// head's first half and the 8 columns half a head further on: the (x_i, x_{i + D/2}) pairs of the rotation.
+			// The accumulator is rounded to bf16 first, as the RoPE kernel would read it from memory.  The table
+			// entries of the whole strip are fetched before the first store (see the residual epilogue below).
+			const int half = g.rope_D >> 1, cph = half >> 3;  // chunks of 8 columns per half head
+			const int j = lane & 7;
+			const int c_lo = (j / cph) * g.rope_D + (j % cph) * 8, c_hi = c_lo + half;
+			const bool rot = gcol0 + c_lo < g.rope_cols;
+			f32x4 tab[4][4];
+			if (rot) {
+#pragma unroll
+				for (int it = 0; it < 4; it++) {
+					const int pos = (grow0 + it * 8 + (lane >> 3)) % g.rope_S;
+					const f32x4* tp = reinterpret_cast<const f32x4*>(g.rope_cs + (int64_t)pos * half + (j % cph) * 8);
+#pragma unroll
+					for (int q = 0; q < 4; q++) tab[it][q] = tp[q];
+				}
+			}
+#pragma unroll
+			for (int it = 0; it < 4; it++) {
+				const int row = it * 8 + (lane >> 3);
+				const float* w = ws + row * PITCH;
+				const f32x4 a0 = *reinterpret_cast<const f32x4*>(w + c_lo), a1 = *reinterpret_cast<const f32x4*>(w + c_lo + 4);
+				const f32x4 b0 = *reinterpret_cast<const f32x4*>(w + c_hi), b1 = *reinterpret_cast<const f32x4*>(w + c_hi + 4);
+				bf16x8 olo, ohi;
+#pragma unroll
+				for (int t = 0; t < 8; t++) {
+					const float a = (float)(bf16_t)(t < 4 ? a0[t] : a1[t - 4]), b = (float)(bf16_t)(t < 4 ? b0[t] : b1[t - 4]);
+					float ra = a, rb = b;
+					if (rot) rope_rot(a, b, tab[it][t >> 1][(t & 1) * 2], tab[it][t >> 1][(t & 1) * 2 + 1], ra, rb);
+					olo[t] = (bf16_t)ra;
+					ohi[t] = (bf16_t)rb;
+				}
+				bf16_t* c = reinterpret_cast<bf16_t*>(g.C) + (int64_t)(grow0 + row) * g.ldc + gcol0;
+				*reinterpret_cast<bf16x8*>(c + c_lo) = olo;
+				*reinterpret_cast<bf16x8*>(c + c_hi) = ohi;
+			}
 		} else if constexpr (EPI == EPI_BF16 || EPI == EPI_BF16_RESID) {
 			// the strip's residual values first, all loads in flight together: read inside the loop below each
 			// one would be awaited (a full trip to HBM) before the store that follows it in program order
@@ -552,6 +593,7 @@ static int launch_epi(const Args& a, int epi, hipStream_t stream) {
 	}
 	if constexpr (!AT && !BT) {
 		if (epi == EPI_BF16_SWIGLU) return launch<NW, RT, AT, BT, EPI_BF16_SWIGLU>(a, stream);
+		if (epi == EPI_BF16_ROPE) return launch<NW, RT, AT, BT, EPI_BF16_ROPE>(a, stream);
 	}
 	if constexpr (NW == 4 && RT == 4 && !AT && BT) {
 		if (epi == EPI_BF16_SWIGLU_BWD) return launch<NW, RT, AT, BT, EPI_BF16_SWIGLU_BWD>(a, stream);
@@ -565,7 +607,7 @@ static int launch_epi(const Args& a, int epi, hipStream_t stream) {
 // Arguments are validated by gemm_bf16() before it dispatches here.
 int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda, const void* B, int64_t ldb, void* C,
                   int64_t ldc, int epi, const void* R, int64_t ldr, int k_splits, int tail_tiles, int bm, hipStream_t stream,
-                  void* C2, int64_t ldc2) {
+                  void* C2, int64_t ldc2, const void* rope_cs, int rope_S, int rope_cols, int rope_D) {
 	ELF_REQUIRE(bm == 256 || bm == 128, "gemm (dma tile): 256- or 128-row tiles");
 	ELF_REQUIRE(M % bm == 0 && N % dma::BN == 0 && K % dma::BKS == 0, "gemm (dma tile): M multiple of %d, N of 256 and K of 64 required", bm);
 	ELF_REQUIRE(bm == 256 || !a_t, "gemm (dma tile): 128-row tiles need a k-contiguous A");
@@ -573,8 +615,10 @@ int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t 
 	ELF_REQUIRE(epi != EPI_BF16_SWIGLU || (C2 && !a_t && !b_t), "gemm (dma tile): the SwiGLU epilogue needs k-contiguous operands and a second output");
 	// the paired rows of the SwiGLU epilogue are addressed with 32-bit byte offsets from the tile's first row
 	ELF_REQUIRE(epi != EPI_BF16_SWIGLU || (int64_t)(N / 2 + 256) * ldb * 2 < (int64_t(1) << 31), "gemm (dma tile): weight too large for the paired-row epilogue");
+	ELF_REQUIRE(epi != EPI_BF16_ROPE || (rope_cs && rope_S > 0 && !a_t && !b_t && (rope_D == 64 || rope_D == 128) && rope_cols % rope_D == 0 && rope_cols <= N),
+	            "gemm (dma tile): the RoPE epilogue needs k-contiguous operands, a table and heads of 64 or 128 columns");
 	dma::Args a{(const bf16_t*)A, (const bf16_t*)B, C, (const bf16_t*)R, (bf16_t*)C2, lda, ldb, ldc, ldr, ldc2, M, N, K, M / bm, N / dma::BN, k_splits < 1 ? 1 : k_splits,
-	            tail_tiles < 0 || tail_tiles > ntiles ? ntiles : tail_tiles, 0};
+	            tail_tiles < 0 || tail_tiles > ntiles ? ntiles : tail_tiles, 0, (const float2*)rope_cs, rope_S, rope_cols, rope_D};
 	// The band walk fetches every row slab of A from HBM in one round only and B once per band; the default
 	// walk wants A in the 256 MB memory-side cache for the whole launch and streams B once.  Inside the stage's
 	// stream (operands cold, per-shape times from a kernel trace) the bands are 0-5 % faster on every shape but

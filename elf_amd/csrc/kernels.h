@@ -14,6 +14,9 @@ enum GemmEpilogue {
 	EPI_BF16_SWIGLU = 4,  // B = [gate rows; up rows]: C(bf16) = acc = [g | u], C2(bf16) = silu(g) * u
 	// k-contiguous A only (see gemm_swiglu_bwd_bf16): R = [g | u] (bf16, N columns each), acc rounded to bf16 = d:
 	EPI_BF16_SWIGLU_BWD = 5,  // C(bf16) = [d silu'(g) u | d silu(g)]
+	// k-contiguous operands (see gemm_rope_bf16): C(bf16) = acc rounded to bf16, then the half-split rotary rotation of
+	// the heads (width rope_D) that lie in the first rope_cols columns, position = row mod rope_S
+	EPI_BF16_ROPE = 6,
 };
 
 int gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda, const void* B, int64_t ldb,
@@ -25,7 +28,16 @@ int gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda,
 // EPI_F32_ACC only: the last tail_tiles tiles (all of them when tail_tiles < 0) are split k_splits ways along K.
 int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda, const void* B, int64_t ldb, void* C,
                   int64_t ldc, int epi, const void* R, int64_t ldr, int k_splits, int tail_tiles, int bm, hipStream_t stream,
-                  void* C2 = nullptr, int64_t ldc2 = 0);
+                  void* C2 = nullptr, int64_t ldc2 = 0, const void* rope_cs = nullptr, int rope_S = 0, int rope_cols = 0, int rope_D = 0);
+
+// The attention block's packed q | k | v projection with the rotary embedding of the q and k heads: C [M, N] =
+// A W^T rounded to bf16, then rope_apply's rotation on the first n_rot_heads heads of width D (cs: the table of
+// rope_table for sequence length S; row r is at position r mod S).  One kernel (rotation in the GEMM epilogue, the
+// projection is not read back) when the shape fits the direct-to-LDS tiles; otherwise the GEMM is followed by the
+// RoPE kernel.  Both ways give the same bits.
+bool gemm_rope_fused(int M, int N, int K, int D);
+int gemm_rope_bf16(int M, int N, int K, const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, const void* cs,
+                   int S, int n_rot_heads, int D, hipStream_t stream);
 
 enum Activation { ACT_GELU = 0, ACT_SWIGLU = 1 };
 // Up-projection of the MLP with its activation: pre = A W^T (A [M, K], W [N, K], N = F for GELU and 2F =

@@ -239,8 +239,9 @@ static int run_forward(Stage* s, MbState& m, const void* x, void* y, FwdMode mod
 		ELF_TRY(buf_alloc(s, bs, B_H1));
 		ELF_TRY(norm_fwd(norm_kind, xin, p.w[P_NORM1_G], p.w[P_NORM1_B], bs.b[B_H1].p, bs.b[B_ST1].p, T, d, s->cfg.eps, st));
 		ELF_TRY(buf_alloc(s, bs, B_QKV));
-		ELF_TRY(gemm_bf16(0, 0, T, s->nqkv, d, bs.b[B_H1].p, d, p.w[P_WQKV], d, bs.b[B_QKV].p, s->nqkv, EPI_BF16, nullptr, 0, 0, 0, st));
-		if (s->llama) ELF_TRY(rope_apply(bs.b[B_QKV].p, s->rope_cs, T, s->S, s->nqkv, s->Hq + s->Hkv, s->D, 0, st));
+		// the packed projection, with the rotary embedding of the q and k heads in the GEMM's epilogue where the shape allows
+		if (s->llama) ELF_TRY(gemm_rope_bf16(T, s->nqkv, d, bs.b[B_H1].p, d, p.w[P_WQKV], d, bs.b[B_QKV].p, s->nqkv, s->rope_cs, s->S, s->Hq + s->Hkv, s->D, st));
+		else ELF_TRY(gemm_bf16(0, 0, T, s->nqkv, d, bs.b[B_H1].p, d, p.w[P_WQKV], d, bs.b[B_QKV].p, s->nqkv, EPI_BF16, nullptr, 0, 0, 0, st));
 		ELF_TRY(buf_alloc(s, bs, B_O));
 		ELF_TRY(buf_alloc(s, bs, B_LSE));
 		{
@@ -392,8 +393,8 @@ static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool gra
 		}
 		if (bs.b[B_QKV].dropped) {
 			ELF_TRY(buf_alloc(s, bs, B_QKV));
-			ELF_TRY(gemm_bf16(0, 0, T, s->nqkv, d, bs.b[B_H1].p, d, p.w[P_WQKV], d, bs.b[B_QKV].p, s->nqkv, EPI_BF16, nullptr, 0, 0, 0, st));
-			if (s->llama) ELF_TRY(rope_apply(bs.b[B_QKV].p, s->rope_cs, T, s->S, s->nqkv, s->Hq + s->Hkv, s->D, 0, st));
+			if (s->llama) ELF_TRY(gemm_rope_bf16(T, s->nqkv, d, bs.b[B_H1].p, d, p.w[P_WQKV], d, bs.b[B_QKV].p, s->nqkv, s->rope_cs, s->S, s->Hq + s->Hkv, s->D, st));
+			else ELF_TRY(gemm_bf16(0, 0, T, s->nqkv, d, bs.b[B_H1].p, d, p.w[P_WQKV], d, bs.b[B_QKV].p, s->nqkv, EPI_BF16, nullptr, 0, 0, 0, st));
 		}
 		if (bs.b[B_LSE].dropped) {  // checkpointed attention core: its output and log-sum-exp are formed again
 			ELF_TRY(buf_alloc(s, bs, B_O));

@@ -69,6 +69,21 @@ def gemm_act(a, w, act):
 	return pre, out
 
 
+def gemm_rope(a, w, cs, S, n_rot_heads, D, fused=True):
+	"""a @ w.T with the rotary embedding applied to the first ``n_rot_heads`` heads of width ``D`` of the result
+	(rows are tokens at position row % S); ``fused=False`` forces the GEMM + RoPE kernel pair (same bits)."""
+	_need(a, torch.bfloat16, "gemm_rope.a")
+	_need(w, torch.bfloat16, "gemm_rope.w")
+	M, K = a.shape
+	N = w.shape[0]
+	if not fused:
+		return rope_apply_(gemm(a, w), cs, S, n_rot_heads, D)
+	c = torch.empty((M, N), dtype=torch.bfloat16, device=a.device)
+	rc = _lib.load().elf_gemm_rope_bf16(M, N, K, _ptr(a), a.stride(0), _ptr(w), w.stride(0), _ptr(c), N, _ptr(cs), S, n_rot_heads, D, _stream())
+	_lib.check(rc, "elf_gemm_rope_bf16")
+	return c
+
+
 def gemm_swiglu_bwd(dy, w2, gu, fused=True):
 	"""dgu [M, 2F]: gradient of gu = [g | u] for d = dy @ w2 (dy [M, K], w2 [K, F]); ``fused=False`` forces the
 	GEMM + activation-backward pair (same bits)."""

@@ -65,6 +65,17 @@ int elf_gemm_act_bf16(int act, int M, int F, int K, const void* A, int64_t lda, 
 int elf_gemm_swiglu_bwd_bf16(int M, int F, int K, const void* dY, int64_t lddy, const void* W, int64_t ldw,
                              const void* gu, int64_t ldgu, void* dgu, int64_t lddgu, void* scratch, void* stream);
 
+/* The attention block's packed q | k | v projection with the rotary embedding of its q and k heads:
+ * C[M, N] = A W^T (A [M, K], W [N, K], both k contiguous) rounded to bf16, then the rotation of elf_rope_apply
+ * on the first n_rot_heads heads of width D (64 or 128); cs is the table of elf_rope_table for sequence length
+ * S, row r of A is the token at position r mod S.  One kernel (rotation in the GEMM epilogue, the projection
+ * is never read back) when M is a multiple of 128, N of 256, K of 64 and the tiles fill the chip; otherwise
+ * elf_gemm_bf16 followed by elf_rope_apply.  Same bits either way.
+ * Replaces: the q / k / v projections of the attention block run through LinearDX.forward
+ *           (elf/zb_utils.py:20); no reference module for the rotary embedding. */
+int elf_gemm_rope_bf16(int M, int N, int K, const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc,
+                       const void* cs, int S, int n_rot_heads, int D, void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Bandwidth-bound stage ops.  bf16 row-major tensors, fp32 math, one rounding on store.
  * kind: 0 = RMSNorm (y = x * rsqrt(mean(x^2)+eps) * gamma; no reference module, textbook form),

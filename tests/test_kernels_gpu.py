@@ -228,6 +228,28 @@ def test_gemm_with_swiglu_backward_epilogue(K, shape):
 	_close(dgu, g32.grad, what="gradient of [g | u]")
 
 
+@pytest.mark.parametrize("shape", [(8192, 6144, 256, 4096, 32, 8, 128), (4096, 2048, 64, 1024, 12, 4, 64), (2048, 4096, 128, 512, 5, 3, 128), (512, 1024, 128, 256, 4, 2, 128)])
+def test_gemm_with_rope_epilogue(K, shape):
+	"""The packed q | k | v projection with the rotary embedding of its q and k heads in the GEMM epilogue:
+	bit for bit against the GEMM followed by the RoPE kernel, and against an fp32 rotation (fp64 angles) of
+	the rounded projection.  Shapes: 256x256 tiles with heads of 128 (the Llama-3-8B projection), 128x256
+	tiles with heads of 64, an odd number of rotated heads (the v heads start in the middle of a tile), and
+	one the fused tiles do not cover (the library runs the two kernels itself)."""
+	M, N, Kd, S, Hq, Hkv, D = shape
+	assert (Hq + 2 * Hkv) * D <= N
+	A = _randn(M, Kd, seed=61)
+	W = _randn(N, Kd, seed=62, scale=0.1)
+	cs = K.rope_table(S, D, 5e5)
+	got = K.gemm_rope(A, W, cs, S, Hq + Hkv, D)
+	two = K.gemm_rope(A, W, cs, S, Hq + Hkv, D, fused=False)
+	assert torch.equal(got, two), "fused rotation differs from the separate kernel"
+	plain = K.gemm(A, W)
+	nrot = (Hq + Hkv) * D
+	assert torch.equal(got[:, nrot:], plain[:, nrot:]), "columns after the rotated heads must be the plain projection"
+	ref = _rope_ref(plain[:, :nrot].float().view(M, Hq + Hkv, D), S, D, 5e5).reshape(M, nrot)
+	_close(got[:, :nrot], ref, what="rotated projection")
+
+
 def test_gemm_with_activation_strided_outputs(K):
 	# outputs that are column slices of wider buffers, as a caller that packs activations would pass
 	from elf_amd import _lib
