@@ -46,6 +46,9 @@ struct AttnBwdArgs {
 	int64_t ldq, ldk, ldv, lddo, lddk, lddv;
 	int B, S, Hq, Hkv;
 	float scale;
+	// non-null: the q and k heads carry a rotary embedding whose backward (the inverse rotation) is applied to
+	// dQ and dK before they are stored; (cos, sin) table [S, D / 2] of rope_table()
+	const float2* rope_cs;
 };
 
 // dQ partials.  Every 128-key tile contributes a [queries, Hq*D] partial dQ; the partials are written
@@ -117,6 +120,58 @@ __device__ __forceinline__ bf16x8 ds_t_frag(const unsigned char* t, int k0, int 
 	s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 ELF_LDS*)(t + ds_t_offset(kk, q)));
 	s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 ELF_LDS*)(t + ds_t_offset(kk + 4, q)));
 	return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+}
+
+// dK^T / dV^T accumulators of one wave -> memory: register r of tile dt <-> d = dt*32 + (r/4)*8 + 4g + r%4, lane <-> key.
+// With a rotary embedding on the k heads, dK (scaled and rounded to bf16, as a separate RoPE pass over the stored
+// gradient would read it) is rotated back first; the partner of column d is d + D/2, same register of tile dt + DT/2.
+template <int D>
+__device__ __forceinline__ void store_dk_dv(const f32x16 (&acc_dk)[D / 32], const f32x16 (&acc_dv)[D / 32], bf16_t* dkp, bf16_t* dvp, float scale, int g,
+                                            const float2* cs_row) {
+	constexpr int DT = D / 32;
+#pragma unroll
+	for (int dt = 0; dt < DT; dt++) {
+#pragma unroll
+		for (int r4 = 0; r4 < 4; r4++) {
+			bf16x4 v4;
+#pragma unroll
+			for (int u = 0; u < 4; u++) v4[u] = (bf16_t)acc_dv[dt][r4 * 4 + u];
+			*reinterpret_cast<bf16x4*>(dvp + dt * 32 + r4 * 8 + 4 * g) = v4;
+		}
+	}
+	if (cs_row == nullptr) {
+#pragma unroll
+		for (int dt = 0; dt < DT; dt++) {
+#pragma unroll
+			for (int r4 = 0; r4 < 4; r4++) {
+				bf16x4 k4;
+#pragma unroll
+				for (int u = 0; u < 4; u++) k4[u] = (bf16_t)(acc_dk[dt][r4 * 4 + u] * scale);
+				*reinterpret_cast<bf16x4*>(dkp + dt * 32 + r4 * 8 + 4 * g) = k4;
+			}
+		}
+		return;
+	}
+#pragma unroll
+	for (int dt = 0; dt < DT / 2; dt++) {
+#pragma unroll
+		for (int r4 = 0; r4 < 4; r4++) {
+			const int i = dt * 32 + r4 * 8 + 4 * g;
+			const f32x4 t0 = *reinterpret_cast<const f32x4*>(cs_row + i), t1 = *reinterpret_cast<const f32x4*>(cs_row + i + 2);
+			bf16x4 lo4, hi4;
+#pragma unroll
+			for (int u = 0; u < 4; u++) {
+				const float lo = (float)(bf16_t)(acc_dk[dt][r4 * 4 + u] * scale), hi = (float)(bf16_t)(acc_dk[dt + DT / 2][r4 * 4 + u] * scale);
+				const float c = (u < 2 ? t0 : t1)[(u & 1) * 2], sn = (u < 2 ? t0 : t1)[(u & 1) * 2 + 1];
+				float rl, rh;
+				rope_rot(lo, hi, c, -sn, rl, rh);
+				lo4[u] = (bf16_t)rl;
+				hi4[u] = (bf16_t)rh;
+			}
+			*reinterpret_cast<bf16x4*>(dkp + i) = lo4;
+			*reinterpret_cast<bf16x4*>(dkp + i + D / 2) = hi4;
+		}
+	}
 }
 
 // One workgroup pass = 128 keys of one (batch, kv head); wave w owns keys [32w, 32w+32) and
@@ -409,20 +464,7 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(AttnBwdArgs a) {
 		// dK^T / dV^T accumulators: register r <-> d = dt*32 + (r/4)*8 + 4g + r%4, lane <-> key
 		bf16_t* dkp = a.dk + (tok0 + wkey0 + kl) * a.lddk + hk * D;
 		bf16_t* dvp = a.dv + (tok0 + wkey0 + kl) * a.lddv + hk * D;
-#pragma unroll
-		for (int dt = 0; dt < DT; dt++) {
-#pragma unroll
-			for (int r4 = 0; r4 < 4; r4++) {
-				bf16x4 k4, v4;
-#pragma unroll
-				for (int u = 0; u < 4; u++) {
-					k4[u] = (bf16_t)(acc_dk[dt][r4 * 4 + u] * a.scale);
-					v4[u] = (bf16_t)acc_dv[dt][r4 * 4 + u];
-				}
-				*reinterpret_cast<bf16x4*>(dkp + dt * 32 + r4 * 8 + 4 * g) = k4;
-				*reinterpret_cast<bf16x4*>(dvp + dt * 32 + r4 * 8 + 4 * g) = v4;
-			}
-		}
+		store_dk_dv<D>(acc_dk, acc_dv, dkp, dvp, a.scale, g, a.rope_cs ? a.rope_cs + (int64_t)(wkey0 + kl) * (D / 2) : nullptr);
 	}
 }
 
@@ -726,50 +768,61 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel_lone(AttnBwdArgs a) {
 		// dK^T / dV^T accumulators: register r <-> d = dt*32 + (r/4)*8 + 4g + r%4, lane <-> key
 		bf16_t* dkp = a.dk + (tok0 + wkey0 + kl) * a.lddk + hk * D;
 		bf16_t* dvp = a.dv + (tok0 + wkey0 + kl) * a.lddv + hk * D;
-#pragma unroll
-		for (int dt = 0; dt < DT; dt++) {
-#pragma unroll
-			for (int r4 = 0; r4 < 4; r4++) {
-				bf16x4 k4, v4;
-#pragma unroll
-				for (int u = 0; u < 4; u++) {
-					k4[u] = (bf16_t)(acc_dk[dt][r4 * 4 + u] * a.scale);
-					v4[u] = (bf16_t)acc_dv[dt][r4 * 4 + u];
-				}
-				*reinterpret_cast<bf16x4*>(dkp + dt * 32 + r4 * 8 + 4 * g) = k4;
-				*reinterpret_cast<bf16x4*>(dvp + dt * 32 + r4 * 8 + 4 * g) = v4;
-			}
-		}
+		store_dk_dv<D>(acc_dk, acc_dv, dkp, dvp, a.scale, g, a.rope_cs ? a.rope_cs + (int64_t)(wkey0 + kl) * (D / 2) : nullptr);
 	}
 }
 
 // dq[b, q, :] (bf16, row stride ld) = scale * sum over the key tiles that meet q of their partial rows,
-// added in fp32 in ascending tile order; 8 columns (16 bytes) per thread.
+// added in fp32 in ascending tile order.  A thread takes 8 columns of a head's first half and the 8 columns
+// half a head further on; with a rotary embedding on the q heads (cs non-null) these are the pairs of the
+// rotation, which is undone on the scaled, bf16-rounded sums before they are stored (what a separate RoPE
+// pass over the stored gradient would compute).
 __global__ __launch_bounds__(256) void dq_reduce_kernel(const bf16_t* __restrict__ part, bf16_t* __restrict__ dq, int B, int S, int cols,
-                                                        int64_t ld, float scale, int causal) {
-	const int cpr = cols / 8;
-	const int64_t n = (int64_t)B * S * cpr;
+                                                        int64_t ld, float scale, int causal, int D, const float2* __restrict__ cs) {
+	const int half = D / 2, cph = half / 8;  // 8-column chunks per half head
+	const int ppr = cols / 16;               // chunk pairs per row
+	const int64_t n = (int64_t)B * S * ppr;
 	const int nkt = S / 128;
 	const int64_t rows_b = part_rows(S, causal);
 	for (int64_t j = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; j < n; j += (int64_t)gridDim.x * blockDim.x) {
 		// last rows first: under a causal mask they sum the most partials, and the launch then ends on the short ones
 		const int64_t i = n - 1 - j;
-		const int64_t row = i / cpr;
-		const int c = (int)(i - row * cpr) * 8;
+		const int64_t row = i / ppr;
+		const int pr = (int)(i - row * ppr);
+		const int c = (pr / cph) * D + (pr % cph) * 8;
 		const int b = (int)(row / S), q = (int)(row - (int64_t)b * S);
 		const int ns = causal ? q / 128 + 1 : nkt;
-		float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+		float lo[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, hi[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 		const bf16_t* pb = part + (int64_t)b * rows_b * cols + c;
-#pragma unroll 8
+#pragma unroll 4
 		for (int kt = 0; kt < ns; kt++) {
-			const bf16x8 v = *reinterpret_cast<const bf16x8*>(pb + (part_row0(kt, S, causal) + q - (causal ? 128 * kt : 0)) * cols);
+			const bf16_t* pr_row = pb + (part_row0(kt, S, causal) + q - (causal ? 128 * kt : 0)) * cols;
+			const bf16x8 v = *reinterpret_cast<const bf16x8*>(pr_row), w = *reinterpret_cast<const bf16x8*>(pr_row + half);
 #pragma unroll
-			for (int t = 0; t < 8; t++) acc[t] += (float)v[t];
+			for (int t = 0; t < 8; t++) {
+				lo[t] += (float)v[t];
+				hi[t] += (float)w[t];
+			}
 		}
-		bf16x8 o;
+		bf16x8 olo, ohi;
 #pragma unroll
-		for (int t = 0; t < 8; t++) o[t] = (bf16_t)(acc[t] * scale);
-		*reinterpret_cast<bf16x8*>(dq + row * ld + c) = o;
+		for (int t = 0; t < 8; t++) {
+			olo[t] = (bf16_t)(lo[t] * scale);
+			ohi[t] = (bf16_t)(hi[t] * scale);
+		}
+		if (cs) {
+			const float2* tab = cs + (int64_t)q * half + (pr % cph) * 8;
+#pragma unroll
+			for (int t = 0; t < 8; t++) {
+				const float2 t2 = tab[t];
+				float rl, rh;
+				rope_rot((float)olo[t], (float)ohi[t], t2.x, -t2.y, rl, rh);
+				olo[t] = (bf16_t)rl;
+				ohi[t] = (bf16_t)rh;
+			}
+		}
+		*reinterpret_cast<bf16x8*>(dq + row * ld + c) = olo;
+		*reinterpret_cast<bf16x8*>(dq + row * ld + c + half) = ohi;
 	}
 }
 
@@ -801,8 +854,9 @@ int64_t attn_bwd_workspace_bytes(int B, int S, int Hq, int D, int causal) {
 int attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* dO, const void* lse, void* dq,
              void* dk, void* dv, void* workspace, int64_t ldq, int64_t ldk, int64_t ldv, int64_t ldo, int64_t lddo,
              int64_t lddq, int64_t lddk, int64_t lddv, int B, int S, int Hq, int Hkv, int D, int causal, float scale,
-             hipStream_t stream) {
+             hipStream_t stream, const void* rope_cs) {
 	ELF_REQUIRE(q && k && v && o && dO && lse && dq && dk && dv && workspace, "attn_bwd: null pointer");
+	ELF_REQUIRE(((uintptr_t)rope_cs % 16) == 0, "attn_bwd: misaligned rotary table");
 	ELF_REQUIRE(B > 0 && S > 0 && S % 128 == 0, "attn_bwd: sequence length must be a multiple of 128 (S=%d)", S);
 	ELF_REQUIRE(Hkv > 0 && Hq % Hkv == 0, "attn_bwd: Hq must be a multiple of Hkv (Hq=%d Hkv=%d)", Hq, Hkv);
 	ELF_REQUIRE(D == 64 || D == 128, "attn_bwd: head_dim must be 64 or 128 (D=%d)", D);
@@ -823,17 +877,17 @@ int attn_bwd(const void* q, const void* k, const void* v, const void* o, const v
 	                   (const bf16_t*)o, (const float*)lse, delta, nlse2, lddo, ldo, B, S, Hq, D);
 	}
 	AttnBwdArgs a{(const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, (const bf16_t*)dO, nlse2, delta, dq_part,
-	              (bf16_t*)dk, (bf16_t*)dv, ldq, ldk, ldv, lddo, lddk, lddv, B, S, Hq, Hkv, scale};
+	              (bf16_t*)dk, (bf16_t*)dv, ldq, ldk, ldv, lddo, lddk, lddv, B, S, Hq, Hkv, scale, (const float2*)rope_cs};
 	const int nkt = S / 128;
 	const dim3 grid((unsigned)((int64_t)B * Hkv * (causal ? (nkt + 1) / 2 : nkt))), block(256);
 	int rc;
 	if (D == 128) rc = causal ? launch_bwd<128, true>(a, grid, stream) : launch_bwd<128, false>(a, grid, stream);
 	else rc = causal ? launch_bwd<64, true>(a, grid, stream) : launch_bwd<64, false>(a, grid, stream);
 	if (rc) return rc;
-	const int64_t n8 = T * (Hq * D / 8);
-	const int64_t blocks = (n8 + 255) / 256;
+	const int64_t n16 = T * (Hq * D / 16);
+	const int64_t blocks = (n16 + 255) / 256;
 	hipLaunchKernelGGL(dq_reduce_kernel, dim3((unsigned)(blocks < 16384 ? blocks : 16384)), dim3(256), 0, stream, dq_part, (bf16_t*)dq, B, S,
-	                   Hq * D, lddq, scale, causal);
+	                   Hq * D, lddq, scale, causal, D, (const float2*)rope_cs);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
 }

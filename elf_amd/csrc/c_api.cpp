@@ -94,6 +94,14 @@ int elf_attn_bwd(const void* q, const void* k, const void* v, const void* o, con
 	                     Hkv, D, causal, scale, S_(stream));
 }
 
+int elf_attn_bwd_rope(const void* q, const void* k, const void* v, const void* o, const void* dO, const void* lse, void* dq,
+                      void* dk, void* dv, void* workspace, int64_t ldq, int64_t ldk, int64_t ldv, int64_t ldo, int64_t lddo,
+                      int64_t lddq, int64_t lddk, int64_t lddv, int B, int S, int Hq, int Hkv, int D, int causal, float scale,
+                      const void* cs, void* stream) {
+	return elf::attn_bwd(q, k, v, o, dO, lse, dq, dk, dv, workspace, ldq, ldk, ldv, ldo, lddo, lddq, lddk, lddv, B, S, Hq,
+	                     Hkv, D, causal, scale, S_(stream), cs);
+}
+
 void elf_prof_enable(int on) { elf::prof_enable(on); }
 int elf_prof_collect(int kind, double* total_ms, double* total_work) {
 	if (kind < 0 || kind >= elf::PROF_COUNT) return -1;

@@ -96,7 +96,9 @@ int64_t attn_bwd_workspace_bytes(int B, int S, int Hq, int D, int causal);
 int attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* dO, const void* lse, void* dq,
              void* dk, void* dv, void* workspace, int64_t ldq, int64_t ldk, int64_t ldv, int64_t ldo, int64_t lddo,
              int64_t lddq, int64_t lddk, int64_t lddv, int B, int S, int Hq, int Hkv, int D, int causal, float scale,
-             hipStream_t stream);
+             hipStream_t stream, const void* rope_cs = nullptr);
+// rope_cs non-null: q and k are the rotated heads (rope_apply with this table); dq and dk come out as the gradients
+// of the heads before the rotation (rope_apply's backward applied to them), bit-identical to the separate pass.
 
 // Optional live timing of kernel launches: when enabled, every launcher brackets its launches
 // with an event pair on the launch stream and books the algorithmic work of the call.

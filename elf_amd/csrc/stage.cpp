@@ -407,11 +407,12 @@ static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool gra
 			const bf16_t* q = (const bf16_t*)bs.b[B_QKV].p;
 			bf16_t* dq = (bf16_t*)bs.b[B_DQKV].p;
 			const int ko = s->Hq * s->D, vo = (s->Hq + s->Hkv) * s->D;
+			// the llama block's q and k carry the rotary embedding: its backward is applied to dQ and dK where they are stored
 			ELF_TRY(attn_bwd(q, q + ko, q + vo, bs.b[B_O].p, d_o.p, bs.b[B_LSE].p, dq, dq + ko, dq + vo, s->attn_ws, s->nqkv, s->nqkv, s->nqkv,
-			                 s->Hq * s->D, s->Hq * s->D, s->nqkv, s->nqkv, s->nqkv, s->B, s->S, s->Hq, s->Hkv, s->D, s->cfg.causal, scale, st));
+			                 s->Hq * s->D, s->Hq * s->D, s->nqkv, s->nqkv, s->nqkv, s->B, s->S, s->Hq, s->Hkv, s->D, s->cfg.causal, scale, st,
+			                 s->llama ? s->rope_cs : nullptr));
 		}
 		d_o.release();
-		if (s->llama) ELF_TRY(rope_apply(bs.b[B_DQKV].p, s->rope_cs, T, s->S, s->nqkv, s->Hq + s->Hkv, s->D, 1, st));
 		if (!(grads_only && i == 0)) {
 			ELF_TRY(gemm_bf16(0, 1, T, d, s->nqkv, bs.b[B_DQKV].p, s->nqkv, p.w[P_WQKV], d, d_h.p, d, EPI_BF16, nullptr, 0, 0, 0, st));
 			void* dxout;

@@ -220,8 +220,9 @@ def attn_fwd(qkv, B, S, Hq, Hkv, D, causal, scale=None):
 	return o, lse
 
 
-def attn_bwd(qkv, o, do, lse, B, S, Hq, Hkv, D, causal, scale=None):
-	"""Returns dqkv packed like qkv."""
+def attn_bwd(qkv, o, do, lse, B, S, Hq, Hkv, D, causal, scale=None, rope_cs=None):
+	"""Returns dqkv packed like qkv.  ``rope_cs``: the q and k heads of ``qkv`` are rotated (``rope_apply_`` with this
+	table); dq and dk then come out with the rotation's backward applied."""
 	T, ld = qkv.shape[0], qkv.stride(0)
 	scale = scale if scale is not None else 1.0 / math.sqrt(D)
 	lib = _lib.load()
@@ -229,7 +230,10 @@ def attn_bwd(qkv, o, do, lse, B, S, Hq, Hkv, D, causal, scale=None):
 	dqkv = torch.empty_like(qkv)
 	q, k, v = qkv[:, : Hq * D], qkv[:, Hq * D : (Hq + Hkv) * D], qkv[:, (Hq + Hkv) * D :]
 	dq, dk, dv = dqkv[:, : Hq * D], dqkv[:, Hq * D : (Hq + Hkv) * D], dqkv[:, (Hq + Hkv) * D :]
-	rc = lib.elf_attn_bwd(_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(lse), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ws),
-	                      ld, ld, ld, o.stride(0), do.stride(0), dqkv.stride(0), dqkv.stride(0), dqkv.stride(0), B, S, Hq, Hkv, D, int(causal), scale, _stream())
-	_lib.check(rc, "elf_attn_bwd")
+	args = (_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(lse), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ws),
+	        ld, ld, ld, o.stride(0), do.stride(0), dqkv.stride(0), dqkv.stride(0), dqkv.stride(0), B, S, Hq, Hkv, D, int(causal), scale)
+	if rope_cs is None:
+		_lib.check(lib.elf_attn_bwd(*args, _stream()), "elf_attn_bwd")
+	else:
+		_lib.check(lib.elf_attn_bwd_rope(*args, _ptr(rope_cs), _stream()), "elf_attn_bwd_rope")
 	return dqkv

@@ -176,6 +176,17 @@ int elf_attn_bwd(const void* q, const void* k, const void* v, const void* o, con
                  int64_t lddv, int B, int S, int Hq, int Hkv, int D, int causal, float scale,
                  void* stream);
 
+/* elf_attn_bwd for q and k heads that carry a rotary embedding (q, k are the rotated heads as elf_rope_apply /
+ * elf_gemm_rope_bf16 left them; cs is that table): dq and dk come out as the gradients of the heads BEFORE the
+ * rotation, i.e. with elf_rope_apply(..., backward = 1) already applied where they are stored (the dQ reduction and
+ * the dK epilogue), bit-identical to elf_attn_bwd followed by that call.  cs = NULL is elf_attn_bwd.
+ * No reference module for the rotary embedding; replaces the autograd backward of the rotation. */
+int elf_attn_bwd_rope(const void* q, const void* k, const void* v, const void* o, const void* dO,
+                      const void* lse, void* dq, void* dk, void* dv, void* workspace, int64_t ldq,
+                      int64_t ldk, int64_t ldv, int64_t ldo, int64_t lddo, int64_t lddq, int64_t lddk,
+                      int64_t lddv, int B, int S, int Hq, int Hkv, int D, int causal, float scale,
+                      const void* cs, void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Stage executor: one pipeline stage = n_blocks transformer blocks on T = mb * seq tokens.
  * It is what PipelineBlock (elf/execution/block.py:134-694) does through nn.Module.__call__ and

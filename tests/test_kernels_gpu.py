@@ -347,3 +347,8 @@ def test_attention_fwd_bwd(K, cfg):
 		_close(dqkv[:, sl], dqkv_ref[:, sl], rel_fro=1.5e-2, what=f"attn {name} {cfg}")
 	# no atomics anywhere in the backward: a second run gives the same bits
 	assert torch.equal(dqkv, K.attn_bwd(qkv, o, do, lse, B, S, Hq, Hkv, D, causal))
+	# the backward of a rotary embedding on q and k, applied where dQ and dK are stored: the bits of the plain
+	# backward followed by the RoPE kernel's backward pass
+	cs = K.rope_table(S, D, 5e5)
+	fused = K.attn_bwd(qkv, o, do, lse, B, S, Hq, Hkv, D, causal, rope_cs=cs)
+	assert torch.equal(fused, K.rope_apply_(dqkv.clone(), cs, S, Hq + Hkv, D, backward=True))
