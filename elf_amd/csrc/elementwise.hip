@@ -231,17 +231,18 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(const bf16_t* __restrict_
 	}
 }
 
-// main_grad[c] += sum_b part[b][which][c].  A workgroup owns 32 columns and one of gridDim.y slices
-// of the partial rows; its 8 row groups stride over the slice and are folded through LDS, the
-// slices meet in the accumulator through fp32 atomics (a few thousand per call).
-__global__ __launch_bounds__(256) void norm_bwd_finalize_kernel(const float* __restrict__ part, int nparts, int d,
-                                                                float* __restrict__ dgamma, float* __restrict__ dbeta) {
-	__shared__ float red[2][8][32];
+// main_grad[c] += sum_b part[b][which][c].  A workgroup owns 32 columns; its 32 row groups stride over the partial
+// rows and are folded through LDS in a fixed order, and each column has one writer: the sums do not depend on
+// the order in which workgroups run (bit-reproducible gamma / beta gradients).
+__global__ __launch_bounds__(1024) void norm_bwd_finalize_kernel(const float* __restrict__ part, int nparts, int d,
+                                                                 float* __restrict__ dgamma, float* __restrict__ dbeta) {
+	__shared__ float red[2][32][33];
 	const int cl = threadIdx.x & 31, rg = threadIdx.x >> 5;
 	const int c = blockIdx.x * 32 + cl;
 	float sg = 0.f, sb = 0.f;
 	if (c < d) {
-		for (int b = blockIdx.y * 8 + rg; b < nparts; b += 8 * gridDim.y) {
+#pragma unroll 4
+		for (int b = rg; b < nparts; b += 32) {
 			sg += part[(int64_t)b * 2 * d + c];
 			if (dbeta) sb += part[(int64_t)b * 2 * d + d + c];
 		}
@@ -252,12 +253,12 @@ __global__ __launch_bounds__(256) void norm_bwd_finalize_kernel(const float* __r
 	if (rg == 0 && c < d) {
 		float tg = 0.f, tb = 0.f;
 #pragma unroll
-		for (int r = 0; r < 8; r++) {
+		for (int r = 0; r < 32; r++) {
 			tg += red[0][r][cl];
 			tb += red[1][r][cl];
 		}
-		unsafeAtomicAdd(dgamma + c, tg);
-		if (dbeta) unsafeAtomicAdd(dbeta + c, tb);
+		dgamma[c] += tg;
+		if (dbeta) dbeta[c] += tb;
 	}
 }
 
@@ -326,11 +327,7 @@ static int norm_bwd_launch(int kind, const void* dy, const void* x, const void* 
 	}
 	if (rc) return rc;
 	const int nparts = norm_bwd_blocks(T, d);
-	const int col_blocks = (d + 31) / 32;
-	int slices = (512 + col_blocks - 1) / col_blocks;  // about two workgroups per CU
-	if (slices > (nparts + 7) / 8) slices = (nparts + 7) / 8;
-	if (slices < 1) slices = 1;
-	hipLaunchKernelGGL(norm_bwd_finalize_kernel, dim3(col_blocks, slices), dim3(256), 0, s, workspace, nparts, d, dgamma,
+	hipLaunchKernelGGL(norm_bwd_finalize_kernel, dim3((d + 31) / 32), dim3(1024), 0, s, workspace, nparts, d, dgamma,
 	                   kind == NORM_LAYER ? dbeta : nullptr);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;

@@ -13,12 +13,24 @@
 // they sit in memory and read with ds_read_b64_tr_b16, the LDS transpose read of gfx950, so
 // no operand is ever transposed through HBM.  Each wave owns a (BM/WR) x (BN/WC) sub-tile
 // built from v_mfma_f32_32x32x16_bf16.
+#include <atomic>
+
 #include "common.h"
 #include "kernels.h"
 
 namespace elf {
 
 constexpr int BK = 64;
+// turn counters of split tiles (see gemm_kernel)
+constexpr int TURN_RS_SLOTS = 4096;
+static __device__ uint32_t turn_rs[TURN_RS_SLOTS];
+
+// One sequence of tags for every launch of every GEMM kernel that splits tiles: a counter value left behind by any
+// earlier launch then never equals a value a later launch waits for.
+uint32_t next_turn_tag() {
+	static std::atomic<uint32_t> launch_tag{0};
+	return (launch_tag.fetch_add(1) % 0xFFFFFFu) + 1;
+}
 constexpr int PAD_R = 8;    // elements of padding per row of an "R" tile ([row][BK+8])
 constexpr int PAD_T = 16;   // elements of padding per row of a "T" tile ([k][rows+16])
 
@@ -31,6 +43,7 @@ struct GemmArgs {
 	int M, N, K;
 	int tiles_m, tiles_n;
 	int k_splits;      // >1: split-K with fp32 atomics (EPI_F32_ACC only)
+	uint32_t turn_tag; // split-K: this launch's tag in the turn counters, 0 = the splits add in any order
 };
 
 template <int ROWS, bool T>
@@ -136,7 +149,33 @@ __global__ __launch_bounds__(WR* WC * 64) void gemm_kernel(GemmArgs g) {
 	const int nk_per = (nk_total + g.k_splits - 1) / g.k_splits;
 	const int kt_begin = ksplit * nk_per;
 	const int kt_end = min(nk_total, kt_begin + nk_per);
-	if (kt_begin >= kt_end) return;
+	// Split tiles add in turn (bit-reproducible sums): split s starts its atomics when turn_rs[tile] holds this
+	// launch's tag with count s and publishes s + 1 when they have been performed.  Splits of lower index are
+	// dispatched first, so the one waited for is running or done; the wait is bounded, and a workgroup that gives
+	// up adds out of turn (the right sum, only its rounding may differ).
+	uint32_t* const my_turn = turn_rs + (((uint32_t)pid + g.turn_tag * 977u) % (uint32_t)TURN_RS_SLOTS);
+	const uint32_t turn_want = (g.turn_tag << 8) | (uint32_t)ksplit;
+	auto take_turn = [&]() {
+		if (g.k_splits > 1 && g.turn_tag) {
+			if (tid == 0 && ksplit > 0) {
+				for (int spin = 0; spin < (1 << 18) && __hip_atomic_load(my_turn, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) != turn_want; spin++)
+					__builtin_amdgcn_s_sleep(16);
+			}
+			__syncthreads();
+		}
+	};
+	auto pass_turn = [&]() {
+		if (g.k_splits > 1 && g.turn_tag) {
+			__threadfence();
+			__syncthreads();
+			if (tid == 0) __hip_atomic_store(my_turn, turn_want + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+		}
+	};
+	if (kt_begin >= kt_end) {
+		take_turn();
+		pass_turn();
+		return;
+	}
 
 	const bf16_t* Ap = AT ? g.A + (int64_t)kt_begin * BK * g.lda + m0 : g.A + (int64_t)m0 * g.lda + (int64_t)kt_begin * BK;
 	const bf16_t* Bp = BT ? g.B + (int64_t)kt_begin * BK * g.ldb + n0 : g.B + (int64_t)n0 * g.ldb + (int64_t)kt_begin * BK;
@@ -193,6 +232,7 @@ __global__ __launch_bounds__(WR* WC * 64) void gemm_kernel(GemmArgs g) {
 
 	// Epilogue. Accumulator register r of a 32x32 tile holds row (r/4)*8 + (lane/32)*4 + r%4,
 	// column lane%32: lanes 0..31 cover 32 consecutive columns of one row.
+	if constexpr (EPI == EPI_F32_ACC) take_turn();
 	const int col_l = lane & 31;
 	const int row_l = (lane >> 5) * 4;
 #pragma unroll
@@ -222,6 +262,7 @@ __global__ __launch_bounds__(WR* WC * 64) void gemm_kernel(GemmArgs g) {
 			}
 		}
 	}
+	if constexpr (EPI == EPI_F32_ACC) pass_turn();
 }
 
 template <int BM, int BN, int WR, int WC, bool AT, bool BT, int EPI>
@@ -237,6 +278,7 @@ static int launch_cfg(const GemmArgs& g, hipStream_t stream) {
 	GemmArgs a = g;
 	a.tiles_m = g.M / BM;
 	a.tiles_n = g.N / BN;
+	a.turn_tag = EPI == EPI_F32_ACC && a.k_splits > 1 && a.tiles_m * a.tiles_n <= TURN_RS_SLOTS ? next_turn_tag() : 0;
 	const int grid = a.tiles_m * a.tiles_n * a.k_splits;
 	hipLaunchKernelGGL(kern, dim3(grid), dim3(WR * WC * 64), smem, stream, a);
 	ELF_CHECK_HIP(hipGetLastError());

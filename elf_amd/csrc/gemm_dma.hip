@@ -64,7 +64,22 @@ struct Args {
 	// EPI_BF16_ROPE: (cos, sin) table [rope_S, rope_D / 2], columns below rope_cols are rotated, heads are rope_D wide
 	const float2* rope_cs;
 	int rope_S, rope_cols, rope_D;
+	// split tiles: this launch's tag in the turn counters (see turn[] below); 0 = the splits add in any order
+	uint32_t turn_tag;
 };
+
+// Turn counters of split tiles.  The workgroups that share a tile along K add their parts with fp32 atomics; to make
+// the sum independent of the order in which they finish, split s only starts adding when turn[slot] holds this
+// launch's tag with count s, and publishes count s + 1 when its adds have been performed.  The tag changes with every
+// launch, so a value left by an earlier launch never matches and nothing has to be cleared.  Workgroups are
+// dispatched in index order and the splits of a tile have consecutive indices, so the one a workgroup waits for is
+// always running or done; the wait is bounded all the same, and a workgroup that gives up (counters shared with a
+// concurrent launch on another stream) adds out of turn: still the right sum, only its rounding may differ.
+// A counter covers one 32-row strip of one wave (up to 16 per tile), so a split starts on a strip as soon as its
+// predecessor is through with that strip and the splits of a tile overlap except for about one strip.
+constexpr int TURN_TILES = 4096, TURN_PER_TILE = 16;
+static __device__ uint32_t turn[TURN_TILES * TURN_PER_TILE];
+constexpr int TURN_SPIN_LIMIT = 1 << 18;  // polls of ~0.5 us
 
 // Byte offsets (relative to the tile origin of the current K slice) of the 16-byte chunks this
 // lane fetches for one operand (< 2^31: 256 rows of at most 64 K elements).  "R" tiles are
@@ -203,6 +218,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 			pid = full + q / splits;
 		}
 	}
+	// split tiles: the turn counter of this tile (tiles of one launch get distinct counters, consecutive launches different ones)
+	const int turn_slot = (int)(((uint32_t)(pid - full) + g.turn_tag * 977u) % (uint32_t)TURN_TILES);
 	int m0, n0;
 	const int nsb = ntiles >> 5, nrem = nsb & 7;
 	if (g.walk && (g.tiles_m & 7) == 0 && (g.tiles_n & 3) == 0 && (nrem == 0 || nrem == 1 || nrem == 2 || nrem == 4)) {
@@ -238,7 +255,19 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	const int nk_per = (nk_total + splits - 1) / splits;
 	const int kt0 = ksplit * nk_per;
 	const int nk = min(nk_total, kt0 + nk_per) - kt0;
-	if (nk <= 0) return;
+	if (nk <= 0) {
+		// a split without a K range of its own still takes and passes its turn on every strip
+		if (splits > 1 && g.turn_tag && lane == 0) {
+			const uint32_t want = (g.turn_tag << 8) | (uint32_t)ksplit;
+			for (int i = 0; i < RT; i++) {
+				uint32_t* t = turn + turn_slot * TURN_PER_TILE + wave * RT + i;
+				for (int spin = 0; ksplit > 0 && spin < TURN_SPIN_LIMIT && __hip_atomic_load(t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != want; spin++)
+					__builtin_amdgcn_s_sleep(8);
+				__hip_atomic_store(t, want + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+			}
+		}
+		return;
+	}
 
 	const bf16_t* Ap = AT ? g.A + (int64_t)kt0 * BKS * g.lda + m0 : g.A + (int64_t)m0 * g.lda + (int64_t)kt0 * BKS;
 	// paired rows: tile column n0 of the (gate | up interleaved) product starts at operand row n0 / 2
@@ -532,6 +561,14 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 			}
 		} else {
 			if (EPI == EPI_F32_ACC && splits > 1) {
+				uint32_t* const my_turn = turn + turn_slot * TURN_PER_TILE + wave * RT + i;
+				if (g.turn_tag && ksplit > 0) {
+					// wait for this split's turn on this strip (see turn[]); every lane polls the same word.  Plain
+					// (cache-bypassing) loads: nothing is read after the wait, the adds are performed at the memory side
+					const uint32_t want = (g.turn_tag << 8) | (uint32_t)ksplit;
+					for (int spin = 0; spin < TURN_SPIN_LIMIT && __hip_atomic_load(my_turn, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != want; spin++)
+						__builtin_amdgcn_s_sleep(8);
+				}
 				// several workgroups add into this tile: fp32 atomics, one scalar per lane so that a wave
 				// instruction covers two whole 128-byte rows of 32 columns (16 bytes per lane would touch a
 				// quarter of eight lines per instruction and run at half the speed)
@@ -541,6 +578,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 					float* c = reinterpret_cast<float*>(g.C) + (int64_t)(grow0 + row) * g.ldc + gcol0 + (lane & 31);
 #pragma unroll
 					for (int cg = 0; cg < 4; cg++) unsafeAtomicAdd(c + cg * 32, ws[row * PITCH + cg * 32 + (lane & 31)]);
+				}
+				if (g.turn_tag) {
+					// wait until this wave's adds have been performed (they complete in vmcnt; no cache write-back is
+					// needed for atomics), then the next split may add to this strip
+					wait_vmcnt<0>();
+					if (lane == 0) __hip_atomic_store(my_turn, (g.turn_tag << 8) | (uint32_t)(ksplit + 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 				}
 				continue;
 			}
@@ -618,7 +661,7 @@ int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t 
 	ELF_REQUIRE(epi != EPI_BF16_ROPE || (rope_cs && rope_S > 0 && !a_t && !b_t && (rope_D == 64 || rope_D == 128) && rope_cols % rope_D == 0 && rope_cols <= N),
 	            "gemm (dma tile): the RoPE epilogue needs k-contiguous operands, a table and heads of 64 or 128 columns");
 	dma::Args a{(const bf16_t*)A, (const bf16_t*)B, C, (const bf16_t*)R, (bf16_t*)C2, lda, ldb, ldc, ldr, ldc2, M, N, K, M / bm, N / dma::BN, k_splits < 1 ? 1 : k_splits,
-	            tail_tiles < 0 || tail_tiles > ntiles ? ntiles : tail_tiles, 0, (const float2*)rope_cs, rope_S, rope_cols, rope_D};
+	            tail_tiles < 0 || tail_tiles > ntiles ? ntiles : tail_tiles, 0, (const float2*)rope_cs, rope_S, rope_cols, rope_D, 0};
 	// The band walk fetches every row slab of A from HBM in one round only and B once per band; the default
 	// walk wants A in the 256 MB memory-side cache for the whole launch and streams B once.  Inside the stage's
 	// stream (operands cold, per-shape times from a kernel trace) the bands are 0-5 % faster on every shape but
@@ -627,6 +670,8 @@ int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t 
 	const int64_t big = int64_t(160) << 20;
 	a.walk = !((int64_t)M * K * 2 < big && (int64_t)N * K * 2 >= big);
 	if (epi != EPI_F32_ACC || a.k_splits == 1) a.k_splits = 1, a.tail_tiles = 0;
+	// split tiles add in a fixed order (bit-reproducible weight gradients) as long as each has a counter of its own
+	a.turn_tag = a.tail_tiles > 0 && a.tail_tiles <= dma::TURN_TILES ? next_turn_tag() : 0;
 	if (bm == 128) {
 		if (!b_t) return dma::launch_epi<4, 2, false, false>(a, epi, stream);
 		return dma::launch_epi<4, 2, false, true>(a, epi, stream);

@@ -39,6 +39,10 @@ bool gemm_rope_fused(int M, int N, int K, int D);
 int gemm_rope_bf16(int M, int N, int K, const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, const void* cs,
                    int S, int n_rot_heads, int D, hipStream_t stream);
 
+// Tag of one GEMM launch whose tiles are split along K (24 bits, never 0, different from launch to launch); see the
+// turn counters in gemm_dma.hip and gemm_bf16.hip.
+uint32_t next_turn_tag();
+
 enum Activation { ACT_GELU = 0, ACT_SWIGLU = 1 };
 // Up-projection of the MLP with its activation: pre = A W^T (A [M, K], W [N, K], N = F for GELU and 2F =
 // [gate rows; up rows] for SwiGLU), out [M, F] = gelu(pre) or silu(pre[:, :F]) * pre[:, F:].  SwiGLU runs

@@ -107,6 +107,27 @@ def test_gemm_direct_to_lds_epilogues_and_k_split(K, tile_cfg, layout):
 			_close(acc, 2 * ref + 0.25, rel_fro=1e-5, rel_max=1e-5, what=f"f32 acc K={Kd} ks={ks}")
 
 
+@pytest.mark.parametrize("dims,ks", [((1024, 1536, 8192), 0), ((512, 768, 4096), 8), ((4096, 6144, 8192), 0), ((2048, 2304, 2048), 4)])
+def test_gemm_k_split_is_bit_reproducible(K, dims, ks):
+	"""Weight-gradient GEMMs whose tiles are shared by several workgroups along K (all tiles split, only the
+	tail of the last round split, an explicit split): the workgroups of a tile add in turn, so repeated runs
+	into equal accumulators give equal bits, and the sum is the unsplit one within fp32 rounding."""
+	M, N, Kd = dims
+	A = _randn(Kd, M, seed=71)
+	B = _randn(Kd, N, seed=72, scale=0.05)
+	start = torch.randn(M, N, device="cuda", generator=torch.Generator(device="cuda").manual_seed(73))
+	runs = []
+	for _ in range(4):
+		acc = start.clone()
+		K.gemm(A, B, a_t=True, b_t=True, out=acc, epilogue=K.EPI_F32_ACC, k_splits=ks)
+		runs.append(acc)
+	for r in runs[1:]:
+		assert torch.equal(r, runs[0]), "split-K accumulation must not depend on the order in which workgroups finish"
+	one = start.clone()
+	K.gemm(A, B, a_t=True, b_t=True, out=one, epilogue=K.EPI_F32_ACC, k_splits=1)
+	assert ((runs[0] - one).norm() / one.norm()).item() <= 1e-5
+
+
 def test_gemm_strided_views(K):
 	# operands that are column slices of wider buffers (leading dimension > row length)
 	big = _randn(512, 1024, seed=6)
