@@ -208,6 +208,32 @@ class Telemetry:
 		return out
 
 
+def hbm_ceiling():
+	"""What the memory system sustains for a plain read, copy and write of 1 GiB (elf_hbm_probe; 20 launches each after
+	3 warm-ups, timed with one event pair): the practical ceiling the bandwidth-bound kernels are compared with."""
+	import torch
+	from elf_amd import _lib
+
+	lib = _lib.load()
+	n = 1 << 30
+	src = torch.randint(0, 255, (n,), dtype=torch.uint8, device="cuda")
+	dst = torch.empty(n, dtype=torch.uint8, device="cuda")
+	st = torch.cuda.current_stream().cuda_stream
+	out = {"bytes": n, "peak_gbs": PEAK_HBM_GBS}
+	for mode, name, moved in ((0, "read", n), (1, "copy", 2 * n), (2, "write", n)):
+		for _ in range(3):
+			_lib.check(lib.elf_hbm_probe(mode, src.data_ptr(), dst.data_ptr(), n, st), "elf_hbm_probe")
+		e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+		e0.record()
+		for _ in range(20):
+			_lib.check(lib.elf_hbm_probe(mode, src.data_ptr(), dst.data_ptr(), n, st), "elf_hbm_probe")
+		e1.record()
+		torch.cuda.synchronize()
+		ms = e0.elapsed_time(e1) / 20
+		out[name] = {"ms": ms, "gbs": moved / ms / 1e6, "frac_of_peak": moved / ms / 1e6 / PEAK_HBM_GBS}
+	return out
+
+
 def main():
 	ap = argparse.ArgumentParser()
 	ap.add_argument("--gpus", type=int, default=1)
@@ -222,6 +248,8 @@ def main():
 	                     "then come from one extra eager step after the timed region (a replay runs no host code that could bracket launches)")
 	ap.add_argument("--telemetry", action="store_true",
 	                help="sample socket power and shader clock on a host thread during the timed steps and report them under \"telemetry\"")
+	ap.add_argument("--hbm-ceiling", action="store_true",
+	                help="also time a plain read / copy / write of 1 GiB (elf_hbm_probe) and report the rates under \"hbm_ceiling\"")
 	ap.add_argument("--calibration-copy", action="store_true",
 	                help="also launch one elf::add_kernel over 2 x 128 MiB in, 128 MiB out: a kernel of known HBM traffic to scale profiler byte counters with")
 	args = ap.parse_args()
@@ -360,6 +388,8 @@ def main():
 		                    "h2d_bytes_per_step": h2d / args.steps, "prefetching_time": w.get("prefetching_time", 1)}
 	if args.telemetry:
 		out["telemetry"] = telemetry.summary(t0, t0 + elapsed)
+	if args.hbm_ceiling:
+		out["hbm_ceiling"] = hbm_ceiling()
 	if cpu_stats is not None:
 		out["cpu_baseline"] = cpu_stats
 	print(json.dumps(out))

@@ -104,6 +104,10 @@ int attn_bwd(const void* q, const void* k, const void* v, const void* o, const v
 // rope_cs non-null: q and k are the rotated heads (rope_apply with this table); dq and dk come out as the gradients
 // of the heads before the rotation (rope_apply's backward applied to them), bit-identical to the separate pass.
 
+// Memory-system yardstick: read (mode 0; dst receives up to 8192 * 256 * 16 bytes of sums), copy (1) or write (2) `bytes`
+// bytes with the simplest possible kernel.
+int hbm_probe(int mode, const void* src, void* dst, int64_t bytes, hipStream_t s);
+
 // Optional live timing of kernel launches: when enabled, every launcher brackets its launches
 // with an event pair on the launch stream and books the algorithmic work of the call.
 enum ProfKind {

@@ -336,6 +336,11 @@ int elf_pinned_pool_free_segment(elf_pinned_pool_t* p, int parent, int i, int64_
  * 6 activation bwd, 7 RoPE, 8 grad scale, 9 add (work = algorithmic bytes).
  * elf_prof_collect waits for the events and returns the number of launches of that kind since
  * elf_prof_enable(1), with their summed duration (ms) and summed work. */
+/* Memory-system yardstick for the bandwidth-bound kernels (no counterpart in the reference): mode 0 reads `bytes`
+ * bytes from src (dst receives at most 8192 * 256 * 16 bytes of per-lane sums), mode 1 copies them to dst, mode 2 writes
+ * `bytes` bytes to dst; 16-byte accesses, each workgroup on contiguous chunks of 16 or 32 KiB.  bench.py --hbm-ceiling
+ * times it. */
+int elf_hbm_probe(int mode, const void* src, void* dst, int64_t bytes, void* stream);
 void elf_prof_enable(int on);
 int elf_prof_collect(int kind, double* total_ms, double* total_work);
 
