@@ -29,7 +29,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per GEMM launch (mean over the launches of one step), from rocprofv3 --pmc FETCH_SIZE and
 # --pmc WRITE_SIZE runs of this script scaled by the same counters' reading for a copy kernel of known
 # size (--calibration-copy); measured per workload, None where it was not.
-GEMM_TRAFFIC_BYTES = {"llama3_8b_zbh1": 1.695e9}
+GEMM_TRAFFIC_BYTES = {"llama3_8b_zbh1": 1.696e9}
 
 WORKLOADS = {
 	# headline configuration: Llama-3-8B-shaped stage, ZB-H1 stream of block 1 in a 4-stage pipeline
