@@ -161,6 +161,16 @@ bool PinnedPool::allocate(int64_t elems, int elem_size, int dtype_key, Block* ou
 	return true;
 }
 
+bool PinnedPool::fits(int64_t elems, int dtype_key) const {
+	const int64_t req = elems < 1 ? 1 : elems;
+	for (const auto& p : parents_) {
+		if (p.dtype_key != dtype_key) continue;
+		for (const auto& seg : p.free_list)
+			if (seg.second >= req) return true;
+	}
+	return false;
+}
+
 void PinnedPool::insert_free(Parent& p, int64_t off, int64_t len) {
 	auto& fl = p.free_list;
 	size_t i = 0;

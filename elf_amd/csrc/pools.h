@@ -61,6 +61,7 @@ class PinnedPool {
 		int64_t length = 0;   // in elements
 	};
 	bool allocate(int64_t elems, int elem_size, int dtype_key, Block* out);
+	bool fits(int64_t elems, int dtype_key) const;  // whether allocate() would find room without a new parent chunk
 	bool free(void* ptr);            // false if ptr is not a live block of this pool
 	bool reserve(int64_t bytes, int elem_size, int dtype_key);
 	int64_t size_bytes() const;      // sum of parent chunk sizes

@@ -118,6 +118,13 @@ struct Stage {
 	void* attn_ws = nullptr;
 	int64_t ws_bytes = 0;  // fixed device workspaces of the stage (norm / attention backward scratch, rope table, gradient sink)
 	float* dummy_grad = nullptr;  // sink for norm weight gradients during gradient recompute
+	// pinned blocks of released micro-batches whose last copy may still be in flight: they go back to the arena
+	// when their event has fired (polled, never waited for inside a step unless the arena would have to grow)
+	struct HostPending {
+		hipEvent_t ev;
+		std::vector<void*> ptrs;
+	};
+	std::vector<HostPending> host_pending;
 	int64_t d2h_bytes = 0, h2d_bytes = 0;
 
 	size_t buf_bytes(int id) const {
@@ -201,6 +208,23 @@ static void destroy_events(MbState& m) {
 }
 
 static int do_offload_block(Stage* s, BlockState& bs, hipStream_t st);
+
+// Return the pinned blocks whose guarding event has fired (all of them, waiting, when `wait`).
+static void poll_host_pending(Stage* s, bool wait) {
+	for (size_t i = 0; i < s->host_pending.size();) {
+		auto& hp = s->host_pending[i];
+		const hipError_t e = wait ? hipEventSynchronize(hp.ev) : hipEventQuery(hp.ev);
+		if (e == hipSuccess) {
+			for (void* p : hp.ptrs) s->pinned->free(p);
+			(void)hipEventDestroy(hp.ev);
+			s->host_pending[i] = std::move(s->host_pending.back());
+			s->host_pending.pop_back();
+		} else {
+			(void)hipGetLastError();
+			i++;
+		}
+	}
+}
 
 // ---------------------------------------------------------------------------------------------
 // remat: ELF_FWD_REMAT_ATTN / ELF_FWD_REMAT_NORM of a forward that keeps its stash: the buffers those module
@@ -486,6 +510,11 @@ static int do_offload_block(Stage* s, BlockState& bs, hipStream_t st) {
 			b.dropped = true;
 			continue;
 		}
+		// blocks of released micro-batches first; the arena only grows when waiting for them does not make room
+		if (!s->host_pending.empty()) {
+			poll_host_pending(s, false);
+			if (!s->pinned->fits((int64_t)(b.bytes / 2), 1)) poll_host_pending(s, true);
+		}
 		if (!s->pinned->allocate((int64_t)(b.bytes / 2), 2, /*bf16*/ 1, &b.host)) return -3;
 		ELF_CHECK_HIP(hipMemcpyAsync(b.host.ptr, b.p, b.bytes, hipMemcpyDeviceToHost, s->offload_stream));
 		s->d2h_bytes += (int64_t)b.bytes;
@@ -561,22 +590,34 @@ static int do_restore(Stage* s, MbState& m, bool async, hipStream_t st) {
 	return 0;
 }
 
+// RELEASE of an offloaded micro-batch (offload.py:392-411): its pinned blocks go back to the arena once the copies
+// that use them are done.  The host does not wait: an event recorded now on the stream those copies were issued on
+// guards the blocks (poll_host_pending).
 static int do_release(Stage* s, MbState& m) {
 	if (!m.offloaded) return 0;
-	for (auto& bs : m.blk) {
-		if (m.prefetched && bs.pre_ev) ELF_CHECK_HIP(hipEventSynchronize(bs.pre_ev));
-		else if (bs.off_ev) ELF_CHECK_HIP(hipEventSynchronize(bs.off_ev));
-	}
+	Stage::HostPending hp;
+	hp.ev = nullptr;
 	for (auto& bs : m.blk)
 		for (int id = 0; id < B_COUNT; id++) {
 			Buf& b = bs.b[id];
 			if (b.offloaded) {
-				s->pinned->free(b.host.ptr);
+				hp.ptrs.push_back(b.host.ptr);
 				b.offloaded = false;
 			}
 		}
+	if (!hp.ptrs.empty()) {
+		// asynchronous prefetch: the host-to-device copies ran on the prefetch stream; otherwise the last user of the
+		// blocks is the offload stream's device-to-host copy (a restore on the compute stream is ordered before any
+		// later offload by that offload's own wait on the compute stream)
+		bool async_restore = false;
+		for (auto& bs : m.blk) async_restore = async_restore || (m.prefetched && bs.pre_ev);
+		ELF_CHECK_HIP(hipEventCreateWithFlags(&hp.ev, hipEventDisableTiming));
+		ELF_CHECK_HIP(hipEventRecord(hp.ev, async_restore ? s->prefetch_stream : s->offload_stream));
+		s->host_pending.push_back(std::move(hp));
+	}
 	m.offloaded = false;
 	m.prefetched = false;
+	poll_host_pending(s, false);
 	return 0;
 }
 
@@ -646,6 +687,7 @@ void elf_stage_destroy(elf_stage_t* h) {
 		destroy_events(kv.second);
 	}
 	s->mbs.clear();
+	poll_host_pending(s, true);
 	if (s->offload_stream) (void)hipStreamDestroy(s->offload_stream);
 	if (s->prefetch_stream) (void)hipStreamDestroy(s->prefetch_stream);
 	if (s->norm_ws) (void)hipFree(s->norm_ws);
@@ -853,6 +895,7 @@ int elf_stage_clear(elf_stage_t* h) {
 	}
 	s->mbs.clear();
 	s->mb_samples.clear();
+	poll_host_pending(s, true);
 	return 0;
 }
 
@@ -860,6 +903,7 @@ int elf_stage_mem_stats(elf_stage_t* h, elf_mem_stats* out) {
 	Stage* s = (Stage*)h;
 	ELF_REQUIRE(s && out, "elf_stage_mem_stats: null argument");
 	s->pool.poll();  // buffers whose copy to the host has finished no longer count as live
+	poll_host_pending(s, false);
 	out->live_bytes = (int64_t)s->pool.live_bytes();
 	out->peak_bytes = (int64_t)s->pool.peak_bytes();
 	out->reserved_bytes = (int64_t)s->pool.reserved_bytes();
