@@ -125,3 +125,49 @@ def test_compute_loss_matches_mean_reduction_after_batch_scaling():
 	ref.backward()
 	assert torch.allclose(loss / 3, ref) and torch.allclose(g / 3, ref_in.grad)
 	assert blk.compute_time[0].name == "loss_forward"
+
+
+@pytest.mark.parametrize("scheduler,placement,nmb", [("1f1b", [0, 1], 4), ("zbh1", [0, 1, 2, 3], 8), ("1f1b", [0, 1, 0, 1], 4), ("afab", [0, 1, 2], 3), ("zbh2", [0, 1, 2, 3], 4)])
+@pytest.mark.parametrize("comm", ["pipelined", "topo", "simulation"])
+def test_sequential_order_lets_one_process_play_every_rank(scheduler, placement, nmb, comm):
+	"""``sequential_order`` (the order ``Pipeline(all_ranks=True)`` runs a multi-rank schedule in): the same ops, every
+	rank's own order kept, each FORWARD after the SEND_FORWARD that feeds it and each BACKWARD_INPUTS after the
+	SEND_BACKWARD of its consumer; the Engine then runs all blocks of the placement on stand-in blocks and the
+	values that come out are those of the chain y = 2^n x."""
+	from elf_amd.pipeline import sequential_order
+
+	sigs = sequential_signatures(placement)
+	schedule = COMM_SCHEDULERS[comm](add_comms(SCHEDULERS[scheduler](placement, nmb), sigs))
+	order = sequential_order(schedule, sigs)
+	assert sorted(map(id, order)) == sorted(map(id, schedule))
+	for r in set(placement):
+		assert [op for op in order if op.rank == r] == [op for op in schedule if op.rank == r]
+	pos = {id(op): i for i, op in enumerate(order)}
+	for op in order:
+		if op.op == T.FORWARD and op.block_id > 0:
+			send = next(o for o in order if o.op == T.SEND_FORWARD and o.block_id == op.block_id - 1 and o.mb_id == op.mb_id and o.options.get("dst") == op.block_id)
+			assert pos[id(send)] < pos[id(op)]
+		if op.op == T.BACKWARD_INPUTS and op.block_id < len(placement) - 1:
+			send = next(o for o in order if o.op == T.SEND_BACKWARD and o.block_id == op.block_id + 1 and o.mb_id == op.mb_id and o.options.get("dst") == op.block_id)
+			assert pos[id(send)] < pos[id(op)]
+	blocks = [FakeBlock(i, placement) for i in range(len(placement))]
+	for b in blocks:
+		b.local_ids = set(range(len(placement)))
+	x = torch.arange(float(2 * nmb)).reshape(nmb, 2)
+	result, losses, _, _ = Engine(blocks, all_ranks=True).train_step([x], torch.zeros(nmb, 2), torch.nn.functional.mse_loss, order, [1] * nmb)
+	assert torch.equal(torch.cat(result), (2 ** len(placement)) * x)
+	assert all(sum(c[0] == k for c in b.calls) == nmb for b in blocks for k in "FBW")
+	left = blocks[0].input_variables[0].to_send
+	assert torch.equal(torch.cat(left), (2 ** (2 * len(placement))) * x)  # dL/dy = 2y / 2, back through the chain
+
+
+def test_sequential_order_reports_a_schedule_that_cannot_run():
+	from elf_amd.pipeline import sequential_order
+	from elf_amd.scheduling import Operation
+
+	sigs = sequential_signatures([0, 1])
+	stuck = [Operation(1, 0, T.FORWARD, 1)]  # nobody ever sends block 1 its input
+	with pytest.raises(RuntimeError, match="deadlock"):
+		sequential_order(stuck, sigs)
+	with pytest.raises(AssertionError):
+		Engine([FakeBlock(0, [0, 1]), FakeBlock(1, [0, 1])])  # two ranks without all_ranks
