@@ -234,6 +234,56 @@ def hbm_ceiling():
 	return out
 
 
+def vendor_gemm(w, seconds=1.0):
+	"""The twelve dense contractions of one block of the workload (forward y = x W^T, input gradient dX = dY W, weight
+	gradient dW = dY^T X for each of the four projections), each run back to back for ``seconds`` through this library
+	and through torch.matmul (the vendor's GEMM library), on the same operands and the same GPU, with socket power and
+	shader clock sampled meanwhile.  A yardstick only: what another bf16 GEMM sustains on this part under its power cap."""
+	import torch
+	from elf_amd import kernels as K
+
+	T, d, F = w["mb"] * w["seq"], w["d"], w["ffn"]
+	nq, nkv = w["heads"] * w["head_dim"], w["kv_heads"] * w["head_dim"]
+	shapes = [("qkv", nq + 2 * nkv, d), ("proj", d, nq), ("up", F * (2 if w["arch"] == "llama" else 1), d), ("down", d, F)]
+
+	def sustained(fn, flops):
+		for _ in range(5):
+			fn()
+		torch.cuda.synchronize()
+		n, t0 = 0, time.perf_counter()
+		with Telemetry(period=0.02) as tel:
+			while time.perf_counter() - t0 < seconds:
+				for _ in range(25):
+					fn()
+				torch.cuda.synchronize()
+				n += 25
+			t1 = time.perf_counter()
+		summ = tel.summary(t0, t1)
+		return {"tflops": flops * n / (t1 - t0) / 1e12, "us": (t1 - t0) / n * 1e6, "power_w": summ.get("power_w", {}).get("mean"), "sclk_mhz": summ.get("sclk_mhz", {}).get("mean")}
+
+	rows, total = [], {"elf": 0.0, "vendor": 0.0}
+	for name, N, Kd in shapes:
+		x = torch.randn(T, Kd, device="cuda").bfloat16()
+		wt = (torch.randn(N, Kd, device="cuda") * 0.02).bfloat16()
+		dy = torch.randn(T, N, device="cuda").bfloat16()
+		y, dx = torch.empty(T, N, device="cuda", dtype=torch.bfloat16), torch.empty(T, Kd, device="cuda", dtype=torch.bfloat16)
+		dw32, dw16 = torch.zeros(N, Kd, device="cuda", dtype=torch.float32), torch.empty(N, Kd, device="cuda", dtype=torch.bfloat16)
+		legs = (
+			("forward", lambda: K.gemm(x, wt, out=y), lambda: torch.matmul(x, wt.t(), out=y)),
+			("dX", lambda: K.gemm(dy, wt, b_t=True, out=dx), lambda: torch.matmul(dy, wt, out=dx)),
+			# this library adds into the fp32 gradient; the vendor leg writes a bf16 product, which is less work
+			("dW", lambda: K.gemm(dy, x, a_t=True, b_t=True, out=dw32, epilogue=K.EPI_F32_ACC), lambda: torch.matmul(dy.t(), x, out=dw16)),
+		)
+		for leg, ours, theirs in legs:
+			r = {"gemm": f"{name}/{leg}", "M": T if leg != "dW" else N, "N": N if leg == "forward" else Kd, "K": Kd if leg == "forward" else (N if leg == "dX" else T)}
+			r["elf"], r["vendor"] = sustained(ours, 2.0 * T * N * Kd), sustained(theirs, 2.0 * T * N * Kd)
+			total["elf"] += r["elf"]["us"]
+			total["vendor"] += r["vendor"]["us"]
+			rows.append(r)
+		del x, wt, dy, y, dx, dw32, dw16
+	return {"seconds_per_leg": seconds, "gemms": rows, "sum_us": total}
+
+
 def main():
 	ap = argparse.ArgumentParser()
 	ap.add_argument("--gpus", type=int, default=1)
@@ -250,6 +300,9 @@ def main():
 	                help="sample socket power and shader clock on a host thread during the timed steps and report them under \"telemetry\"")
 	ap.add_argument("--hbm-ceiling", action="store_true",
 	                help="also time a plain read / copy / write of 1 GiB (elf_hbm_probe) and report the rates under \"hbm_ceiling\"")
+	ap.add_argument("--vendor-gemm", action="store_true",
+	                help="also run the twelve GEMMs of one block back to back through this library and through torch.matmul (the vendor's "
+	                     "library), with power and clock, and report both under \"vendor_gemm\"")
 	ap.add_argument("--calibration-copy", action="store_true",
 	                help="also launch one elf::add_kernel over 2 x 128 MiB in, 128 MiB out: a kernel of known HBM traffic to scale profiler byte counters with")
 	args = ap.parse_args()
@@ -390,6 +443,8 @@ def main():
 		out["telemetry"] = telemetry.summary(t0, t0 + elapsed)
 	if args.hbm_ceiling:
 		out["hbm_ceiling"] = hbm_ceiling()
+	if args.vendor_gemm:
+		out["vendor_gemm"] = vendor_gemm(w)
 	if cpu_stats is not None:
 		out["cpu_baseline"] = cpu_stats
 	print(json.dumps(out))

@@ -241,7 +241,8 @@ __global__ __launch_bounds__(1024) void norm_bwd_finalize_kernel(const float* __
 	const int c = blockIdx.x * 32 + cl;
 	float sg = 0.f, sb = 0.f;
 	if (c < d) {
-#pragma unroll 4
+		// 16 loads in flight per lane: the kernel is a chain of dependent trips to memory otherwise
+#pragma unroll 16
 		for (int b = rg; b < nparts; b += 32) {
 			sg += part[(int64_t)b * 2 * d + c];
 			if (dbeta) sb += part[(int64_t)b * 2 * d + d + c];
@@ -265,7 +266,9 @@ __global__ __launch_bounds__(1024) void norm_bwd_finalize_kernel(const float* __
 static inline int norm_bwd_blocks(int T, int d) {
 	const int rows_per_block = d <= 2048 ? ROWS_PER_BLOCK : 1;
 	const int want = (T + rows_per_block - 1) / rows_per_block;
-	return want < 1024 ? want : 1024;
+	// narrow rows: fewer, longer workgroups - the partial rows are overhead traffic that the fold kernel reads back
+	const int cap = d <= 1024 ? 512 : 1024;
+	return want < cap ? want : cap;
 }
 
 template <bool LN>

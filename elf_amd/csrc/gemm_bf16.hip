@@ -17,6 +17,7 @@
 
 #include "common.h"
 #include "kernels.h"
+#include "lds_dma.h"
 
 namespace elf {
 
@@ -155,20 +156,23 @@ __global__ __launch_bounds__(WR* WC * 64) void gemm_kernel(GemmArgs g) {
 	// up adds out of turn (the right sum, only its rounding may differ).
 	uint32_t* const my_turn = turn_rs + (((uint32_t)pid + g.turn_tag * 977u) % (uint32_t)TURN_RS_SLOTS);
 	const uint32_t turn_want = (g.turn_tag << 8) | (uint32_t)ksplit;
+	// The poll and the publication are relaxed: the adds are atomics performed at the memory side, so what has to
+	// be known is only that they have been performed - every lane awaits the acknowledgement of its own
+	// (vmcnt(0)) before the workgroup barrier that precedes the publication.
 	auto take_turn = [&]() {
 		if (g.k_splits > 1 && g.turn_tag) {
 			if (tid == 0 && ksplit > 0) {
-				for (int spin = 0; spin < (1 << 18) && __hip_atomic_load(my_turn, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) != turn_want; spin++)
-					__builtin_amdgcn_s_sleep(16);
+				for (int spin = 0; spin < (1 << 18) && __hip_atomic_load(my_turn, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != turn_want; spin++)
+					__builtin_amdgcn_s_sleep(4);
 			}
 			__syncthreads();
 		}
 	};
 	auto pass_turn = [&]() {
 		if (g.k_splits > 1 && g.turn_tag) {
-			__threadfence();
+			wait_vmcnt<0>();
 			__syncthreads();
-			if (tid == 0) __hip_atomic_store(my_turn, turn_want + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+			if (tid == 0) __hip_atomic_store(my_turn, turn_want + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 		}
 	};
 	if (kt_begin >= kt_end) {

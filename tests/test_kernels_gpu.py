@@ -107,7 +107,7 @@ def test_gemm_direct_to_lds_epilogues_and_k_split(K, tile_cfg, layout):
 			_close(acc, 2 * ref + 0.25, rel_fro=1e-5, rel_max=1e-5, what=f"f32 acc K={Kd} ks={ks}")
 
 
-@pytest.mark.parametrize("dims,ks", [((1024, 1536, 8192), 0), ((512, 768, 4096), 8), ((4096, 6144, 8192), 0), ((2048, 2304, 2048), 4)])
+@pytest.mark.parametrize("dims,ks", [((1024, 1536, 8192), 0), ((768, 768, 8192), 0), ((512, 768, 4096), 8), ((4096, 6144, 8192), 0), ((2048, 2304, 2048), 4)])
 def test_gemm_k_split_is_bit_reproducible(K, dims, ks):
 	"""Weight-gradient GEMMs whose tiles are shared by several workgroups along K (all tiles split, only the
 	tail of the last round split, an explicit split): the workgroups of a tile add in turn, so repeated runs
