@@ -22,7 +22,9 @@ static hipEvent_t get_event() {
 		return e;
 	}
 	hipEvent_t e = nullptr;
-	(void)hipEventCreate(&e);
+	// timing only: without the system-scope fence a recorded event neither writes the caches back nor invalidates
+	// them, so bracketing a launch does not disturb the launches after it
+	(void)hipEventCreateWithFlags(&e, hipEventDisableSystemFence);
 	return e;
 }
 
