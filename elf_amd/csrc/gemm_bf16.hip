@@ -367,6 +367,16 @@ int gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda,
 	g.K = K;
 	g.tiles_m = g.tiles_n = 0;
 	g.k_splits = k_splits;
+	// small weight gradients (24..128 tiles of 128x256, e.g. 2304x768 or 2048x2048 at K = 8192): 128x256 tiles with K
+	// split so that the workgroups just fill the chip once - 7-28 % faster than 256x256 tiles split further
+	if (tile_cfg <= 0 && epi == EPI_F32_ACC && a_t && b_t && k_splits <= 0 && M % 128 == 0 && N % 256 == 0 && K >= 4096) {
+		const int64_t tiles = (int64_t)(M / 128) * (N / 256);
+		if (tiles >= 24 && tiles <= 128) {
+			int ks = (int)(256 / tiles);
+			if (ks > K / 64 / 32) ks = K / 64 / 32;
+			return gemm_bf16_dma(a_t, b_t, M, N, K, A, lda, B, ldb, C, ldc, epi, R, ldr, ks < 1 ? 1 : ks, -1, 128, stream);
+		}
+	}
 	// Tile choice when the caller leaves it open: the direct-to-LDS 256x256 kernel whenever its
 	// tiles can fill the chip, the register-staged kernels (smaller tiles) otherwise.
 	if (tile_cfg <= 0 && M % 256 == 0 && N % 256 == 0) {
@@ -396,7 +406,7 @@ int gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda,
 		}
 		return gemm_bf16_dma(a_t, b_t, M, N, K, A, lda, B, ldb, C, ldc, epi, R, ldr, k_splits, tail_tiles, 256, stream);
 	}
-	if (tile_cfg == 8) return gemm_bf16_dma(a_t, b_t, M, N, K, A, lda, B, ldb, C, ldc, epi, R, ldr, 1, 0, 128, stream);
+	if (tile_cfg == 8) return gemm_bf16_dma(a_t, b_t, M, N, K, A, lda, B, ldb, C, ldc, epi, R, ldr, epi == EPI_F32_ACC && k_splits > 1 ? k_splits : 1, -1, 128, stream);
 	if (!a_t && !b_t) return launch_epi<false, false>(g, epi, tile_cfg, stream);
 	if (!a_t && b_t) return launch_epi<false, true>(g, epi, tile_cfg, stream);
 	if (a_t && b_t) return launch_epi<true, true>(g, epi, tile_cfg, stream);

@@ -83,19 +83,24 @@ constexpr int TURN_SPIN_LIMIT = 1 << 18;  // polls of ~0.5 us
 
 // Byte offsets (relative to the tile origin of the current K slice) of the 16-byte chunks this
 // lane fetches for one operand (< 2^31: 256 rows of at most 64 K elements).  "R" tiles are
-// [256 rows][128 B], "T" tiles [64 k][512 B]; LDS chunk slot s of a row holds global chunk
+// [256 rows][128 B], "T" tiles [64 k][512 B] ([64 k][256 B] for the 128 rows of A in a 128x256 tile); LDS chunk slot s of a row holds global chunk
 // s ^ f(row) with f chosen so that the lanes of a fragment read spread over all banks: an "R"
 // read takes one chunk from each of 32 rows (f = (row / 2) % 8), a "T" transpose read takes 64
 // contiguous bytes from each of four k rows per half-wave (f = 4 * (k % 8): the four rows land in
 // four different 64-byte bank groups; with 2 * (k % 8) pairs of rows shared one and the bank-conflict
 // counter read half of the LDS-active cycles).
 // chunk swizzle of reduction-major ("T") tiles as a function of the k row
-__device__ __forceinline__ int t_swz(int k) { return ((k & 7) << 2) ^ (((k >> 3) & 1) << 1); }
+// ROWS = 128 (a k row is 256 bytes, exactly one row of banks): the four k rows of a half-wave's transpose read
+// are moved into four different 64-byte groups by (k % 4) * 4 chunks, rows k and k + 8 apart by two chunks
+template <int ROWS = 256>
+__device__ __forceinline__ int t_swz(int k) {
+	return ((k & (ROWS == 256 ? 7 : 3)) << 2) ^ (((k >> 3) & 1) << 1);
+}
 
 // PAIRED (k-contiguous operands only): the 256 tile rows are not 256 consecutive operand rows but, for
 // each 128-row half, 64 consecutive rows followed by the 64 rows `pair_rows` further down — the gate and
 // up rows of the same 64 SwiGLU columns, which thereby land in one wave's accumulators.
-template <bool T, int LPO, bool PAIRED = false>
+template <bool T, int LPO, bool PAIRED = false, int ROWS = 256>
 __device__ __forceinline__ void lane_offsets(int wave, int lane, int64_t ld, uint32_t (&off)[LPO], int64_t pair_rows = 0) {
 #pragma unroll
 	for (int i = 0; i < LPO; i++) {
@@ -105,8 +110,9 @@ __device__ __forceinline__ void lane_offsets(int wave, int lane, int64_t ld, uin
 			const int64_t grow = PAIRED ? (row >> 7) * 64 + (row & 63) + ((row >> 6) & 1) * pair_rows : row;
 			off[i] = (uint32_t)((grow * ld + ((slot ^ ((row >> 1) & 7)) << 3)) * 2);
 		} else {
-			const int krow = q * 2 + (lane >> 5), slot = lane & 31;
-			off[i] = (uint32_t)((krow * ld + ((slot ^ t_swz(krow)) << 3)) * 2);
+			constexpr int CPR = ROWS / 8;  // 16-byte chunks per k row; a 1 KiB piece holds 64 / CPR k rows
+			const int krow = q * (64 / CPR) + lane / CPR, slot = lane % CPR;
+			off[i] = (uint32_t)((krow * ld + ((slot ^ t_swz<ROWS>(krow)) << 3)) * 2);
 		}
 	}
 }
@@ -115,7 +121,7 @@ __device__ __forceinline__ void lane_offsets(int wave, int lane, int64_t ld, uin
 // of the current slice: lane l holds row (or column) row0 + l % 16 at k = 32 kq + 8 (l / 16) .. + 7.
 // "R" tiles give it with one 16-byte read; "T" tiles with two transpose reads, each of which hands
 // the 16 lanes of a group the 4 (k) x 16 (rows) block they address row-wise.
-template <bool T>
+template <bool T, int ROWS = 256>
 __device__ __forceinline__ bf16x8 frag(const unsigned char* base, int row0, int kq, int lane) {
 	if constexpr (!T) {
 		const int r = row0 + (lane & 15);
@@ -125,10 +131,10 @@ __device__ __forceinline__ bf16x8 frag(const unsigned char* base, int row0, int 
 		const int j = lane & 15;
 		const int m = row0 + 4 * (j & 3);
 		const int kk = kq * 32 + 8 * (lane >> 4) + (j >> 2);
-		const int c0 = (m >> 3) ^ t_swz(kk);
-		const int c1 = (m >> 3) ^ t_swz(kk + 4);
-		const unsigned char* p0 = base + kk * 512 + c0 * 16 + (j & 1) * 8;
-		const unsigned char* p1 = base + (kk + 4) * 512 + c1 * 16 + (j & 1) * 8;
+		const int c0 = (m >> 3) ^ t_swz<ROWS>(kk);
+		const int c1 = (m >> 3) ^ t_swz<ROWS>(kk + 4);
+		const unsigned char* p0 = base + kk * (ROWS * 2) + c0 * 16 + (j & 1) * 8;
+		const unsigned char* p1 = base + (kk + 4) * (ROWS * 2) + c1 * 16 + (j & 1) * 8;
 		s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 ELF_LDS*)(p0));
 		s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 ELF_LDS*)(p1));
 		return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
@@ -137,16 +143,17 @@ __device__ __forceinline__ bf16x8 frag(const unsigned char* base, int row0, int 
 
 // The two byte offsets (within the operand tile of stage 0, k32 half 0) that frag<true> reads for the
 // 16-row slab at row0, and the fragment read from them for k32 half kq of the tile at `base`.
+template <int ROWS = 256>
 __device__ __forceinline__ void frag_t_offsets(int row0, int lane, uint32_t (&o)[2]) {
 	const int j = lane & 15;
 	const int m = row0 + 4 * (j & 3);
 	const int kk = 8 * (lane >> 4) + (j >> 2);
-	o[0] = (uint32_t)(kk * 512 + (((m >> 3) ^ t_swz(kk)) << 4) + (j & 1) * 8);
-	o[1] = (uint32_t)((kk + 4) * 512 + (((m >> 3) ^ t_swz(kk + 4)) << 4) + (j & 1) * 8);
+	o[0] = (uint32_t)(kk * (ROWS * 2) + (((m >> 3) ^ t_swz<ROWS>(kk)) << 4) + (j & 1) * 8);
+	o[1] = (uint32_t)((kk + 4) * (ROWS * 2) + (((m >> 3) ^ t_swz<ROWS>(kk + 4)) << 4) + (j & 1) * 8);
 }
 // o: LDS byte addresses; imm: a compile-time byte offset (stage and k32 half) that ends up in the
 // instructions' offset fields.  t_swz only looks at k % 16, so the second k32 half of a tile lies 32 rows
-// of 512 bytes further on.
+// (of 2 * ROWS bytes) further on.
 __device__ __forceinline__ bf16x8 frag_t_at(const uint32_t (&o)[2], uint32_t imm) {
 	s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 ELF_LDS*)(uintptr_t)(o[0] + imm));
 	s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 ELF_LDS*)(uintptr_t)(o[1] + imm));
@@ -163,8 +170,7 @@ __device__ __forceinline__ bf16x8 frag_t_at(const uint32_t (&o)[2], uint32_t imm
 // NW = 8, RT = 2: 256x256 workgroup tile, two waves per SIMD with 64x128 wave tiles (12 fragment reads per
 // k32 and 32 MFMAs); the two waves fill each other's issue gaps and barrier waits.  Used when both
 // operands are reduction-major (dW): each of their fragments costs two transpose reads and an address.
-// NW = 4, RT = 2: 128x256 workgroup tile for outputs with too few 256x256 tiles to fill the chip
-// (A must be k-contiguous: the reduction-major tile layout below assumes 256 rows).  One wave per SIMD
+// NW = 4, RT = 2: 128x256 workgroup tile for outputs with too few 256x256 tiles to fill the chip.  One wave per SIMD
 // as well, so it runs the same interleaved loop (+35-40 % on the GPT-2-small shapes over read bursts).
 // acc += a b as one in-place instruction on accumulator registers — the builtin leaves source and
 // destination accumulators untied, and when all 256 accumulator registers are live (128x128 wave tiles) the
@@ -180,7 +186,6 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	using Sh = Shape<NW, RT>;
 	constexpr int BM = Sh::BM, A_BYTES = Sh::A_BYTES, STAGE_BYTES = Sh::STAGE_BYTES;
 	constexpr int LOADS_A = Sh::LOADS_A, LOADS_B = Sh::LOADS_B, LOADS_PER_STAGE = Sh::LOADS_PER_STAGE;
-	static_assert(BM == 256 || !AT, "reduction-major A tiles are laid out for 256 rows");
 	constexpr bool PAIRED = EPI == EPI_BF16_SWIGLU;
 	static_assert(!PAIRED || !BT, "the paired row order is defined for a k-contiguous B");
 	extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
@@ -275,7 +280,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	const int64_t a_step = AT ? (int64_t)BKS * g.lda : BKS;
 	const int64_t b_step = BT ? (int64_t)BKS * g.ldb : BKS;
 	uint32_t aoff[LOADS_A], boff[LOADS_B];
-	lane_offsets<AT, LOADS_A>(wave, lane, g.lda, aoff);
+	lane_offsets<AT, LOADS_A, false, BM>(wave, lane, g.lda, aoff);
 	lane_offsets<BT, LOADS_B, PAIRED>(wave, lane, g.ldb, boff, g.N / 2);
 
 	// this wave's first 1 KiB piece of each operand in stage 0
@@ -335,7 +340,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	auto load_a = [&](int buf, int step, int kq) {
 		const unsigned char* sa = smem + (step % NST) * A_BYTES;
 #pragma unroll
-		for (int i = 0; i < RF; i++) fa[buf][i] = frag<AT>(sa, wr * (RT * 32) + i * 16, kq, lane);
+		for (int i = 0; i < RF; i++) fa[buf][i] = frag<AT, BM>(sa, wr * (RT * 32) + i * 16, kq, lane);
 	};
 	auto load_b = [&](int buf, int step, int kq, int h) {
 		const unsigned char* sb = smem + NST * A_BYTES + (step % NST) * B_BYTES;
@@ -356,7 +361,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 		if constexpr (AT)
 #pragma unroll
 			for (int i = 0; i < RF; i++) {
-				frag_t_offsets(wr * (RT * 32) + i * 16, lane, ta[i]);
+				frag_t_offsets<BM>(wr * (RT * 32) + i * 16, lane, ta[i]);
 				ta[i][0] += lds_addr(smem), ta[i][1] += lds_addr(smem);
 				// opaque from here on: folded into these, the tile's base would push the loop's offsets past 16 bits
 				asm volatile("" : "+v"(ta[i][0]), "+v"(ta[i][1]));
@@ -386,8 +391,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 					else fb[pb_buf][r] = frag<BT>(sb, wc * 128 + (pb_h * 4 + r) * 16, pb_kq, lane);
 				} else if constexpr (r - 4 < RF) {
 					if (pa) {
-						if constexpr (AT) fa[pa_buf][r - 4] = frag_t_at(ta[r - 4], (uint32_t)(SA * A_BYTES + pa_kq * (32 * 512)));
-						else fa[pa_buf][r - 4] = frag<AT>(sa, wr * (RT * 32) + (r - 4) * 16, pa_kq, lane);
+						if constexpr (AT) fa[pa_buf][r - 4] = frag_t_at(ta[r - 4], (uint32_t)(SA * A_BYTES + pa_kq * (32 * BM * 2)));
+						else fa[pa_buf][r - 4] = frag<AT, BM>(sa, wr * (RT * 32) + (r - 4) * 16, pa_kq, lane);
 					}
 				}
 			}
@@ -653,7 +658,6 @@ int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t 
                   void* C2, int64_t ldc2, const void* rope_cs, int rope_S, int rope_cols, int rope_D) {
 	ELF_REQUIRE(bm == 256 || bm == 128, "gemm (dma tile): 256- or 128-row tiles");
 	ELF_REQUIRE(M % bm == 0 && N % dma::BN == 0 && K % dma::BKS == 0, "gemm (dma tile): M multiple of %d, N of 256 and K of 64 required", bm);
-	ELF_REQUIRE(bm == 256 || !a_t, "gemm (dma tile): 128-row tiles need a k-contiguous A");
 	const int ntiles = (M / bm) * (N / dma::BN);
 	ELF_REQUIRE(epi != EPI_BF16_SWIGLU || (C2 && !a_t && !b_t), "gemm (dma tile): the SwiGLU epilogue needs k-contiguous operands and a second output");
 	// the paired rows of the SwiGLU epilogue are addressed with 32-bit byte offsets from the tile's first row
@@ -673,8 +677,11 @@ int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t 
 	// split tiles add in a fixed order (bit-reproducible weight gradients) as long as each has a counter of its own
 	a.turn_tag = a.tail_tiles > 0 && a.tail_tiles <= dma::TURN_TILES ? next_turn_tag() : 0;
 	if (bm == 128) {
-		if (!b_t) return dma::launch_epi<4, 2, false, false>(a, epi, stream);
-		return dma::launch_epi<4, 2, false, true>(a, epi, stream);
+		if (!a_t && !b_t) return dma::launch_epi<4, 2, false, false>(a, epi, stream);
+		if (!a_t && b_t) return dma::launch_epi<4, 2, false, true>(a, epi, stream);
+		if (a_t && b_t) return dma::launch_epi<4, 2, true, true>(a, epi, stream);
+		set_error("gemm: layout A=T,B=R is not used by any stage contraction");
+		return -1;
 	}
 	// k-contiguous A (forward, dX): four waves with 128x128 wave tiles; both operands reduction-major (dW): eight
 	// waves with 64x128 wave tiles (with two transpose reads per fragment on both operands the lone wave wins on
