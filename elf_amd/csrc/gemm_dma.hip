@@ -24,7 +24,7 @@ namespace elf {
 
 namespace dma {
 
-constexpr int BN = 256, BKS = 64, NST = 2;
+constexpr int BN = 256, BKS = 64;
 constexpr int B_BYTES = BN * BKS * 2;  // 32 KiB per stage
 
 // Shape of one workgroup: NW waves arranged (NW / 2) x 2, each owning RT x 4 accumulator tiles of
@@ -32,6 +32,10 @@ constexpr int B_BYTES = BN * BKS * 2;  // 32 KiB per stage
 template <int NW, int RT>
 struct Shape {
 	static constexpr int BM = (NW / 2) * RT * 32;
+	// K slices in the LDS ring: two of 64 KiB for the 256-row tile; the 128-row tile's slices are 48 KiB and three of
+	// them fit, so its loads run two slices ahead of their use (its shapes are the small ones, whose short K
+	// ranges per workgroup leave a slice's loads less than a trip to memory when fetched one slice ahead)
+	static constexpr int NST = BM == 128 ? 3 : 2;
 	static constexpr int A_BYTES = BM * BKS * 2;
 	static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
 	// 1 KiB pieces (one wave instruction each) per wave, stage and operand
@@ -185,7 +189,7 @@ template <int NW, int RT, bool AT, bool BT, int EPI>
 __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	using Sh = Shape<NW, RT>;
 	constexpr int BM = Sh::BM, A_BYTES = Sh::A_BYTES, STAGE_BYTES = Sh::STAGE_BYTES;
-	constexpr int LOADS_A = Sh::LOADS_A, LOADS_B = Sh::LOADS_B, LOADS_PER_STAGE = Sh::LOADS_PER_STAGE;
+	constexpr int LOADS_A = Sh::LOADS_A, LOADS_B = Sh::LOADS_B, LOADS_PER_STAGE = Sh::LOADS_PER_STAGE, NST = Sh::NST;
 	constexpr bool PAIRED = EPI == EPI_BF16_SWIGLU;
 	static_assert(!PAIRED || !BT, "the paired row order is defined for a k-contiguous B");
 	extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
@@ -301,7 +305,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	auto slice_loads = [&](int step) {
 		const bool ok = step < nk;
 		const int sc = ok ? step : nk - 1;
-		const uint32_t st = (uint32_t)(sc & 1);
+		const uint32_t st = (uint32_t)(sc % NST);
 		return SliceLoads{Ap + (int64_t)sc * a_step, Bp + (int64_t)sc * b_step, ok ? lds_a + st * A_BYTES : lds_dummy, ok ? lds_b + st * B_BYTES : lds_dummy};
 	};
 	auto issue_piece = [&](const SliceLoads& sl, auto pc) {
@@ -329,10 +333,14 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	// kt+2 starts a full slice ahead of its use.
 	constexpr int HALF = LOADS_PER_STAGE / 2;
 	{
-		const SliceLoads s0 = slice_loads(0), s1 = slice_loads(1);
-		static_for<LOADS_PER_STAGE>([&](auto pc) { issue_piece(s0, pc); });
-		static_for<HALF>([&](auto pc) { issue_piece(s1, pc); });
-		wait_vmcnt<HALF>();
+		// slices 0 .. NST-2 whole and the first half of slice NST-1; slice 0 has to have landed
+		static_for<NST - 1>([&](auto sc) {
+			const SliceLoads sl = slice_loads(decltype(sc)::value);
+			static_for<LOADS_PER_STAGE>([&](auto pc) { issue_piece(sl, pc); });
+		});
+		const SliceLoads sh = slice_loads(NST - 1);
+		static_for<HALF>([&](auto pc) { issue_piece(sh, pc); });
+		wait_vmcnt<(NST - 2) * LOADS_PER_STAGE + HALF>();
 	}
 	__syncthreads();
 
@@ -405,27 +413,30 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	auto slice = [&](auto sc, int kt) {
 		constexpr int S = decltype(sc)::value;
 		constexpr std::integral_constant<int, S> CUR{};
-		constexpr std::integral_constant<int, 1 - S> NXT{};
+		constexpr std::integral_constant<int, (S + 1) % NST> NXT{};
 		constexpr std::integral_constant<int, 0> H0{};
 		constexpr std::integral_constant<int, 1> H1{};
 		constexpr std::integral_constant<int, -1> NO_DMA{};
 		// where this slice's loads go: scalar work
-		const SliceLoads next1 = slice_loads(kt + 1), next2 = slice_loads(kt + 2);
+		const SliceLoads next1 = slice_loads(kt + NST - 1), next2 = slice_loads(kt + NST);
 		half_step(0, 0, H0, 1, CUR, 0, 1, false, 0, CUR, 0, next1, std::integral_constant<int, HALF>{});
 		half_step(0, 1, H1, 0, CUR, 1, 0, true, 1, CUR, 1, next1, NO_DMA);
 		half_step(1, 0, H0, 1, CUR, 1, 1, false, 0, CUR, 0, next1, NO_DMA);
-		wait_counters<0, 0>();  // vmcnt(0): slice kt+1 landed; lgkmcnt(0): slice kt fully read
+		// vmcnt: slice kt+1 landed (with three stages slice kt+2's loads may still be in flight); lgkmcnt(0): slice kt fully read
+		wait_counters<(NST - 2) * LOADS_PER_STAGE, 0>();
 		__syncthreads();
-		// with the first half of slice kt+2's loads into the stage the barrier just freed; past the end the
+		// with the first half of slice kt+NST's loads into the stage the barrier just freed; past the end the
 		// fragment reads hit a stale stage and their values are unused
 		half_step(1, 1, H1, 0, NXT, 0, 0, true, 0, NXT, 0, next2, std::integral_constant<int, 0>{});
 	};
 
 	load_a(0, 0, 0);
 	load_b(0, 0, 0, 0);
-	for (int kt = 0; kt < nk; kt += 2) {
+	for (int kt = 0; kt < nk; kt += NST) {
 		slice(std::integral_constant<int, 0>{}, kt);
 		if (kt + 1 < nk) slice(std::integral_constant<int, 1>{}, kt + 1);
+		if constexpr (NST == 3)
+			if (kt + 2 < nk) slice(std::integral_constant<int, 2>{}, kt + 2);
 	}
 
 	// Epilogue through LDS (free once every wave has left the main loop).  Register r of a 16x16
@@ -618,7 +629,7 @@ static int launch(const Args& a, hipStream_t stream) {
 	// the ring + the target of the loads past the end of K (as many KiB as a wave issues loads per
 	// operand); the epilogue needs a 32 x 136 fp32 strip per wave
 	using Sh = Shape<NW, RT>;
-	constexpr int ring = NST * Sh::STAGE_BYTES + (Sh::LOADS_A > Sh::LOADS_B ? Sh::LOADS_A : Sh::LOADS_B) * 1024, epi = NW * 32 * 136 * 4;
+	constexpr int ring = Sh::NST * Sh::STAGE_BYTES + (Sh::LOADS_A > Sh::LOADS_B ? Sh::LOADS_A : Sh::LOADS_B) * 1024, epi = NW * 32 * 136 * 4;
 	constexpr int smem = ring > epi ? ring : epi;
 	auto kern = gemm_dma_kernel<NW, RT, AT, BT, EPI>;
 	static bool attr_set = false;
