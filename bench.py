@@ -29,7 +29,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per GEMM launch (mean over the launches of one step), from rocprofv3 --pmc FETCH_SIZE and
 # --pmc WRITE_SIZE runs of this script scaled by the same counters' reading for a copy kernel of known
 # size (--calibration-copy); measured per workload, None where it was not.
-GEMM_TRAFFIC_BYTES = {"llama3_8b_zbh1": 1.696e9}
+GEMM_TRAFFIC_BYTES = {"llama3_8b_zbh1": 1.698e9}
 
 WORKLOADS = {
 	# headline configuration: Llama-3-8B-shaped stage, ZB-H1 stream of block 1 in a 4-stage pipeline
@@ -234,7 +234,7 @@ def hbm_ceiling():
 	return out
 
 
-def vendor_gemm(w, seconds=1.0):
+def vendor_gemm(w, seconds=1.5):
 	"""The twelve dense contractions of one block of the workload (forward y = x W^T, input gradient dX = dY W, weight
 	gradient dW = dY^T X for each of the four projections), each run back to back for ``seconds`` through this library
 	and through torch.matmul (the vendor's GEMM library), on the same operands and the same GPU, with socket power and
@@ -247,9 +247,11 @@ def vendor_gemm(w, seconds=1.0):
 	shapes = [("qkv", nq + 2 * nkv, d), ("proj", d, nq), ("up", F * (2 if w["arch"] == "llama" else 1), d), ("down", d, F)]
 
 	def sustained(fn, flops):
-		for _ in range(5):
-			fn()
-		torch.cuda.synchronize()
+		t0 = time.perf_counter()
+		while time.perf_counter() - t0 < 0.3 * seconds:  # untimed: lets the governor and the smoothed power reading settle
+			for _ in range(25):
+				fn()
+			torch.cuda.synchronize()
 		n, t0 = 0, time.perf_counter()
 		with Telemetry(period=0.02) as tel:
 			while time.perf_counter() - t0 < seconds:
