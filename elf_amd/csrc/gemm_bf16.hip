@@ -162,7 +162,7 @@ __global__ __launch_bounds__(WR* WC * 64) void gemm_kernel(GemmArgs g) {
 	auto take_turn = [&]() {
 		if (g.k_splits > 1 && g.turn_tag) {
 			if (tid == 0 && ksplit > 0) {
-				for (int spin = 0; spin < (1 << 18) && __hip_atomic_load(my_turn, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != turn_want; spin++)
+				for (int spin = 0; spin < (1 << 15) && __hip_atomic_load(my_turn, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != turn_want; spin++)
 					__builtin_amdgcn_s_sleep(4);
 			}
 			__syncthreads();

@@ -83,7 +83,7 @@ struct Args {
 // predecessor is through with that strip and the splits of a tile overlap except for about one strip.
 constexpr int TURN_TILES = 4096, TURN_PER_TILE = 16;
 static __device__ uint32_t turn[TURN_TILES * TURN_PER_TILE];
-constexpr int TURN_SPIN_LIMIT = 1 << 18;  // polls of ~0.5 us
+constexpr int TURN_SPIN_LIMIT = 1 << 15;  // polls of ~1 us: far beyond the length of a predecessor's epilogue
 
 // Byte offsets (relative to the tile origin of the current K slice) of the 16-byte chunks this
 // lane fetches for one operand (< 2^31: 256 rows of at most 64 K elements).  "R" tiles are
@@ -448,6 +448,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	__syncthreads();
 	constexpr int PITCH = 136;
 	float* ws = reinterpret_cast<float*>(smem) + wave * (32 * PITCH);
+	[[maybe_unused]] int turn_patience = TURN_SPIN_LIMIT;
 	const int col_l = lane & 15;
 	const int row_l = (lane >> 4) * 4;
 #pragma unroll
@@ -582,8 +583,11 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 					// wait for this split's turn on this strip (see turn[]); every lane polls the same word.  Plain
 					// (cache-bypassing) loads: nothing is read after the wait, the adds are performed at the memory side
 					const uint32_t want = (g.turn_tag << 8) | (uint32_t)ksplit;
-					for (int spin = 0; spin < TURN_SPIN_LIMIT && __hip_atomic_load(my_turn, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != want; spin++)
+					int spin = 0;
+					for (; spin < turn_patience && __hip_atomic_load(my_turn, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != want; spin++)
 						__builtin_amdgcn_s_sleep(8);
+					// a wave that gave up once (its counters are shared with a concurrent launch) does not wait again
+					if (spin >= turn_patience) turn_patience = 0;
 				}
 				// several workgroups add into this tile: fp32 atomics, one scalar per lane so that a wave
 				// instruction covers two whole 128-byte rows of 32 columns (16 bytes per lane would touch a
