@@ -837,7 +837,7 @@ int launch_bwd(const AttnBwdArgs& a, dim3 grid, hipStream_t stream) {
 		ELF_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
 		attr_set = true;
 	}
-	hipLaunchKernelGGL(kern, grid, dim3(256), smem, stream, a);
+	ELF_LAUNCH(kern, grid, dim3(256), smem, stream, a);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
 }
@@ -873,7 +873,7 @@ int attn_bwd(const void* q, const void* k, const void* v, const void* o, const v
 	{
 		const int64_t rows = T * Hq, per_block = 256 / (D / 8);
 		const int64_t want = (rows + per_block - 1) / per_block;
-		hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)(want < 8192 ? want : 8192)), dim3(256), 0, stream, (const bf16_t*)dO,
+		ELF_LAUNCH(attn_delta_kernel, dim3((unsigned)(want < 8192 ? want : 8192)), dim3(256), 0, stream, (const bf16_t*)dO,
 	                   (const bf16_t*)o, (const float*)lse, delta, nlse2, lddo, ldo, B, S, Hq, D);
 	}
 	AttnBwdArgs a{(const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, (const bf16_t*)dO, nlse2, delta, dq_part,
@@ -886,7 +886,7 @@ int attn_bwd(const void* q, const void* k, const void* v, const void* o, const v
 	if (rc) return rc;
 	const int64_t n16 = T * (Hq * D / 16);
 	const int64_t blocks = (n16 + 255) / 256;
-	hipLaunchKernelGGL(dq_reduce_kernel, dim3((unsigned)(blocks < 16384 ? blocks : 16384)), dim3(256), 0, stream, dq_part, (bf16_t*)dq, B, S,
+	ELF_LAUNCH(dq_reduce_kernel, dim3((unsigned)(blocks < 16384 ? blocks : 16384)), dim3(256), 0, stream, dq_part, (bf16_t*)dq, B, S,
 	                   Hq * D, lddq, scale, causal, D, (const float2*)rope_cs);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;

@@ -202,7 +202,7 @@ int launch_fwd(const AttnArgs& a, dim3 grid, hipStream_t stream) {
 		ELF_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
 		attr_set = true;
 	}
-	hipLaunchKernelGGL(kern, grid, dim3(256), smem, stream, a);
+	ELF_LAUNCH(kern, grid, dim3(256), smem, stream, a);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
 }

@@ -276,7 +276,7 @@ static int norm_fwd_dispatch(const void* x, const void* gamma, const void* beta,
                              float eps, hipStream_t s) {
 	const dim3 block(256);
 #define ELF_NORM_FWD(N, W)                                                                                          \
-	hipLaunchKernelGGL((norm_fwd_kernel<N, W, LN>), dim3(W == 1 ? (T + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK : T), block, 0, \
+	ELF_LAUNCH((norm_fwd_kernel<N, W, LN>), dim3(W == 1 ? (T + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK : T), block, 0, \
 	                   s, (const bf16_t*)x, (const bf16_t*)gamma, (const bf16_t*)beta, (bf16_t*)y, (float2*)stats, T, d, eps)
 	if (d <= 512) ELF_NORM_FWD(1, 1);
 	else if (d <= 1024) ELF_NORM_FWD(2, 1);
@@ -307,7 +307,7 @@ static int norm_bwd_dispatch(const void* dy, const void* x, const void* gamma, c
                              void* dx, float* part, int T, int d, hipStream_t s) {
 	const dim3 grid(norm_bwd_blocks(T, d)), block(256);
 #define ELF_NORM_BWD(N, W)                                                                                      \
-	hipLaunchKernelGGL((norm_bwd_kernel<N, W, LN>), grid, block, 0, s, (const bf16_t*)dy, (const bf16_t*)x,       \
+	ELF_LAUNCH((norm_bwd_kernel<N, W, LN>), grid, block, 0, s, (const bf16_t*)dy, (const bf16_t*)x,       \
 	                   (const bf16_t*)gamma, (const float2*)stats, (const bf16_t*)dres, (bf16_t*)dx, part, T, d)
 	if (d <= 512) ELF_NORM_BWD(1, 1);
 	else if (d <= 1024) ELF_NORM_BWD(2, 1);
@@ -330,7 +330,7 @@ static int norm_bwd_launch(int kind, const void* dy, const void* x, const void* 
 	}
 	if (rc) return rc;
 	const int nparts = norm_bwd_blocks(T, d);
-	hipLaunchKernelGGL(norm_bwd_finalize_kernel, dim3((d + 31) / 32), dim3(1024), 0, s, workspace, nparts, d, dgamma,
+	ELF_LAUNCH(norm_bwd_finalize_kernel, dim3((d + 31) / 32), dim3(1024), 0, s, workspace, nparts, d, dgamma,
 	                   kind == NORM_LAYER ? dbeta : nullptr);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
@@ -450,14 +450,14 @@ static inline int ew_grid(int64_t nchunks) {
 int gelu_fwd(const void* x, void* y, int64_t n, hipStream_t s) {
 	ELF_REQUIRE(n > 0 && n % 8 == 0 && x && y, "gelu_fwd: n must be a positive multiple of 8");
 	ProfScope prof(PROF_ACT_FWD, 4.0 * n, s);
-	hipLaunchKernelGGL(gelu_fwd_kernel, dim3(ew_grid(n / 8)), dim3(256), 0, s, (const bf16_t*)x, (bf16_t*)y, n / 8);
+	ELF_LAUNCH(gelu_fwd_kernel, dim3(ew_grid(n / 8)), dim3(256), 0, s, (const bf16_t*)x, (bf16_t*)y, n / 8);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
 }
 int gelu_bwd(const void* dy, const void* x, void* dx, int64_t n, hipStream_t s) {
 	ELF_REQUIRE(n > 0 && n % 8 == 0 && x && dy && dx, "gelu_bwd: n must be a positive multiple of 8");
 	ProfScope prof(PROF_ACT_BWD, 6.0 * n, s);
-	hipLaunchKernelGGL(gelu_bwd_kernel, dim3(ew_grid(n / 8)), dim3(256), 0, s, (const bf16_t*)dy, (const bf16_t*)x,
+	ELF_LAUNCH(gelu_bwd_kernel, dim3(ew_grid(n / 8)), dim3(256), 0, s, (const bf16_t*)dy, (const bf16_t*)x,
 	                   (bf16_t*)dx, n / 8);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
@@ -465,14 +465,14 @@ int gelu_bwd(const void* dy, const void* x, void* dx, int64_t n, hipStream_t s) 
 int swiglu_fwd(const void* gu, void* h, int64_t T, int F, hipStream_t s) {
 	ELF_REQUIRE(T > 0 && F > 0 && F % 8 == 0 && gu && h, "swiglu_fwd: F must be a positive multiple of 8");
 	ProfScope prof(PROF_ACT_FWD, 6.0 * T * F, s);
-	hipLaunchKernelGGL(swiglu_fwd_kernel, dim3(ew_grid(T * (F / 8))), dim3(256), 0, s, (const bf16_t*)gu, (bf16_t*)h, T, F);
+	ELF_LAUNCH(swiglu_fwd_kernel, dim3(ew_grid(T * (F / 8))), dim3(256), 0, s, (const bf16_t*)gu, (bf16_t*)h, T, F);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
 }
 int swiglu_bwd(const void* dh, const void* gu, void* dgu, int64_t T, int F, hipStream_t s) {
 	ELF_REQUIRE(T > 0 && F > 0 && F % 8 == 0 && gu && dh && dgu, "swiglu_bwd: F must be a positive multiple of 8");
 	ProfScope prof(PROF_ACT_BWD, 10.0 * T * F, s);
-	hipLaunchKernelGGL(swiglu_bwd_kernel, dim3(ew_grid(T * (F / 8))), dim3(256), 0, s, (const bf16_t*)dh,
+	ELF_LAUNCH(swiglu_bwd_kernel, dim3(ew_grid(T * (F / 8))), dim3(256), 0, s, (const bf16_t*)dh,
 	                   (const bf16_t*)gu, (bf16_t*)dgu, T, F);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
@@ -496,7 +496,7 @@ __global__ void rope_table_kernel(float2* __restrict__ cs, int S, int half, doub
 int rope_table(void* cs, int S, int D, double theta, hipStream_t s) {
 	ELF_REQUIRE(cs && S > 0 && D > 0 && D % 16 == 0, "rope_table: head_dim must be a multiple of 16");
 	const int n = S * (D / 2);
-	hipLaunchKernelGGL(rope_table_kernel, dim3((n + 255) / 256), dim3(256), 0, s, (float2*)cs, S, D / 2, theta);
+	ELF_LAUNCH(rope_table_kernel, dim3((n + 255) / 256), dim3(256), 0, s, (float2*)cs, S, D / 2, theta);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
 }
@@ -529,7 +529,7 @@ int rope_apply(void* buf, const void* cs, int64_t T, int S, int ld, int n_heads,
 	ELF_REQUIRE(D % 16 == 0 && ld % 8 == 0 && n_heads * D <= ld, "rope: bad head layout");
 	const int64_t n = T * n_heads * (D / 16);
 	ProfScope prof(PROF_ROPE, 4.0 * T * n_heads * D, s);
-	hipLaunchKernelGGL(rope_kernel, dim3(ew_grid(n)), dim3(256), 0, s, (bf16_t*)buf, (const float2*)cs, T, S, ld, n_heads,
+	ELF_LAUNCH(rope_kernel, dim3(ew_grid(n)), dim3(256), 0, s, (bf16_t*)buf, (const float2*)cs, T, S, ld, n_heads,
 	                   D, backward ? -1.f : 1.f);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
@@ -563,7 +563,7 @@ int scale_grads(void* acc_f32, void* out_bf16, int64_t n, float scale, hipStream
 	ELF_REQUIRE(acc_f32 && n > 0, "scale_grads: empty");
 	ELF_REQUIRE(((uintptr_t)acc_f32 % 16) == 0 && (!out_bf16 || ((uintptr_t)out_bf16 % 8) == 0), "scale_grads: misaligned");
 	ProfScope prof(PROF_SCALE, (out_bf16 ? 10.0 : 8.0) * n, s);
-	hipLaunchKernelGGL(scale_grads_kernel, dim3(ew_grid(n / 4 + 1)), dim3(256), 0, s, (float*)acc_f32, (bf16_t*)out_bf16,
+	ELF_LAUNCH(scale_grads_kernel, dim3(ew_grid(n / 4 + 1)), dim3(256), 0, s, (float*)acc_f32, (bf16_t*)out_bf16,
 	                   n / 4, n, scale);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
@@ -582,7 +582,7 @@ __global__ __launch_bounds__(256) void add_kernel(const bf16_t* __restrict__ a, 
 int add_bf16(const void* a, const void* b, void* out, int64_t n, hipStream_t s) {
 	ELF_REQUIRE(n > 0 && n % 8 == 0 && a && b && out, "add: n must be a positive multiple of 8");
 	ProfScope prof(PROF_ADD, 6.0 * n, s);
-	hipLaunchKernelGGL(add_kernel, dim3(ew_grid(n / 8)), dim3(256), 0, s, (const bf16_t*)a, (const bf16_t*)b, (bf16_t*)out, n / 8);
+	ELF_LAUNCH(add_kernel, dim3(ew_grid(n / 8)), dim3(256), 0, s, (const bf16_t*)a, (const bf16_t*)b, (bf16_t*)out, n / 8);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
 }
@@ -621,7 +621,7 @@ int colsum_bf16(const void* x, int64_t ld, void* out_f32, int64_t T, int N, hipS
 	const int col_blocks = (N + 255) / 256;
 	int64_t slices = (2048 + col_blocks - 1) / col_blocks;  // about eight workgroups per CU
 	if (slices > (T + 7) / 8) slices = (T + 7) / 8;
-	hipLaunchKernelGGL(colsum_kernel, dim3(col_blocks, (unsigned)slices), dim3(256), 0, s, (const bf16_t*)x, ld, (float*)out_f32, T, N);
+	ELF_LAUNCH(colsum_kernel, dim3(col_blocks, (unsigned)slices), dim3(256), 0, s, (const bf16_t*)x, ld, (float*)out_f32, T, N);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
 }
@@ -667,7 +667,7 @@ __global__ __launch_bounds__(256) void embedding_bwd_kernel(const int64_t* __res
 int embedding_fwd(const void* ids, const void* table, void* out, int64_t T, int d, int V, hipStream_t s) {
 	ELF_REQUIRE(ids && table && out && T > 0 && V > 0 && d > 0 && d % 8 == 0, "embedding_fwd: bad argument (d must be a multiple of 8)");
 	ProfScope prof(PROF_EMBED, 4.0 * T * d, s);
-	hipLaunchKernelGGL(embedding_fwd_kernel, dim3(ew_grid(T * (d / 8))), dim3(256), 0, s, (const int64_t*)ids, (const bf16_t*)table,
+	ELF_LAUNCH(embedding_fwd_kernel, dim3(ew_grid(T * (d / 8))), dim3(256), 0, s, (const int64_t*)ids, (const bf16_t*)table,
 	                   (bf16_t*)out, T, d, V);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
@@ -675,7 +675,7 @@ int embedding_fwd(const void* ids, const void* table, void* out, int64_t T, int 
 int embedding_bwd(const void* ids, const void* dx, void* dtable_f32, int64_t T, int d, int V, hipStream_t s) {
 	ELF_REQUIRE(ids && dx && dtable_f32 && T > 0 && V > 0 && d > 0 && d % 8 == 0, "embedding_bwd: bad argument (d must be a multiple of 8)");
 	ProfScope prof(PROF_EMBED, 10.0 * T * d, s);
-	hipLaunchKernelGGL(embedding_bwd_kernel, dim3(ew_grid(T * (d / 8))), dim3(256), 0, s, (const int64_t*)ids, (const bf16_t*)dx,
+	ELF_LAUNCH(embedding_bwd_kernel, dim3(ew_grid(T * (d / 8))), dim3(256), 0, s, (const int64_t*)ids, (const bf16_t*)dx,
 	                   (float*)dtable_f32, T, d, V);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;

@@ -284,7 +284,7 @@ static int launch_cfg(const GemmArgs& g, hipStream_t stream) {
 	a.tiles_n = g.N / BN;
 	a.turn_tag = EPI == EPI_F32_ACC && a.k_splits > 1 && a.tiles_m * a.tiles_n <= TURN_RS_SLOTS ? next_turn_tag() : 0;
 	const int grid = a.tiles_m * a.tiles_n * a.k_splits;
-	hipLaunchKernelGGL(kern, dim3(grid), dim3(WR * WC * 64), smem, stream, a);
+	ELF_LAUNCH(kern, dim3(grid), dim3(WR * WC * 64), smem, stream, a);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
 }

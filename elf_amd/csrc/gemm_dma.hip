@@ -641,7 +641,7 @@ static int launch(const Args& a, hipStream_t stream) {
 		ELF_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
 		attr_set = true;
 	}
-	hipLaunchKernelGGL(kern, dim3(a.tiles_m * a.tiles_n + a.tail_tiles * (a.k_splits - 1)), dim3(NW * 64), smem, stream, a);
+	ELF_LAUNCH(kern, dim3(a.tiles_m * a.tiles_n + a.tail_tiles * (a.k_splits - 1)), dim3(NW * 64), smem, stream, a);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
 }

@@ -1,7 +1,11 @@
 // Internal launcher prototypes shared by the C-ABI layer and the stage executor.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
+
+#include <tuple>
+#include <utility>
 
 namespace elf {
 
@@ -121,7 +125,31 @@ struct ProfScope {
 	~ProfScope();
 	int slot;
 	hipStream_t stream;
+	ProfScope* outer;
 };
+// The timing events of the innermost open scope of this thread, to be attached to the next kernel launch: the start
+// event for the scope's first launch only, the stop event for every launch (the last one keeps it).  False when
+// nothing is being timed.
+bool prof_launch_events(hipEvent_t* start, hipEvent_t* stop);
+
+// A launch that carries its scope's timing events in the dispatch itself (hipExtLaunchKernel): the kernel's own start
+// and end timestamps, with no barrier packets between the launches of a stream (an event recorded before and after
+// each launch costs two of them, about 3 us per launch).
+template <class... P, size_t... I, class... A>
+inline void launch_timed(void (*kern)(P...), dim3 grid, dim3 block, unsigned smem, hipStream_t s, hipEvent_t e0, hipEvent_t e1,
+                         std::index_sequence<I...>, A&&... a) {
+	static_assert(sizeof...(P) == sizeof...(A), "kernel argument count");
+	std::tuple<P...> formal{static_cast<P>(a)...};
+	void* ptrs[] = {(void*)&std::get<I>(formal)...};
+	(void)hipExtLaunchKernel(reinterpret_cast<const void*>(kern), grid, block, ptrs, smem, s, e0, e1, 0);
+}
+template <class... P, class... A>
+inline void launch_kernel(void (*kern)(P...), dim3 grid, dim3 block, unsigned smem, hipStream_t s, A&&... a) {
+	hipEvent_t e0 = nullptr, e1 = nullptr;
+	if (prof_launch_events(&e0, &e1)) launch_timed(kern, grid, block, smem, s, e0, e1, std::index_sequence_for<P...>{}, a...);
+	else hipLaunchKernelGGL(kern, grid, block, smem, s, static_cast<P>(a)...);
+}
+#define ELF_LAUNCH(kern, grid, block, smem, stream, ...) elf::launch_kernel(kern, grid, block, smem, stream, __VA_ARGS__)
 // Waits for the recorded events; totals since the last prof_enable(1). Returns the launch count.
 int prof_collect(int kind, double* total_ms, double* total_work);
 

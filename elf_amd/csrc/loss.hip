@@ -238,7 +238,7 @@ template <int G, int C>
 void launch_rows(const LossArgs& a, hipStream_t s) {
 	constexpr int BLOCK = G < 256 ? 256 : G;
 	constexpr int ROWS = BLOCK / G;
-	hipLaunchKernelGGL((cross_entropy_kernel<G, C>), dim3((unsigned)((a.rows + ROWS - 1) / ROWS)), dim3(BLOCK), 0, s, a);
+	ELF_LAUNCH((cross_entropy_kernel<G, C>), dim3((unsigned)((a.rows + ROWS - 1) / ROWS)), dim3(BLOCK), 0, s, a);
 }
 
 }  // namespace
@@ -260,15 +260,15 @@ int cross_entropy(const void* logits, int64_t ld, const void* target, int64_t ro
 	if (width <= 64 * 2 * 8) launch_rows<64, 2>(a, s);
 	else if (width <= 64 * 8 * 8) launch_rows<64, 8>(a, s);
 	else if (width <= 256 * 8 * 8) launch_rows<256, 8>(a, s);
-	else if (width <= 65536) hipLaunchKernelGGL(cross_entropy_stream_kernel<256>, dim3((unsigned)rows), dim3(256), 0, s, a);
-	else hipLaunchKernelGGL(cross_entropy_stream_kernel<1024>, dim3((unsigned)rows), dim3(1024), 0, s, a);
+	else if (width <= 65536) ELF_LAUNCH(cross_entropy_stream_kernel<256>, dim3((unsigned)rows), dim3(256), 0, s, a);
+	else ELF_LAUNCH(cross_entropy_stream_kernel<1024>, dim3((unsigned)rows), dim3(1024), 0, s, a);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
 }
 
 int cross_entropy_reduce(const void* row_loss, const void* target, int64_t rows, int64_t ignore_index, void* out2, hipStream_t s) {
 	ELF_REQUIRE(target && out2 && rows > 0, "cross_entropy_reduce: bad argument");
-	hipLaunchKernelGGL(cross_entropy_reduce_kernel, dim3(1), dim3(1024), 0, s, (const float*)row_loss, (const int64_t*)target, rows,
+	ELF_LAUNCH(cross_entropy_reduce_kernel, dim3(1), dim3(1024), 0, s, (const float*)row_loss, (const int64_t*)target, rows,
 	                   ignore_index, (float*)out2);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;

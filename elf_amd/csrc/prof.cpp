@@ -1,4 +1,5 @@
-// Live per-launch timing with HIP events on the launch stream (see ProfScope in kernels.h).
+// Live per-launch timing with HIP events on the launch stream (see ProfScope and launch_kernel in kernels.h): the
+// events travel in the kernel dispatches themselves and read the kernels' own start and end timestamps.
 #include <vector>
 
 #include "common.h"
@@ -10,10 +11,12 @@ struct ProfRec {
 	int kind;
 	double work;
 	hipEvent_t e0, e1;
+	bool started;  // a launch has taken the start event
 };
 static bool g_on = false;
 static std::vector<ProfRec> g_recs;
 static std::vector<hipEvent_t> g_free_events;
+static thread_local ProfScope* t_scope = nullptr;
 
 static hipEvent_t get_event() {
 	if (!g_free_events.empty()) {
@@ -38,23 +41,33 @@ void prof_enable(int on) {
 }
 bool prof_on() { return g_on; }
 
-ProfScope::ProfScope(int kind, double work, hipStream_t s) : slot(-1), stream(s) {
+ProfScope::ProfScope(int kind, double work, hipStream_t s) : slot(-1), stream(s), outer(nullptr) {
 	if (!g_on) return;
-	ProfRec r{kind, work, get_event(), get_event()};
+	ProfRec r{kind, work, get_event(), get_event(), false};
 	if (!r.e0 || !r.e1) return;
-	(void)hipEventRecord(r.e0, s);
 	slot = (int)g_recs.size();
 	g_recs.push_back(r);
+	outer = t_scope;
+	t_scope = this;
 }
 ProfScope::~ProfScope() {
-	if (slot >= 0) (void)hipEventRecord(g_recs[slot].e1, stream);
+	if (slot >= 0) t_scope = outer;
+}
+
+bool prof_launch_events(hipEvent_t* start, hipEvent_t* stop) {
+	if (!t_scope || t_scope->slot < 0 || t_scope->slot >= (int)g_recs.size()) return false;
+	ProfRec& r = g_recs[t_scope->slot];
+	*start = r.started ? nullptr : r.e0;
+	*stop = r.e1;
+	r.started = true;
+	return true;
 }
 
 int prof_collect(int kind, double* total_ms, double* total_work) {
 	int n = 0;
 	double ms = 0, work = 0;
 	for (auto& r : g_recs) {
-		if (r.kind != kind) continue;
+		if (r.kind != kind || !r.started) continue;
 		if (hipEventSynchronize(r.e1) != hipSuccess) continue;
 		float t = 0;
 		if (hipEventElapsedTime(&t, r.e0, r.e1) != hipSuccess) continue;
@@ -104,9 +117,9 @@ int hbm_probe(int mode, const void* src, void* dst, int64_t bytes, hipStream_t s
 	const int64_t n16 = bytes / 16;
 	const dim3 block(256);
 	// the best of unroll 4 / 8, 1024 / 2048 / 8192 workgroups and plain / non-temporal stores for each pattern at 1 GiB
-	if (mode == 0) hipLaunchKernelGGL((hbm_probe_kernel<0, 4, 0>), dim3(1024), block, 0, s, (const u32x4*)src, (u32x4*)dst, n16);
-	else if (mode == 1) hipLaunchKernelGGL((hbm_probe_kernel<1, 4, 1>), dim3(8192), block, 0, s, (const u32x4*)src, (u32x4*)dst, n16);
-	else hipLaunchKernelGGL((hbm_probe_kernel<2, 8, 0>), dim3(8192), block, 0, s, (const u32x4*)src, (u32x4*)dst, n16);
+	if (mode == 0) ELF_LAUNCH((hbm_probe_kernel<0, 4, 0>), dim3(1024), block, 0, s, (const u32x4*)src, (u32x4*)dst, n16);
+	else if (mode == 1) ELF_LAUNCH((hbm_probe_kernel<1, 4, 1>), dim3(8192), block, 0, s, (const u32x4*)src, (u32x4*)dst, n16);
+	else ELF_LAUNCH((hbm_probe_kernel<2, 8, 0>), dim3(8192), block, 0, s, (const u32x4*)src, (u32x4*)dst, n16);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
 }
