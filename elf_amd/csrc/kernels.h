@@ -146,7 +146,10 @@ inline void launch_timed(void (*kern)(P...), dim3 grid, dim3 block, unsigned sme
 template <class... P, class... A>
 inline void launch_kernel(void (*kern)(P...), dim3 grid, dim3 block, unsigned smem, hipStream_t s, A&&... a) {
 	hipEvent_t e0 = nullptr, e1 = nullptr;
-	if (prof_launch_events(&e0, &e1)) launch_timed(kern, grid, block, smem, s, e0, e1, std::index_sequence_for<P...>{}, a...);
+	hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+	// a stream under graph capture takes plain launches only
+	if (prof_launch_events(&e0, &e1) && hipStreamIsCapturing(s, &capture) == hipSuccess && capture == hipStreamCaptureStatusNone)
+		launch_timed(kern, grid, block, smem, s, e0, e1, std::index_sequence_for<P...>{}, a...);
 	else hipLaunchKernelGGL(kern, grid, block, smem, s, static_cast<P>(a)...);
 }
 #define ELF_LAUNCH(kern, grid, block, smem, stream, ...) elf::launch_kernel(kern, grid, block, smem, stream, __VA_ARGS__)

@@ -148,3 +148,35 @@ def test_capture_refuses_offload_schedules():
 	schedule = COMM_SCHEDULERS["pipelined"](add_comms(sched(placement, 4), sequential_signatures(placement)))
 	with pytest.raises(NotImplementedError):
 		Engine([blk]).capture(None, None, None, [op for op in schedule if op.block_id == 1], [2] * 4)
+
+
+def test_capture_with_live_kernel_timing_switched_on():
+	"""Kernel timing events travel in the dispatches; a stream under capture must get plain launches all the
+	same, and the captured kernels must replay correctly."""
+	from elf_amd import _lib
+	from elf_amd import kernels as K
+
+	lib = _lib.load()
+	g = torch.Generator(device="cuda").manual_seed(11)
+	a = torch.randn(512, 256, device="cuda", generator=g).bfloat16()
+	w = (torch.randn(768, 256, device="cuda", generator=g) * 0.05).bfloat16()
+	out = torch.empty(512, 768, device="cuda", dtype=torch.bfloat16)
+	ref = K.gemm(a, w).clone()
+	lib.elf_prof_enable(1)
+	try:
+		K.gemm(a, w, out=out)  # timed, eager
+		torch.cuda.synchronize()
+		graph = torch.cuda.CUDAGraph()
+		side = torch.cuda.Stream()
+		side.wait_stream(torch.cuda.current_stream())
+		with torch.cuda.stream(side):
+			with torch.cuda.graph(graph, stream=side):
+				K.gemm(a, w, out=out)
+		torch.cuda.current_stream().wait_stream(side)
+		for _ in range(3):
+			out.zero_()
+			graph.replay()
+			torch.cuda.synchronize()
+			assert torch.equal(out, ref)
+	finally:
+		lib.elf_prof_enable(0)
