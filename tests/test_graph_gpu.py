@@ -1,8 +1,8 @@
 """A stage step captured as a HIP graph (Engine.capture, Pipeline.capture_step) against the same step
 run eagerly: every replay is checked, with eager kernels and device synchronisations between the
-replays and with new input data written into the buffers the graph reads.  Outputs of F are
-bit-identical; gradients agree to 2e-3 (dQ and split-K weight gradients add with fp32 atomics, whose
-order differs from run to run)."""
+replays and with new input data written into the buffers the graph reads.  Outputs, input gradients
+and weight gradients of a middle stage are bit-identical: every accumulation of the path has a fixed order
+(the embedding table of a first stage, whose rows add with atomics, is compared to 2e-3)."""
 
 import pytest
 import torch
@@ -68,10 +68,10 @@ def test_captured_stage_stream_replays_like_the_eager_one():
 		torch.cuda.synchronize()
 		for m in range(nmb):
 			assert torch.equal(sent_y[m], y0[m]), f"replay {rep}: y[{m}]"
-			assert_close(sent_dx[m], dx0[m], f"replay {rep}: dx[{m}]", rel_max=2e-3, rel_fro=2e-3)
+			assert torch.equal(sent_dx[m], dx0[m]), f"replay {rep}: dx[{m}]"
 		got = product_grads(stage)
 		for name in sorted(g0):
-			assert_close(got[name], g0[name], f"replay {rep}: grad {name}", rel_max=2e-3, rel_fro=2e-3)
+			assert torch.equal(got[name], g0[name]), f"replay {rep}: grad {name}"
 		# eager work of the same library and a synchronisation between replays
 		K.gemm(a, a)
 		K.norm_fwd(K.NORM_RMS, a, torch.ones(512, dtype=torch.bfloat16, device="cuda"), None, 1e-5)
@@ -91,7 +91,7 @@ def test_captured_stage_stream_replays_like_the_eager_one():
 	for m in range(nmb):
 		assert torch.equal(y_rep[m], y1[m]) and not torch.equal(y1[m], y0[m])
 	for name in sorted(g1):
-		assert_close(g_rep[name], g1[name], f"new data: grad {name}", rel_max=2e-3, rel_fro=2e-3)
+		assert torch.equal(g_rep[name], g1[name]), f"new data: grad {name}"
 
 
 @pytest.mark.parametrize("loss_kind", ["fused", "torch"])
@@ -132,6 +132,7 @@ def test_captured_pipeline_step(loss_kind):
 		for a, b in zip(got_out, want_out):
 			assert torch.equal(a.cpu(), b.cpu())
 		for have, (n, p) in zip(got, pipe.named_parameters()):
+			# the embedding table's rows add with atomics (one per occurrence of a token), in no fixed order
 			assert_close(have, p.main_grad, f"replay {rep}: grad {n}", rel_max=2e-3, rel_fro=2e-3)
 
 
