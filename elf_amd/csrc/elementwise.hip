@@ -648,20 +648,59 @@ __global__ __launch_bounds__(256) void embedding_fwd_kernel(const int64_t* __res
 		store8(out + t * d + c, x);
 	}
 }
-// dtable[ids[t], :] += dx[t, :] in fp32 (tokens repeat within a micro-batch: atomics).
+// dtable[ids[t], :] += dx[t, :] in fp32.  One workgroup per token position.  The workgroup of a token's first
+// occurrence sums the rows of all its occurrences in ascending position and is the only writer of that table
+// row: no atomics, and the sums do not depend on the order in which workgroups run.  The other workgroups find an
+// earlier occurrence and leave (the ids are a few KiB and stay in cache).
 __global__ __launch_bounds__(256) void embedding_bwd_kernel(const int64_t* __restrict__ ids, const bf16_t* __restrict__ dx,
-                                                            float* __restrict__ dtable, int64_t T, int d, int V) {
+                                                            float* __restrict__ dtable, int T, int d, int V) {
+	__shared__ unsigned long long hit[4];
+	const int t = blockIdx.x;
+	const int64_t id = ids[t];
+	if (id < 0 || id >= V) return;
+	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+	for (int base = 0; base < t; base += 256) {
+		const int u = base + threadIdx.x;
+		if (__syncthreads_or(u < t && ids[u] == id)) return;
+	}
+	constexpr int MAXC = 4;  // d <= 8192: at most four 8-column chunks per lane
 	const int cpr = d / 8;
-	const int64_t n = T * cpr;
-	for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
-		const int64_t t = i / cpr;
-		const int c = (int)(i - t * cpr) * 8;
-		const int64_t id = ids[t];
-		if (id < 0 || id >= V) continue;
-		const Chunk x = load8(dx + t * d + c);
-		float* g = dtable + id * d + c;
+	float acc[MAXC][8];
 #pragma unroll
-		for (int j = 0; j < 8; j++) unsafeAtomicAdd(g + j, x.v[j]);
+	for (int i = 0; i < MAXC; i++)
+#pragma unroll
+		for (int k = 0; k < 8; k++) acc[i][k] = 0.f;
+	for (int base = t; base < T; base += 256) {
+		const int u = base + threadIdx.x;
+		const unsigned long long b = __ballot(u < T && ids[u] == id);
+		if (lane == 0) hit[wave] = b;
+		__syncthreads();
+		for (int w = 0; w < 4; w++) {
+			unsigned long long bits = hit[w];
+			while (bits) {
+				const int64_t row = base + w * 64 + (__ffsll(bits) - 1);
+				bits &= bits - 1;
+#pragma unroll
+				for (int i = 0; i < MAXC; i++) {
+					const int ch = threadIdx.x + i * 256;
+					if (ch < cpr) {
+						const Chunk x = load8(dx + row * d + ch * 8);
+#pragma unroll
+						for (int k = 0; k < 8; k++) acc[i][k] += x.v[k];
+					}
+				}
+			}
+		}
+		__syncthreads();
+	}
+#pragma unroll
+	for (int i = 0; i < MAXC; i++) {
+		const int ch = threadIdx.x + i * 256;
+		if (ch < cpr) {
+			float* g = dtable + id * d + ch * 8;
+#pragma unroll
+			for (int k = 0; k < 8; k++) g[k] += acc[i][k];
+		}
 	}
 }
 int embedding_fwd(const void* ids, const void* table, void* out, int64_t T, int d, int V, hipStream_t s) {
@@ -673,10 +712,10 @@ int embedding_fwd(const void* ids, const void* table, void* out, int64_t T, int 
 	return 0;
 }
 int embedding_bwd(const void* ids, const void* dx, void* dtable_f32, int64_t T, int d, int V, hipStream_t s) {
-	ELF_REQUIRE(ids && dx && dtable_f32 && T > 0 && V > 0 && d > 0 && d % 8 == 0, "embedding_bwd: bad argument (d must be a multiple of 8)");
+	ELF_REQUIRE(ids && dx && dtable_f32 && T > 0 && V > 0 && d > 0 && d % 8 == 0 && d <= 8192 && T < (int64_t(1) << 31),
+	            "embedding_bwd: bad argument (d must be a multiple of 8 and at most 8192)");
 	ProfScope prof(PROF_EMBED, 10.0 * T * d, s);
-	ELF_LAUNCH(embedding_bwd_kernel, dim3(ew_grid(T * (d / 8))), dim3(256), 0, s, (const int64_t*)ids, (const bf16_t*)dx,
-	                   (float*)dtable_f32, T, d, V);
+	ELF_LAUNCH(embedding_bwd_kernel, dim3((unsigned)T), dim3(256), 0, s, (const int64_t*)ids, (const bf16_t*)dx, (float*)dtable_f32, (int)T, d, V);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
 }

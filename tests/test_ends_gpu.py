@@ -33,8 +33,39 @@ def test_embedding_kernels_match_torch():
 	K.embedding_bwd_(ids, dx, dtab)
 	want = torch.full((V, d), 0.25, dtype=torch.float32, device="cuda").index_add_(0, ids, dx.float())
 	assert_close(dtab, want, "embedding dtable", rel_max=1e-5, rel_fro=1e-5)
+	again = torch.full((V, d), 0.25, dtype=torch.float32, device="cuda")
+	K.embedding_bwd_(ids, dx, again)
+	assert torch.equal(again, dtab), "a table row has one writer that adds its tokens in order: equal bits from run to run"
 	K.embedding_bwd_(bad, dx, dtab.zero_())
 	assert dtab.abs().sum().item() > 0  # out-of-range ids are skipped, the rest still lands
+
+
+@pytest.mark.parametrize("V,d,T", [(50, 4096, 1000), (3, 8192, 777), (128256, 1024, 8192)])
+def test_embedding_backward_ragged_sizes_and_heavy_repeats(V, d, T):
+	"""Token counts that are not multiples of the workgroup size, rows wider than one pass of the workgroup, a
+	vocabulary so small that every row collects hundreds of tokens: the sum in position order, exactly."""
+	from elf_amd import kernels as K
+
+	g = torch.Generator().manual_seed(V + d)
+	ids = torch.randint(0, V, (T,), generator=g).cuda()
+	dx = torch.randn(T, d, generator=g).to(torch.bfloat16).cuda()
+	start = torch.randn(V, d, generator=g).cuda()
+	got = start.clone()
+	K.embedding_bwd_(ids, dx, got)
+	# position order, row by row, as the kernel adds: the tokens' sum first, then the row's old value
+	touched = torch.unique(ids)
+	want = start.clone()
+	for tok in touched[:64].tolist():
+		acc = torch.zeros(d, device="cuda")
+		for t in (ids == tok).nonzero().flatten().tolist():
+			acc += dx[t].float()
+		want[tok] += acc
+		assert torch.equal(got[tok], want[tok]), f"row {tok}"
+	full = start.clone().index_add_(0, ids, dx.float())
+	assert_close(got, full, "embedding dtable", rel_max=1e-5, rel_fro=1e-5)
+	untouched = torch.ones(V, dtype=torch.bool, device="cuda")
+	untouched[touched] = False
+	assert torch.equal(got[untouched], start[untouched])
 
 
 def _end_stage(kind, vocab_in, vocab_out, final_norm, seed):
