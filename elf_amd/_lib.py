@@ -24,7 +24,8 @@ _SIGNATURES = {
 	"elf_norm_bwd_workspace_floats": (c_int64, [c_int, c_int]),
 	"elf_norm_bwd": (c_int, [c_int, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, _P]),
 	"elf_gemm_rope_bf16": (c_int, [c_int, c_int, c_int, _P, c_int64, _P, c_int64, _P, c_int64, _P, c_int, c_int, c_int, _P]),
-	"elf_colsum_bf16": (c_int, [_P, c_int64, _P, c_int64, c_int, _P]),
+	"elf_colsum_workspace_floats": (c_int64, [c_int64, c_int]),
+	"elf_colsum_bf16": (c_int, [_P, c_int64, _P, c_int64, c_int, _P, _P]),
 	"elf_norm_bwd_noalloc": (c_int, [c_int, _P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, _P]),
 	"elf_gelu_fwd": (c_int, [_P, _P, c_int64, _P]),
 	"elf_gelu_bwd": (c_int, [_P, _P, _P, c_int64, _P]),

@@ -65,8 +65,9 @@ int elf_scale_grads(void* acc_f32, void* out_bf16, int64_t n, float scale, void*
 int elf_add_bf16(const void* a, const void* b, void* out, int64_t n, void* stream) {
 	return elf::add_bf16(a, b, out, n, S_(stream));
 }
-int elf_colsum_bf16(const void* x, int64_t ld, void* out_f32, int64_t T, int N, void* stream) {
-	return elf::colsum_bf16(x, ld, out_f32, T, N, S_(stream));
+int64_t elf_colsum_workspace_floats(int64_t T, int N) { return elf::colsum_workspace_floats(T, N); }
+int elf_colsum_bf16(const void* x, int64_t ld, void* out_f32, int64_t T, int N, float* workspace, void* stream) {
+	return elf::colsum_bf16(x, ld, out_f32, T, N, workspace, S_(stream));
 }
 int elf_embedding_fwd(const void* ids, const void* table, void* out, int64_t T, int d, int V, void* stream) {
 	return elf::embedding_fwd(ids, table, out, T, d, V, S_(stream));

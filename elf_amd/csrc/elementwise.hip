@@ -590,9 +590,9 @@ int add_bf16(const void* a, const void* b, void* out, int64_t n, hipStream_t s) 
 // ------------------------------------------------------------------------------------------
 // Bias gradient of a split linear layer (elf/zb_utils.py:247-252: go.sum(0) added to bias.grad in
 // LinearDW.backward): out[c] += sum_t x[t, c] in fp32.  A workgroup owns 256 columns and one of gridDim.y
-// slices of the rows; its 8 row groups are folded through LDS and the slices meet in the accumulator
-// through fp32 atomics.
-__global__ __launch_bounds__(256) void colsum_kernel(const bf16_t* __restrict__ x, int64_t ld, float* __restrict__ out, int64_t T, int N) {
+// slices of the rows; its 8 row groups are folded through LDS and the slice's sums go to part[slice][c].  A second
+// kernel adds the slices in ascending order, one writer per column: equal bits from run to run.
+__global__ __launch_bounds__(256) void colsum_kernel(const bf16_t* __restrict__ x, int64_t ld, float* __restrict__ part, int64_t T, int N) {
 	__shared__ float red[8][256];
 	const int cl = threadIdx.x & 31, rg = threadIdx.x >> 5;
 	const int c0 = (blockIdx.x * 32 + cl) * 8;
@@ -612,16 +612,31 @@ __global__ __launch_bounds__(256) void colsum_kernel(const bf16_t* __restrict__ 
 		float t = 0.f;
 #pragma unroll
 		for (int r = 0; r < 8; r++) t += red[r][threadIdx.x];
-		unsafeAtomicAdd(out + c, t);
+		part[(int64_t)blockIdx.y * N + c] = t;
 	}
 }
-int colsum_bf16(const void* x, int64_t ld, void* out_f32, int64_t T, int N, hipStream_t s) {
-	ELF_REQUIRE(x && out_f32 && T > 0 && N > 0 && N % 8 == 0 && ld % 8 == 0 && ld >= N, "colsum: N and the row stride must be multiples of 8 (T=%lld N=%d ld=%lld)",
-	            (long long)T, N, (long long)ld);
+__global__ __launch_bounds__(256) void colsum_fold_kernel(const float* __restrict__ part, int slices, int N, float* __restrict__ out) {
+	const int c = blockIdx.x * 256 + threadIdx.x;
+	if (c >= N) return;
+	float t = 0.f;
+#pragma unroll 8
+	for (int sl = 0; sl < slices; sl++) t += part[(int64_t)sl * N + c];
+	out[c] += t;
+}
+static inline int colsum_slices(int64_t T, int N) {
 	const int col_blocks = (N + 255) / 256;
-	int64_t slices = (2048 + col_blocks - 1) / col_blocks;  // about eight workgroups per CU
+	int64_t slices = (1024 + col_blocks - 1) / col_blocks;  // about four workgroups per CU
+	if (slices > 64) slices = 64;
 	if (slices > (T + 7) / 8) slices = (T + 7) / 8;
-	ELF_LAUNCH(colsum_kernel, dim3(col_blocks, (unsigned)slices), dim3(256), 0, s, (const bf16_t*)x, ld, (float*)out_f32, T, N);
+	return (int)(slices < 1 ? 1 : slices);
+}
+int64_t colsum_workspace_floats(int64_t T, int N) { return T > 0 && N > 0 ? (int64_t)colsum_slices(T, N) * N : 0; }
+int colsum_bf16(const void* x, int64_t ld, void* out_f32, int64_t T, int N, float* workspace, hipStream_t s) {
+	ELF_REQUIRE(x && out_f32 && workspace && T > 0 && N > 0 && N % 8 == 0 && ld % 8 == 0 && ld >= N,
+	            "colsum: null pointer, or N and the row stride are not multiples of 8 (T=%lld N=%d ld=%lld)", (long long)T, N, (long long)ld);
+	const int col_blocks = (N + 255) / 256, slices = colsum_slices(T, N);
+	ELF_LAUNCH(colsum_kernel, dim3(col_blocks, (unsigned)slices), dim3(256), 0, s, (const bf16_t*)x, ld, workspace, T, N);
+	ELF_LAUNCH(colsum_fold_kernel, dim3(col_blocks), dim3(256), 0, s, (const float*)workspace, slices, N, (float*)out_f32);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
 }

@@ -88,7 +88,8 @@ int rope_apply(void* buf, const void* cs, int64_t T, int S, int ld, int n_heads,
 int scale_grads(void* acc_f32, void* out_bf16, int64_t n, float scale, hipStream_t s);
 int add_bf16(const void* a, const void* b, void* out, int64_t n, hipStream_t s);
 // out[c] (fp32) += sum over the T rows of x[t, c] (bf16 [T, N], row stride ld)
-int colsum_bf16(const void* x, int64_t ld, void* out_f32, int64_t T, int N, hipStream_t s);
+int64_t colsum_workspace_floats(int64_t T, int N);
+int colsum_bf16(const void* x, int64_t ld, void* out_f32, int64_t T, int N, float* workspace, hipStream_t s);
 // ids: int64 [T]; table bf16 [V, d]; dtable fp32 [V, d] (+=)
 int embedding_fwd(const void* ids, const void* table, void* out, int64_t T, int d, int V, hipStream_t s);
 int embedding_bwd(const void* ids, const void* dx, void* dtable_f32, int64_t T, int d, int V, hipStream_t s);

@@ -183,7 +183,9 @@ def colsum_(x, out_f32):
 	"""out_f32 [N] += x.sum(0) for x: bf16 [T, N]."""
 	_need(x, torch.bfloat16, "colsum.x")
 	_need(out_f32, torch.float32, "colsum.out")
-	_lib.check(_lib.load().elf_colsum_bf16(_ptr(x), x.stride(0), _ptr(out_f32), x.shape[0], x.shape[1], _stream()), "elf_colsum_bf16")
+	lib = _lib.load()
+	ws = torch.empty(max(1, lib.elf_colsum_workspace_floats(x.shape[0], x.shape[1])), dtype=torch.float32, device=x.device)
+	_lib.check(lib.elf_colsum_bf16(_ptr(x), x.stride(0), _ptr(out_f32), x.shape[0], x.shape[1], _ptr(ws), _stream()), "elf_colsum_bf16")
 	return out_f32
 
 

@@ -128,9 +128,12 @@ int elf_scale_grads(void* acc_f32, void* out_bf16, int64_t n, float scale, void*
 int elf_add_bf16(const void* a, const void* b, void* out, int64_t n, void* stream);
 
 /* out_f32[c] += sum over the T rows of x[t, c] (x: bf16 [T, N], row stride ld; N and ld multiples of 8).
+ * workspace: elf_colsum_workspace_floats(T, N) floats of partial sums, added by one writer per column in a fixed
+ * order (equal bits from run to run).
  * Replaces the bias gradient of LinearDW.backward, go.sum(0) added to bias.grad (elf/zb_utils.py:247-252),
  * with fp32 accumulation. */
-int elf_colsum_bf16(const void* x, int64_t ld, void* out_f32, int64_t T, int N, void* stream);
+int64_t elf_colsum_workspace_floats(int64_t T, int N);
+int elf_colsum_bf16(const void* x, int64_t ld, void* out_f32, int64_t T, int N, float* workspace, void* stream);
 
 /* Token embedding of a first pipeline stage: out[t, :] = table[ids[t], :] (ids: int64 [T], table: bf16
  * [V, d], d % 8 == 0; an id outside [0, V) gives a zero row) and its weight gradient dtable[ids[t], :] +=

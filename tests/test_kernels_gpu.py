@@ -371,3 +371,20 @@ def test_attention_fwd_bwd(K, cfg):
 	cs = K.rope_table(S, D, 5e5)
 	fused = K.attn_bwd(qkv, o, do, lse, B, S, Hq, Hkv, D, causal, rope_cs=cs)
 	assert torch.equal(fused, K.rope_apply_(dqkv.clone(), cs, S, Hq + Hkv, D, backward=True))
+
+
+@pytest.mark.parametrize("T,N,ld", [(8192, 768, 768), (1000, 2304, 2304), (7, 64, 128), (4096, 8, 8), (333, 4104, 4104)])
+def test_colsum_is_exact_to_rounding_and_repeatable(K, T, N, ld):
+	"""The bias gradient of a split linear layer: column sums of a bf16 [T, N] view (row stride ld) added to an fp32
+	accumulator, equal bits from run to run (one writer per column, slices added in a fixed order)."""
+	buf = _randn(T, ld, seed=91)
+	x = buf[:, :N]
+	start = torch.randn(N, device="cuda", generator=torch.Generator(device="cuda").manual_seed(92))
+	runs = []
+	for _ in range(3):
+		acc = start.clone()
+		K.colsum_(x, acc)
+		runs.append(acc)
+	assert torch.equal(runs[0], runs[1]) and torch.equal(runs[0], runs[2])
+	want = start.double() + x.double().sum(0)
+	assert ((runs[0].double() - want).abs().max() / want.abs().max()).item() <= 1e-5
