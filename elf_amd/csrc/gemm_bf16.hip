@@ -341,6 +341,18 @@ static int launch_epi(GemmArgs& g, int epi, int tile_cfg, hipStream_t stream) {
 	}
 }
 
+// Which direct-to-LDS tile a forward / input-gradient product runs on: 256 rows when 192 or more such tiles fill
+// the chip, else 128 rows (k-contiguous A) when 128 or more of those do, else neither (0).  A choice by estimated
+// rounds of workgroups x time per workgroup - 128-row tiles where the 256-row ones leave a mostly empty last round,
+// e.g. 8192 x 2304 x 768 - wins 4-11 % back to back on operands that stay cached and loses 3.6 % inside the
+// GPT-2-small stream, where they are cold and the narrower tile fetches B twice as often: not used.
+static int dma_tile_rows(bool a_t, int M, int N, int K) {
+	if (N % 256 != 0 || K % 64 != 0) return 0;
+	if (M % 256 == 0 && (int64_t)(M / 256) * (N / 256) >= 192) return 256;
+	if (M % 128 == 0 && !a_t && (int64_t)(M / 128) * (N / 256) >= 128) return 128;
+	return 0;
+}
+
 int gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda, const void* B, int64_t ldb,
               void* C, int64_t ldc, int epi, const void* R, int64_t ldr, int tile_cfg, int k_splits,
               hipStream_t stream) {
@@ -379,13 +391,15 @@ int gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda,
 	}
 	// Tile choice when the caller leaves it open: the direct-to-LDS 256x256 kernel whenever its
 	// tiles can fill the chip, the register-staged kernels (smaller tiles) otherwise.
-	if (tile_cfg <= 0 && M % 256 == 0 && N % 256 == 0) {
-		const int64_t tiles = (int64_t)(M / 256) * (N / 256);
+	if (tile_cfg <= 0 && epi == EPI_F32_ACC && M % 256 == 0 && N % 256 == 0 && K % 64 == 0) {
 		// weight gradients (long K, fp32 accumulate) also when the tiles are few: K is split instead
-		if (tiles >= 192 || (epi == EPI_F32_ACC && tiles >= 24 && K >= 4096)) tile_cfg = 7;
+		const int64_t tiles = (int64_t)(M / 256) * (N / 256);
+		if (tiles >= 192 || (tiles >= 24 && K >= 4096)) tile_cfg = 7;
 	}
-	// narrower outputs (e.g. N = 768 at M = 8192): 128x256 tiles of the same kernel fill the chip
-	if (tile_cfg <= 0 && !a_t && M % 128 == 0 && N % 256 == 0 && (int64_t)(M / 128) * (N / 256) >= 128) tile_cfg = 8;
+	if (tile_cfg <= 0 && epi != EPI_F32_ACC) {
+		const int rows = dma_tile_rows(a_t, M, N, K);
+		tile_cfg = rows == 256 ? 7 : rows == 128 ? 8 : tile_cfg;
+	}
 	if (tile_cfg == 7) {
 		int tail_tiles = -1;  // an explicit k_splits splits every tile
 		if (epi == EPI_F32_ACC && k_splits <= 0) {
@@ -424,8 +438,7 @@ int gemm_act_bf16(int act, int M, int F, int K, const void* A, int64_t lda, cons
 	int bm = 0;
 	if (act == ACT_SWIGLU && K % 64 == 0 && N % 256 == 0 && lda % 8 == 0 && ldw % 8 == 0 && ldpre >= N && ldout >= F && ldpre % 8 == 0 && ldout % 8 == 0 &&
 	    ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0 && ((uintptr_t)pre % 16) == 0 && ((uintptr_t)out % 16) == 0 && lda >= K && ldw >= K) {
-		if (M % 256 == 0 && (int64_t)(M / 256) * (N / 256) >= 192) bm = 256;
-		else if (M % 128 == 0 && (int64_t)(M / 128) * (N / 256) >= 128) bm = 128;
+		bm = dma_tile_rows(false, M, N, K);
 	}
 	if (bm) {
 		ProfScope prof(PROF_GEMM, 2.0 * M * N * K, stream);
@@ -440,7 +453,7 @@ int gemm_act_bf16(int act, int M, int F, int K, const void* A, int64_t lda, cons
 bool gemm_rope_fused(int M, int N, int K, int D) {
 	if (!(M > 0 && N > 0 && K > 0 && K % 64 == 0 && N % 256 == 0 && (D == 64 || D == 128))) return false;
 	// the tile choice gemm_bf16 makes for this shape
-	return (M % 256 == 0 && (int64_t)(M / 256) * (N / 256) >= 192) || (M % 128 == 0 && (int64_t)(M / 128) * (N / 256) >= 128);
+	return dma_tile_rows(false, M, N, K) != 0;
 }
 
 int gemm_rope_bf16(int M, int N, int K, const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, const void* cs,
@@ -451,7 +464,7 @@ int gemm_rope_bf16(int M, int N, int K, const void* A, int64_t lda, const void* 
 	    ((uintptr_t)W % 16) == 0 && ((uintptr_t)C % 16) == 0 && ((uintptr_t)cs % 16) == 0) {
 		// the rotation's arithmetic is not counted: the figure stays the GEMM's
 		ProfScope prof(PROF_GEMM, 2.0 * M * N * K, stream);
-		const int bm = (M % 256 == 0 && (int64_t)(M / 256) * (N / 256) >= 192) ? 256 : 128;
+		const int bm = dma_tile_rows(false, M, N, K);
 		return gemm_bf16_dma(0, 0, M, N, K, A, lda, W, ldw, C, ldc, EPI_BF16_ROPE, nullptr, 0, 1, 0, bm, stream, nullptr, 0, cs, S, n_rot_heads * D, D);
 	}
 	if (int rc = gemm_bf16(0, 0, M, N, K, A, lda, W, ldw, C, ldc, EPI_BF16, nullptr, 0, 0, 0, stream)) return rc;
