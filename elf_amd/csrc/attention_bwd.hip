@@ -208,8 +208,17 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(AttnBwdArgs a) {
 	const int g = lane >> 5, kl = lane & 31;
 	const int nkt = a.S / BKV;
 	const int npair = CAUSAL ? (nkt + 1) / 2 : nkt;
-	const int pair = blockIdx.x % npair;
-	const int bh = blockIdx.x / npair;
+	int pair = blockIdx.x % npair;
+	int bh = blockIdx.x / npair;
+	{
+		// all key-tile workgroups of a (batch, kv head) group on one XCD (workgroup w runs on XCD w % 8)
+		const int ngroups = (int)(gridDim.x / npair);
+		if (ngroups % 8 == 0) {
+			const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+			bh = xcd + 8 * (slot / npair);
+			pair = slot % npair;
+		}
+	}
 	const int hk = bh % a.Hkv, b = bh / a.Hkv;
 	const int G = a.Hq / a.Hkv;
 	const int64_t tok0 = (int64_t)b * a.S;
@@ -496,8 +505,17 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel_lone(AttnBwdArgs a) {
 	const int g = lane >> 5, kl = lane & 31;
 	const int nkt = a.S / BKV;
 	const int npair = CAUSAL ? (nkt + 1) / 2 : nkt;
-	const int pair = blockIdx.x % npair;
-	const int bh = blockIdx.x / npair;
+	int pair = blockIdx.x % npair;
+	int bh = blockIdx.x / npair;
+	{
+		// all key-tile workgroups of a (batch, kv head) group on one XCD (workgroup w runs on XCD w % 8)
+		const int ngroups = (int)(gridDim.x / npair);
+		if (ngroups % 8 == 0) {
+			const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+			bh = xcd + 8 * (slot / npair);
+			pair = slot % npair;
+		}
+	}
 	const int hk = bh % a.Hkv, b = bh / a.Hkv;
 	const int G = a.Hq / a.Hkv;
 	const int64_t tok0 = (int64_t)b * a.S;
