@@ -286,6 +286,52 @@ def vendor_gemm(w, seconds=1.5):
 	return {"seconds_per_leg": seconds, "gemms": rows, "sum_us": total}
 
 
+def vendor_attention(w, repeats=20):
+	"""The attention of one block at the workload's shape, forward and backward, through this library and through
+	torch's scaled_dot_product_attention (the vendor's flash attention), same values, back to back.  A yardstick only."""
+	import torch
+	import torch.nn.functional as F
+	from elf_amd import kernels as K
+
+	B, S, Hq, Hkv, D, causal = w["mb"], w["seq"], w["heads"], w["kv_heads"], w["head_dim"], w["causal"]
+	g = torch.Generator(device="cuda").manual_seed(3)
+	qkv = torch.randn(B * S, (Hq + 2 * Hkv) * D, device="cuda", generator=g).bfloat16()
+	do = torch.randn(B * S, Hq * D, device="cuda", generator=g).bfloat16()
+	flops_f = (2.0 if causal else 4.0) * B * Hq * S * S * D
+
+	def timed(fn):
+		for _ in range(3):
+			fn()
+		torch.cuda.synchronize()
+		t0 = time.perf_counter()
+		for _ in range(repeats):
+			fn()
+		torch.cuda.synchronize()
+		return (time.perf_counter() - t0) / repeats
+
+	o, lse = K.attn_fwd(qkv, B, S, Hq, Hkv, D, causal)
+	t_f = timed(lambda: K.attn_fwd(qkv, B, S, Hq, Hkv, D, causal))
+	t_b = timed(lambda: K.attn_bwd(qkv, o, do, lse, B, S, Hq, Hkv, D, causal))
+	out = {"shape": {"B": B, "S": S, "Hq": Hq, "Hkv": Hkv, "D": D, "causal": causal},
+	       "elf": {"fwd_us": t_f * 1e6, "fwd_tflops": flops_f / t_f / 1e12, "bwd_us": t_b * 1e6, "bwd_tflops": 2 * flops_f / t_b / 1e12}}
+	# [B, H, S, D] views of the same values for torch
+	q, k, v = (t.view(B, S, -1, D).transpose(1, 2).contiguous().requires_grad_(True)
+	           for t in (qkv[:, : Hq * D], qkv[:, Hq * D : (Hq + Hkv) * D], qkv[:, (Hq + Hkv) * D :]))
+	do4 = do.view(B, S, Hq, D).transpose(1, 2).contiguous()
+	try:
+		fwd = lambda: F.scaled_dot_product_attention(q, k, v, is_causal=causal, enable_gqa=Hq != Hkv)
+		t_vf = timed(fwd)
+
+		def both():
+			fwd().backward(do4)
+
+		t_vfb = timed(both)
+		out["vendor"] = {"fwd_us": t_vf * 1e6, "fwd_tflops": flops_f / t_vf / 1e12, "bwd_us": (t_vfb - t_vf) * 1e6, "bwd_tflops": 2 * flops_f / (t_vfb - t_vf) / 1e12}
+	except Exception as e:  # no fused kernel for this shape in this torch build
+		out["vendor"] = {"error": f"{type(e).__name__}: {e}"[:200]}
+	return out
+
+
 def main():
 	ap = argparse.ArgumentParser()
 	ap.add_argument("--gpus", type=int, default=1)
@@ -305,6 +351,9 @@ def main():
 	ap.add_argument("--vendor-gemm", action="store_true",
 	                help="also run the twelve GEMMs of one block back to back through this library and through torch.matmul (the vendor's "
 	                     "library), with power and clock, and report both under \"vendor_gemm\"")
+	ap.add_argument("--vendor-attention", action="store_true",
+	                help="also time the block's attention, forward and backward, through this library and through torch's scaled_dot_product_attention, "
+	                     "and report both under \"vendor_attention\"")
 	ap.add_argument("--calibration-copy", action="store_true",
 	                help="also launch one elf::add_kernel over 2 x 128 MiB in, 128 MiB out: a kernel of known HBM traffic to scale profiler byte counters with")
 	args = ap.parse_args()
@@ -447,6 +496,8 @@ def main():
 		out["hbm_ceiling"] = hbm_ceiling()
 	if args.vendor_gemm:
 		out["vendor_gemm"] = vendor_gemm(w)
+	if args.vendor_attention:
+		out["vendor_attention"] = vendor_attention(w)
 	if cpu_stats is not None:
 		out["cpu_baseline"] = cpu_stats
 	print(json.dumps(out))
