@@ -388,3 +388,24 @@ def test_colsum_is_exact_to_rounding_and_repeatable(K, T, N, ld):
 	assert torch.equal(runs[0], runs[1]) and torch.equal(runs[0], runs[2])
 	want = start.double() + x.double().sum(0)
 	assert ((runs[0].double() - want).abs().max() / want.abs().max()).item() <= 1e-5
+
+
+def test_split_k_gemms_on_two_streams_stay_correct(K):
+	"""Weight-gradient GEMMs launched concurrently on two streams share the turn counters of their split tiles; whatever
+	the interleaving, every sum must be the right one to fp32 rounding (a workgroup that finds its counter taken by
+	the other launch adds out of turn)."""
+	M, N, Kd = 768, 768, 8192
+	A = [_randn(Kd, M, seed=110 + i) for i in range(2)]
+	B = [_randn(Kd, N, seed=120 + i, scale=0.05) for i in range(2)]
+	ref = [A[i].float().t() @ B[i].float() for i in range(2)]
+	acc = [torch.zeros(M, N, device="cuda") for _ in range(2)]
+	streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+	torch.cuda.synchronize()
+	reps = 12
+	for _ in range(reps):
+		for i in range(2):
+			with torch.cuda.stream(streams[i]):
+				K.gemm(A[i], B[i], a_t=True, b_t=True, out=acc[i], epilogue=K.EPI_F32_ACC, k_splits=4, tile_cfg=7 if i == 0 else 8)
+	torch.cuda.synchronize()
+	for i in range(2):
+		assert ((acc[i] - reps * ref[i]).norm() / (reps * ref[i]).norm()).item() <= 1e-5
