@@ -176,6 +176,15 @@ __device__ __forceinline__ bf16x8 frag_t_at(const uint32_t (&o)[2], uint32_t imm
 // operands are reduction-major (dW): each of their fragments costs two transpose reads and an address.
 // NW = 4, RT = 2: 128x256 workgroup tile for outputs with too few 256x256 tiles to fill the chip.  One wave per SIMD
 // as well, so it runs the same interleaved loop (+35-40 % on the GPT-2-small shapes over read bursts).
+// Which of the `half` load pieces dealt over a half-step of `nm` MFMAs goes out after MFMA n (-1: none): piece k after
+// MFMA 2 * floor(k * (nm / 2) / half) - always an even one, because the fragment reads go out after the odd ones and a
+// read and a load behind the same MFMA do not fit under it.
+constexpr int piece_in_slot(int n, int nm, int half) {
+	for (int k = 0; k < half; k++)
+		if (2 * ((k * (nm / 2)) / half) == n) return k;
+	return -1;
+}
+
 // acc += a b as one in-place instruction on accumulator registers — the builtin leaves source and
 // destination accumulators untied, and when all 256 accumulator registers are live (128x128 wave tiles) the
 // allocator then copies accumulator tiles around inside the loop (192 copies per K slice).  Every
@@ -404,7 +413,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 					}
 				}
 			}
-			if constexpr (PIECE0 >= 0 && (n + 1) * HALF / NM != n * HALF / NM) issue_piece(sl, std::integral_constant<int, (PIECE0 < 0 ? 0 : PIECE0) + n * HALF / NM>{});
+			if constexpr (PIECE0 >= 0 && piece_in_slot(n, NM, HALF) >= 0) issue_piece(sl, std::integral_constant<int, (PIECE0 < 0 ? 0 : PIECE0) + (piece_in_slot(n, NM, HALF) < 0 ? 0 : piece_in_slot(n, NM, HALF))>{});
 			__builtin_amdgcn_sched_barrier(0);
 		});
 		if constexpr (NW == 8) __builtin_amdgcn_s_setprio(0);
