@@ -185,6 +185,16 @@ constexpr int piece_in_slot(int n, int nm, int half) {
 	return -1;
 }
 
+// every piece has a slot of its own within the half-step
+constexpr bool pieces_have_slots(int nm, int half) {
+	for (int k = 0; k < half; k++) {
+		int hits = 0;
+		for (int n = 0; n < nm; n++) hits += piece_in_slot(n, nm, half) == k;
+		if (hits != 1) return false;
+	}
+	return true;
+}
+
 // acc += a b as one in-place instruction on accumulator registers — the builtin leaves source and
 // destination accumulators untied, and when all 256 accumulator registers are live (128x128 wave tiles) the
 // allocator then copies accumulator tiles around inside the loop (192 copies per K slice).  Every
@@ -341,6 +351,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	// last fragments are in registers), so the same barrier frees that stage and the fetch of slice
 	// kt+2 starts a full slice ahead of its use.
 	constexpr int HALF = LOADS_PER_STAGE / 2;
+	static_assert(pieces_have_slots(RF * 4, HALF), "a half-step has too few even MFMA slots for half a slice's loads");
 	{
 		// slices 0 .. NST-2 whole and the first half of slice NST-1; slice 0 has to have landed
 		static_for<NST - 1>([&](auto sc) {
