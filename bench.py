@@ -89,6 +89,120 @@ def op_stream(w, sched=None):
 	return [op for op in schedule if op.block_id == BLOCK_ID]
 
 
+def make_block(w, stage):
+	"""The stage executor of block ``BLOCK_ID`` as Pipeline builds it: a stage that runs under a memory budget holds the lean stash."""
+	from elf_amd.execution import HipStageBlock
+	from elf_amd.partitioners.utils import sequential_signatures
+
+	placement = w.get("placement", PLACEMENT)
+	return HipStageBlock(stage, BLOCK_ID, placement, sequential_signatures(placement)[BLOCK_ID], mb_size=w["mb"], lean_stash=bool(w.get("memory_budget_mib")))
+
+
+def plan_stream(w, block):
+	"""(op stream of the workload, remat record or None).  Under a memory budget the stage is profiled on the native
+	executor, the remat ILP is solved for a pipeline of such stages and the block's rewritten stream is returned."""
+	import torch
+
+	if not w.get("memory_budget_mib"):
+		return op_stream(w), None
+	from elf_amd.registry import SCHEDULERS
+	from elf_amd.scheduling.ilp import RematScheduler, profile_stage, solve_remat
+
+	placement = w.get("placement", PLACEMENT)
+	stats, _ = profile_stage(block, n_iter=3)
+	# The budget is for everything this process holds on the device.  The ILP's memory model covers weights,
+	# fp32 gradient accumulators, the stage's fixed scratch (2 x Mparams) and the activations; what is resident
+	# beyond that comes off the budget it is given: the boundary tensors of all micro-batches (inputs and
+	# output gradients now, outputs and input gradients as the step produces them; a pipeline would pass them
+	# on one at a time) and the bf16 copies of the gradients that scale_grads leaves behind.
+	unmodelled_mib = max(0.0, torch.cuda.memory_allocated() / 2**20 + stats["Mworkspace"] - 2 * stats["Mparams"])
+	unmodelled_mib += w["n_mb"] * (stats["Minput"] + stats["Moutput"]) + sum(p.numel() * 2 for p in block._fused_w) / 2**20
+	t_ilp = time.perf_counter()
+	solution = solve_remat([stats] * len(placement), placement, SCHEDULERS[w["scheduler"]], w["n_mb"], w["memory_budget_mib"] - unmodelled_mib)
+	t_ilp = time.perf_counter() - t_ilp
+	remat = {
+		"memory_budget_mib": w["memory_budget_mib"], "unmodelled_resident_mib": unmodelled_mib, "ilp_seconds": t_ilp, "ilp_makespan_ms": solution["objective"],
+		"ilp_peak_mib_rank": solution["peak_mems"][placement[BLOCK_ID]],
+		"decisions_block": {k: int(sum(solution[k][BLOCK_ID])) for k in ("full_fwd", "activations_bwd", "full_bwd")},
+		"profile": {k: stats[k] for k in ("T", "M", "Mpeak", "Mpeak_ckpt", "Mparams", "Mba", "Mbg", "Minput")},
+	}
+	return op_stream(w, RematScheduler(SCHEDULERS[w["scheduler"]], solution)), remat
+
+
+def plain_stream(w):
+	"""(name, op stream) of the stream the workload's own stream must reproduce bit for bit on the same stage: the
+	scheduler without the remat rewrite, without the offload wrapper, or - for the split-backward ZB-H1 stream -
+	plain 1F1B, which runs the same F, B and W per micro-batch with every accumulation in the same order; a plain
+	1F1B workload is compared with a second run of itself."""
+	from elf_amd.registry import SCHEDULERS
+
+	if w.get("memory_budget_mib"):
+		return f"{w['scheduler']} without the remat rewrite", op_stream(w, SCHEDULERS[w["scheduler"]])
+	if w.get("offload"):
+		return f"{w['scheduler']} without activation offload", op_stream(w, SCHEDULERS[w["scheduler"]])
+	if w["scheduler"] != "1f1b":
+		return "1f1b", op_stream(w, SCHEDULERS["1f1b"])
+	return "a second run of the same stream", op_stream(w)
+
+
+def run_and_keep(block, engine, stream, mb_sizes, xs, dys):
+	"""One step of ``stream`` from zeroed accumulators with everything the stage produces kept: what SEND_FORWARD and
+	SEND_BACKWARD would ship per micro-batch, a copy of every fused fp32 gradient accumulator, the library's counters."""
+	import torch
+
+	block.set_boundary(inputs=xs, grads=dys, keep_sent=True)
+	block.zero_grad()
+	block.reset_peak()
+	torch.cuda.reset_peak_memory_stats()
+	before = block.mem_stats()
+	engine.train_step(None, None, None, stream, mb_sizes)
+	torch.cuda.synchronize()
+	mem = block.mem_stats()
+	peak = mem["peak_bytes"] + mem["workspace_bytes"] + torch.cuda.max_memory_allocated()  # before the copies below are made
+	kept = {"y": dict(block.sent_forward), "dx": dict(block.sent_backward), "grads": [g.clone() for g in block._fused_g], "mem": mem,
+	        "d2h": mem["d2h_bytes"] - before["d2h_bytes"], "h2d": mem["h2d_bytes"] - before["h2d_bytes"], "peak_bytes": peak}
+	block.set_boundary(inputs=xs, grads=dys)
+	return kept
+
+
+def compare_kept(a, b):
+	"""Bit equality of two ``run_and_keep`` records, and the largest difference relative to the tensor's largest
+	magnitude where they differ."""
+	import torch
+
+	out = {"micro_batches": len(a["y"]), "outputs_equal": True, "input_grads_equal": True, "weight_grads_equal": True, "max_rel_diff": 0.0}
+
+	def cmp(x, y, key):
+		if x.shape != y.shape or not torch.equal(x, y):
+			out[key] = False
+			d = (x.float() - y.float()).abs().max().item() / (y.float().abs().max().item() + 1e-30) if x.shape == y.shape else float("inf")
+			out["max_rel_diff"] = max(out["max_rel_diff"], d)
+
+	if set(a["y"]) != set(b["y"]) or set(a["dx"]) != set(b["dx"]) or len(a["grads"]) != len(b["grads"]):
+		return dict(out, outputs_equal=False, input_grads_equal=False, weight_grads_equal=False, max_rel_diff=float("inf"))
+	for m in a["y"]:
+		cmp(a["y"][m], b["y"][m], "outputs_equal")
+	for m in a["dx"]:
+		cmp(a["dx"][m], b["dx"][m], "input_grads_equal")
+	for x, y in zip(a["grads"], b["grads"]):
+		cmp(x, y, "weight_grads_equal")
+	return out
+
+
+def check_stream(w, block, engine, stream, mb_sizes, xs, dys):
+	"""The reference's own criterion, "the pipeline gives what the plain model gives" (benchmarks/benchmark_utils.py:
+	215-292), at the workload's full size: the workload's stream and its plain counterpart (``plain_stream``) run on
+	the same stage from the same boundary tensors and must agree bit for bit in every stage output, every input
+	gradient and every accumulated weight gradient."""
+	name, plain = plain_stream(w)
+	got = run_and_keep(block, engine, stream, mb_sizes, xs, dys)
+	want = run_and_keep(block, engine, plain, mb_sizes, xs, dys)
+	out = compare_kept(got, want)
+	out.update({"against": name, "peak_bytes": got["peak_bytes"], "plain_peak_bytes": want["peak_bytes"], "d2h_bytes": got["d2h"], "h2d_bytes": got["h2d"]})
+	out["ok"] = bool(out["outputs_equal"] and out["input_grads_equal"] and out["weight_grads_equal"] and got["d2h"] == got["h2d"])
+	return out
+
+
 def cpu_baseline(w, stage_module, repeats=3):
 	"""Oracle stage on the host cores: F, B, W of ONE micro-batch through ONE block, fp32; one untimed
 	warm-up pass, then the median of ``repeats`` timed passes."""
@@ -354,6 +468,9 @@ def main():
 	ap.add_argument("--vendor-attention", action="store_true",
 	                help="also time the block's attention, forward and backward, through this library and through torch's scaled_dot_product_attention, "
 	                     "and report both under \"vendor_attention\"")
+	ap.add_argument("--check", action="store_true",
+	                help="after the timed region run the workload's stream and its plain counterpart (no remat rewrite / no offload / 1F1B for ZB-H1) once "
+	                     "each on the same stage and report under \"check\" whether every output, input gradient and weight gradient agrees bit for bit")
 	ap.add_argument("--calibration-copy", action="store_true",
 	                help="also launch one elf::add_kernel over 2 x 128 MiB in, 128 MiB out: a kernel of known HBM traffic to scale profiler byte counters with")
 	args = ap.parse_args()
@@ -363,8 +480,7 @@ def main():
 
 	import torch
 	from elf_amd import _lib
-	from elf_amd.execution import Engine, HipStageBlock
-	from elf_amd.partitioners.utils import sequential_signatures
+	from elf_amd.execution import Engine
 	from elf_amd.synthetic import make_boundary
 
 	if not torch.cuda.is_available():
@@ -379,35 +495,10 @@ def main():
 	if not args.no_cpu_baseline:
 		cpu_stats = cpu_baseline(w, stage)
 	placement = w.get("placement", PLACEMENT)
-	# as Pipeline does: a stage that runs under a memory budget holds the lean stash
-	block = HipStageBlock(stage, BLOCK_ID, placement, sequential_signatures(placement)[BLOCK_ID], mb_size=w["mb"], lean_stash=bool(w.get("memory_budget_mib")))
+	block = make_block(w, stage)
 	xs, dys = make_boundary(w["mb"], w["seq"], w["d"], w["n_mb"], seed=1, device="cuda")
 	block.set_boundary(inputs=xs, grads=dys)
-	remat = None
-	if w.get("memory_budget_mib"):
-		from elf_amd.registry import SCHEDULERS
-		from elf_amd.scheduling.ilp import RematScheduler, profile_stage, solve_remat
-
-		stats, _ = profile_stage(block, n_iter=3)
-		# The budget is for everything this process holds on the device.  The ILP's memory model covers weights,
-		# fp32 gradient accumulators, the stage's fixed scratch (2 x Mparams) and the activations; what is resident
-		# beyond that comes off the budget it is given: the boundary tensors of all micro-batches (inputs and
-		# output gradients now, outputs and input gradients as the step produces them; a pipeline would pass them
-		# on one at a time) and the bf16 copies of the gradients that scale_grads leaves behind.
-		unmodelled_mib = max(0.0, torch.cuda.memory_allocated() / 2**20 + stats["Mworkspace"] - 2 * stats["Mparams"])
-		unmodelled_mib += w["n_mb"] * (stats["Minput"] + stats["Moutput"]) + sum(p.numel() * 2 for p in block._fused_w) / 2**20
-		t_ilp = time.perf_counter()
-		solution = solve_remat([stats] * len(placement), placement, SCHEDULERS[w["scheduler"]], w["n_mb"], w["memory_budget_mib"] - unmodelled_mib)
-		t_ilp = time.perf_counter() - t_ilp
-		remat = {
-			"memory_budget_mib": w["memory_budget_mib"], "unmodelled_resident_mib": unmodelled_mib, "ilp_seconds": t_ilp, "ilp_makespan_ms": solution["objective"],
-			"ilp_peak_mib_rank": solution["peak_mems"][placement[BLOCK_ID]],
-			"decisions_block": {k: int(sum(solution[k][BLOCK_ID])) for k in ("full_fwd", "activations_bwd", "full_bwd")},
-			"profile": {k: stats[k] for k in ("T", "M", "Mpeak", "Mpeak_ckpt", "Mparams", "Mba", "Mbg", "Minput")},
-		}
-		stream = op_stream(w, RematScheduler(SCHEDULERS[w["scheduler"]], solution))
-	else:
-		stream = op_stream(w)
+	stream, remat = plan_stream(w, block)
 	engine = Engine([block])
 	mb_sizes = [w["mb"]] * w["n_mb"]
 
@@ -500,7 +591,11 @@ def main():
 		out["vendor_attention"] = vendor_attention(w)
 	if cpu_stats is not None:
 		out["cpu_baseline"] = cpu_stats
+	if args.check:
+		out["check"] = check_stream(w, block, engine, stream, mb_sizes, xs, dys)
 	print(json.dumps(out))
+	if args.check and not out["check"]["ok"]:
+		sys.exit(3)
 
 
 if __name__ == "__main__":

@@ -105,6 +105,11 @@ int elf_attn_bwd_rope(const void* q, const void* k, const void* v, const void* o
 
 int elf_hbm_probe(int mode, const void* src, void* dst, int64_t bytes, void* stream) { return elf::hbm_probe(mode, src, dst, bytes, S_(stream)); }
 
+int elf_gemm_turn_giveups(uint64_t* out) {
+	if (!out) return -1;
+	return elf::gemm_turn_giveups(out);
+}
+
 void elf_prof_enable(int on) { elf::prof_enable(on); }
 int elf_prof_collect(int kind, double* total_ms, double* total_work) {
 	if (kind < 0 || kind >= elf::PROF_COUNT) return -1;

@@ -8,6 +8,7 @@
 // (benchmarks/models/simple.py:44-52 GELU FFN, :444-445 LayerNorm, :460/:466 residual adds;
 // elf/execution/block.py:518-527 scale_grads).  RMSNorm, RoPE and SwiGLU have no reference
 // module; their definitions are the textbook ones stated next to each kernel.
+#include <atomic>
 #include <mutex>
 
 #include "common.h"
@@ -353,7 +354,7 @@ int norm_bwd(int kind, const void* dy, const void* x, const void* gamma, const v
 constexpr int64_t NORM_BWD_SCRATCH_FLOATS = (int64_t)1024 * 2 * 8192;
 static __device__ __align__(256) float scratch[NORM_BWD_SCRATCH_FLOATS];
 constexpr int MAX_DEVICES = 64;
-static float* scratch_ptr[MAX_DEVICES] = {};
+static std::atomic<float*> scratch_ptr[MAX_DEVICES] = {};  // written once per device under the mutex, read lock-free
 static std::mutex scratch_mutex;
 
 int norm_bwd_scratch_prepare() {
@@ -361,11 +362,11 @@ int norm_bwd_scratch_prepare() {
 	ELF_CHECK_HIP(hipGetDevice(&dev));
 	ELF_REQUIRE(dev >= 0 && dev < MAX_DEVICES, "norm_bwd_noalloc: device index %d out of range", dev);
 	std::lock_guard<std::mutex> lock(scratch_mutex);
-	if (!scratch_ptr[dev]) {
+	if (!scratch_ptr[dev].load(std::memory_order_acquire)) {
 		float* p = nullptr;
 		ELF_CHECK_HIP(hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch)));
 		ELF_REQUIRE(p != nullptr, "norm_bwd_noalloc: no device address for the scratch array");
-		scratch_ptr[dev] = p;
+		scratch_ptr[dev].store(p, std::memory_order_release);
 	}
 	return 0;
 }
@@ -380,11 +381,14 @@ int norm_bwd_noalloc(int kind, const void* dy, const void* x, const void* gamma,
 	int dev = -1;
 	ELF_CHECK_HIP(hipGetDevice(&dev));
 	ELF_REQUIRE(dev >= 0 && dev < MAX_DEVICES, "norm_bwd_noalloc: device index %d out of range", dev);
-	if (!scratch_ptr[dev]) {
+	float* ptr = scratch_ptr[dev].load(std::memory_order_acquire);
+	if (!ptr) {
+		// first call on this device: the address lookup (no allocation; the array is part of the loaded code object)
 		if (int rc = norm_bwd_scratch_prepare()) return rc;
+		ptr = scratch_ptr[dev].load(std::memory_order_acquire);
 	}
 	// every workgroup writes its whole partial row before the fold reads it: nothing has to start at zero
-	return norm_bwd_launch(kind, dy, x, gamma, stats, dres, dx, dgamma, dbeta, scratch_ptr[dev], T, d, s);
+	return norm_bwd_launch(kind, dy, x, gamma, stats, dres, dx, dgamma, dbeta, ptr, T, d, s);
 }
 
 // ------------------------------------------------------------------------------------------

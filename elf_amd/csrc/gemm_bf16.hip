@@ -25,12 +25,26 @@ constexpr int BK = 64;
 // turn counters of split tiles (see gemm_kernel)
 constexpr int TURN_RS_SLOTS = 4096;
 static __device__ uint32_t turn_rs[TURN_RS_SLOTS];
+// polls of ~1 us: about a millisecond, several times a predecessor's epilogue; a workgroup that uses them up is counted
+constexpr int TURN_RS_SPIN_LIMIT = 1 << 10;
+static __device__ unsigned int turn_rs_giveups;
 
 // One sequence of tags for every launch of every GEMM kernel that splits tiles: a counter value left behind by any
 // earlier launch then never equals a value a later launch waits for.
 uint32_t next_turn_tag() {
 	static std::atomic<uint32_t> launch_tag{0};
 	return (launch_tag.fetch_add(1) % 0xFFFFFFu) + 1;
+}
+int dma_turn_giveups(uint64_t* out);  // gemm_dma.hip
+// Split-K workgroups / waves (both GEMM kernel families, this device) that stopped waiting for their turn and added out
+// of turn since the library was loaded: the sums are right, only bit-reproducibility lapsed for those launches.
+int gemm_turn_giveups(uint64_t* out) {
+	unsigned int n = 0;
+	uint64_t d = 0;
+	ELF_CHECK_HIP(hipMemcpyFromSymbol(&n, HIP_SYMBOL(turn_rs_giveups), sizeof(n)));
+	if (int rc = dma_turn_giveups(&d)) return rc;
+	*out = d + n;
+	return 0;
 }
 constexpr int PAD_R = 8;    // elements of padding per row of an "R" tile ([row][BK+8])
 constexpr int PAD_T = 16;   // elements of padding per row of a "T" tile ([k][rows+16])
@@ -162,8 +176,10 @@ __global__ __launch_bounds__(WR* WC * 64) void gemm_kernel(GemmArgs g) {
 	auto take_turn = [&]() {
 		if (g.k_splits > 1 && g.turn_tag) {
 			if (tid == 0 && ksplit > 0) {
-				for (int spin = 0; spin < (1 << 15) && __hip_atomic_load(my_turn, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != turn_want; spin++)
-					__builtin_amdgcn_s_sleep(4);
+				int spin = 0;
+				for (; spin < TURN_RS_SPIN_LIMIT && __hip_atomic_load(my_turn, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != turn_want; spin++)
+					__builtin_amdgcn_s_sleep(8);
+				if (spin >= TURN_RS_SPIN_LIMIT) atomicAdd(&turn_rs_giveups, 1u);
 			}
 			__syncthreads();
 		}
@@ -364,6 +380,8 @@ int gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda,
 	ELF_REQUIRE(lda >= (a_t ? M : K) && ldb >= (b_t ? N : K) && ldc >= N, "gemm: leading dimension too small");
 	// ldr == 0: R is one row of N values added to every row of C (the bias of a linear layer)
 	ELF_REQUIRE(epi != EPI_BF16_RESID || (R != nullptr && (ldr >= N || ldr == 0)), "gemm: residual epilogue needs R");
+	// the turn counters of split tiles hold the split index in 8 bits next to the launch tag
+	ELF_REQUIRE(k_splits <= 255, "gemm: k_splits must be at most 255 (got %d)", k_splits);
 	ProfScope prof(PROF_GEMM, 2.0 * M * N * K, stream);
 	GemmArgs g;
 	g.A = (const bf16_t*)A;

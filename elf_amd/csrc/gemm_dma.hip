@@ -83,7 +83,12 @@ struct Args {
 // predecessor is through with that strip and the splits of a tile overlap except for about one strip.
 constexpr int TURN_TILES = 4096, TURN_PER_TILE = 16;
 static __device__ uint32_t turn[TURN_TILES * TURN_PER_TILE];
-constexpr int TURN_SPIN_LIMIT = 1 << 15;  // polls of ~1 us: far beyond the length of a predecessor's epilogue
+// polls of ~1 us each: about a millisecond in all, several times what a predecessor's epilogue takes (the splits of a
+// tile start together and run equal K ranges).  One budget per wave for the whole epilogue; a wave that uses it up is
+// counted in turn_giveups (gemm_turn_giveups() reads it) and adds out of turn from then on.
+constexpr int TURN_SPIN_LIMIT = 1 << 10;
+static __device__ unsigned int turn_giveups;
+__device__ __forceinline__ void note_turn_giveup() { atomicAdd(&turn_giveups, 1u); }
 
 // Byte offsets (relative to the tile origin of the current K slice) of the 16-byte chunks this
 // lane fetches for one operand (< 2^31: 256 rows of at most 64 K elements).  "R" tiles are
@@ -287,10 +292,18 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 		// a split without a K range of its own still takes and passes its turn on every strip
 		if (splits > 1 && g.turn_tag && lane == 0) {
 			const uint32_t want = (g.turn_tag << 8) | (uint32_t)ksplit;
+			int patience = TURN_SPIN_LIMIT;
 			for (int i = 0; i < RT; i++) {
 				uint32_t* t = turn + turn_slot * TURN_PER_TILE + wave * RT + i;
-				for (int spin = 0; ksplit > 0 && spin < TURN_SPIN_LIMIT && __hip_atomic_load(t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != want; spin++)
+				int spin = 0;
+				for (; ksplit > 0 && spin < patience && __hip_atomic_load(t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != want; spin++)
 					__builtin_amdgcn_s_sleep(8);
+				if (ksplit > 0 && spin >= patience) {
+					if (patience > 0) note_turn_giveup();
+					patience = 0;
+				} else {
+					patience -= spin;
+				}
 				__hip_atomic_store(t, want + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 			}
 		}
@@ -607,7 +620,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 					for (; spin < turn_patience && __hip_atomic_load(my_turn, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != want; spin++)
 						__builtin_amdgcn_s_sleep(8);
 					// a wave that gave up once (its counters are shared with a concurrent launch) does not wait again
-					if (spin >= turn_patience) turn_patience = 0;
+					if (spin >= turn_patience) {
+						if (turn_patience > 0 && lane == 0) note_turn_giveup();
+						turn_patience = 0;
+					} else {
+						turn_patience -= spin;
+					}
 				}
 				// several workgroups add into this tile: fp32 atomics, one scalar per lane so that a wave
 				// instruction covers two whole 128-byte rows of 32 columns (16 bytes per lane would touch a
@@ -686,6 +704,14 @@ static int launch_epi(const Args& a, int epi, hipStream_t stream) {
 }
 
 }  // namespace dma
+
+// Waves of this file's kernels that stopped waiting for their turn since the library was loaded (this device).
+int dma_turn_giveups(uint64_t* out) {
+	unsigned int n = 0;
+	ELF_CHECK_HIP(hipMemcpyFromSymbol(&n, HIP_SYMBOL(dma::turn_giveups), sizeof(n)));
+	*out = n;
+	return 0;
+}
 
 // Arguments are validated by gemm_bf16() before it dispatches here.
 int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda, const void* B, int64_t ldb, void* C,

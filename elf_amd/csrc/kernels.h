@@ -46,6 +46,10 @@ int gemm_rope_bf16(int M, int N, int K, const void* A, int64_t lda, const void* 
 // Tag of one GEMM launch whose tiles are split along K (24 bits, never 0, different from launch to launch); see the
 // turn counters in gemm_dma.hip and gemm_bf16.hip.
 uint32_t next_turn_tag();
+// Waves / workgroups of split-K launches on the current device that used up their bounded wait for their turn and added
+// out of turn (right sums, rounding order not fixed) since the library was loaded.  Synchronous (one 4-byte copy each
+// from two device counters).
+int gemm_turn_giveups(uint64_t* out);
 
 enum Activation { ACT_GELU = 0, ACT_SWIGLU = 1 };
 // Up-projection of the MLP with its activation: pre = A W^T (A [M, K], W [N, K], N = F for GELU and 2F =

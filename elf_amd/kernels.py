@@ -50,6 +50,15 @@ def gemm(a, b, *, a_t=False, b_t=False, out=None, epilogue=EPI_BF16, residual=No
 	return out
 
 
+def gemm_turn_giveups():
+	"""Waves of split-K GEMM launches on the current device that added out of turn since the library was loaded."""
+	import ctypes
+
+	n = ctypes.c_uint64()
+	_lib.check(_lib.load().elf_gemm_turn_giveups(ctypes.byref(n)), "elf_gemm_turn_giveups")
+	return n.value
+
+
 ACT_GELU, ACT_SWIGLU = 0, 1
 
 

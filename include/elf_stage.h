@@ -34,8 +34,9 @@ int elf_abi_version(void);
  *             added to every row of C, the bias of nn.Linear);
  *             2 C(fp32) += acc; 3 C(fp32) = acc.
  *   tile_cfg = 0 picks a tile shape from M,N (1: 256x256, 2: 128x128, 3: 64x64, 5: 256x128 register-staged;
- *   7: 256x256 with direct-to-LDS loads; 8: 128x256 with direct-to-LDS loads, a_t = 0 only);
- *   k_splits = 0 picks a K split (epilogue 2 only).
+ *   7: 256x256 with direct-to-LDS loads; 8: 128x256 with direct-to-LDS loads: a_t = 1 is accepted only together with
+ *   b_t = 1, and k_splits is honoured for epilogue 2);
+ *   k_splits = 0 picks a K split (epilogue 2 only; at most 255).
  * Replaces: F.linear in LinearDX.forward (elf/zb_utils.py:20)            -> a_t=0,b_t=0
  *           torch.mm(grad_output, weight) in LinearDX.backward (:34-37)  -> a_t=0,b_t=1
  *           torch.mm(go.t(), inp) + weight.grad.add_ in LinearDW.backward (:238-244) -> a_t=1,b_t=1, epilogue 2
@@ -43,6 +44,14 @@ int elf_abi_version(void);
 int elf_gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda, const void* B,
                   int64_t ldb, void* C, int64_t ldc, int epilogue, const void* R, int64_t ldr,
                   int tile_cfg, int k_splits, void* stream);
+/* Epilogue 2 with a split K: the workgroups that share a tile add their parts in the order of their K ranges (turn
+ * counters in device memory, tagged per launch), so the fp32 sums are bit-identical from run to run.  The counters are
+ * shared by every stream of the process: split-K launches that overlap in time on two streams can make a wave wait for a
+ * turn that is not its launch's; the wait is bounded (about a millisecond), after which the wave adds out of turn - still
+ * the right sum, but its rounding order is no longer fixed.  *out receives how many waves did so on the current device
+ * since the library was loaded (0 as long as split-K launches do not overlap).  Synchronous.  No counterpart in the
+ * reference (torch.mm's split-K is not reproducible either way). */
+int elf_gemm_turn_giveups(uint64_t* out);
 
 /* The MLP's up-projection with its activation: pre = A W^T with A [M, K] and W [N, K], both k contiguous;
  * act 0 (GELU): N = F, out[M, F] = gelu(pre); act 1 (SwiGLU): N = 2F, W = [gate rows; up rows],
@@ -197,8 +206,12 @@ int elf_attn_bwd_rope(const void* q, const void* k, const void* v, const void* o
  * The caller (torch) owns the boundary tensors X, Y, dY, dX, the weights and the fp32 gradient
  * accumulators; the library owns the per-micro-batch activation stash, the W stash (input X and
  * output gradient dY of every linear layer), temporaries, the pinned-host arena and the two side
- * streams of activation offload.  All calls for one stage come from one host thread and use one
- * stream; the external X of a micro-batch must stay valid until its B (and until its recompute
+ * streams of activation offload.  All calls for one stage come from one host thread and use ONE
+ * stream for the stage's whole life (the offload copies, the release of pinned blocks and the reuse of
+ * pooled device blocks are ordered against that stream only; a caller that must change streams
+ * synchronises the device first).  The fp32 gradient accumulators, too, are updated by plain
+ * read-modify-writes with one writer per element: two streams must not accumulate into the same
+ * gradient buffer at the same time.  The external X of a micro-batch must stay valid until its B (and until its recompute
  * ops), the external dY until its W. */
 typedef struct elf_stage elf_stage_t;
 

@@ -199,6 +199,19 @@ def test_reference_small_configuration_through_pipeline(loss_kind, scheduler, pl
 	logits = ref_last(ref_first(ids))
 	want_loss = F.cross_entropy(logits.view(-1, V), tgt.view(-1), reduction="sum") / (S * mb * nmb)
 	want_loss.backward()
+	# the same model in the reference's own arithmetic (bf16 modules under PyTorch autograd): how far bf16 itself is from
+	# the fp32 truth per parameter gradient.  Every gradient meets rel 2e-2 of its largest magnitude; the relative
+	# Frobenius bound is 1e-2 or 1.25 x PyTorch's bf16 error, whichever is larger (the query / key projections of the
+	# deeper blocks sit at 1.1-1.2 % in PyTorch's bf16 as well: four blocks of roundings in front of a softmax).
+	bf_first, bf_last = copy.deepcopy(first).cuda(), copy.deepcopy(last).cuda()
+	(F.cross_entropy(bf_last(bf_first(ids)).float().view(-1, V), tgt.view(-1), reduction="sum") / (S * mb * nmb)).backward()
+	fro_bound = {}
+	for tag, bf_mod, ref_mod in (("first", bf_first, ref_first), ("last", bf_last, ref_last)):
+		ref_params = dict(ref_mod.named_parameters())
+		for name, p in bf_mod.named_parameters():
+			r = ref_params[name].grad.double()
+			fro_bound[tag, name] = max(1e-2, 1.25 * ((p.grad.double() - r).norm() / (r.norm() + 1e-12)).item())
+	del bf_first, bf_last
 
 	pipe = Pipeline([first, last], ids[:mb], scheduler=scheduler, partitioner=False, placement=placement, all_ranks=len(set(placement)) > 1)
 	pipe.zero_grad()
@@ -218,11 +231,11 @@ def test_reference_small_configuration_through_pipeline(loss_kind, scheduler, pl
 	assert len(result) == nmb and tuple(result[0].shape) == (mb, S, V)
 	assert_close(torch.cat([r.float() for r in result]), logits.detach(), "logits")
 	assert abs(float(loss) - float(want_loss.detach())) <= 1e-2 * float(want_loss.detach())
-	for mod, ref_mod in ((first, ref_first), (last, ref_last)):
+	for tag, mod, ref_mod in (("first", first, ref_first), ("last", last, ref_last)):
 		ref_params = dict(ref_mod.named_parameters())
 		for name, p in mod.named_parameters():
-			assert_close(p.main_grad, ref_params[name].grad, f"grad {name}", rel_max=3e-2, rel_fro=2e-2)
-			assert_close(p.grad, ref_params[name].grad, f"bf16 grad {name}", rel_max=4e-2, rel_fro=2e-2)
+			assert_close(p.main_grad, ref_params[name].grad, f"grad {tag}.{name}", rel_fro=fro_bound[tag, name])
+			assert_close(p.grad, ref_params[name].grad, f"bf16 grad {tag}.{name}", rel_fro=fro_bound[tag, name])
 
 
 def test_memory_budget_with_first_and_last_stage():

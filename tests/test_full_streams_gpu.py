@@ -1,0 +1,136 @@
+"""The full operation streams the benchmark times, at full size, checked the way the reference checks a pipeline:
+"what comes out equals what the plain model gives" (benchmarks/benchmark_utils.py:215-292).
+
+Every variant of the stage path (remat rewrite, activation offload, split backward) is built to reproduce the plain
+F -> B -> W sequence bit for bit, so each full stream is run once next to its plain counterpart on the same stage
+and from the same boundary tensors, and every stage output, every input gradient and every accumulated fp32 weight
+gradient is compared with ``torch.equal``:
+
+  llama3_8b_remat     8 blocks, 1 x 8192 tokens x 16 micro-batches, lean stash, the stream rewritten by the remat ILP
+                      under a 48 GB budget (the benchmark's own profile -> solve -> rewrite)  vs  plain 1F1B;
+                      the measured peak stays under the budget
+  llama3_70b_offload  2 blocks at the 70B shape, 1 x 8192 tokens x 8 micro-batches, every micro-batch offloaded and
+                      prefetched  vs  1F1B without offload; bytes to the host == bytes back
+  llama3_8b_zbh1      4 blocks, 2 x 4096 tokens x 16 micro-batches, ZB-H1 (W deferred)  vs  1F1B; and the sum over the
+                      16 micro-batches of the first block's weight gradients against the oracle stage in fp32 on the
+                      GPU driven through the same 16 micro-batches
+
+The streams come from bench.py (``plan_stream`` / ``plain_stream``), the functions its ``--check`` flag runs."""
+
+import gc
+
+import pytest
+import torch
+
+from tests.helpers import assert_close_dev, cfg_from_stage, oracle_params_from_stage, product_grads
+
+pytestmark = pytest.mark.gpu
+
+
+def _setup(name):
+	import bench
+	from elf_amd.execution import Engine
+	from elf_amd.synthetic import make_boundary
+
+	w = dict(bench.WORKLOADS[name])
+	print(f"[case] full stream {name}: {w}", flush=True)
+	stage = bench.build_stage(w)
+	block = bench.make_block(w, stage)
+	xs, dys = make_boundary(w["mb"], w["seq"], w["d"], w["n_mb"], seed=1, device="cuda")
+	block.set_boundary(inputs=xs, grads=dys)
+	return bench, w, stage, block, Engine([block]), xs, dys, [w["mb"]] * w["n_mb"]
+
+
+def _free():
+	gc.collect()
+	torch.cuda.empty_cache()
+
+
+def _assert_equal(out, name):
+	print(f"[check] {name}: {out}", flush=True)
+	assert out["micro_batches"] > 0
+	assert out["outputs_equal"], f"{name}: stage outputs differ from the plain stream's (max rel diff {out['max_rel_diff']:.3g})"
+	assert out["input_grads_equal"], f"{name}: input gradients differ from the plain stream's (max rel diff {out['max_rel_diff']:.3g})"
+	assert out["weight_grads_equal"], f"{name}: accumulated weight gradients differ from the plain stream's (max rel diff {out['max_rel_diff']:.3g})"
+
+
+def test_remat_stream_equals_plain_1f1b_and_fits_the_budget():
+	bench, w, stage, block, engine, xs, dys, mb_sizes = _setup("llama3_8b_remat")
+	stream, remat = bench.plan_stream(w, block)
+	decisions = remat["decisions_block"]
+	print(f"[remat] decisions {decisions}, ILP peak {remat['ilp_peak_mib_rank']:.0f} MiB, unmodelled {remat['unmodelled_resident_mib']:.0f} MiB", flush=True)
+	assert sum(decisions.values()) > 0, "a 48 GB budget forces recomputation at this shape"
+	assert [str(op) for op in stream] != [str(op) for op in bench.plain_stream(w)[1]], "the ILP's decisions rewrite the stream"
+	out = bench.check_stream(w, block, engine, stream, mb_sizes, xs, dys)
+	_assert_equal(out, "llama3_8b_remat")
+	assert out["ok"]
+	# the rewritten stream holds less than the plain one and fits the budget it was solved for.  The boundary tensors
+	# kept for the comparison (what SEND_* shipped, 2 x 16 x 64 MiB) are part of the measured peak although a pipeline
+	# would have passed them on; they are inside "unmodelled" only as allocations, so they are taken off here.
+	kept_for_check = 2 * w["n_mb"] * xs[0].numel() * 2
+	budget = w["memory_budget_mib"] * 2**20
+	assert out["peak_bytes"] < out["plain_peak_bytes"]
+	assert out["peak_bytes"] - kept_for_check <= budget, f"peak {out['peak_bytes'] / 2**30:.2f} GiB over the budget of {budget / 2**30:.2f} GiB"
+	del block, engine, stage
+	_free()
+
+
+def test_offloaded_stream_equals_plain_1f1b():
+	bench, w, stage, block, engine, xs, dys, mb_sizes = _setup("llama3_70b_offload")
+	stream, _ = bench.plan_stream(w, block)
+	out = bench.check_stream(w, block, engine, stream, mb_sizes, xs, dys)
+	_assert_equal(out, "llama3_70b_offload")
+	assert out["d2h_bytes"] == out["h2d_bytes"] and out["d2h_bytes"] > w["n_mb"] * (1 << 30), "every micro-batch's stash crosses the link once each way"
+	assert out["ok"]
+	assert block.mem_stats()["live_bytes"] == 0
+	del block, engine, stage
+	_free()
+
+
+def test_zbh1_stream_equals_1f1b_and_the_oracle_over_all_micro_batches():
+	from oracle import stage_ref as R
+
+	bench, w, stage, block, engine, xs, dys, mb_sizes = _setup("llama3_8b_zbh1")
+	stream, _ = bench.plan_stream(w, block)
+	out = bench.check_stream(w, block, engine, stream, mb_sizes, xs, dys)
+	_assert_equal(out, "llama3_8b_zbh1")
+	assert out["ok"]
+	# the accumulators now hold the plain stream's sums over the 16 micro-batches, scaled by 1 / 32 sequences
+	got = {k: v.clone() for k, v in product_grads(stage).items() if k.startswith("0.")}
+	block.set_boundary(inputs=xs, grads=dys, keep_sent=True)
+	block.zero_grad()
+	engine.train_step(None, None, None, stream, mb_sizes)
+	torch.cuda.synchronize()
+	last = w["n_mb"] - 1
+	y_last, dx_last = block.sent_forward[last].clone(), block.sent_backward[last].clone()
+	params = oracle_params_from_stage(stage)
+	cfg = cfg_from_stage(stage, w["mb"])
+	del block, engine
+	_free()
+	# how far bf16 arithmetic itself (the reference's: PyTorch kernels on bf16 tensors) is from the fp32 truth after
+	# four blocks, on the last micro-batch: the Frobenius bound is 1e-2 or 1.25 x that error, whichever is larger
+	ref = R.RefStage(cfg, params, device="cuda")
+	ref16 = R.RefStage(cfg, params, compute_dtype=torch.bfloat16, device="cuda")
+	y16, dx16 = ref16.forward(last, xs[last]), ref16.backward_inputs(last, dys[last])
+	del ref16
+	bound = 1e-2
+	for m in range(w["n_mb"]):
+		y = ref.forward(m, xs[m])
+		dx = ref.backward_inputs(m, dys[m])
+		ref.backward_params(m)
+		if m == last:
+			fro16 = {"y": ((y16.double() - y.double()).norm() / y.double().norm()).item(), "dx": ((dx16.double() - dx.double()).norm() / dx.double().norm()).item()}
+			bound = max(1e-2, 1.25 * max(fro16.values()))
+			print(f"[bf16 torch vs fp32] 4 blocks: y {fro16['y']:.4g}, dx {fro16['dx']:.4g} -> Frobenius bound {bound:.4g}", flush=True)
+			_, fy = assert_close_dev(y_last, y, "zbh1 y[last]", rel_fro=max(1e-2, 1.25 * fro16["y"]))
+			_, fdx = assert_close_dev(dx_last, dx, "zbh1 dx[last]", rel_fro=max(1e-2, 1.25 * fro16["dx"]))
+			print(f"[hip vs fp32 oracle] 4 blocks: y {fy:.4g}, dx {fdx:.4g}", flush=True)
+			del y16, dx16
+		del y, dx
+	ref.scale_grads(w["mb"] * w["n_mb"])
+	want = ref.grads()
+	for k in sorted(got):
+		err, fro = assert_close_dev(got[k], want[k], f"zbh1 sum over {w['n_mb']} micro-batches, grad {k}", rel_fro=bound)
+		print(f"[hip vs fp32 oracle] grad {k}: max {err:.4g}, fro {fro:.4g}", flush=True)
+	del ref, want, got, stage
+	_free()

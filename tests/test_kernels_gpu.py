@@ -390,6 +390,28 @@ def test_colsum_is_exact_to_rounding_and_repeatable(K, T, N, ld):
 	assert ((runs[0].double() - want).abs().max() / want.abs().max()).item() <= 1e-5
 
 
+def test_split_k_on_one_stream_never_gives_up_its_turn_and_wide_splits_are_refused(K):
+	"""Back-to-back split-K launches on one stream keep their turns (the counter of waves that added out of turn does not
+	move, which is what bit-reproducible weight gradients rest on), and a split count that would not fit the 8 bits the
+	turn counters give it is refused."""
+	from elf_amd import _lib
+
+	M, N, Kd = 768, 768, 8192
+	A, B = _randn(Kd, M, seed=130), _randn(Kd, N, seed=131, scale=0.05)
+	before = K.gemm_turn_giveups()
+	runs = []
+	for _ in range(3):
+		acc = torch.zeros(M, N, device="cuda")
+		for cfg in (7, 8, 1):
+			K.gemm(A, B, a_t=True, b_t=True, out=acc, epilogue=K.EPI_F32_ACC, k_splits=4, tile_cfg=cfg)
+		runs.append(acc)
+	torch.cuda.synchronize()
+	assert K.gemm_turn_giveups() == before
+	assert torch.equal(runs[0], runs[1]) and torch.equal(runs[0], runs[2])
+	with pytest.raises(_lib.ElfStageError):
+		K.gemm(A, B, a_t=True, b_t=True, out=runs[0], epilogue=K.EPI_F32_ACC, k_splits=256, tile_cfg=7)
+
+
 def test_split_k_gemms_on_two_streams_stay_correct(K):
 	"""Weight-gradient GEMMs launched concurrently on two streams share the turn counters of their split tiles; whatever
 	the interleaving, every sum must be the right one to fp32 rounding (a workgroup that finds its counter taken by

@@ -235,11 +235,11 @@ def test_autograd_stage_block_on_a_generic_module(variant):
 	for name, p in blk.model.named_parameters():
 		got = p.main_grad if getattr(p, "main_grad", None) is not None else p.grad
 		assert got is not None, name
-		assert_close(got, ref_params[name].grad, f"{variant} grad {name}", rel_max=3e-2, rel_fro=2e-2)
+		assert_close(got, ref_params[name].grad, f"{variant} grad {name}")
 	blk.scale_grads(4)
 	for name, p in blk.model.named_parameters():
 		assert p.grad.dtype == torch.bfloat16
-		assert_close(p.grad, ref_params[name].grad / 4, f"{variant} scaled grad {name}", rel_max=4e-2, rel_fro=2e-2)
+		assert_close(p.grad, ref_params[name].grad / 4, f"{variant} scaled grad {name}")
 
 
 @pytest.mark.parametrize("scheduler,placement", [("afab", [0, 0]), ("1f1b", [0, 1]), ("zbh1", [0, 1])])
@@ -281,4 +281,4 @@ def test_pipeline_builds_generic_stages_for_other_modules(scheduler, placement):
 	for stage, ref in zip(stages, refs):
 		ref_params = dict(ref.named_parameters())
 		for name, p in stage.named_parameters():
-			assert_close(p.grad, ref_params[name].grad, f"grad {name}", rel_max=5e-2, rel_fro=3e-2)
+			assert_close(p.grad, ref_params[name].grad, f"grad {name}")

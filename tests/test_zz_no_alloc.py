@@ -63,3 +63,58 @@ def test_norm_bwd_noalloc_refuses_what_the_array_cannot_hold():
 	dg = torch.zeros(16384, dtype=torch.float32, device="cuda")
 	with pytest.raises(_lib.ElfStageError):
 		K.norm_bwd_noalloc(K.NORM_RMS, x, x, g, st, dg, torch.empty_like(x))
+
+
+def _inputs(K, kind, T, d, seed):
+	g = torch.Generator(device="cuda").manual_seed(seed)
+	rnd = lambda *shape: torch.randn(*shape, generator=g, device="cuda")
+	x = (rnd(T, d) * 2 + 0.5).to(torch.bfloat16)
+	dy = rnd(T, d).to(torch.bfloat16)
+	gamma = (1 + 0.1 * rnd(d)).to(torch.bfloat16)
+	_, stats = K.norm_fwd(kind, x, gamma, None)
+	return x, dy, gamma, stats
+
+
+def test_norm_bwd_noalloc_takes_no_device_memory():
+	"""What the entry point exists for: across a call neither torch's allocator nor the driver's free-memory
+	figure moves (after one earlier call on the device, which looks the array's address up)."""
+	from elf_amd import kernels as K
+
+	T, d = 4096, 4096
+	x, dy, gamma, stats = _inputs(K, K.NORM_RMS, T, d, 5)
+	dg, dx = torch.zeros(d, dtype=torch.float32, device="cuda"), torch.empty_like(x)
+	K.norm_bwd_noalloc(K.NORM_RMS, dy, x, gamma, stats, dg, dx)
+	torch.cuda.synchronize()
+	allocated, reserved, free = torch.cuda.memory_allocated(), torch.cuda.memory_reserved(), torch.cuda.mem_get_info()[0]
+	for _ in range(3):
+		K.norm_bwd_noalloc(K.NORM_RMS, dy, x, gamma, stats, dg, dx)
+	torch.cuda.synchronize()
+	assert torch.cuda.memory_allocated() == allocated and torch.cuda.memory_reserved() == reserved
+	assert torch.cuda.mem_get_info()[0] == free, "the driver's free memory moved across elf_norm_bwd_noalloc"
+
+
+def test_norm_bwd_noalloc_under_graph_capture():
+	"""Captured into a HIP graph (where hipMalloc is not allowed) and replayed three times with eager work and
+	synchronisations in between; every replay equals the eager call bit for bit."""
+	from elf_amd import kernels as K
+
+	T, d = 2048, 4096
+	x, dy, gamma, stats = _inputs(K, K.NORM_RMS, T, d, 6)
+	want_dg = torch.zeros(d, dtype=torch.float32, device="cuda")
+	want_dx = torch.empty_like(x)
+	K.norm_bwd_noalloc(K.NORM_RMS, dy, x, gamma, stats, want_dg, want_dx)  # eager; also the first call on the device
+	torch.cuda.synchronize()
+	dg, dx = torch.zeros(d, dtype=torch.float32, device="cuda"), torch.empty_like(x)
+	graph = torch.cuda.CUDAGraph()
+	with torch.cuda.graph(graph):
+		K.norm_bwd_noalloc(K.NORM_RMS, dy, x, gamma, stats, dg, dx)
+	for replay in range(3):
+		dg.zero_()
+		dx.fill_(7.0)
+		# eager work on the shared array between the replays: another shape leaves other partial sums in it
+		x2, dy2, g2, st2 = _inputs(K, K.NORM_RMS, 512, 1024, 70 + replay)
+		K.norm_bwd_noalloc(K.NORM_RMS, dy2, x2, g2, st2, torch.zeros(1024, dtype=torch.float32, device="cuda"), torch.empty_like(x2))
+		torch.cuda.synchronize()
+		graph.replay()
+		torch.cuda.synchronize()
+		assert torch.equal(dx, want_dx) and torch.equal(dg, want_dg), f"replay {replay} differs from the eager call"
