@@ -25,6 +25,7 @@ namespace elf {
 namespace dma {
 
 constexpr int BN = 256, BKS = 64;
+constexpr int PERS_WORKGROUPS = 256;  // one per compute unit: the persistent kernel's grid
 constexpr int B_BYTES = BN * BKS * 2;  // 32 KiB per stage
 
 // Shape of one workgroup: NW waves arranged (NW / 2) x 2, each owning RT x 4 accumulator tiles of
@@ -209,6 +210,40 @@ __device__ __forceinline__ void mfma_acc(f32x4& acc, const bf16x8& a, const bf16
 	asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
 }
 
+
+// Origin (m0, n0) of tile `pid` of the launch: see "Tile assignment" in gemm_dma_kernel for the two walks.
+template <int BM>
+__device__ __forceinline__ void tile_origin(const Args& g, int pid, int& m0, int& n0) {
+	const int ntiles = g.tiles_m * g.tiles_n;
+	const int nsb = ntiles >> 5, nrem = nsb & 7;
+	if (g.walk && (g.tiles_m & 7) == 0 && (g.tiles_n & 3) == 0 && (nrem == 0 || nrem == 1 || nrem == 2 || nrem == 4)) {
+		const int x = pid & 7, i = pid >> 3, nfull = nsb >> 3;
+		int sb, jj;
+		if (i < nfull * 32) {
+			sb = (i >> 5) * 8 + x;
+			jj = i & 31;
+		} else {
+			const int k = 8 / nrem;
+			sb = nfull * 8 + x / k;
+			jj = (x % k) * (32 / k) + (i - nfull * 32);
+		}
+		const int nsb_n = g.tiles_n >> 2, nsb_m = g.tiles_m >> 3;
+		const int band = sb / (2 * nsb_n), within = sb - band * 2 * nsb_n;
+		const bool pair = 2 * band + 1 < nsb_m;
+		const int sbm = 2 * band + (pair ? within & 1 : 0), sbn = pair ? within >> 1 : within;
+		m0 = (sbm * 8 + (jj & 7)) * BM;
+		n0 = (sbn * 4 + (jj >> 3)) * BN;
+	} else {
+		if ((ntiles & 7) == 0) pid = (pid & 7) * (ntiles >> 3) + (pid >> 3);
+		constexpr int GROUP_M = 8;
+		const int per_group = GROUP_M * g.tiles_n;
+		const int first_m = (pid / per_group) * GROUP_M;
+		const int gsz = min(g.tiles_m - first_m, GROUP_M);
+		m0 = (first_m + (pid % per_group) % gsz) * BM;
+		n0 = ((pid % per_group) / gsz) * BN;
+	}
+}
+
 template <int NW, int RT, bool AT, bool BT, int EPI>
 __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	using Sh = Shape<NW, RT>;
@@ -254,33 +289,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	// split tiles: the turn counter of this tile (tiles of one launch get distinct counters, consecutive launches different ones)
 	const int turn_slot = (int)(((uint32_t)(pid - full) + g.turn_tag * 977u) % (uint32_t)TURN_TILES);
 	int m0, n0;
-	const int nsb = ntiles >> 5, nrem = nsb & 7;
-	if (g.walk && (g.tiles_m & 7) == 0 && (g.tiles_n & 3) == 0 && (nrem == 0 || nrem == 1 || nrem == 2 || nrem == 4)) {
-		const int x = pid & 7, i = pid >> 3, nfull = nsb >> 3;
-		int sb, jj;
-		if (i < nfull * 32) {
-			sb = (i >> 5) * 8 + x;
-			jj = i & 31;
-		} else {
-			const int k = 8 / nrem;
-			sb = nfull * 8 + x / k;
-			jj = (x % k) * (32 / k) + (i - nfull * 32);
-		}
-		const int nsb_n = g.tiles_n >> 2, nsb_m = g.tiles_m >> 3;
-		const int band = sb / (2 * nsb_n), within = sb - band * 2 * nsb_n;
-		const bool pair = 2 * band + 1 < nsb_m;
-		const int sbm = 2 * band + (pair ? within & 1 : 0), sbn = pair ? within >> 1 : within;
-		m0 = (sbm * 8 + (jj & 7)) * BM;
-		n0 = (sbn * 4 + (jj >> 3)) * BN;
-	} else {
-		if ((ntiles & 7) == 0) pid = (pid & 7) * (ntiles >> 3) + (pid >> 3);
-		constexpr int GROUP_M = 8;
-		const int per_group = GROUP_M * g.tiles_n;
-		const int first_m = (pid / per_group) * GROUP_M;
-		const int gsz = min(g.tiles_m - first_m, GROUP_M);
-		m0 = (first_m + (pid % per_group) % gsz) * BM;
-		n0 = ((pid % per_group) / gsz) * BN;
-	}
+	tile_origin<BM>(g, pid, m0, n0);
 	m0 = __builtin_amdgcn_readfirstlane(m0);
 	n0 = __builtin_amdgcn_readfirstlane(n0);
 
@@ -666,6 +675,320 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	}
 }
 
+
+// ------------------------------------------------------------------------------------------------------------
+// Persistent forward kernel: both operands k-contiguous, 256x256 tiles, four waves with 128x128 wave tiles - the loop
+// of gemm_dma_kernel<4, 4, false, false, .> with two changes that take the tile boundary out of the matrix pipe's way.
+//
+//  * The epilogue leaves from registers.  The MFMA operands are swapped (the weight rows feed the m side), so a lane
+//    holds four consecutive columns of ONE output row per accumulator tile, and the order in which weight rows enter
+//    the four column slabs of a half-step is permuted (slab jj, m slot 4 g + r  <-  column 32 (jj / 2) + 8 g + 4 (jj % 2) + r)
+//    so that the lane's 16 values of a half-step are two runs of 8 consecutive columns: one 16-byte store each, the four
+//    lane groups of a row together 64 contiguous bytes.  No LDS staging, no barrier, a quarter of the instructions.
+//    For column slab jj of half h and k32 half kq lane l reads tile row wc * 128 + h * 64 + 32 (jj / 2) + 8 ((l % 16) / 4)
+//    + 4 (jj % 2) + l % 4 at k = 32 kq + 8 (l / 16) .. + 7; the B tile's chunk swizzle follows these rows (rb_swz) so
+//    that the 16 lanes of a k chunk still hit 16 different 16-byte bank groups.
+//  * A workgroup walks tiles pid, pid + grid, ... and its K-slice pipeline never drains: the last two slices of a tile
+//    fetch the first two of the next (the loop's "slice past the end of K" is the next tile's slice 0), the LDS ring is
+//    not needed by the epilogue, and the first MFMAs of a tile write their accumulators (C = 0 form) instead of adding
+//    to cleared ones.  K / 64 must be even so that a tile starts in ring stage 0.
+// Results are bit-identical to gemm_dma_kernel's: same products, same accumulation order along K, same roundings.
+__device__ __forceinline__ int rb_swz(int row) { return (((row >> 3) & 3) << 1) | ((row >> 1) & 1); }
+
+template <bool PAIRED>
+__device__ __forceinline__ void lane_offsets_rb(int wave, int lane, int64_t ld, uint32_t (&off)[8], int64_t pair_rows) {
+#pragma unroll
+	for (int i = 0; i < 8; i++) {
+		const int q = wave * 8 + i;
+		const int row = q * 8 + (lane >> 3), slot = lane & 7;
+		const int64_t grow = PAIRED ? (row >> 7) * 64 + (row & 63) + ((row >> 6) & 1) * pair_rows : row;
+		off[i] = (uint32_t)((grow * ld + ((slot ^ rb_swz(row)) << 3)) * 2);
+	}
+}
+
+// acc = a b: the first MFMA of an accumulator tile in a tile's K loop
+__device__ __forceinline__ void mfma_init(f32x4& acc, const bf16x8& a, const bf16x8& b) {
+	asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=a"(acc) : "v"(a), "v"(b));
+}
+
+template <int EPI>
+__global__ __launch_bounds__(256) void gemm_pers_kernel(Args g) {
+	using Sh = Shape<4, 4>;
+	constexpr int BM = 256, RT = 4, RF = 8, NST = 2, A_BYTES = Sh::A_BYTES, STAGE_BYTES = Sh::STAGE_BYTES;
+	constexpr int LOADS_A = Sh::LOADS_A, LOADS_B = Sh::LOADS_B, LOADS_PER_STAGE = Sh::LOADS_PER_STAGE, HALF = LOADS_PER_STAGE / 2;
+	constexpr bool PAIRED = EPI == EPI_BF16_SWIGLU;
+	static_assert(Sh::NST == 2 && LOADS_A == 8 && LOADS_B == 8, "ring of two 64 KiB stages");
+	extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+	const int tid = threadIdx.x;
+	const int lane = tid & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+	const int wr = wave >> 1, wc = wave & 1;
+	const int ntiles = g.tiles_m * g.tiles_n;
+	const int nk = g.K / BKS;  // even
+
+	uint32_t aoff[LOADS_A], boff[LOADS_B];
+	lane_offsets<false, LOADS_A, false, BM>(wave, lane, g.lda, aoff);
+	lane_offsets_rb<PAIRED>(wave, lane, g.ldb, boff, g.N / 2);
+	const uint32_t lds_a = lds_addr(smem) + wave * (LOADS_A * 1024);
+	const uint32_t lds_b = lds_addr(smem) + NST * A_BYTES + wave * (LOADS_B * 1024);
+	const uint32_t lds_dummy = lds_addr(smem) + NST * STAGE_BYTES;
+
+	auto tile_ptrs = [&](int tile, int& m0, int& n0, const bf16_t*& Ap, const bf16_t*& Bp) {
+		tile_origin<BM>(g, tile, m0, n0);
+		m0 = __builtin_amdgcn_readfirstlane(m0);
+		n0 = __builtin_amdgcn_readfirstlane(n0);
+		Ap = g.A + (int64_t)m0 * g.lda;
+		Bp = g.B + (int64_t)(PAIRED ? n0 / 2 : n0) * g.ldb;
+	};
+	int tile = blockIdx.x, m0, n0, m0_n = 0, n0_n = 0;
+	const bf16_t *Ap, *Bp, *Ap_n, *Bp_n;
+	tile_ptrs(tile, m0, n0, Ap, Bp);
+	Ap_n = Ap, Bp_n = Bp;
+	bool has_next = false;
+
+	struct SliceLoads {
+		const bf16_t* pa;
+		const bf16_t* pb;
+		uint32_t la, lb;
+	};
+	// slice `step` of the current tile; steps nk and nk + 1 are slices 0 and 1 of the next tile (same ring stage: nk is
+	// even), or, behind the workgroup's last tile, loads nobody reads into the scratch area behind the ring
+	auto slice_loads = [&](int step) {
+		const bool cur = step < nk;
+		const int sc = cur ? step : step - nk;
+		const bool ok = cur || has_next;
+		const uint32_t st = (uint32_t)(sc & 1);
+		return SliceLoads{(cur ? Ap : Ap_n) + (int64_t)sc * BKS, (cur ? Bp : Bp_n) + (int64_t)sc * BKS, ok ? lds_a + st * A_BYTES : lds_dummy,
+		                  ok ? lds_b + st * B_BYTES : lds_dummy};
+	};
+	auto issue_piece = [&](const SliceLoads& sl, auto pc) {
+		constexpr int P = decltype(pc)::value;
+		if constexpr (P < LOADS_A) dma16_at<P * 1024>(sl.pa, aoff[P], sl.la);
+		else dma16_at<(P - LOADS_A) * 1024>(sl.pb, boff[P - LOADS_A], sl.lb);
+	};
+
+	f32x4 acc[RF][8];
+	bf16x8 fa[2][RF], fb[2][4];
+	static_assert(pieces_have_slots(RF * 4, HALF), "a half-step has too few even MFMA slots for half a slice's loads");
+	{
+		const SliceLoads s0 = slice_loads(0);
+		static_for<LOADS_PER_STAGE>([&](auto pc) { issue_piece(s0, pc); });
+		const SliceLoads s1 = slice_loads(1);
+		static_for<HALF>([&](auto pc) { issue_piece(s1, pc); });
+		wait_vmcnt<HALF>();
+	}
+	__syncthreads();
+	// Per-lane LDS addresses of the fragment reads for the two k32 halves of a slice (the chunk swizzles only look at
+	// lane bits); stage, row slab and column slab are compile-time byte offsets in the read instructions.
+	uint32_t a_lane[2], b_lane[2];
+	{
+		const int l15 = lane & 15, q4 = lane >> 4;
+#pragma unroll
+		for (int kq = 0; kq < 2; kq++) {
+			a_lane[kq] = lds_addr(smem) + (uint32_t)((wr * 128 + l15) * 128 + (((4 * kq + q4) ^ ((l15 >> 1) & 7)) << 4));
+			b_lane[kq] = lds_addr(smem) + NST * A_BYTES + (uint32_t)((wc * 128 + 8 * (l15 >> 2) + (l15 & 3)) * 128 + (((4 * kq + q4) ^ rb_swz(8 * (l15 >> 2) + (l15 & 3))) << 4));
+			asm volatile("" : "+v"(a_lane[kq]), "+v"(b_lane[kq]));
+		}
+	}
+	auto read_a = [&](auto stage, int kq, auto ic) -> bf16x8 {
+		constexpr uint32_t IMM = decltype(stage)::value * A_BYTES + decltype(ic)::value * (16 * 128);
+		return *reinterpret_cast<const bf16x8 ELF_LDS*>((uintptr_t)(a_lane[kq] + IMM));
+	};
+	auto read_b = [&](auto stage, int kq, int h, auto jc) -> bf16x8 {
+		constexpr int JJ = decltype(jc)::value;
+		constexpr uint32_t IMM = decltype(stage)::value * B_BYTES + (32 * (JJ >> 1) + 4 * (JJ & 1)) * 128;
+		return *reinterpret_cast<const bf16x8 ELF_LDS*>((uintptr_t)(b_lane[kq] + IMM + (uint32_t)h * (64 * 128)));
+	};
+	static_for<RF>([&](auto ic) { fa[0][decltype(ic)::value] = read_a(std::integral_constant<int, 0>{}, 0, ic); });
+	static_for<4>([&](auto jc) { fb[0][decltype(jc)::value] = read_b(std::integral_constant<int, 0>{}, 0, 0, jc); });
+
+	// One half-step (see gemm_dma_kernel): RF * 4 MFMAs, the next half-step's fragment reads behind the odd ones, half of
+	// a slice's loads behind even ones.  FIRST: the accumulator tiles of this half-step are written, not added to.
+	auto half_step = [&](int abuf, int bbuf, auto hc, auto first, int pb_buf, auto pb_stage, int pb_kq, int pb_h, bool pa, int pa_buf, auto pa_stage, int pa_kq,
+	                     const SliceLoads& sl, auto piece0) {
+		constexpr int PIECE0 = decltype(piece0)::value, H = decltype(hc)::value, NM = RF * 4;
+		constexpr int SA = decltype(pa_stage)::value, SB = decltype(pb_stage)::value;
+		constexpr bool FIRST = decltype(first)::value;
+		static_for<NM>([&](auto nc) {
+			constexpr int n = decltype(nc)::value, i = n / 4, j = n % 4;
+			if constexpr (FIRST) mfma_init(acc[i][H * 4 + j], fb[bbuf][j], fa[abuf][i]);
+			else mfma_acc(acc[i][H * 4 + j], fb[bbuf][j], fa[abuf][i]);
+			if constexpr (n % 2 == 1) {
+				constexpr int r = n / 2;
+				if constexpr (r < 4) {
+					fb[pb_buf][r] = read_b(std::integral_constant<int, SB>{}, pb_kq, pb_h, std::integral_constant<int, r>{});
+				} else if constexpr (r - 4 < RF) {
+					if (pa) fa[pa_buf][r - 4] = read_a(std::integral_constant<int, SA>{}, pa_kq, std::integral_constant<int, r - 4>{});
+				}
+			}
+			if constexpr (PIECE0 >= 0 && piece_in_slot(n, NM, HALF) >= 0) issue_piece(sl, std::integral_constant<int, (PIECE0 < 0 ? 0 : PIECE0) + (piece_in_slot(n, NM, HALF) < 0 ? 0 : piece_in_slot(n, NM, HALF))>{});
+			__builtin_amdgcn_sched_barrier(0);
+		});
+	};
+	auto slice = [&](auto sc, auto first, int kt) {
+		constexpr int S = decltype(sc)::value;
+		constexpr std::integral_constant<int, S> CUR{};
+		constexpr std::integral_constant<int, (S + 1) % NST> NXT{};
+		constexpr std::integral_constant<int, 0> H0{};
+		constexpr std::integral_constant<int, 1> H1{};
+		constexpr std::integral_constant<int, -1> NO_DMA{};
+		constexpr std::false_type ADD{};
+		const SliceLoads next1 = slice_loads(kt + 1), next2 = slice_loads(kt + 2);
+		half_step(0, 0, H0, first, 1, CUR, 0, 1, false, 0, CUR, 0, next1, std::integral_constant<int, HALF>{});
+		half_step(0, 1, H1, first, 0, CUR, 1, 0, true, 1, CUR, 1, next1, NO_DMA);
+		half_step(1, 0, H0, ADD, 1, CUR, 1, 1, false, 0, CUR, 0, next1, NO_DMA);
+		wait_counters<0, 0>();  // slice kt + 1 landed (and the previous tile's stores acknowledged); slice kt fully read
+		__syncthreads();
+		half_step(1, 1, H1, ADD, 0, NXT, 0, 0, true, 0, NXT, 0, next2, std::integral_constant<int, 0>{});
+	};
+
+	const int g4 = lane >> 4, rr = lane & 15;
+	for (;;) {
+		const int tile_n = tile + (int)gridDim.x;
+		has_next = tile_n < ntiles;
+		if (has_next) tile_ptrs(tile_n, m0_n, n0_n, Ap_n, Bp_n);
+
+		slice(std::integral_constant<int, 0>{}, std::true_type{}, 0);
+		slice(std::integral_constant<int, 1>{}, std::false_type{}, 1);
+		for (int kt = 2; kt < nk; kt += 2) {
+			slice(std::integral_constant<int, 0>{}, std::false_type{}, kt);
+			slice(std::integral_constant<int, 1>{}, std::false_type{}, kt + 1);
+		}
+
+		// Epilogue from registers, while the next tile's first two slices are on their way into the ring.  The MFMAs were
+		// issued through inline assembly, so the compiler places no wait states between the last of them and the first
+		// read of an accumulator: 32 of them here (an 8-pass MFMA needs 11).
+		asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+		const int grow0 = m0 + wr * 128 + rr;
+		const int gcol0 = n0 + wc * 128;
+		// the lane's run t (0..3) of 8 consecutive columns: columns (t / 2) * 64 + (t % 2) * 32 + 8 g4 .. + 7 of the wave's 128
+		auto run = [&](int i, int t, float (&v)[8]) {
+#pragma unroll
+			for (int e = 0; e < 8; e++) v[e] = acc[i][(t >> 1) * 4 + (t & 1) * 2 + (e >> 2)][e & 3];
+		};
+		auto run_col = [&](int t) { return (t >> 1) * 64 + (t & 1) * 32 + g4 * 8; };
+		if constexpr (EPI == EPI_BF16_SWIGLU) {
+			// the wave's columns are 64 gate columns (first half-step) and the 64 up columns of the same outputs (second)
+			const int F = g.N / 2, cg0 = n0 / 2 + wc * 64;
+#pragma unroll
+			for (int i = 0; i < RF; i++) {
+				const int64_t row = grow0 + i * 16;
+#pragma unroll
+				for (int t = 0; t < 2; t++) {
+					float gv[8], uv[8];
+					run(i, t, gv);
+					run(i, 2 + t, uv);
+					bf16x8 og, ou, oa;
+#pragma unroll
+					for (int e = 0; e < 8; e++) {
+						og[e] = (bf16_t)gv[e];
+						ou[e] = (bf16_t)uv[e];
+						oa[e] = (bf16_t)swiglu_f((float)og[e], (float)ou[e]);
+					}
+					const int c = cg0 + t * 32 + g4 * 8;
+					bf16_t* cp = reinterpret_cast<bf16_t*>(g.C) + row * g.ldc + c;
+					*reinterpret_cast<bf16x8*>(cp) = og;
+					*reinterpret_cast<bf16x8*>(cp + F) = ou;
+					*reinterpret_cast<bf16x8*>(g.C2 + row * g.ldc2 + c) = oa;
+				}
+			}
+		} else if constexpr (EPI == EPI_BF16_ROPE) {
+			// heads of 128: the wave's strip is one head, its halves are the two half-steps (runs t and t + 2); heads of
+			// 64: each half-step is a head, its halves are runs t = 0 and 1 (2 and 3).  Rounded to bf16 before the rotation,
+			// as the RoPE kernel would read the projection from memory.
+			const int half = g.rope_D >> 1;
+			auto rope_rows = [&](auto widec) {
+				constexpr bool WIDE = decltype(widec)::value;
+#pragma unroll
+				for (int i = 0; i < RF; i++) {
+					const int64_t row = grow0 + i * 16;
+					const int pos = (int)(row % g.rope_S);
+					bf16_t* cp = reinterpret_cast<bf16_t*>(g.C) + row * g.ldc + gcol0;
+#pragma unroll
+					for (int p = 0; p < 2; p++) {
+						// pair p: runs (lo, hi) = (p, p + 2) for heads of 128, (2 p, 2 p + 1) for heads of 64
+						const int tlo = WIDE ? p : 2 * p, thi = WIDE ? p + 2 : 2 * p + 1;
+						const int c_in_head = WIDE ? p * 32 + g4 * 8 : g4 * 8;  // first of the lane's 8 columns within the head's first half
+						const bool rot = gcol0 + run_col(tlo) < g.rope_cols;
+						float a[8], b[8];
+						run(i, tlo, a);
+						run(i, thi, b);
+						bf16x8 olo, ohi;
+						f32x4 tab[4] = {};
+						if (rot) {
+							const f32x4* tp = reinterpret_cast<const f32x4*>(g.rope_cs + (int64_t)pos * half + c_in_head);
+#pragma unroll
+							for (int q = 0; q < 4; q++) tab[q] = tp[q];
+						}
+#pragma unroll
+						for (int e = 0; e < 8; e++) {
+							const float x = (float)(bf16_t)a[e], y = (float)(bf16_t)b[e];
+							float ra = x, rb = y;
+							if (rot) rope_rot(x, y, tab[e >> 1][(e & 1) * 2], tab[e >> 1][(e & 1) * 2 + 1], ra, rb);
+							olo[e] = (bf16_t)ra;
+							ohi[e] = (bf16_t)rb;
+						}
+						*reinterpret_cast<bf16x8*>(cp + run_col(tlo)) = olo;
+						*reinterpret_cast<bf16x8*>(cp + run_col(thi)) = ohi;
+					}
+				}
+			};
+			if (g.rope_D == 128) rope_rows(std::true_type{});
+			else rope_rows(std::false_type{});
+		} else {
+			static_assert(EPI == EPI_BF16 || EPI == EPI_BF16_RESID, "epilogues of the persistent forward kernel");
+			// residual (or bias row, ldr = 0): the loads of four rows of accumulator tiles in flight together
+#pragma unroll
+			for (int ib = 0; ib < RF; ib += 4) {
+				bf16x8 rs[EPI == EPI_BF16_RESID ? 4 : 1][4];
+				if constexpr (EPI == EPI_BF16_RESID) {
+#pragma unroll
+					for (int i = 0; i < 4; i++)
+#pragma unroll
+						for (int t = 0; t < 4; t++)
+							rs[i][t] = *reinterpret_cast<const bf16x8*>(g.R + (int64_t)(grow0 + (ib + i) * 16) * g.ldr + gcol0 + run_col(t));
+				}
+#pragma unroll
+				for (int i = 0; i < 4; i++) {
+					bf16_t* cp = reinterpret_cast<bf16_t*>(g.C) + (int64_t)(grow0 + (ib + i) * 16) * g.ldc + gcol0;
+#pragma unroll
+					for (int t = 0; t < 4; t++) {
+						float v[8];
+						run(ib + i, t, v);
+						bf16x8 o;
+#pragma unroll
+						for (int e = 0; e < 8; e++) {
+							if constexpr (EPI == EPI_BF16_RESID) v[e] += (float)rs[i][t][e];
+							o[e] = (bf16_t)v[e];
+						}
+						*reinterpret_cast<bf16x8*>(cp + run_col(t)) = o;
+					}
+				}
+			}
+		}
+		if (!has_next) break;
+		tile = tile_n, m0 = m0_n, n0 = n0_n, Ap = Ap_n, Bp = Bp_n;
+		asm volatile("s_nop 7" ::: "memory");  // accumulator reads above, accumulator writes by the next tile's first MFMAs
+	}
+	wait_vmcnt<0>();  // the loads past the last tile land in LDS too
+}
+
+template <int EPI>
+static int launch_pers(const Args& a, hipStream_t stream) {
+	using Sh = Shape<4, 4>;
+	constexpr int smem = Sh::NST * Sh::STAGE_BYTES + Sh::LOADS_A * 1024;
+	auto kern = gemm_pers_kernel<EPI>;
+	static bool attr_set = false;
+	if (!attr_set) {
+		ELF_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+		attr_set = true;
+	}
+	const int ntiles = a.tiles_m * a.tiles_n;
+	ELF_LAUNCH(kern, dim3(ntiles < PERS_WORKGROUPS ? ntiles : PERS_WORKGROUPS), dim3(256), smem, stream, a);
+	ELF_CHECK_HIP(hipGetLastError());
+	return 0;
+}
+
 template <int NW, int RT, bool AT, bool BT, int EPI>
 static int launch(const Args& a, hipStream_t stream) {
 	// the ring + the target of the loads past the end of K (as many KiB as a wave issues loads per
@@ -747,6 +1070,15 @@ int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t 
 	// k-contiguous A (forward, dX): four waves with 128x128 wave tiles; both operands reduction-major (dW): eight
 	// waves with 64x128 wave tiles (with two transpose reads per fragment on both operands the lone wave wins on
 	// some shapes by 2-3 % and loses on most by 1-10 %)
+	if (!a_t && !b_t && (K / dma::BKS) % 2 == 0 && !getenv("ELF_NO_PERSISTENT_GEMM")) {
+		// forward shapes: persistent workgroups, register epilogue
+		switch (epi) {
+			case EPI_BF16: return dma::launch_pers<EPI_BF16>(a, stream);
+			case EPI_BF16_RESID: return dma::launch_pers<EPI_BF16_RESID>(a, stream);
+			case EPI_BF16_SWIGLU: return dma::launch_pers<EPI_BF16_SWIGLU>(a, stream);
+			case EPI_BF16_ROPE: return dma::launch_pers<EPI_BF16_ROPE>(a, stream);
+		}
+	}
 	if (!a_t && !b_t) return dma::launch_epi<4, 4, false, false>(a, epi, stream);
 	if (!a_t && b_t) return dma::launch_epi<4, 4, false, true>(a, epi, stream);
 	if (a_t && b_t) return dma::launch_epi<8, 2, true, true>(a, epi, stream);

@@ -126,6 +126,36 @@ def test_gemm_k_split_is_bit_reproducible(K, dims, ks):
 	assert ((runs[0] - one).norm() / one.norm()).item() <= 1e-5
 
 
+@pytest.mark.parametrize("shape", [(256, 256, 128), (512, 768, 256), (4096, 1280, 1152), (8192, 4096, 1024), (2048, 28672, 256)])
+def test_persistent_forward_gemm_equals_the_tile_kernel_bit_for_bit(K, monkeypatch, shape):
+	"""Forward GEMMs on 256x256 tiles run as persistent workgroups that walk several tiles and store from registers
+	(operands swapped on the MFMA, permuted weight rows); the one-tile-per-workgroup kernel with its LDS-staged epilogue
+	(ELF_NO_PERSISTENT_GEMM=1) forms the same products in the same order: equal bits for every epilogue, from one tile
+	per workgroup (1, 6 tiles) to several with a ragged last round (80, 512, 896 tiles), also against fp32 torch."""
+	M, N, Kd = shape
+	a, w, r, bias = _randn(M, Kd, seed=61), _randn(N, Kd, seed=62, scale=0.05), _randn(M, N, seed=63), _randn(1, N, seed=64)
+	F = N // 2
+	S, D = 256, 128
+	cs = K.rope_table(S, D, 5e5)
+	n_rot = (N // D) // 2
+
+	def run():
+		return (K.gemm(a, w, tile_cfg=7), K.gemm(a, w, tile_cfg=7, epilogue=K.EPI_BF16_RESID, residual=r),
+		        K.gemm(a, w, tile_cfg=7, epilogue=K.EPI_BF16_RESID, residual=bias, residual_ld=0), *K.gemm_act(a, w, K.ACT_SWIGLU), K.gemm_rope(a, w, cs, S, n_rot, D))
+
+	new = run()
+	monkeypatch.setenv("ELF_NO_PERSISTENT_GEMM", "1")
+	old = run()
+	monkeypatch.delenv("ELF_NO_PERSISTENT_GEMM")
+	for i, (x, y) in enumerate(zip(new, old)):
+		assert torch.equal(x, y), f"output {i} of the persistent kernel differs from the tile kernel's at {shape}"
+	ref = a.float() @ w.float().t()
+	_close(new[0], ref, what="persistent bf16")
+	_close(new[1], ref + r.float(), what="persistent residual")
+	_close(new[2], ref + bias.float(), what="persistent bias row")
+	_close(new[4], torch.nn.functional.silu(new[3][:, :F].float()) * new[3][:, F:].float(), what="persistent swiglu")
+
+
 def test_gemm_strided_views(K):
 	# operands that are column slices of wider buffers (leading dimension > row length)
 	big = _randn(512, 1024, seed=6)
