@@ -334,13 +334,14 @@ def hbm_ceiling():
 	dst = torch.empty(n, dtype=torch.uint8, device="cuda")
 	st = torch.cuda.current_stream().cuda_stream
 	out = {"bytes": n, "peak_gbs": PEAK_HBM_GBS}
-	for mode, name, moved in ((0, "read", n), (1, "copy", 2 * n), (2, "write", n)):
+	# "read3_write1": three input streams of n / 4 bytes each and one output stream (a norm backward's pattern)
+	for mode, name, size, moved in ((0, "read", n, n), (1, "copy", n, 2 * n), (2, "write", n, n), (3, "read3_write1", n // 4, n)):
 		for _ in range(3):
-			_lib.check(lib.elf_hbm_probe(mode, src.data_ptr(), dst.data_ptr(), n, st), "elf_hbm_probe")
+			_lib.check(lib.elf_hbm_probe(mode, src.data_ptr(), dst.data_ptr(), size, st), "elf_hbm_probe")
 		e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
 		e0.record()
 		for _ in range(20):
-			_lib.check(lib.elf_hbm_probe(mode, src.data_ptr(), dst.data_ptr(), n, st), "elf_hbm_probe")
+			_lib.check(lib.elf_hbm_probe(mode, src.data_ptr(), dst.data_ptr(), size, st), "elf_hbm_probe")
 		e1.record()
 		torch.cuda.synchronize()
 		ms = e0.elapsed_time(e1) / 20

@@ -148,28 +148,45 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(const bf16_t* __restrict_
 		for (int j = 0; j < 8; j++) dg[i][j] = db[i][j] = 0.f;
 	}
 	const int row_step = WPR == 1 ? gridDim.x * ROWS_PER_BLOCK : gridDim.x;
-	for (int row = WPR == 1 ? blockIdx.x * ROWS_PER_BLOCK + wave : blockIdx.x; row < T; row += row_step) {
-		const float2 st = stats[row];
-		const float mean = st.x, rstd = st.y;
-		const bf16_t* xr = x + (int64_t)row * d;
-		const bf16_t* dyr = dy + (int64_t)row * d;
-		Chunk xh[NCH], gy[NCH];
+	// the next row's operands (dy, x, the residual gradient, the row statistics) are fetched while the current row is
+	// reduced: a row costs two or three trips through the workgroup's reduction, during which nothing else would be in flight
+	bf16x8 nx[NCH], ndy[NCH], nres[NCH];  // the row in flight
+	float2 nst = make_float2(0.f, 0.f);
+	auto fetch = [&](int r) {
+		if (r < T) {
+			nst = stats[r];
+#pragma unroll
+			for (int i = 0; i < NCH; i++) {
+				const int ch = tr + i * TPR;
+				if (ch < nchunks) {
+					nx[i] = *reinterpret_cast<const bf16x8*>(x + (int64_t)r * d + ch * 8);
+					ndy[i] = *reinterpret_cast<const bf16x8*>(dy + (int64_t)r * d + ch * 8);
+					if (dres) nres[i] = *reinterpret_cast<const bf16x8*>(dres + (int64_t)r * d + ch * 8);
+				}
+			}
+		}
+	};
+	int row = WPR == 1 ? blockIdx.x * ROWS_PER_BLOCK + wave : blockIdx.x;
+	fetch(row);
+	for (; row < T; row += row_step) {
+		// the current row stays in its 16-bit form; xhat and dy * gamma are formed again for dx rather than kept as floats
+		bf16x8 rx[NCH], rdy[NCH], rres[NCH];
+		const float mean = nst.x, rstd = nst.y;
+#pragma unroll
+		for (int i = 0; i < NCH; i++) rx[i] = nx[i], rdy[i] = ndy[i], rres[i] = nres[i];
+		fetch(row + row_step);
 		float s1 = 0.f, s2 = 0.f;
 #pragma unroll
 		for (int i = 0; i < NCH; i++) {
 			const int ch = tr + i * TPR;
 			if (ch < nchunks) {
-				xh[i] = load8(xr + ch * 8);
-				gy[i] = load8(dyr + ch * 8);
 #pragma unroll
 				for (int j = 0; j < 8; j++) {
-					const float xhat = (xh[i].v[j] - mean) * rstd;
-					const float dyv = gy[i].v[j];
+					const float xhat = ((float)rx[i][j] - mean) * rstd;
+					const float dyv = (float)rdy[i][j];
 					dg[i][j] += dyv * xhat;
 					if (LN) db[i][j] += dyv;
 					const float gv = dyv * g[i].v[j];
-					xh[i].v[j] = xhat;
-					gy[i].v[j] = gv;
 					s1 += gv;
 					s2 += gv * xhat;
 				}
@@ -184,11 +201,11 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(const bf16_t* __restrict_
 			if (ch < nchunks) {
 				Chunk o;
 #pragma unroll
-				for (int j = 0; j < 8; j++) o.v[j] = rstd * (gy[i].v[j] - m1 - xh[i].v[j] * m2);
-				if (dres) {
-					Chunk r = load8(dres + (int64_t)row * d + ch * 8);
-#pragma unroll
-					for (int j = 0; j < 8; j++) o.v[j] += r.v[j];
+				for (int j = 0; j < 8; j++) {
+					const float xhat = ((float)rx[i][j] - mean) * rstd;
+					const float gv = (float)rdy[i][j] * g[i].v[j];
+					o.v[j] = rstd * (gv - m1 - xhat * m2);
+					if (dres) o.v[j] += (float)rres[i][j];
 				}
 				store8(dxr + ch * 8, o);
 			}
@@ -264,7 +281,174 @@ __global__ __launch_bounds__(1024) void norm_bwd_finalize_kernel(const float* __
 	}
 }
 
+
+// ------------------------------------------------------------------------------------------
+// Narrow rows (d = 256, 512 or 768; the GPT-2-small width 768 is three 16-byte chunks per lane): half a
+// wave per row, so that no lane idles in a partly filled chunk and a wave has two rows' loads in flight; reductions
+// stay inside the half-wave (butterfly over 16 .. 1).  Forward: each wave takes PAIRS consecutive row pairs, all
+// loads issued before the first reduction.
+__device__ __forceinline__ float half_wave_sum(float v) {
+#pragma unroll
+	for (int o = 16; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+	return v;
+}
+
+template <int NCH, bool LN, int PAIRS>
+__global__ __launch_bounds__(256) void norm_fwd_half_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ gamma,
+                                                            const bf16_t* __restrict__ beta, bf16_t* __restrict__ y,
+                                                            float2* __restrict__ stats, int T, float eps) {
+	constexpr int d = NCH * 256;
+	const int l32 = threadIdx.x & 31;
+	const int row0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * (2 * PAIRS) + ((threadIdx.x >> 5) & 1);
+	bf16x8 raw[PAIRS][NCH];
+#pragma unroll
+	for (int p = 0; p < PAIRS; p++) {
+		const int row = row0 + 2 * p;
+		if (row < T)
+#pragma unroll
+			for (int i = 0; i < NCH; i++) raw[p][i] = *reinterpret_cast<const bf16x8*>(x + (int64_t)row * d + (l32 + 32 * i) * 8);
+	}
+	Chunk g[NCH], b[NCH];
+#pragma unroll
+	for (int i = 0; i < NCH; i++) {
+		g[i] = load8(gamma + (l32 + 32 * i) * 8);
+		if (LN) b[i] = load8(beta + (l32 + 32 * i) * 8);
+	}
+#pragma unroll
+	for (int p = 0; p < PAIRS; p++) {
+		const int row = row0 + 2 * p;
+		if (row >= T) continue;  // uniform per half-wave; the shuffles below stay inside it
+		float c[NCH][8];
+		float s = 0.f, ss = 0.f;
+#pragma unroll
+		for (int i = 0; i < NCH; i++)
+#pragma unroll
+			for (int j = 0; j < 8; j++) {
+				c[i][j] = (float)raw[p][i][j];
+				s += c[i][j];
+				ss += c[i][j] * c[i][j];
+			}
+		float mean = 0.f, rstd;
+		if (LN) {
+			mean = half_wave_sum(s) / d;
+			float var = 0.f;
+#pragma unroll
+			for (int i = 0; i < NCH; i++)
+#pragma unroll
+				for (int j = 0; j < 8; j++) {
+					const float t = c[i][j] - mean;
+					var += t * t;
+				}
+			rstd = rsqrtf(half_wave_sum(var) / d + eps);
+		} else {
+			rstd = rsqrtf(half_wave_sum(ss) / d + eps);
+		}
+		if (l32 == 0) stats[row] = make_float2(mean, rstd);
+#pragma unroll
+		for (int i = 0; i < NCH; i++) {
+			Chunk o;
+#pragma unroll
+			for (int j = 0; j < 8; j++) o.v[j] = LN ? (c[i][j] - mean) * rstd * g[i].v[j] + b[i].v[j] : c[i][j] * rstd * g[i].v[j];
+			store8(y + (int64_t)row * d + (l32 + 32 * i) * 8, o);
+		}
+	}
+}
+
+// Backward for the same rows: a wave walks row pairs with the next pair's loads in flight while it reduces the current
+// one; the eight rows a workgroup holds at a time are folded through LDS into one partial row per workgroup.
+template <int NCH, bool LN>
+__global__ __launch_bounds__(256) void norm_bwd_half_kernel(const bf16_t* __restrict__ dy, const bf16_t* __restrict__ x,
+                                                            const bf16_t* __restrict__ gamma, const float2* __restrict__ stats,
+                                                            const bf16_t* __restrict__ dres, bf16_t* __restrict__ dx,
+                                                            float* __restrict__ part, int T) {
+	constexpr int d = NCH * 256;
+	__shared__ float fold[4][NCH * 256];
+	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31;
+	Chunk g[NCH];
+	float dg[NCH][8], db[NCH][8];
+#pragma unroll
+	for (int i = 0; i < NCH; i++) {
+		g[i] = load8(gamma + (l32 + 32 * i) * 8);
+#pragma unroll
+		for (int j = 0; j < 8; j++) dg[i][j] = db[i][j] = 0.f;
+	}
+	const int row_step = gridDim.x * 8;
+	int row = blockIdx.x * 8 + wave * 2 + (lane >> 5);
+	bf16x8 nx[NCH], ndy[NCH], nres[NCH];  // the row pair in flight
+	float2 nst = make_float2(0.f, 0.f);
+	auto fetch = [&](int r) {
+		if (r < T) {
+			nst = stats[r];
+#pragma unroll
+			for (int i = 0; i < NCH; i++) {
+				nx[i] = *reinterpret_cast<const bf16x8*>(x + (int64_t)r * d + (l32 + 32 * i) * 8);
+				ndy[i] = *reinterpret_cast<const bf16x8*>(dy + (int64_t)r * d + (l32 + 32 * i) * 8);
+				if (dres) nres[i] = *reinterpret_cast<const bf16x8*>(dres + (int64_t)r * d + (l32 + 32 * i) * 8);
+			}
+		}
+	};
+	fetch(row);
+	for (; row < T; row += row_step) {
+		bf16x8 rx[NCH], rdy[NCH], rres[NCH];
+		const float mean = nst.x, rstd = nst.y;
+#pragma unroll
+		for (int i = 0; i < NCH; i++) rx[i] = nx[i], rdy[i] = ndy[i], rres[i] = nres[i];
+		fetch(row + row_step);  // the next pair's loads travel while this one is reduced and stored
+		float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+		for (int i = 0; i < NCH; i++)
+#pragma unroll
+			for (int j = 0; j < 8; j++) {
+				const float xhat = ((float)rx[i][j] - mean) * rstd;
+				const float dyv = (float)rdy[i][j];
+				dg[i][j] += dyv * xhat;
+				if (LN) db[i][j] += dyv;
+				const float gv = dyv * g[i].v[j];
+				s1 += gv;
+				s2 += gv * xhat;
+			}
+		const float m2 = half_wave_sum(s2) / d;
+		const float m1 = LN ? half_wave_sum(s1) / d : 0.f;
+#pragma unroll
+		for (int i = 0; i < NCH; i++) {
+			Chunk o;
+#pragma unroll
+			for (int j = 0; j < 8; j++) {
+				const float xhat = ((float)rx[i][j] - mean) * rstd;
+				const float gv = (float)rdy[i][j] * g[i].v[j];
+				o.v[j] = rstd * (gv - m1 - xhat * m2);
+				if (dres) o.v[j] += (float)rres[i][j];
+			}
+			store8(dx + (int64_t)row * d + (l32 + 32 * i) * 8, o);
+		}
+	}
+	// fold: the two rows of a wave by a shuffle, the four waves through LDS, in a fixed order
+	float* pg = part + (int64_t)blockIdx.x * 2 * d;
+	for (int which = 0; which < (LN ? 2 : 1); which++) {
+		__syncthreads();
+#pragma unroll
+		for (int i = 0; i < NCH; i++)
+#pragma unroll
+			for (int j = 0; j < 8; j++) {
+				float v = which ? db[i][j] : dg[i][j];
+				v += __shfl_xor(v, 32, 64);
+				if (lane < 32) fold[wave][(l32 + 32 * i) * 8 + j] = v;
+			}
+		__syncthreads();
+		for (int col = threadIdx.x; col < d; col += 256) pg[which * d + col] = (fold[0][col] + fold[1][col]) + (fold[2][col] + fold[3][col]);
+	}
+}
+
+// (at d = 1024 the backward's four chunks per lane of three tensors, current and next row, fill the register file and the
+// full-wave kernel is faster)
+static inline bool norm_half_rows(int d) { return d % 256 == 0 && d <= 768; }
+
 static inline int norm_bwd_blocks(int T, int d) {
+	if (norm_half_rows(d)) {
+		// eight rows per workgroup at a time, at most two workgroups per compute unit: 512 partial rows for the fold
+		const int want = (T + 7) / 8;
+		return want < 512 ? want : 512;
+	}
 	const int rows_per_block = d <= 2048 ? ROWS_PER_BLOCK : 1;
 	const int want = (T + rows_per_block - 1) / rows_per_block;
 	// fewer, longer workgroups for narrow rows and for the widest ones: the partial rows are overhead traffic that the fold
@@ -277,6 +461,19 @@ template <bool LN>
 static int norm_fwd_dispatch(const void* x, const void* gamma, const void* beta, void* y, void* stats, int T, int d,
                              float eps, hipStream_t s) {
 	const dim3 block(256);
+	if (norm_half_rows(d)) {
+		constexpr int PAIRS = 2;  // 16 rows per workgroup
+		const dim3 grid((T + 16 - 1) / 16);
+#define ELF_NORM_FWD_HALF(N) ELF_LAUNCH((norm_fwd_half_kernel<N, LN, PAIRS>), grid, block, 0, s, (const bf16_t*)x, (const bf16_t*)gamma, (const bf16_t*)beta, (bf16_t*)y, (float2*)stats, T, eps)
+		switch (d / 256) {
+			case 1: ELF_NORM_FWD_HALF(1); break;
+			case 2: ELF_NORM_FWD_HALF(2); break;
+			default: ELF_NORM_FWD_HALF(3); break;
+		}
+#undef ELF_NORM_FWD_HALF
+		ELF_CHECK_HIP(hipGetLastError());
+		return 0;
+	}
 #define ELF_NORM_FWD(N, W)                                                                                          \
 	ELF_LAUNCH((norm_fwd_kernel<N, W, LN>), dim3(W == 1 ? (T + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK : T), block, 0, \
 	                   s, (const bf16_t*)x, (const bf16_t*)gamma, (const bf16_t*)beta, (bf16_t*)y, (float2*)stats, T, d, eps)
@@ -308,6 +505,17 @@ template <bool LN>
 static int norm_bwd_dispatch(const void* dy, const void* x, const void* gamma, const void* stats, const void* dres,
                              void* dx, float* part, int T, int d, hipStream_t s) {
 	const dim3 grid(norm_bwd_blocks(T, d)), block(256);
+	if (norm_half_rows(d)) {
+#define ELF_NORM_BWD_HALF(N) ELF_LAUNCH((norm_bwd_half_kernel<N, LN>), grid, block, 0, s, (const bf16_t*)dy, (const bf16_t*)x, (const bf16_t*)gamma, (const float2*)stats, (const bf16_t*)dres, (bf16_t*)dx, part, T)
+		switch (d / 256) {
+			case 1: ELF_NORM_BWD_HALF(1); break;
+			case 2: ELF_NORM_BWD_HALF(2); break;
+			default: ELF_NORM_BWD_HALF(3); break;
+		}
+#undef ELF_NORM_BWD_HALF
+		ELF_CHECK_HIP(hipGetLastError());
+		return 0;
+	}
 #define ELF_NORM_BWD(N, W)                                                                                      \
 	ELF_LAUNCH((norm_bwd_kernel<N, W, LN>), grid, block, 0, s, (const bf16_t*)dy, (const bf16_t*)x,       \
 	                   (const bf16_t*)gamma, (const float2*)stats, (const bf16_t*)dres, (bf16_t*)dx, part, T, d)

@@ -369,6 +369,26 @@ static int dma_tile_rows(bool a_t, int M, int N, int K) {
 	return 0;
 }
 
+// K split of a weight gradient on 256x256 direct-to-LDS tiles when the caller leaves it open: *k_splits ways for the last
+// *tail_tiles tiles (-1: all of them).
+static void dw_split_plan(int M, int N, int K, int* k_splits, int* tail_tiles) {
+	const int64_t tiles = (int64_t)(M / 256) * (N / 256);
+	const int nk = K / 64;
+	*k_splits = 1;
+	*tail_tiles = -1;
+	if (tiles < 256) {
+		// too few tiles for the chip: split them all, down to 32 slices per workgroup (shorter
+		// ranges pay more in pipeline fill and atomics than the extra workgroups bring)
+		while (tiles * *k_splits * 2 <= 256 && nk / (*k_splits * 2) >= 32 && *k_splits < 16) *k_splits *= 2;
+	} else if (const int rem = (int)(tiles % 256); rem != 0 && rem <= 128) {
+		// the last round of workgroups would leave at least half of the CUs idle: split just those
+		// tiles so that they fill it with proportionally shorter workgroups
+		*k_splits = rem <= 64 ? 4 : 2;
+		*tail_tiles = rem;
+		if (nk / *k_splits < 16) *k_splits = 1;
+	}
+}
+
 int gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda, const void* B, int64_t ldb,
               void* C, int64_t ldc, int epi, const void* R, int64_t ldr, int tile_cfg, int k_splits,
               hipStream_t stream) {
@@ -397,13 +417,15 @@ int gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda,
 	g.K = K;
 	g.tiles_m = g.tiles_n = 0;
 	g.k_splits = k_splits;
-	// small weight gradients (24..128 tiles of 128x256, e.g. 2304x768 or 2048x2048 at K = 8192): 128x256 tiles with K
-	// split so that the workgroups just fill the chip once - 7-28 % faster than 256x256 tiles split further
+	// small weight gradients (12..128 tiles of 128x256, e.g. 2304x768 or 2048x2048 at K = 8192): 128x256 tiles with K
+	// split so that the workgroups just fill the chip once - 7-28 % faster than 256x256 tiles split further.  A split
+	// keeps at least 32 K slices, 16 where the tiles are so few (768x768: 18) that half of the chip would idle otherwise
 	if (tile_cfg <= 0 && epi == EPI_F32_ACC && a_t && b_t && k_splits <= 0 && M % 128 == 0 && N % 256 == 0 && K >= 4096) {
 		const int64_t tiles = (int64_t)(M / 128) * (N / 256);
-		if (tiles >= 24 && tiles <= 128) {
+		if (tiles >= 12 && tiles <= 128) {
 			int ks = (int)(256 / tiles);
-			if (ks > K / 64 / 32) ks = K / 64 / 32;
+			const int min_slices = tiles < 24 ? 16 : 32;
+			if (ks > K / 64 / min_slices) ks = K / 64 / min_slices;
 			return gemm_bf16_dma(a_t, b_t, M, N, K, A, lda, B, ldb, C, ldc, epi, R, ldr, ks < 1 ? 1 : ks, -1, 128, stream);
 		}
 	}
@@ -420,22 +442,7 @@ int gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda,
 	}
 	if (tile_cfg == 7) {
 		int tail_tiles = -1;  // an explicit k_splits splits every tile
-		if (epi == EPI_F32_ACC && k_splits <= 0) {
-			const int64_t tiles = (int64_t)(M / 256) * (N / 256);
-			const int nk = K / 64;
-			k_splits = 1;
-			if (tiles < 256) {
-				// too few tiles for the chip: split them all, down to 32 slices per workgroup (shorter
-				// ranges pay more in pipeline fill and atomics than the extra workgroups bring)
-				while (tiles * k_splits * 2 <= 256 && nk / (k_splits * 2) >= 32 && k_splits < 16) k_splits *= 2;
-			} else if (const int rem = (int)(tiles % 256); rem != 0 && rem <= 128) {
-				// the last round of workgroups would leave at least half of the CUs idle: split just those
-				// tiles so that they fill it with proportionally shorter workgroups
-				k_splits = rem <= 64 ? 4 : 2;
-				tail_tiles = rem;
-				if (nk / k_splits < 16) k_splits = 1;
-			}
-		}
+		if (epi == EPI_F32_ACC && k_splits <= 0) dw_split_plan(M, N, K, &k_splits, &tail_tiles);
 		return gemm_bf16_dma(a_t, b_t, M, N, K, A, lda, B, ldb, C, ldc, epi, R, ldr, k_splits, tail_tiles, 256, stream);
 	}
 	if (tile_cfg == 8) return gemm_bf16_dma(a_t, b_t, M, N, K, A, lda, B, ldb, C, ldc, epi, R, ldr, epi == EPI_F32_ACC && k_splits > 1 ? k_splits : 1, -1, 128, stream);
@@ -466,6 +473,23 @@ int gemm_act_bf16(int act, int M, int F, int K, const void* A, int64_t lda, cons
 	ELF_REQUIRE(ldpre == N && ldout == F, "gemm_act: the unfused path needs dense outputs");
 	if (int rc = gemm_bf16(0, 0, M, N, K, A, lda, W, ldw, pre, ldpre, EPI_BF16, nullptr, 0, 0, 0, stream)) return rc;
 	return act == ACT_SWIGLU ? swiglu_fwd(pre, out, M, F, stream) : gelu_fwd(pre, out, (int64_t)M * F, stream);
+}
+
+int gemm_dw_final(int M, int N, int K, const void* dY, int64_t lddy, const void* X, int64_t ldx, float* acc, void* grad_bf16, float scale,
+                  hipStream_t stream) {
+	ELF_REQUIRE(M > 0 && N > 0 && K > 0 && dY && X && acc && grad_bf16, "gemm_dw_final: bad argument");
+	const bool fused = M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && (int64_t)(M / 256) * (N / 256) >= 192 && lddy % 8 == 0 && ldx % 8 == 0 && lddy >= M &&
+	                   ldx >= N && ((uintptr_t)dY % 16) == 0 && ((uintptr_t)X % 16) == 0 && ((uintptr_t)acc % 16) == 0 && ((uintptr_t)grad_bf16 % 8) == 0;
+	if (fused) {
+		// the same K split as the plain weight gradient (same rounding); tiles shared by several workgroups along K have no
+		// single epilogue that could scale them: a small kernel behind the GEMM does those
+		int k_splits, tail_tiles;
+		dw_split_plan(M, N, K, &k_splits, &tail_tiles);
+		ProfScope prof(PROF_GEMM, 2.0 * M * N * K, stream);
+		return gemm_bf16_dma(1, 1, M, N, K, dY, lddy, X, ldx, acc, N, EPI_F32_ACC_SCALE, nullptr, 0, k_splits, tail_tiles, 256, stream, grad_bf16, N, nullptr, 0, 0, 0, scale);
+	}
+	if (int rc = gemm_bf16(1, 1, M, N, K, dY, lddy, X, ldx, acc, N, EPI_F32_ACC, nullptr, 0, 0, 0, stream)) return rc;
+	return scale_grads(acc, grad_bf16, (int64_t)M * N, scale, stream);
 }
 
 bool gemm_rope_fused(int M, int N, int K, int D) {

@@ -71,6 +71,7 @@ struct Args {
 	int rope_S, rope_cols, rope_D;
 	// split tiles: this launch's tag in the turn counters (see turn[] below); 0 = the splits add in any order
 	uint32_t turn_tag;
+	float scale;  // EPI_F32_ACC_SCALE
 };
 
 // Turn counters of split tiles.  The workgroups that share a tile along K add their parts with fp32 atomics; to make
@@ -619,7 +620,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 				*reinterpret_cast<bf16x8*>(reinterpret_cast<bf16_t*>(g.C) + (int64_t)(grow0 + row) * g.ldc + gcol0 + c8) = o;
 			}
 		} else {
-			if (EPI == EPI_F32_ACC && splits > 1) {
+			if ((EPI == EPI_F32_ACC || EPI == EPI_F32_ACC_SCALE) && splits > 1) {  // (split tiles of a scaling launch are scaled by scale_tail_kernel)
 				uint32_t* const my_turn = turn + turn_slot * TURN_PER_TILE + wave * RT + i;
 				if (g.turn_tag && ksplit > 0) {
 					// wait for this split's turn on this strip (see turn[]); every lane polls the same word.  Plain
@@ -657,8 +658,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 			// fp32 accumulate: the strip's 16 loads of C all in flight before the first store (left inside the
 			// loop each load is awaited on its own, 16 trips to HBM in a row per strip: 43 k cycles of a
 			// 360 k-cycle dW tile)
-			f32x4 cv[EPI == EPI_F32_ACC ? 16 : 1];
-			if constexpr (EPI == EPI_F32_ACC) {
+			constexpr bool ACCUM = EPI == EPI_F32_ACC || EPI == EPI_F32_ACC_SCALE;
+			f32x4 cv[ACCUM ? 16 : 1];
+			if constexpr (ACCUM) {
 #pragma unroll
 				for (int it = 0; it < 16; it++)
 					cv[it] = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(g.C) + (int64_t)(grow0 + it * 2 + (lane >> 5)) * g.ldc + gcol0 + (lane & 31) * 4);
@@ -668,7 +670,16 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 				const int row = it * 2 + (lane >> 5), c4 = (lane & 31) * 4;
 				f32x4 v = *reinterpret_cast<const f32x4*>(ws + row * PITCH + c4);
 				float* c = reinterpret_cast<float*>(g.C) + (int64_t)(grow0 + row) * g.ldc + gcol0 + c4;
-				if constexpr (EPI == EPI_F32_ACC) v += cv[it];
+				if constexpr (ACCUM) v += cv[it];
+				if constexpr (EPI == EPI_F32_ACC_SCALE) {
+					// the step's last weight-gradient pass: the gradient scale and the bf16 copy that scale_grads would make
+					// in a pass of its own over the accumulator (same operations on the same values: same bits)
+					v *= g.scale;
+					bf16x4 o;
+#pragma unroll
+					for (int t = 0; t < 4; t++) o[t] = (bf16_t)v[t];
+					*reinterpret_cast<bf16x4*>(g.C2 + (int64_t)(grow0 + row) * g.ldc2 + gcol0 + c4) = o;
+				}
 				*reinterpret_cast<f32x4*>(c) = v;
 			}
 		}
@@ -989,6 +1000,29 @@ static int launch_pers(const Args& a, hipStream_t stream) {
 	return 0;
 }
 
+
+// The split tiles of a launch with the scaling accumulate epilogue: their workgroups add partial sums and none of them
+// holds the finished tile, so the scale and the bf16 copy of those (few, at most 128) tiles are applied here, behind the
+// GEMM on the same stream.  One workgroup per tile; tile index and origin as in the GEMM.
+__global__ __launch_bounds__(256) void scale_tail_kernel(Args g) {
+	const int ntiles = g.tiles_m * g.tiles_n;
+	const int pid = ntiles - g.tail_tiles + (int)blockIdx.x;
+	int m0, n0;
+	tile_origin<256>(g, pid, m0, n0);
+	float* C = reinterpret_cast<float*>(g.C);
+	for (int i = threadIdx.x; i < 256 * 64; i += 256) {
+		const int row = i >> 6, c4 = (i & 63) * 4;
+		float* c = C + (int64_t)(m0 + row) * g.ldc + n0 + c4;
+		f32x4 v = *reinterpret_cast<const f32x4*>(c);
+		v *= g.scale;
+		bf16x4 o;
+#pragma unroll
+		for (int t = 0; t < 4; t++) o[t] = (bf16_t)v[t];
+		*reinterpret_cast<f32x4*>(c) = v;
+		*reinterpret_cast<bf16x4*>(g.C2 + (int64_t)(m0 + row) * g.ldc2 + n0 + c4) = o;
+	}
+}
+
 template <int NW, int RT, bool AT, bool BT, int EPI>
 static int launch(const Args& a, hipStream_t stream) {
 	// the ring + the target of the loads past the end of K (as many KiB as a wave issues loads per
@@ -1022,6 +1056,9 @@ static int launch_epi(const Args& a, int epi, hipStream_t stream) {
 	if constexpr (NW == 4 && RT == 4 && !AT && BT) {
 		if (epi == EPI_BF16_SWIGLU_BWD) return launch<NW, RT, AT, BT, EPI_BF16_SWIGLU_BWD>(a, stream);
 	}
+	if constexpr (NW == 8 && AT && BT) {
+		if (epi == EPI_F32_ACC_SCALE) return launch<NW, RT, AT, BT, EPI_F32_ACC_SCALE>(a, stream);
+	}
 	set_error("gemm: unknown epilogue %d", epi);
 	return -1;
 }
@@ -1039,17 +1076,18 @@ int dma_turn_giveups(uint64_t* out) {
 // Arguments are validated by gemm_bf16() before it dispatches here.
 int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda, const void* B, int64_t ldb, void* C,
                   int64_t ldc, int epi, const void* R, int64_t ldr, int k_splits, int tail_tiles, int bm, hipStream_t stream,
-                  void* C2, int64_t ldc2, const void* rope_cs, int rope_S, int rope_cols, int rope_D) {
+                  void* C2, int64_t ldc2, const void* rope_cs, int rope_S, int rope_cols, int rope_D, float scale) {
 	ELF_REQUIRE(bm == 256 || bm == 128, "gemm (dma tile): 256- or 128-row tiles");
 	ELF_REQUIRE(M % bm == 0 && N % dma::BN == 0 && K % dma::BKS == 0, "gemm (dma tile): M multiple of %d, N of 256 and K of 64 required", bm);
 	const int ntiles = (M / bm) * (N / dma::BN);
 	ELF_REQUIRE(epi != EPI_BF16_SWIGLU || (C2 && !a_t && !b_t), "gemm (dma tile): the SwiGLU epilogue needs k-contiguous operands and a second output");
 	// the paired rows of the SwiGLU epilogue are addressed with 32-bit byte offsets from the tile's first row
 	ELF_REQUIRE(epi != EPI_BF16_SWIGLU || (int64_t)(N / 2 + 256) * ldb * 2 < (int64_t(1) << 31), "gemm (dma tile): weight too large for the paired-row epilogue");
+	ELF_REQUIRE(epi != EPI_F32_ACC_SCALE || (C2 && a_t && b_t && bm == 256), "gemm (dma tile): the scaling accumulate epilogue needs reduction-major operands, 256-row tiles and a bf16 output");
 	ELF_REQUIRE(epi != EPI_BF16_ROPE || (rope_cs && rope_S > 0 && !a_t && !b_t && (rope_D == 64 || rope_D == 128) && rope_cols % rope_D == 0 && rope_cols <= N),
 	            "gemm (dma tile): the RoPE epilogue needs k-contiguous operands, a table and heads of 64 or 128 columns");
 	dma::Args a{(const bf16_t*)A, (const bf16_t*)B, C, (const bf16_t*)R, (bf16_t*)C2, lda, ldb, ldc, ldr, ldc2, M, N, K, M / bm, N / dma::BN, k_splits < 1 ? 1 : k_splits,
-	            tail_tiles < 0 || tail_tiles > ntiles ? ntiles : tail_tiles, 0, (const float2*)rope_cs, rope_S, rope_cols, rope_D, 0};
+	            tail_tiles < 0 || tail_tiles > ntiles ? ntiles : tail_tiles, 0, (const float2*)rope_cs, rope_S, rope_cols, rope_D, 0, scale};
 	// The band walk fetches every row slab of A from HBM in one round only and B once per band; the default
 	// walk wants A in the 256 MB memory-side cache for the whole launch and streams B once.  Inside the stage's
 	// stream (operands cold, per-shape times from a kernel trace) the bands are 0-5 % faster on every shape but
@@ -1057,7 +1095,7 @@ int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t 
 	// slower), which keeps the default.
 	const int64_t big = int64_t(160) << 20;
 	a.walk = !((int64_t)M * K * 2 < big && (int64_t)N * K * 2 >= big);
-	if (epi != EPI_F32_ACC || a.k_splits == 1) a.k_splits = 1, a.tail_tiles = 0;
+	if ((epi != EPI_F32_ACC && epi != EPI_F32_ACC_SCALE) || a.k_splits == 1) a.k_splits = 1, a.tail_tiles = 0;
 	// split tiles add in a fixed order (bit-reproducible weight gradients) as long as each has a counter of its own
 	a.turn_tag = a.tail_tiles > 0 && a.tail_tiles <= dma::TURN_TILES ? next_turn_tag() : 0;
 	if (bm == 128) {
@@ -1081,7 +1119,14 @@ int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t 
 	}
 	if (!a_t && !b_t) return dma::launch_epi<4, 4, false, false>(a, epi, stream);
 	if (!a_t && b_t) return dma::launch_epi<4, 4, false, true>(a, epi, stream);
-	if (a_t && b_t) return dma::launch_epi<8, 2, true, true>(a, epi, stream);
+	if (a_t && b_t) {
+		if (int rc = dma::launch_epi<8, 2, true, true>(a, epi, stream)) return rc;
+		if (epi == EPI_F32_ACC_SCALE && a.tail_tiles > 0) {
+			ELF_LAUNCH(dma::scale_tail_kernel, dim3(a.tail_tiles), dim3(256), 0, stream, a);
+			ELF_CHECK_HIP(hipGetLastError());
+		}
+		return 0;
+	}
 	set_error("gemm: layout A=T,B=R is not used by any stage contraction");
 	return -1;
 }

@@ -21,6 +21,8 @@ enum GemmEpilogue {
 	// k-contiguous operands (see gemm_rope_bf16): C(bf16) = acc rounded to bf16, then the half-split rotary rotation of
 	// the heads (width rope_D) that lie in the first rope_cols columns, position = row mod rope_S
 	EPI_BF16_ROPE = 6,
+	// both operands reduction-major, 256x256 direct-to-LDS tiles without a K split (see gemm_dw_final):
+	EPI_F32_ACC_SCALE = 7,  // C(fp32) = (C + acc) * scale, C2(bf16) = bf16 of that
 };
 
 int gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda, const void* B, int64_t ldb,
@@ -32,7 +34,16 @@ int gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda,
 // EPI_F32_ACC only: the last tail_tiles tiles (all of them when tail_tiles < 0) are split k_splits ways along K.
 int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t lda, const void* B, int64_t ldb, void* C,
                   int64_t ldc, int epi, const void* R, int64_t ldr, int k_splits, int tail_tiles, int bm, hipStream_t stream,
-                  void* C2 = nullptr, int64_t ldc2 = 0, const void* rope_cs = nullptr, int rope_S = 0, int rope_cols = 0, int rope_D = 0);
+                  void* C2 = nullptr, int64_t ldc2 = 0, const void* rope_cs = nullptr, int rope_S = 0, int rope_cols = 0, int rope_D = 0,
+                  float scale = 1.f);
+
+// The weight gradient of the step's last micro-batch with the step's gradient scale folded in: acc [M, N] (fp32, dense)
+// = (acc + dY^T X) * scale and grad_bf16 [M, N] = bf16(acc), with dY [K, M] and X [K, N] (both reduction-major).  One
+// kernel when the shape fills the chip with whole 256x256 tiles (the scale and the bf16 copy leave from the epilogue
+// that holds the fp32 tile anyway); otherwise gemm_bf16 (epilogue 2) followed by scale_grads.  Same bits either way:
+// one fp32 add, one fp32 multiply, one rounding to bf16 per element.
+int gemm_dw_final(int M, int N, int K, const void* dY, int64_t lddy, const void* X, int64_t ldx, float* acc, void* grad_bf16, float scale,
+                  hipStream_t stream);
 
 // The attention block's packed q | k | v projection with the rotary embedding of the q and k heads: C [M, N] =
 // A W^T rounded to bf16, then rope_apply's rotation on the first n_rot_heads heads of width D (cs: the table of

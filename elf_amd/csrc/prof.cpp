@@ -83,7 +83,8 @@ int prof_collect(int kind, double* total_ms, double* total_work) {
 // ---------------------------------------------------------------------------------------------
 // What this GPU's memory system sustains for the simplest access patterns: the yardstick the bandwidth-bound
 // kernels are compared with.  mode 0: read n bytes (every lane sums 16-byte loads; one value per workgroup is
-// written), 1: copy n bytes, 2: write n bytes.
+// written), 1: copy n bytes, 2: write n bytes, 3: read three streams of n bytes (src, src + n, src + 2 n) and write one
+// (their XOR): the pattern of a normalisation backward (dy, x, residual gradient in; dx out).
 // A workgroup takes contiguous chunks of 256 lanes x U x 16 bytes and strides over the buffer by the grid; V = 1 uses
 // non-temporal stores.
 template <int MODE, int U, int V>
@@ -96,6 +97,7 @@ __global__ __launch_bounds__(256) void hbm_probe_kernel(const u32x4* __restrict_
 		for (int u = 0; u < U; u++) {
 			const int64_t i = base + u * 256 + threadIdx.x;
 			if constexpr (MODE == 2) v[u] = u32x4{(uint32_t)i, 1u, 2u, 3u};
+			else if constexpr (MODE == 3) v[u] = i < n16 ? src[i] ^ src[i + n16] ^ src[i + 2 * n16] : u32x4{0u, 0u, 0u, 0u};
 			else v[u] = i < n16 ? src[i] : u32x4{0u, 0u, 0u, 0u};
 		}
 #pragma unroll
@@ -112,13 +114,14 @@ __global__ __launch_bounds__(256) void hbm_probe_kernel(const u32x4* __restrict_
 }
 
 int hbm_probe(int mode, const void* src, void* dst, int64_t bytes, hipStream_t s) {
-	ELF_REQUIRE(mode >= 0 && mode <= 2 && dst && (mode == 2 || src) && bytes >= 16 && bytes % 16 == 0, "hbm_probe: bad argument");
+	ELF_REQUIRE(mode >= 0 && mode <= 3 && dst && (mode == 2 || src) && bytes >= 16 && bytes % 16 == 0, "hbm_probe: bad argument");
 	ELF_REQUIRE(((uintptr_t)src % 16) == 0 && ((uintptr_t)dst % 16) == 0, "hbm_probe: buffers must be 16-byte aligned");
 	const int64_t n16 = bytes / 16;
 	const dim3 block(256);
 	// the best of unroll 4 / 8, 1024 / 2048 / 8192 workgroups and plain / non-temporal stores for each pattern at 1 GiB
 	if (mode == 0) ELF_LAUNCH((hbm_probe_kernel<0, 4, 0>), dim3(1024), block, 0, s, (const u32x4*)src, (u32x4*)dst, n16);
 	else if (mode == 1) ELF_LAUNCH((hbm_probe_kernel<1, 4, 1>), dim3(8192), block, 0, s, (const u32x4*)src, (u32x4*)dst, n16);
+	else if (mode == 3) ELF_LAUNCH((hbm_probe_kernel<3, 4, 1>), dim3(8192), block, 0, s, (const u32x4*)src, (u32x4*)dst, n16);
 	else ELF_LAUNCH((hbm_probe_kernel<2, 8, 0>), dim3(8192), block, 0, s, (const u32x4*)src, (u32x4*)dst, n16);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;

@@ -49,9 +49,11 @@ static const unsigned WIN_MASK = (1u << B_H1) | (1u << B_O) | (1u << B_H2) | (1u
 // link twice (a third of the stash bytes; the same kernels on the same inputs: bit-identical).  A stage with a
 // lean stash (elf_stage_set_lean_stash) does the same for every micro-batch, to hold less between F and B.
 static const unsigned REFORM_MASK = (1u << B_H1) | (1u << B_H2) | (1u << B_A);
-// An offloaded micro-batch also leaves out the QKV projection's output: one GEMM over the re-formed norm
-// output (plus RoPE) costs a third of the link time its 2 x 168 MB would take at the 70B shape.
-static const unsigned OFFLOAD_REFORM_MASK = REFORM_MASK | (1u << B_QKV);
+// An offloaded micro-batch also leaves out the outputs of the two projections that a GEMM over buffers it holds anyway
+// gives back for a third of their link time: the QKV projection's output (one GEMM over the re-formed norm output, plus
+// RoPE: 1.0 ms against 2 x 3.4 ms of link time for its 168 MB at the 70B shape) and the attention residual x2 = x + o Wo^T
+// (0.8 ms against 2 x 2.7 ms for 134 MB; the forward's own GEMM call with its residual epilogue: bit-identical).
+static const unsigned OFFLOAD_REFORM_MASK = REFORM_MASK | (1u << B_QKV) | (1u << B_X2);
 static const unsigned WGRAD_MASK = (1u << B_DY) | (1u << B_DGU) | (1u << B_DX2) | (1u << B_DQKV);
 
 enum ParamId { P_NORM1_G = 0, P_NORM1_B, P_WQKV, P_WO, P_NORM2_G, P_NORM2_B, P_W1, P_W2, P_COUNT };
@@ -69,10 +71,12 @@ struct Buf {
 
 struct BlockState {
 	Buf b[B_COUNT];
-	// offload copies run block by block: this block's device->host copies are done at off_ev,
-	// its host->device copies, which come in the order B needs them, at pre_ffn (gate/up product), pre_x2
-	// (+ the FFN norm's input) and pre_ev (everything)
-	hipEvent_t off_ev = nullptr, pre_ev = nullptr, pre_ffn = nullptr, pre_x2 = nullptr;
+	// offload copies run block by block: this block's device->host copies are done at off_ev; its host->device copies
+	// come in the order B needs them: the FFN pre-activation in row chunks (pre_gu[c] after chunk c: B's activation
+	// backward and the GEMM behind it run chunk by chunk while the rest is still on the link), then everything else (pre_ev)
+	static constexpr int MAX_GU_CHUNKS = 4;
+	hipEvent_t off_ev = nullptr, pre_ev = nullptr, pre_gu[MAX_GU_CHUNKS] = {};
+	int gu_chunks = 1;  // row chunks of the last restore
 };
 
 struct MbState {
@@ -90,6 +94,7 @@ struct MbState {
 struct BlockParams {
 	void* w[P_COUNT] = {};
 	float* g[P_COUNT] = {};
+	void* g16[P_COUNT] = {};  // bf16 copies of the scaled gradients (elf_stage_bind_grad_bf16), linear layers only
 };
 
 enum FwdMode { SAVE_ALL, SAVE_WIN, SAVE_NONE };
@@ -106,6 +111,7 @@ struct Stage {
 	bool lean = false;  // elf_stage_set_lean_stash: F keeps no REFORM_MASK buffer, B forms them again
 	void* xw[XP_COUNT] = {};
 	float* xg[XP_COUNT] = {};
+	void* xg16[XP_COUNT] = {};
 	std::map<int, MbState> mbs;
 	// micro-batches with fewer sequences than cfg.mb (the last one of a batch the split size does not
 	// divide): T and B above are set from here at every entry point (one host thread per stage)
@@ -201,9 +207,11 @@ static void destroy_events(MbState& m) {
 	for (auto& bs : m.blk) {
 		if (bs.off_ev) (void)hipEventDestroy(bs.off_ev);
 		if (bs.pre_ev) (void)hipEventDestroy(bs.pre_ev);
-		if (bs.pre_ffn) (void)hipEventDestroy(bs.pre_ffn);
-		if (bs.pre_x2) (void)hipEventDestroy(bs.pre_x2);
-		bs.off_ev = bs.pre_ev = bs.pre_ffn = bs.pre_x2 = nullptr;
+		for (auto& ev : bs.pre_gu) {
+			if (ev) (void)hipEventDestroy(ev);
+			ev = nullptr;
+		}
+		bs.off_ev = bs.pre_ev = nullptr;
 	}
 }
 
@@ -377,26 +385,73 @@ static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool gra
 		// FFN: dY W2 and the activation's backward, in one kernel for SwiGLU where the shape allows (a prefetched
 		// micro-batch keeps them apart: the GEMM then runs while the gate/up product is still on the link)
 		ELF_TRY(buf_alloc(s, bs, B_DGU));
+		PoolTmp d_h(s->pool, (size_t)T * d * 2);
+		if (!d_h.p) return -3;
 		if (s->llama && !pre && gemm_swiglu_bwd_fused(T, F, d)) {
 			ELF_TRY(gemm_swiglu_bwd_bf16(T, F, d, dyin, d, p.w[P_W2], F, bs.b[B_GU].p, s->ffn_in, bs.b[B_DGU].p, s->ffn_in, nullptr, st));
+			if (reform && bs.b[B_A].dropped) {
+				ELF_TRY(buf_alloc(s, bs, B_A));
+				ELF_TRY(swiglu_fwd(bs.b[B_GU].p, bs.b[B_A].p, T, F, st));
+			}
+			ELF_TRY(gemm_bf16(0, 1, T, d, s->ffn_in, bs.b[B_DGU].p, s->ffn_in, p.w[P_W1], d, d_h.p, d, EPI_BF16, nullptr, 0, 0, 0, st));
 		} else {
 			PoolTmp d_a(s->pool, (size_t)T * F * 2);
 			if (!d_a.p) return -3;
 			ELF_TRY(gemm_bf16(0, 1, T, F, d, dyin, d, p.w[P_W2], F, d_a.p, F, EPI_BF16, nullptr, 0, 0, 0, st));
-			if (pre) ELF_CHECK_HIP(hipStreamWaitEvent(st, bs.pre_ffn, 0));
-			if (s->llama) ELF_TRY(swiglu_bwd(d_a.p, bs.b[B_GU].p, bs.b[B_DGU].p, T, F, st));
-			else ELF_TRY(gelu_bwd(d_a.p, bs.b[B_GU].p, bs.b[B_DGU].p, (int64_t)T * F, st));
+			const bool form_a = reform && bs.b[B_A].dropped;
+			if (form_a) ELF_TRY(buf_alloc(s, bs, B_A));
+			// a prefetched micro-batch: row chunk by row chunk as the pre-activation arrives (elementwise kernels and a
+			// GEMM whose rows are independent: the same bits as in one piece)
+			const int nch = pre ? bs.gu_chunks : 1;
+			const int Tc = T / nch;
+			for (int c = 0; c < nch; c++) {
+				if (pre) ELF_CHECK_HIP(hipStreamWaitEvent(st, bs.pre_gu[c], 0));
+				const bf16_t* gu_c = (const bf16_t*)bs.b[B_GU].p + (size_t)c * Tc * s->ffn_in;
+				bf16_t* dgu_c = (bf16_t*)bs.b[B_DGU].p + (size_t)c * Tc * s->ffn_in;
+				const bf16_t* da_c = (const bf16_t*)d_a.p + (size_t)c * Tc * F;
+				if (s->llama) ELF_TRY(swiglu_bwd(da_c, gu_c, dgu_c, Tc, F, st));
+				else ELF_TRY(gelu_bwd(da_c, gu_c, dgu_c, (int64_t)Tc * F, st));
+				if (form_a) {
+					bf16_t* a_c = (bf16_t*)bs.b[B_A].p + (size_t)c * Tc * F;
+					if (s->llama) ELF_TRY(swiglu_fwd(gu_c, a_c, Tc, F, st));
+					else ELF_TRY(gelu_fwd(gu_c, a_c, (int64_t)Tc * F, st));
+				}
+				ELF_TRY(gemm_bf16(0, 1, Tc, d, s->ffn_in, dgu_c, s->ffn_in, p.w[P_W1], d, (bf16_t*)d_h.p + (size_t)c * Tc * d, d, EPI_BF16, nullptr, 0, 0, 0, st));
+			}
 		}
-		if (reform && bs.b[B_A].dropped) {
-			ELF_TRY(buf_alloc(s, bs, B_A));
-			if (s->llama) ELF_TRY(swiglu_fwd(bs.b[B_GU].p, bs.b[B_A].p, T, F, st));
-			else ELF_TRY(gelu_fwd(bs.b[B_GU].p, bs.b[B_A].p, (int64_t)T * F, st));
-		}
-		PoolTmp d_h(s->pool, (size_t)T * d * 2);
-		if (!d_h.p) return -3;
-		ELF_TRY(gemm_bf16(0, 1, T, d, s->ffn_in, bs.b[B_DGU].p, s->ffn_in, p.w[P_W1], d, d_h.p, d, EPI_BF16, nullptr, 0, 0, 0, st));
 		ELF_TRY(buf_alloc(s, bs, B_DX2));
-		if (pre) ELF_CHECK_HIP(hipStreamWaitEvent(st, bs.pre_x2, 0));
+		if (pre) ELF_CHECK_HIP(hipStreamWaitEvent(st, bs.pre_ev, 0));  // the rest of the block's stash
+		// what the attention backward reads and the offload / lean stash / module checkpoints dropped, formed again with the
+		// forward's own calls: the first norm's output and statistics, the QKV projection, the attention output and log-sum-exp
+		auto reform_attention_inputs = [&]() -> int {
+			if ((bs.b[B_H1].dropped && (reform || bs.b[B_QKV].dropped)) || bs.b[B_ST1].dropped) {
+				ELF_TRY(buf_alloc(s, bs, B_H1));
+				ELF_TRY(buf_alloc(s, bs, B_ST1));
+				ELF_TRY(norm_fwd(norm_kind, bs.b[B_X].p, p.w[P_NORM1_G], p.w[P_NORM1_B], bs.b[B_H1].p, bs.b[B_ST1].p, T, d, s->cfg.eps, st));
+			}
+			if (bs.b[B_QKV].dropped) {
+				ELF_TRY(buf_alloc(s, bs, B_QKV));
+				if (s->llama) ELF_TRY(gemm_rope_bf16(T, s->nqkv, d, bs.b[B_H1].p, d, p.w[P_WQKV], d, bs.b[B_QKV].p, s->nqkv, s->rope_cs, s->S, s->Hq + s->Hkv, s->D, st));
+				else ELF_TRY(gemm_bf16(0, 0, T, s->nqkv, d, bs.b[B_H1].p, d, p.w[P_WQKV], d, bs.b[B_QKV].p, s->nqkv, EPI_BF16, nullptr, 0, 0, 0, st));
+			}
+			if (bs.b[B_LSE].dropped) {  // checkpointed attention core: its output and log-sum-exp are formed again
+				ELF_TRY(buf_alloc(s, bs, B_O));
+				ELF_TRY(buf_alloc(s, bs, B_LSE));
+				const bf16_t* q = (const bf16_t*)bs.b[B_QKV].p;
+				ELF_TRY(attn_fwd(q, q + s->Hq * s->D, q + (s->Hq + s->Hkv) * s->D, bs.b[B_O].p, bs.b[B_LSE].p, s->nqkv, s->nqkv, s->nqkv,
+				                 s->Hq * s->D, s->B, s->S, s->Hq, s->Hkv, s->D, s->cfg.causal, scale, st));
+			}
+			return 0;
+		};
+		bool attention_inputs_ready = false;
+		if (bs.b[B_X2].dropped && bs.b[B_LSE].dropped) {  // x2 needs the attention output, which a checkpointed attention core dropped as well
+			ELF_TRY(reform_attention_inputs());
+			attention_inputs_ready = true;
+		}
+		if (bs.b[B_X2].dropped) {  // not moved over the host link: x2 = x + o Wo^T, the forward's own call
+			ELF_TRY(buf_alloc(s, bs, B_X2));
+			ELF_TRY(gemm_bf16(0, 0, T, d, s->Hq * s->D, bs.b[B_O].p, s->Hq * s->D, p.w[P_WO], s->Hq * s->D, bs.b[B_X2].p, d, EPI_BF16_RESID, bs.b[B_X].p, d, 0, 0, st));
+		}
 		if ((reform && bs.b[B_H2].dropped) || bs.b[B_ST2].dropped) {  // dropped by the lean stash / offload, or a checkpointed norm
 			ELF_TRY(buf_alloc(s, bs, B_H2));
 			ELF_TRY(buf_alloc(s, bs, B_ST2));
@@ -409,24 +464,7 @@ static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool gra
 		if (!d_o.p) return -3;
 		ELF_TRY(gemm_bf16(0, 1, T, s->Hq * s->D, d, bs.b[B_DX2].p, d, p.w[P_WO], s->Hq * s->D, d_o.p, s->Hq * s->D, EPI_BF16, nullptr, 0, 0, 0, st));
 		ELF_TRY(buf_alloc(s, bs, B_DQKV));
-		if (pre) ELF_CHECK_HIP(hipStreamWaitEvent(st, bs.pre_ev, 0));
-		if ((bs.b[B_H1].dropped && (reform || bs.b[B_QKV].dropped)) || bs.b[B_ST1].dropped) {
-			ELF_TRY(buf_alloc(s, bs, B_H1));
-			ELF_TRY(buf_alloc(s, bs, B_ST1));
-			ELF_TRY(norm_fwd(norm_kind, bs.b[B_X].p, p.w[P_NORM1_G], p.w[P_NORM1_B], bs.b[B_H1].p, bs.b[B_ST1].p, T, d, s->cfg.eps, st));
-		}
-		if (bs.b[B_QKV].dropped) {
-			ELF_TRY(buf_alloc(s, bs, B_QKV));
-			if (s->llama) ELF_TRY(gemm_rope_bf16(T, s->nqkv, d, bs.b[B_H1].p, d, p.w[P_WQKV], d, bs.b[B_QKV].p, s->nqkv, s->rope_cs, s->S, s->Hq + s->Hkv, s->D, st));
-			else ELF_TRY(gemm_bf16(0, 0, T, s->nqkv, d, bs.b[B_H1].p, d, p.w[P_WQKV], d, bs.b[B_QKV].p, s->nqkv, EPI_BF16, nullptr, 0, 0, 0, st));
-		}
-		if (bs.b[B_LSE].dropped) {  // checkpointed attention core: its output and log-sum-exp are formed again
-			ELF_TRY(buf_alloc(s, bs, B_O));
-			ELF_TRY(buf_alloc(s, bs, B_LSE));
-			const bf16_t* q = (const bf16_t*)bs.b[B_QKV].p;
-			ELF_TRY(attn_fwd(q, q + s->Hq * s->D, q + (s->Hq + s->Hkv) * s->D, bs.b[B_O].p, bs.b[B_LSE].p, s->nqkv, s->nqkv, s->nqkv,
-			                 s->Hq * s->D, s->B, s->S, s->Hq, s->Hkv, s->D, s->cfg.causal, scale, st));
-		}
+		if (!attention_inputs_ready) ELF_TRY(reform_attention_inputs());
 		{
 			const bf16_t* q = (const bf16_t*)bs.b[B_QKV].p;
 			bf16_t* dq = (bf16_t*)bs.b[B_DQKV].p;
@@ -468,20 +506,25 @@ static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool gra
 	return 0;
 }
 
-static int run_backward_params(Stage* s, MbState& m, hipStream_t st) {
+// scale != 0: the step's last W pass; every linear layer's accumulator leaves it multiplied by `scale`, with its bf16
+// copy written (PipelineBlock.scale_grads, elf/execution/block.py:518-527, folded into the pass that holds the tiles).
+static int run_backward_params(Stage* s, MbState& m, hipStream_t st, float scale = 0.f) {
 	const int T = s->T, d = s->d, F = s->F;
+	// dW[N_out, K_in] += dY[T, N_out]^T X[T, K_in]
+	auto dw = [&](int M, int N, const void* dy, int64_t lddy, const void* x, int64_t ldx, float* acc, void* g16) -> int {
+		if (scale != 0.f) return gemm_dw_final(M, N, T, dy, lddy, x, ldx, acc, g16, scale, st);
+		return gemm_bf16(1, 1, M, N, T, dy, lddy, x, ldx, acc, N, EPI_F32_ACC, nullptr, 0, 0, 0, st);
+	};
 	for (int i = 0; i < s->cfg.n_blocks; i++) {
 		BlockState& bs = m.blk[i];
 		const BlockParams& p = s->params[i];
 		const int hd = s->Hq * s->D;
-		// dW[N_out, K_in] += dY[T, N_out]^T X[T, K_in]
-		ELF_TRY(gemm_bf16(1, 1, d, F, T, bs.b[B_DY].p, d, bs.b[B_A].p, F, p.g[P_W2], F, EPI_F32_ACC, nullptr, 0, 0, 0, st));
-		ELF_TRY(gemm_bf16(1, 1, s->ffn_in, d, T, bs.b[B_DGU].p, s->ffn_in, bs.b[B_H2].p, d, p.g[P_W1], d, EPI_F32_ACC, nullptr, 0, 0, 0, st));
-		ELF_TRY(gemm_bf16(1, 1, d, hd, T, bs.b[B_DX2].p, d, bs.b[B_O].p, hd, p.g[P_WO], hd, EPI_F32_ACC, nullptr, 0, 0, 0, st));
-		ELF_TRY(gemm_bf16(1, 1, s->nqkv, d, T, bs.b[B_DQKV].p, s->nqkv, bs.b[B_H1].p, d, p.g[P_WQKV], d, EPI_F32_ACC, nullptr, 0, 0, 0, st));
+		ELF_TRY(dw(d, F, bs.b[B_DY].p, d, bs.b[B_A].p, F, p.g[P_W2], p.g16[P_W2]));
+		ELF_TRY(dw(s->ffn_in, d, bs.b[B_DGU].p, s->ffn_in, bs.b[B_H2].p, d, p.g[P_W1], p.g16[P_W1]));
+		ELF_TRY(dw(d, hd, bs.b[B_DX2].p, d, bs.b[B_O].p, hd, p.g[P_WO], p.g16[P_WO]));
+		ELF_TRY(dw(s->nqkv, d, bs.b[B_DQKV].p, s->nqkv, bs.b[B_H1].p, d, p.g[P_WQKV], p.g16[P_WQKV]));
 	}
-	if (s->vocab_out)
-		ELF_TRY(gemm_bf16(1, 1, s->vld, d, T, m.head.b[B_DQKV].p, s->vld, m.head.b[B_H1].p, d, s->xg[XP_HEAD], d, EPI_F32_ACC, nullptr, 0, 0, 0, st));
+	if (s->vocab_out) ELF_TRY(dw(s->vld, d, m.head.b[B_DQKV].p, s->vld, m.head.b[B_H1].p, d, s->xg[XP_HEAD], s->xg16[XP_HEAD]));
 	free_mask(s, m, WIN_MASK | WGRAD_MASK);
 	m.has_win = m.has_wgrad = false;
 	return 0;
@@ -559,23 +602,41 @@ static int do_restore(Stage* s, MbState& m, bool async, hipStream_t st) {
 		ELF_CHECK_HIP(hipStreamWaitEvent(cs, now, 0));
 		ELF_CHECK_HIP(hipEventDestroy(now));
 	}
+	// Row chunks of the FFN pre-activation (by far the largest buffer: 940 of 1210 MB per block at the 70B shape): as
+	// many as keep each chunk's GEMM in B on the tiles the whole GEMM uses (at least 192 tiles of 256 x 256), so that
+	// chunked and whole give the same bits.
+	int nch = 1;
+	for (int n : {4, 2})
+		if (nch == 1 && n <= BlockState::MAX_GU_CHUNKS && s->T % (n * 256) == 0 && s->d % 256 == 0 && (int64_t)(s->T / n / 256) * (s->d / 256) >= 192) nch = n;
 	for (int i = (int)m.blk.size() - 1; i >= 0; i--) {
 		BlockState& bs = m.blk[i];
 		if (bs.off_ev) ELF_CHECK_HIP(hipStreamWaitEvent(cs, bs.off_ev, 0));
-		// in the order B reads them: the gate/up product (activation backward, after one GEMM), the FFN norm's
-		// input and statistics, then the attention's and the first norm's buffers
-		static const int order[] = {B_GU, B_X2, B_ST2, B_O, B_LSE, B_QKV, B_X, B_ST1};
+		// in the order B reads them: the gate/up product (activation backward, after one GEMM), then the block input and
+		// the attention's buffers (x2, the norm outputs and the QKV projection are formed again from these)
+		static const int order[] = {B_GU, B_X, B_ST1, B_ST2, B_O, B_LSE, B_X2, B_QKV};
 		static_assert(sizeof(order) / sizeof(order[0]) == 8, "every ACT_MASK buffer outside REFORM_MASK is listed");
+		bs.gu_chunks = async ? nch : 1;
 		for (int id : order) {
 			Buf& b = bs.b[id];
+			if (id == B_GU && b.offloaded && async) {
+				const size_t piece = b.bytes / nch;  // whole rows: bytes = T * ffn_in * 2 and T % nch == 0
+				for (int c = 0; c < nch; c++) {
+					ELF_CHECK_HIP(hipMemcpyAsync((char*)b.p + c * piece, (const char*)b.host.ptr + c * piece, piece, hipMemcpyHostToDevice, cs));
+					if (!bs.pre_gu[c]) ELF_CHECK_HIP(hipEventCreateWithFlags(&bs.pre_gu[c], hipEventDisableTiming));
+					ELF_CHECK_HIP(hipEventRecord(bs.pre_gu[c], cs));
+				}
+				s->h2d_bytes += (int64_t)b.bytes;
+				continue;
+			}
 			if (b.offloaded) {
 				ELF_CHECK_HIP(hipMemcpyAsync(b.p, b.host.ptr, b.bytes, hipMemcpyHostToDevice, cs));
 				s->h2d_bytes += (int64_t)b.bytes;
 			}
-			if (async && (id == B_GU || id == B_ST2)) {
-				hipEvent_t& ev = id == B_GU ? bs.pre_ffn : bs.pre_x2;
-				if (!ev) ELF_CHECK_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
-				ELF_CHECK_HIP(hipEventRecord(ev, cs));
+			if (id == B_GU && async) {  // nothing to copy (the buffer was small enough to stay): its events fire at once
+				for (int c = 0; c < nch; c++) {
+					if (!bs.pre_gu[c]) ELF_CHECK_HIP(hipEventCreateWithFlags(&bs.pre_gu[c], hipEventDisableTiming));
+					ELF_CHECK_HIP(hipEventRecord(bs.pre_gu[c], cs));
+				}
 			}
 		}
 		if (async) {
@@ -813,9 +874,36 @@ int elf_stage_backward_inputs(elf_stage_t* h, int mb, const void* x, const void*
 	return 0;
 }
 
-int elf_stage_backward_params(elf_stage_t* h, int mb, void* stream) {
+int elf_stage_bind_grad_bf16(elf_stage_t* h, int block, int which, void* grad_bf16) {
 	Stage* s = (Stage*)h;
-	ELF_REQUIRE(s && mb >= 0, "elf_stage_backward_params: bad argument");
+	ELF_REQUIRE(s && grad_bf16 && ((uintptr_t)grad_bf16 % 16) == 0, "elf_stage_bind_grad_bf16: null stage or null / misaligned pointer");
+	if (block == -1) {
+		ELF_REQUIRE(which == ELF_P_HEAD, "elf_stage_bind_grad_bf16: of the stage-level parameters only the output head (%d) is a linear layer", ELF_P_HEAD);
+		s->xg16[XP_HEAD] = grad_bf16;
+		return 0;
+	}
+	ELF_REQUIRE(block >= 0 && block < s->cfg.n_blocks, "elf_stage_bind_grad_bf16: block %d out of range", block);
+	ELF_REQUIRE(which == P_WQKV || which == P_WO || which == P_W1 || which == P_W2, "elf_stage_bind_grad_bf16: parameter %d is not a linear layer's weight", which);
+	s->params[block].g16[which] = grad_bf16;
+	return 0;
+}
+
+static int backward_params_entry(elf_stage_t* h, int mb, float scale, void* stream, const char* who);
+
+int elf_stage_backward_params_scaled(elf_stage_t* h, int mb, float scale, void* stream) {
+	Stage* s = (Stage*)h;
+	ELF_REQUIRE(s && scale != 0.f && scale == scale, "elf_stage_backward_params_scaled: null stage or a scale that is zero or not a number");
+	for (int i = 0; i < s->cfg.n_blocks; i++)
+		for (int w : {P_WQKV, P_WO, P_W1, P_W2}) ELF_REQUIRE(s->params[i].g16[w] != nullptr, "elf_stage_backward_params_scaled: bf16 gradient buffer %d of block %d not bound", w, i);
+	ELF_REQUIRE(!s->vocab_out || s->xg16[XP_HEAD], "elf_stage_backward_params_scaled: bf16 gradient buffer of the output head not bound");
+	return backward_params_entry(h, mb, scale, stream, "elf_stage_backward_params_scaled");
+}
+
+int elf_stage_backward_params(elf_stage_t* h, int mb, void* stream) { return backward_params_entry(h, mb, 0.f, stream, "elf_stage_backward_params"); }
+
+static int backward_params_entry(elf_stage_t* h, int mb, float scale, void* stream, const char* who) {
+	Stage* s = (Stage*)h;
+	ELF_REQUIRE(s && mb >= 0, "%s: bad argument", who);
 	auto it = s->mbs.find(mb);
 	ELF_REQUIRE(it != s->mbs.end() && it->second.has_win && it->second.has_wgrad,
 	            "elf_stage_backward_params: micro-batch %d has no saved inputs / output gradients (run B, or the recompute ops, first)", mb);
@@ -823,7 +911,7 @@ int elf_stage_backward_params(elf_stage_t* h, int mb, void* stream) {
 		for (int w : {P_WQKV, P_WO, P_W1, P_W2}) ELF_REQUIRE(s->params[i].g[w] != nullptr, "elf_stage_backward_params: gradient buffer not bound");
 	ELF_REQUIRE(!s->vocab_out || s->xg[XP_HEAD], "elf_stage_backward_params: gradient buffer of the output head not bound");
 	use_mb(s, mb);
-	ELF_TRY(run_backward_params(s, it->second, (hipStream_t)stream));
+	ELF_TRY(run_backward_params(s, it->second, (hipStream_t)stream, scale));
 	return 0;
 }
 

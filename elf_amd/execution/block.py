@@ -100,6 +100,8 @@ for _name, _ret, _args in [
 	("elf_stage_forward", _I, [_P, _I, _P, _P, ctypes.c_uint32, _P]),
 	("elf_stage_backward_inputs", _I, [_P, _I, _P, _P, _P, ctypes.c_uint32, _P]),
 	("elf_stage_backward_params", _I, [_P, _I, _P]),
+	("elf_stage_bind_grad_bf16", _I, [_P, _I, _I, _P]),
+	("elf_stage_backward_params_scaled", _I, [_P, _I, ctypes.c_float, _P]),
 	("elf_stage_recompute_forward", _I, [_P, _I, _P, _I, _P]),
 	("elf_stage_recompute_backward_inputs", _I, [_P, _I, _P, _P]),
 	("elf_stage_offload", _I, [_P, _I, _P]),
@@ -273,6 +275,8 @@ class HipStageBlock(StageBlockBase):
 		self.blocks = blocks
 		dev = torch.device("cuda", self.device)
 		self._fused_w, self._fused_g, self._fused_bf16_grad = [], [], []  # the fused buffers (kept alive here)
+		self._w_scaled = []  # indices of the fused buffers of linear layers: what a W with the folded gradient scale covers
+		self._folded_scale = None  # 1 / batch size that the step's last W applied, until scale_grads has run
 		self._param_loc = {}  # parameter -> (fused buffer index, first row, rows)
 		self.main_grads = {}  # parameter -> fp32 accumulator view
 		handle = ctypes.c_void_p()
@@ -301,6 +305,15 @@ class HipStageBlock(StageBlockBase):
 			self._fused_bf16_grad.append(None)
 			return w, g
 
+		def bind(block, pid, w, g):
+			_lib.check(self.lib.elf_stage_bind_param(self._handle, block, pid, w.data_ptr(), g.data_ptr()), "elf_stage_bind_param")
+			if pid in (P_WQKV, P_WO, P_W1, P_W2, P_HEAD):
+				# linear layers: the bf16 gradient the step's last W writes together with the scaled accumulator
+				i = len(self._fused_w) - 1
+				self._fused_bf16_grad[i] = torch.empty_like(w)
+				self._w_scaled.append(i)
+				_lib.check(self.lib.elf_stage_bind_grad_bf16(self._handle, block, pid, self._fused_bf16_grad[i].data_ptr()), "elf_stage_bind_grad_bf16")
+
 		for i, b in enumerate(blocks):
 			m = b.mlp
 			groups = {
@@ -316,7 +329,7 @@ class HipStageBlock(StageBlockBase):
 				if any(p.dtype != torch.bfloat16 for p in params):
 					raise _lib.ElfStageError("HipStageBlock: parameters must be bf16")
 				w, g = fuse(params)
-				_lib.check(self.lib.elf_stage_bind_param(self._handle, i, pid, w.data_ptr(), g.data_ptr()), "elf_stage_bind_param")
+				bind(i, pid, w, g)
 		self.T = mb_size * seq
 		self.d = b0.dim
 		self.mb_size, self.seq = mb_size, seq
@@ -341,7 +354,7 @@ class HipStageBlock(StageBlockBase):
 				if any(p.dtype != torch.bfloat16 for p in params):
 					raise _lib.ElfStageError("HipStageBlock: parameters must be bf16")
 				w, g = fuse(params, pad)
-				_lib.check(self.lib.elf_stage_bind_param(self._handle, -1, pid, w.data_ptr(), g.data_ptr()), "elf_stage_bind_param")
+				bind(-1, pid, w, g)
 
 	def __del__(self):
 		try:
@@ -515,10 +528,19 @@ class HipStageBlock(StageBlockBase):
 		if rg:
 			outs[0].set(outs[0].to_process, mb_id, dy)
 
+	folds_grad_scale = True  # Engine may pass ``final_scale`` to the step's last backward_params
+
 	def backward_params(self, mb_id, **options):
-		"""W: fp32 dW += dY^T X for every linear layer of the stage."""
+		"""W: fp32 dW += dY^T X for every linear layer of the stage.  ``final_scale`` (set by the Engine on the step's
+		last W when a gradient scale follows it): the linear layers' accumulators leave this pass multiplied by it,
+		with their bf16 copies written; ``scale_grads`` then only has the small rest to do."""
+		scale = options.get("final_scale")
 		with self._timed(f"backward_params({self.id}:{mb_id})"):
-			_lib.check(self.lib.elf_stage_backward_params(self._handle, mb_id, _stream()), "elf_stage_backward_params")
+			if scale:
+				_lib.check(self.lib.elf_stage_backward_params_scaled(self._handle, mb_id, float(scale), _stream()), "elf_stage_backward_params_scaled")
+				self._folded_scale = ctypes.c_float(float(scale)).value  # as the library received it
+			else:
+				_lib.check(self.lib.elf_stage_backward_params(self._handle, mb_id, _stream()), "elf_stage_backward_params")
 		self._kept.pop(mb_id, None)
 
 	def recompute_forward(self, mb_id, **options):
@@ -546,7 +568,16 @@ class HipStageBlock(StageBlockBase):
 	def scale_grads(self, batch_size):
 		"""main_grad /= batch_size, and param.grad = bf16(main_grad) (block.py:518-527)."""
 		inv = 1.0 / float(batch_size)
+		done = ()
+		if self._folded_scale is not None:
+			# the step's last W has scaled the linear layers already (and written their bf16 copies)
+			if self._folded_scale != ctypes.c_float(inv).value:
+				raise _lib.ElfStageError(f"{self}: the last W folded a gradient scale of {self._folded_scale}, scale_grads is asked for {inv}")
+			done = self._w_scaled
+			self._folded_scale = None
 		for i, (w, g) in enumerate(zip(self._fused_w, self._fused_g)):
+			if i in done:
+				continue
 			if self._fused_bf16_grad[i] is None:
 				self._fused_bf16_grad[i] = torch.empty_like(w)
 			_lib.check(self.lib.elf_scale_grads(g.data_ptr(), self._fused_bf16_grad[i].data_ptr(), g.numel(), inv, _stream()), "elf_scale_grads")
@@ -554,6 +585,7 @@ class HipStageBlock(StageBlockBase):
 			p.grad = self._fused_bf16_grad[i][r : r + n]
 
 	def zero_grad(self):
+		self._folded_scale = None
 		for g in self._fused_g:
 			g.zero_()
 		for p in self.main_grads:

@@ -115,6 +115,22 @@ class Engine:
 				offloaders[key] = self._offloader(block, mb)
 			return offloaders[key]
 
+		# The step's last W of a block that can fold the gradient scale into it (HipStageBlock): that W is told the scale
+		# the ALL_REDUCE_PARAM_GRADS op behind it will apply (block.scale_grads then skips what the W has already done).
+		final_w = {}
+		for i, op in enumerate(schedule):
+			blk = self.id_to_block.get(op.block_id)
+			if blk is None or not getattr(blk, "folds_grad_scale", False):
+				continue
+			if op.op == OperationType.BACKWARD_PARAMS:
+				final_w[op.block_id] = [i, False]
+			elif op.op == OperationType.ALL_REDUCE_PARAM_GRADS and op.block_id in final_w:
+				final_w[op.block_id][1] = True
+			elif op.op == OperationType.ALL_REDUCE_PARAM_GRADS:
+				final_w[op.block_id] = [-1, False]
+		final_w = {i for i, scaled in final_w.values() if scaled and i >= 0}
+		final_scale = 1.0 / float(sum(mb_sizes))
+
 		result, losses, grad_fns = [], [], deque()
 		if precise_timings:
 			if dist.is_available() and dist.is_initialized():
@@ -126,7 +142,7 @@ class Engine:
 		memories, peak_memories = OrderedDict(), OrderedDict()
 		T = OperationType
 
-		for op in schedule:
+		for op_index, op in enumerate(schedule):
 			block = self.id_to_block.get(op.block_id)
 			if block is None:
 				continue
@@ -155,7 +171,10 @@ class Engine:
 				if op.options.get(OpOptions.ACTIVATION_OFFLOAD):
 					offloader(block, op.mb_id).release()
 			elif kind == T.BACKWARD_PARAMS:
-				block.backward_params(op.mb_id, **op.options)
+				if op_index in final_w:
+					block.backward_params(op.mb_id, final_scale=final_scale, **op.options)
+				else:
+					block.backward_params(op.mb_id, **op.options)
 			elif kind == T.SEND_FORWARD:
 				dst = self.id_to_block.get(op.options.get("dst"))
 				if dst is not None:

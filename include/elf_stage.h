@@ -306,6 +306,14 @@ int elf_stage_backward_inputs(elf_stage_t* s, int mb, const void* x, const void*
 /* W: PipelineBlock.backward_params + LinearDW.backward (block.py:376-391, zb_utils.py:215-256):
  * grad_f32 += dY^T X for every linear layer, then the W stash of the micro-batch is dropped. */
 int elf_stage_backward_params(elf_stage_t* s, int mb, void* stream);
+/* W of the step's LAST micro-batch with the step's gradient scale folded in: every linear layer's accumulator leaves
+ * the pass as (grad_f32 + dY^T X) * scale, and bf16(grad_f32) is written to the buffer bound with
+ * elf_stage_bind_grad_bf16 (same shape as the weight).  Replaces that W followed by PipelineBlock.scale_grads
+ * (block.py:518-527: grad /= batch size at ALL_REDUCE_PARAM_GRADS) for the linear layers, bit for bit, without the
+ * extra pass over every gradient; the norm gains / biases and the token embedding, whose gradients accumulate in B, are
+ * still scaled by elf_scale_grads.  The caller decides which W is the last one (the schedule is static). */
+int elf_stage_bind_grad_bf16(elf_stage_t* s, int block, int which, void* grad_bf16);
+int elf_stage_backward_params_scaled(elf_stage_t* s, int mb, float scale, void* stream);
 /* RF: PipelineBlock.recompute_forward (block.py:308-338). save = 0 refills only the W-stash inputs,
  * save != 0 rebuilds the whole activation stash. */
 int elf_stage_recompute_forward(elf_stage_t* s, int mb, const void* x, int save, void* stream);
@@ -314,9 +322,10 @@ int elf_stage_recompute_forward(elf_stage_t* s, int mb, const void* x, int save,
 int elf_stage_recompute_backward_inputs(elf_stage_t* s, int mb, const void* dy, void* stream);
 /* Offload life cycle (OffloadToCPU, offload.py:166-411): offload is also implied by
  * ELF_FWD_OFFLOAD; prefetch = PREFETCH_ACTIVATIONS; release returns the pinned blocks.  Of the
- * stash, the two norm outputs, the FFN activation and the QKV projection's output are not copied:
- * backward_inputs forms them again from the restored buffers with the forward's kernels
- * (bit-identical). */
+ * stash, the two norm outputs, the FFN activation, the QKV projection's output and the attention
+ * residual (x + o Wo^T) are not copied: backward_inputs forms them again from the restored buffers
+ * with the forward's own kernel calls (bit-identical).  A prefetch brings the FFN pre-activation
+ * back in row chunks and backward_inputs works through it chunk by chunk as they arrive. */
 int elf_stage_offload(elf_stage_t* s, int mb, void* stream);
 int elf_stage_prefetch(elf_stage_t* s, int mb, void* stream);
 int elf_stage_release(elf_stage_t* s, int mb);
@@ -354,8 +363,9 @@ int elf_pinned_pool_free_segment(elf_pinned_pool_t* p, int parent, int i, int64_
  * elf_prof_enable(1), with their summed duration (ms) and summed work. */
 /* Memory-system yardstick for the bandwidth-bound kernels (no counterpart in the reference): mode 0 reads `bytes`
  * bytes from src (dst receives at most 8192 * 256 * 16 bytes of per-lane sums), mode 1 copies them to dst, mode 2 writes
- * `bytes` bytes to dst; 16-byte accesses, each workgroup on contiguous chunks of 16 or 32 KiB.  bench.py --hbm-ceiling
- * times it. */
+ * `bytes` bytes to dst, mode 3 reads three streams of `bytes` bytes each (src, src + bytes, src + 2 bytes: src holds
+ * 3 * bytes) and writes their XOR to dst (the traffic pattern of a normalisation backward with a residual gradient);
+ * 16-byte accesses, each workgroup on contiguous chunks of 16 or 32 KiB.  bench.py --hbm-ceiling times it. */
 int elf_hbm_probe(int mode, const void* src, void* dst, int64_t bytes, void* stream);
 void elf_prof_enable(int on);
 int elf_prof_collect(int kind, double* total_ms, double* total_work);

@@ -97,6 +97,16 @@ def test_zbh1_stream_equals_1f1b_and_the_oracle_over_all_micro_batches():
 	assert out["ok"]
 	# the accumulators now hold the plain stream's sums over the 16 micro-batches, scaled by 1 / 32 sequences
 	got = {k: v.clone() for k, v in product_grads(stage).items() if k.startswith("0.")}
+	# the gradient scale folded into the step's last W (what the Engine does for this block) against the same stream
+	# with the scale as a pass of its own behind it: fp32 accumulators and bf16 gradients bit for bit
+	folded = bench.run_and_keep(block, engine, stream, mb_sizes, xs, dys)
+	folded16 = [g.clone() for g in block._fused_bf16_grad]
+	block.folds_grad_scale = False
+	apart = bench.run_and_keep(block, engine, stream, mb_sizes, xs, dys)
+	del block.folds_grad_scale
+	assert bench.compare_kept(folded, apart)["weight_grads_equal"], "the folded gradient scale changes the accumulators"
+	assert all(torch.equal(a, b) for a, b in zip(folded16, block._fused_bf16_grad)), "the folded gradient scale changes the bf16 gradients"
+	del folded, apart, folded16
 	block.set_boundary(inputs=xs, grads=dys, keep_sent=True)
 	block.zero_grad()
 	engine.train_step(None, None, None, stream, mb_sizes)
@@ -119,12 +129,17 @@ def test_zbh1_stream_equals_1f1b_and_the_oracle_over_all_micro_batches():
 		dx = ref.backward_inputs(m, dys[m])
 		ref.backward_params(m)
 		if m == last:
-			fro16 = {"y": ((y16.double() - y.double()).norm() / y.double().norm()).item(), "dx": ((dx16.double() - dx.double()).norm() / dx.double().norm()).item()}
+			rel = lambda a, b: ((a.double() - b.double()).norm() / b.double().norm()).item()
+			mx = lambda a, b: ((a.float() - b.float()).abs().max() / b.float().abs().max()).item()
+			fro16 = {"y": rel(y16, y), "dx": rel(dx16, dx)}
+			max16 = {"y": mx(y16, y), "dx": mx(dx16, dx)}
 			bound = max(1e-2, 1.25 * max(fro16.values()))
-			print(f"[bf16 torch vs fp32] 4 blocks: y {fro16['y']:.4g}, dx {fro16['dx']:.4g} -> Frobenius bound {bound:.4g}", flush=True)
-			_, fy = assert_close_dev(y_last, y, "zbh1 y[last]", rel_fro=max(1e-2, 1.25 * fro16["y"]))
-			_, fdx = assert_close_dev(dx_last, dx, "zbh1 dx[last]", rel_fro=max(1e-2, 1.25 * fro16["dx"]))
-			print(f"[hip vs fp32 oracle] 4 blocks: y {fy:.4g}, dx {fdx:.4g}", flush=True)
+			print(f"[bf16 torch vs fp32] 4 blocks: y fro {fro16['y']:.4g} max {max16['y']:.4g}, dx fro {fro16['dx']:.4g} max {max16['dx']:.4g}", flush=True)
+			# four blocks deep the largest element (|dx| up to 140 against a root mean square near 1) sits three bf16 steps from
+			# the fp32 value in PyTorch's own bf16 run as well: both bounds are the stated ones or 1.25 x PyTorch's, whichever is larger
+			ey, fy = assert_close_dev(y_last, y, "zbh1 y[last]", rel_max=max(2e-2, 1.25 * max16["y"]), rel_fro=max(1e-2, 1.25 * fro16["y"]))
+			edx, fdx = assert_close_dev(dx_last, dx, "zbh1 dx[last]", rel_max=max(2e-2, 1.25 * max16["dx"]), rel_fro=max(1e-2, 1.25 * fro16["dx"]))
+			print(f"[hip vs fp32 oracle] 4 blocks: y fro {fy:.4g} max {ey:.4g}, dx fro {fdx:.4g} max {edx:.4g}", flush=True)
 			del y16, dx16
 		del y, dx
 	ref.scale_grads(w["mb"] * w["n_mb"])

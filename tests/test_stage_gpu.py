@@ -172,11 +172,13 @@ def test_remat_and_offload_variants_equal_plain(kind, variant, lean):
 			torch.cuda.synchronize()
 			st = blk.mem_stats()
 			assert st["d2h_bytes"] > 0 and st["pinned_bytes"] >= st["d2h_bytes"]
-			# what crosses the link: the stage-owned buffers above 1 MiB minus the two norm outputs, the FFN
-			# activation and the QKV projection's output, which B forms again from the restored buffers
+			# what crosses the link: the stage-owned buffers above 1 MiB minus the two norm outputs, the FFN activation,
+			# the QKV projection's output and the attention residual, which B forms again from the restored buffers:
+			# per block the attention output, its log-sum-exp and the FFN pre-activation, plus the inputs of the blocks
+			# behind the first
 			T, d, hq, hkv, hd = mb * cfg["seq"], cfg["d_model"], cfg["n_heads"], cfg["n_kv_heads"], cfg["head_dim"]
 			ffn_in = cfg["ffn"] * (2 if kind == "llama" else 1)
-			per_block = [T * hq * hd * 2, mb * hq * cfg["seq"] * 4, T * d * 2, T * ffn_in * 2]
+			per_block = [T * hq * hd * 2, mb * hq * cfg["seq"] * 4, T * ffn_in * 2]
 			moved = sum(b for b in per_block if b > 1 << 20) * cfg["n_blocks"] + (T * d * 2 if T * d * 2 > 1 << 20 else 0) * (cfg["n_blocks"] - 1)
 			assert st["d2h_bytes"] == 2 * moved
 		for m in range(2):
@@ -354,6 +356,43 @@ def test_engine_runs_1f1b_and_zbh1_streams():
 			assert_close(got[name], want[name], f"{sched_name} grad {name}")
 		assert list(detailed["memories"]) == [str(op) for op in stream]
 		assert set(stats) == {"total", "idle", "start_idle", "end_idle", "bubble"}
+
+
+def test_gradient_scale_folded_into_the_last_w_equals_the_separate_pass():
+	"""The Engine tells the step's last W the scale that ALL_REDUCE_PARAM_GRADS applies behind it; the accumulators and
+	the bf16 gradients must be those of the plain order, W then scale_grads (elf/execution/block.py:518-527), bit for
+	bit - here at a shape whose weight gradients take the unfused route inside the library; the benchmark shapes, which
+	scale in the GEMM epilogue, are compared the same way in tests/test_full_streams_gpu.py."""
+	from elf_amd.execution import Engine
+	from elf_amd.partitioners.utils import sequential_signatures
+	from elf_amd.registry import COMM_SCHEDULERS, SCHEDULERS
+	from elf_amd.scheduling import add_comms
+
+	mb, nmb, placement = 2, 4, [0, 1, 2, 3]
+	out = {}
+	for fold in (True, False):
+		stage = _stage("llama")
+		R, cfg, _ = _oracle(stage, mb)
+		xs, dys = R.make_boundary(cfg, nmb, seed=33)
+		blk = _block(stage, mb)
+		if not fold:
+			blk.folds_grad_scale = False
+		blk.zero_grad()
+		blk.set_boundary(inputs=[x.cuda() for x in xs], grads=[d.cuda() for d in dys])
+		schedule = COMM_SCHEDULERS["pipelined"](add_comms(SCHEDULERS["zbh1"](placement, nmb), sequential_signatures(placement)))
+		Engine([blk]).train_step(None, None, None, [op for op in schedule if op.block_id == 1], [mb] * nmb)
+		torch.cuda.synchronize()
+		out[fold] = ({k: v.clone() for k, v in product_grads(stage).items()}, {k: v.clone() for k, v in product_grads(stage, "grad").items()})
+	for k in out[True][0]:
+		assert torch.equal(out[True][0][k], out[False][0][k]), f"fp32 accumulator {k}"
+		assert out[True][1][k].dtype == torch.bfloat16 and torch.equal(out[True][1][k], out[False][1][k]), f"bf16 gradient {k}"
+	# a scale that is not the one the last W folded is refused
+	blk = _block(_stage("llama"), mb)
+	blk._folded_scale = 0.5  # as if the last W had folded 1 / 2
+	from elf_amd._lib import ElfStageError
+
+	with pytest.raises(ElfStageError):
+		blk.scale_grads(8)
 
 
 def test_profile_stage_feeds_the_remat_ilp_and_the_stream_fits_the_budget():
