@@ -26,10 +26,22 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA peak
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per GEMM launch (mean over the launches of one step), from rocprofv3 --pmc FETCH_SIZE and
-# --pmc WRITE_SIZE runs of this script scaled by the same counters' reading for a copy kernel of known
-# size (--calibration-copy); measured per workload, None where it was not.
-GEMM_TRAFFIC_BYTES = {"llama3_8b_zbh1": 1.698e9}
+
+
+def gemm_traffic_bytes(workload):
+	"""HBM bytes per GEMM launch (mean over the launches of one step) of ``workload``: read from the line the counter
+	summary under profiles/ ends with (rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs of this script, scaled by
+	the same counters' reading for a copy kernel of known size, --calibration-copy), so that the figure has one
+	source; None where no counter run was summarised."""
+	import re
+
+	try:
+		text = open(os.path.join(ROOT, "profiles", f"stage_kernels_{workload}.md")).read()
+	except OSError:
+		return None
+	m = re.search(r"\(([0-9.e+]+) bytes: bench\.py's `roofline\.traffic`\)", text)
+	return float(m.group(1)) if m else None
+
 
 WORKLOADS = {
 	# headline configuration: Llama-3-8B-shaped stage, ZB-H1 stream of block 1 in a 4-stage pipeline
@@ -565,8 +577,8 @@ def main():
 			"seq_len": w["seq"], "micro_batch": w["mb"], "n_micro_batches": w["n_mb"], "op_stream": f"{w['scheduler']} block {BLOCK_ID} of placement {placement}",
 			"tokens_per_step": tokens, "ops_per_step": len(stream), "offload": bool(w.get("offload")), "hip_graph": bool(args.graph),
 		},
-		"roofline": {"bound": "mfma", "achieved": g["tflops"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": g["tflops"] / PEAK_BF16_TFLOPS, "traffic": GEMM_TRAFFIC_BYTES.get(args.workload),
-		             "kernel": "elf::dma::gemm_dma_kernel / elf::gemm_kernel (bf16 MFMA GEMM, all layouts)", "launches": g["launches"], "avg_launch_ms": g["avg_ms"]},
+		"roofline": {"bound": "mfma", "achieved": g["tflops"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": g["tflops"] / PEAK_BF16_TFLOPS, "traffic": gemm_traffic_bytes(args.workload),
+		             "kernel": "elf::dma::gemm_pers_kernel / elf::dma::gemm_dma_kernel / elf::gemm_kernel (bf16 MFMA GEMM, all layouts)", "launches": g["launches"], "avg_launch_ms": g["avg_ms"]},
 		"stream_mfu": stream_flops(w) / (elapsed / args.steps) / (PEAK_BF16_TFLOPS * 1e12),
 		"kernels": per_kernel,
 		"peak_stage_memory_bytes": mem["peak_bytes"] + mem["workspace_bytes"] + torch.cuda.max_memory_allocated(),

@@ -775,7 +775,8 @@ __global__ __launch_bounds__(256) void scale_grads_kernel(float* __restrict__ ac
 int scale_grads(void* acc_f32, void* out_bf16, int64_t n, float scale, hipStream_t s) {
 	ELF_REQUIRE(acc_f32 && n > 0, "scale_grads: empty");
 	ELF_REQUIRE(((uintptr_t)acc_f32 % 16) == 0 && (!out_bf16 || ((uintptr_t)out_bf16 % 8) == 0), "scale_grads: misaligned");
-	ProfScope prof(PROF_SCALE, (out_bf16 ? 10.0 : 8.0) * n, s);
+	// buffers under a MiB (norm gains and biases) are launch-bound, not bandwidth-bound: they stay out of the bandwidth figure
+	ProfScope prof(PROF_SCALE, (out_bf16 ? 10.0 : 8.0) * n, s, /*record=*/n >= (1 << 18));
 	ELF_LAUNCH(scale_grads_kernel, dim3(ew_grid(n / 4 + 1)), dim3(256), 0, s, (float*)acc_f32, (bf16_t*)out_bf16,
 	                   n / 4, n, scale);
 	ELF_CHECK_HIP(hipGetLastError());

@@ -137,7 +137,8 @@ enum ProfKind {
 void prof_enable(int on);
 bool prof_on();
 struct ProfScope {
-	ProfScope(int kind, double work, hipStream_t stream);
+	// record = false: an inert scope (launches inside it are not timed)
+	ProfScope(int kind, double work, hipStream_t stream, bool record = true);
 	~ProfScope();
 	int slot;
 	hipStream_t stream;

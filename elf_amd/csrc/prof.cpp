@@ -41,8 +41,8 @@ void prof_enable(int on) {
 }
 bool prof_on() { return g_on; }
 
-ProfScope::ProfScope(int kind, double work, hipStream_t s) : slot(-1), stream(s), outer(nullptr) {
-	if (!g_on) return;
+ProfScope::ProfScope(int kind, double work, hipStream_t s, bool record) : slot(-1), stream(s), outer(nullptr) {
+	if (!g_on || !record) return;
 	ProfRec r{kind, work, get_event(), get_event(), false};
 	if (!r.e0 || !r.e1) return;
 	slot = (int)g_recs.size();
