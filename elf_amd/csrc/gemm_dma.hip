@@ -883,6 +883,7 @@ __global__ __launch_bounds__(256) void gemm_pers_kernel(Args g) {
 			const int F = g.N / 2, cg0 = n0 / 2 + wc * 64;
 #pragma unroll
 			for (int i = 0; i < RF; i++) {
+				__builtin_amdgcn_sched_barrier(0);  // one row group at a time (see the residual epilogue below)
 				const int64_t row = grow0 + i * 16;
 #pragma unroll
 				for (int t = 0; t < 2; t++) {
@@ -910,70 +911,81 @@ __global__ __launch_bounds__(256) void gemm_pers_kernel(Args g) {
 			const int half = g.rope_D >> 1;
 			auto rope_rows = [&](auto widec) {
 				constexpr bool WIDE = decltype(widec)::value;
+				// pair p of a row: runs (lo, hi) = (p, p + 2) for heads of 128, (2 p, 2 p + 1) for heads of 64; the lane's 8
+				// columns within the head's first half start at c_in_head
+				const int c_in_head[2] = {g4 * 8, WIDE ? 32 + g4 * 8 : g4 * 8};
+				const bool rot[2] = {gcol0 + run_col(0) < g.rope_cols, gcol0 + run_col(WIDE ? 1 : 2) < g.rope_cols};
+				// (cos, sin) of row i's 2 x 8 column pairs: fetched two rows ahead of their use - a lone wave has nothing
+				// else to cover a trip to the cache with
+				f32x4 tab[3][2][4] = {};
+				auto fetch = [&](int i, int slot) {
+					const int pos = (int)((grow0 + i * 16) % g.rope_S);
 #pragma unroll
-				for (int i = 0; i < RF; i++) {
-					const int64_t row = grow0 + i * 16;
-					const int pos = (int)(row % g.rope_S);
-					bf16_t* cp = reinterpret_cast<bf16_t*>(g.C) + row * g.ldc + gcol0;
+					for (int p = 0; p < 2; p++)
+						if (rot[p]) {
+							const f32x4* tp = reinterpret_cast<const f32x4*>(g.rope_cs + (int64_t)pos * half + c_in_head[p]);
+#pragma unroll
+							for (int q = 0; q < 4; q++) tab[slot][p][q] = tp[q];
+						}
+				};
+				fetch(0, 0);
+				fetch(1, 1);
+				static_for<RF>([&](auto ic) {
+					constexpr int i = decltype(ic)::value;
+					__builtin_amdgcn_sched_barrier(0);  // one row group at a time, its table entries fetched two groups earlier
+					if constexpr (i + 2 < RF) fetch(i + 2, (i + 2) % 3);
+					bf16_t* cp = reinterpret_cast<bf16_t*>(g.C) + (int64_t)(grow0 + i * 16) * g.ldc + gcol0;
 #pragma unroll
 					for (int p = 0; p < 2; p++) {
-						// pair p: runs (lo, hi) = (p, p + 2) for heads of 128, (2 p, 2 p + 1) for heads of 64
 						const int tlo = WIDE ? p : 2 * p, thi = WIDE ? p + 2 : 2 * p + 1;
-						const int c_in_head = WIDE ? p * 32 + g4 * 8 : g4 * 8;  // first of the lane's 8 columns within the head's first half
-						const bool rot = gcol0 + run_col(tlo) < g.rope_cols;
 						float a[8], b[8];
 						run(i, tlo, a);
 						run(i, thi, b);
 						bf16x8 olo, ohi;
-						f32x4 tab[4] = {};
-						if (rot) {
-							const f32x4* tp = reinterpret_cast<const f32x4*>(g.rope_cs + (int64_t)pos * half + c_in_head);
-#pragma unroll
-							for (int q = 0; q < 4; q++) tab[q] = tp[q];
-						}
 #pragma unroll
 						for (int e = 0; e < 8; e++) {
 							const float x = (float)(bf16_t)a[e], y = (float)(bf16_t)b[e];
 							float ra = x, rb = y;
-							if (rot) rope_rot(x, y, tab[e >> 1][(e & 1) * 2], tab[e >> 1][(e & 1) * 2 + 1], ra, rb);
+							if (rot[p]) rope_rot(x, y, tab[i % 3][p][e >> 1][(e & 1) * 2], tab[i % 3][p][e >> 1][(e & 1) * 2 + 1], ra, rb);
 							olo[e] = (bf16_t)ra;
 							ohi[e] = (bf16_t)rb;
 						}
 						*reinterpret_cast<bf16x8*>(cp + run_col(tlo)) = olo;
 						*reinterpret_cast<bf16x8*>(cp + run_col(thi)) = ohi;
 					}
-				}
+				});
 			};
 			if (g.rope_D == 128) rope_rows(std::true_type{});
 			else rope_rows(std::false_type{});
 		} else {
 			static_assert(EPI == EPI_BF16 || EPI == EPI_BF16_RESID, "epilogues of the persistent forward kernel");
-			// residual (or bias row, ldr = 0): the loads of four rows of accumulator tiles in flight together
+			// residual (or bias row, ldr = 0): every load of the wave's 128 x 128 share goes out before the first store (a lone
+			// wave has nothing else to cover the trips to memory with; inside the store loop each would be awaited alone)
+			bf16x8 rs[EPI == EPI_BF16_RESID ? RF : 1][4];
+			if constexpr (EPI == EPI_BF16_RESID) {
 #pragma unroll
-			for (int ib = 0; ib < RF; ib += 4) {
-				bf16x8 rs[EPI == EPI_BF16_RESID ? 4 : 1][4];
-				if constexpr (EPI == EPI_BF16_RESID) {
+				for (int i = 0; i < RF; i++)
 #pragma unroll
-					for (int i = 0; i < 4; i++)
+					for (int t = 0; t < 4; t++) rs[i][t] = *reinterpret_cast<const bf16x8*>(g.R + (int64_t)(grow0 + i * 16) * g.ldr + gcol0 + run_col(t));
+			}
+			// (left to itself the scheduler reads all 256 accumulators into vector registers first and then has room for
+			// two loads at a time: the row groups are fenced off from each other and from the loads)
+			__builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-						for (int t = 0; t < 4; t++)
-							rs[i][t] = *reinterpret_cast<const bf16x8*>(g.R + (int64_t)(grow0 + (ib + i) * 16) * g.ldr + gcol0 + run_col(t));
-				}
+			for (int i = 0; i < RF; i++) {
+				__builtin_amdgcn_sched_barrier(0);
+				bf16_t* cp = reinterpret_cast<bf16_t*>(g.C) + (int64_t)(grow0 + i * 16) * g.ldc + gcol0;
 #pragma unroll
-				for (int i = 0; i < 4; i++) {
-					bf16_t* cp = reinterpret_cast<bf16_t*>(g.C) + (int64_t)(grow0 + (ib + i) * 16) * g.ldc + gcol0;
+				for (int t = 0; t < 4; t++) {
+					float v[8];
+					run(i, t, v);
+					bf16x8 o;
 #pragma unroll
-					for (int t = 0; t < 4; t++) {
-						float v[8];
-						run(ib + i, t, v);
-						bf16x8 o;
-#pragma unroll
-						for (int e = 0; e < 8; e++) {
-							if constexpr (EPI == EPI_BF16_RESID) v[e] += (float)rs[i][t][e];
-							o[e] = (bf16_t)v[e];
-						}
-						*reinterpret_cast<bf16x8*>(cp + run_col(t)) = o;
+					for (int e = 0; e < 8; e++) {
+						if constexpr (EPI == EPI_BF16_RESID) v[e] += (float)rs[i][t][e];
+						o[e] = (bf16_t)v[e];
 					}
+					*reinterpret_cast<bf16x8*>(cp + run_col(t)) = o;
 				}
 			}
 		}
