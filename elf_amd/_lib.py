@@ -44,6 +44,7 @@ _SIGNATURES = {
 	"elf_attn_fwd": (c_int, [_P, _P, _P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_float, _P]),
 	"elf_attn_bwd_workspace_bytes": (c_int64, [c_int, c_int, c_int, c_int, c_int]),
 	"elf_gemm_turn_giveups": (c_int, [POINTER(ctypes.c_uint64)]),
+	"elf_gemm_dw_group": (c_int, [c_int, _P, c_int, c_float, _P]),
 	"elf_hbm_probe": (c_int, [c_int, _P, _P, c_int64, _P]),
 	"elf_prof_enable": (None, [c_int]),
 	"elf_prof_collect": (c_int, [c_int, POINTER(c_double), POINTER(c_double)]),

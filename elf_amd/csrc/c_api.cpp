@@ -15,6 +15,14 @@ int elf_gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t 
 	                      (hipStream_t)stream);
 }
 
+int elf_gemm_dw_group(int n, const elf_dw_problem* problems, int K, float scale, void* stream) {
+	// the header's plain-C problem record and the launcher's are the same eight fields in the same order
+	static_assert(sizeof(elf_dw_problem) == sizeof(elf::DwProblem) && offsetof(elf_dw_problem, acc) == offsetof(elf::DwProblem, acc) &&
+	                  offsetof(elf_dw_problem, N) == offsetof(elf::DwProblem, N),
+	              "elf_dw_problem and elf::DwProblem differ");
+	return elf::gemm_dw_group(n, reinterpret_cast<const elf::DwProblem*>(problems), K, scale, (hipStream_t)stream);
+}
+
 int elf_gemm_act_bf16(int act, int M, int F, int K, const void* A, int64_t lda, const void* W, int64_t ldw,
                       void* pre, int64_t ldpre, void* out, int64_t ldout, void* stream) {
 	return elf::gemm_act_bf16(act, M, F, K, A, lda, W, ldw, pre, ldpre, out, ldout, (hipStream_t)stream);

@@ -72,6 +72,7 @@ struct Args {
 	// split tiles: this launch's tag in the turn counters (see turn[] below); 0 = the splits add in any order
 	uint32_t turn_tag;
 	float scale;  // EPI_F32_ACC_SCALE
+	uint32_t turn_base;  // split tiles: the first of this problem's turn counters
 };
 
 // Turn counters of split tiles.  The workgroups that share a tile along K add their parts with fp32 atomics; to make
@@ -215,9 +216,14 @@ __device__ __forceinline__ void mfma_acc(f32x4& acc, const bf16x8& a, const bf16
 // Origin (m0, n0) of tile `pid` of the launch: see "Tile assignment" in gemm_dma_kernel for the two walks.
 template <int BM>
 __device__ __forceinline__ void tile_origin(const Args& g, int pid, int& m0, int& n0) {
+	if (g.walk == 2) {  // tiles in plain order, down the rows first (the launch places them on the XCDs itself)
+		m0 = (pid % g.tiles_m) * BM;
+		n0 = (pid / g.tiles_m) * BN;
+		return;
+	}
 	const int ntiles = g.tiles_m * g.tiles_n;
 	const int nsb = ntiles >> 5, nrem = nsb & 7;
-	if (g.walk && (g.tiles_m & 7) == 0 && (g.tiles_n & 3) == 0 && (nrem == 0 || nrem == 1 || nrem == 2 || nrem == 4)) {
+	if (g.walk == 1 && (g.tiles_m & 7) == 0 && (g.tiles_n & 3) == 0 && (nrem == 0 || nrem == 1 || nrem == 2 || nrem == 4)) {
 		const int x = pid & 7, i = pid >> 3, nfull = nsb >> 3;
 		int sb, jj;
 		if (i < nfull * 32) {
@@ -245,36 +251,14 @@ __device__ __forceinline__ void tile_origin(const Args& g, int pid, int& m0, int
 	}
 }
 
-template <int NW, int RT, bool AT, bool BT, int EPI>
-__global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
-	using Sh = Shape<NW, RT>;
-	constexpr int BM = Sh::BM, A_BYTES = Sh::A_BYTES, STAGE_BYTES = Sh::STAGE_BYTES;
-	constexpr int LOADS_A = Sh::LOADS_A, LOADS_B = Sh::LOADS_B, LOADS_PER_STAGE = Sh::LOADS_PER_STAGE, NST = Sh::NST;
-	constexpr bool PAIRED = EPI == EPI_BF16_SWIGLU;
-	static_assert(!PAIRED || !BT, "the paired row order is defined for a k-contiguous B");
-	extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-	const int tid = threadIdx.x;
-	const int lane = tid & 63;
-	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-	const int wr = wave >> 1, wc = wave & 1;
-
-	// Tile assignment.  Workgroup w runs on XCD w % 8, whose 32 CUs hold 32 tiles at a time (a round);
-	// both walks give an XCD 8 tile rows x 4 tile columns per round (12 operand slabs through its L2 for
-	// 32 tiles) and differ in where the 8 XCDs are relative to each other:
-	//  * default: each XCD owns a contiguous run of tiles (8 tile rows at a time, along the columns).  The
-	//    XCDs work on different row groups; a row slab of A is needed in as many rounds as the row has
-	//    column groups, so A has to stay in the memory-side cache between them;
-	//  * walk = 1: the 8 XCDs share a 16 x 16 block of tiles per round, bands of 16 tile rows walked along the
-	//    columns; a row slab of A is live for one band only, B is fetched once per band (weight gradient of
-	//    the gate/up projection, 28672 x 4096 at K = 8192, A = 470 MB: 5-7 % faster).  A last, partly filled
-	//    round shares each 8 x 4 block between several XCDs.
-	// The first ntiles - tail_tiles tiles
-	// are computed whole, one workgroup each; each of the last tail_tiles is shared by k_splits
-	// workgroups that take a K range each and add their part with atomics.  Splitting only the tail
-	// turns the last, partly filled round of workgroups of a launch into a full round of shorter ones.
+// Tile, K range and turn counter of workgroup `bid` of the problem `g` (the block index of a launch with one problem).
+// The first ntiles - tail_tiles tiles are computed whole, one workgroup each; each of the last tail_tiles is shared by
+// k_splits workgroups that take a K range each and add their part with atomics.  Splitting only the tail turns the
+// last, partly filled round of workgroups of a launch into a full round of shorter ones.
+__device__ __forceinline__ void locate_tile(const Args& g, const int bid, int& pid, int& ksplit, int& splits, int& turn_slot) {
 	const int ntiles = g.tiles_m * g.tiles_n;
 	const int full = ntiles - g.tail_tiles;
-	int pid = blockIdx.x, ksplit = 0, splits = 1;
+	pid = bid, ksplit = 0, splits = 1;
 	if (pid >= full) {
 		const int q = pid - full;
 		splits = g.k_splits;
@@ -288,7 +272,34 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 		}
 	}
 	// split tiles: the turn counter of this tile (tiles of one launch get distinct counters, consecutive launches different ones)
-	const int turn_slot = (int)(((uint32_t)(pid - full) + g.turn_tag * 977u) % (uint32_t)TURN_TILES);
+	turn_slot = (int)(((uint32_t)(pid - full) + g.turn_base) % (uint32_t)TURN_TILES);
+}
+
+// One workgroup: tile `pid` of the problem `g`, K range `ksplit` of `splits`; a split tile's turn counters are those of
+// `turn_slot`.
+template <int NW, int RT, bool AT, bool BT, int EPI>
+__device__ __forceinline__ void gemm_dma_tile(const Args& g, const int pid, const int ksplit, const int splits, const int turn_slot) {
+	using Sh = Shape<NW, RT>;
+	constexpr int BM = Sh::BM, A_BYTES = Sh::A_BYTES, STAGE_BYTES = Sh::STAGE_BYTES;
+	constexpr int LOADS_A = Sh::LOADS_A, LOADS_B = Sh::LOADS_B, LOADS_PER_STAGE = Sh::LOADS_PER_STAGE, NST = Sh::NST;
+	constexpr bool PAIRED = EPI == EPI_BF16_SWIGLU;
+	static_assert(!PAIRED || !BT, "the paired row order is defined for a k-contiguous B");
+	extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+	const int tid = threadIdx.x;
+	const int lane = tid & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+	const int wr = wave >> 1, wc = wave & 1;
+
+	// Tile assignment (tile_origin).  Workgroup w runs on XCD w % 8, whose 32 CUs hold 32 tiles at a time (a round);
+	// both walks give an XCD 8 tile rows x 4 tile columns per round (12 operand slabs through its L2 for
+	// 32 tiles) and differ in where the 8 XCDs are relative to each other:
+	//  * default: each XCD owns a contiguous run of tiles (8 tile rows at a time, along the columns).  The
+	//    XCDs work on different row groups; a row slab of A is needed in as many rounds as the row has
+	//    column groups, so A has to stay in the memory-side cache between them;
+	//  * walk = 1: the 8 XCDs share a 16 x 16 block of tiles per round, bands of 16 tile rows walked along the
+	//    columns; a row slab of A is live for one band only, B is fetched once per band (weight gradient of
+	//    the gate/up projection, 28672 x 4096 at K = 8192, A = 470 MB: 5-7 % faster).  A last, partly filled
+	//    round shares each 8 x 4 block between several XCDs.
 	int m0, n0;
 	tile_origin<BM>(g, pid, m0, n0);
 	m0 = __builtin_amdgcn_readfirstlane(m0);
@@ -686,6 +697,64 @@ __global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
 	}
 }
 
+template <int NW, int RT, bool AT, bool BT, int EPI>
+__global__ __launch_bounds__(NW * 64) void gemm_dma_kernel(Args g) {
+	int pid, ksplit, splits, turn_slot;
+	locate_tile(g, (int)blockIdx.x, pid, ksplit, splits, turn_slot);
+	gemm_dma_tile<NW, RT, AT, BT, EPI>(g, pid, ksplit, splits, turn_slot);
+}
+
+// Several weight gradients in one launch (the W pass of a stage: every linear layer's dW += dY^T X over the same
+// tokens).  The chip's workgroup slots refill across problem boundaries, so only the launch's last round is partly
+// filled, and small problems that would each need their tiles split many ways to fill the chip fill it together.
+//  * compact = 0 (a problem of 256 tiles or more among them): the workgroups of problem p are first[p] .. first[p] +
+//    count[p] - 1, each first[p] a multiple of 8 so that a workgroup's index within its problem names its XCD as in a
+//    launch of its own (the workgroups in the gaps leave at once); every problem keeps its own walk and its own tail.
+//  * compact = 1 (small problems only): the tiles of all problems form one sequence (problem after problem, down the
+//    rows first; first[p] = problem p's first tile in it) and XCD x takes a contiguous eighth of its whole tiles, then
+//    of its split tiles with the `splits` workgroups of a tile side by side: the 32 tiles an XCD holds at a time are
+//    neighbours that share their operand slabs in its L2 (taken in launch order, neighbouring tiles of a 3-row problem
+//    land on different XCDs and every slab is fetched by all eight).
+constexpr int GROUP_MAX = 16;
+struct GroupArgs {
+	int n, compact;
+	int tiles, tail, splits;  // compact: all tiles of the launch, how many of the last are split, and how many ways
+	uint32_t turn_base;
+	int first[GROUP_MAX], count[GROUP_MAX];
+	Args a[GROUP_MAX];
+};
+template <int EPI>
+__global__ __launch_bounds__(512) void gemm_dw_group_kernel(GroupArgs ga) {
+	int p = 0, pid, ksplit = 0, splits = 1, turn_slot = 0;
+	if (ga.compact) {
+		const int x = blockIdx.x & 7, slot = blockIdx.x >> 3;
+		const int full = ga.tiles - ga.tail, chunk_f = (full + 7) >> 3, chunk_t = (ga.tail + 7) >> 3;
+		int gt;
+		if (slot < chunk_f) {
+			gt = x * chunk_f + slot;
+			if (gt >= full) return;
+		} else {
+			const int q = slot - chunk_f, tt = x * chunk_t + q / ga.splits;
+			if (tt >= ga.tail) return;
+			gt = full + tt;
+			ksplit = q % ga.splits;
+			splits = ga.splits;
+			turn_slot = (int)(((uint32_t)tt + ga.turn_base) % (uint32_t)TURN_TILES);
+		}
+		for (int i = 1; i < ga.n; i++)
+			if (gt >= ga.first[i]) p = i;
+		p = __builtin_amdgcn_readfirstlane(p);
+		pid = gt - ga.first[p];
+	} else {
+		for (int i = 1; i < ga.n; i++)
+			if ((int)blockIdx.x >= ga.first[i]) p = i;
+		p = __builtin_amdgcn_readfirstlane(p);
+		const int bid = (int)blockIdx.x - ga.first[p];
+		if (bid >= ga.count[p]) return;
+		locate_tile(ga.a[p], bid, pid, ksplit, splits, turn_slot);
+	}
+	gemm_dma_tile<8, 2, true, true, EPI>(ga.a[p], pid, ksplit, splits, turn_slot);
+}
 
 // ------------------------------------------------------------------------------------------------------------
 // Persistent forward kernel: both operands k-contiguous, 256x256 tiles, four waves with 128x128 wave tiles - the loop
@@ -1110,6 +1179,7 @@ int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t 
 	if ((epi != EPI_F32_ACC && epi != EPI_F32_ACC_SCALE) || a.k_splits == 1) a.k_splits = 1, a.tail_tiles = 0;
 	// split tiles add in a fixed order (bit-reproducible weight gradients) as long as each has a counter of its own
 	a.turn_tag = a.tail_tiles > 0 && a.tail_tiles <= dma::TURN_TILES ? next_turn_tag() : 0;
+	a.turn_base = a.turn_tag * 977u;  // consecutive launches on different counters
 	if (bm == 128) {
 		if (!a_t && !b_t) return dma::launch_epi<4, 2, false, false>(a, epi, stream);
 		if (!a_t && b_t) return dma::launch_epi<4, 2, false, true>(a, epi, stream);
@@ -1141,6 +1211,87 @@ int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t 
 	}
 	set_error("gemm: layout A=T,B=R is not used by any stage contraction");
 	return -1;
+}
+
+bool gemm_dw_groupable(int M, int N, int K, const void* dY, int64_t lddy, const void* X, int64_t ldx, const void* acc) {
+	return M > 0 && N > 0 && K > 0 && M % 256 == 0 && N % dma::BN == 0 && K % dma::BKS == 0 && lddy % 8 == 0 && ldx % 8 == 0 && lddy >= M && ldx >= N &&
+	       ((uintptr_t)dY % 16) == 0 && ((uintptr_t)X % 16) == 0 && ((uintptr_t)acc % 16) == 0;
+}
+
+int gemm_dw_group(int n, const DwProblem* pr, int K, float scale, hipStream_t stream) {
+	ELF_REQUIRE(n > 0 && n <= dma::GROUP_MAX && pr, "gemm_dw_group: 1..%d problems", dma::GROUP_MAX);
+	int64_t tiles = 0;
+	double flops = 0;
+	for (int i = 0; i < n; i++) {
+		ELF_REQUIRE(pr[i].dY && pr[i].X && pr[i].acc && gemm_dw_groupable(pr[i].M, pr[i].N, K, pr[i].dY, pr[i].lddy, pr[i].X, pr[i].ldx, pr[i].acc),
+		            "gemm_dw_group: problem %d (M=%d N=%d K=%d) needs M, N multiples of 256, K of 64 and 16-byte aligned operands", i, pr[i].M, pr[i].N, K);
+		ELF_REQUIRE(scale == 0.f || (pr[i].grad_bf16 && ((uintptr_t)pr[i].grad_bf16 % 8) == 0), "gemm_dw_group: a scaling pass needs the bf16 gradient buffers");
+		tiles += (int64_t)(pr[i].M / 256) * (pr[i].N / dma::BN);
+		flops += 2.0 * pr[i].M * pr[i].N * K;
+	}
+	// Whole tiles, one workgroup each, except in the launch's last round: when that round would fill at most half of the
+	// chip, its tiles (the last ones of the last problems) are split along K so that proportionally shorter workgroups
+	// fill it - at least 16 K slices each, and no more than 8 ways (the splits of a tile add with atomics, one after the
+	// other: past that their adds cost more than the idle compute units).
+	const int nk = K / dma::BKS;
+	int splits = 1, tail = 0;
+	if (const int rem = (int)(tiles % 256); rem != 0 && rem <= 128 && rem <= dma::TURN_TILES) {
+		splits = 256 / rem < 8 ? 256 / rem : 8;
+		while (splits > 1 && nk / splits < 16) splits--;
+		if (splits > 1) tail = rem;
+	}
+	dma::GroupArgs ga{};
+	ga.n = n;
+	ga.compact = 1;
+	for (int i = 0; i < n; i++)
+		if ((pr[i].M / 256) * (pr[i].N / dma::BN) >= 256) ga.compact = 0;
+	ga.tiles = (int)tiles, ga.tail = tail, ga.splits = splits;
+	const uint32_t tag = tail ? next_turn_tag() : 0;
+	uint32_t turn_base = tag * 977u;
+	ga.turn_base = turn_base;
+	const int64_t big = int64_t(160) << 20;
+	int64_t before = 0;  // tiles of the problems ahead of this one
+	int next = 0;
+	for (int i = 0; i < n; i++) {
+		const DwProblem& q = pr[i];
+		const int ntiles = (q.M / 256) * (q.N / dma::BN);
+		// this problem's share of the launch's last `tail` tiles
+		const int64_t tail_from = tiles - tail;
+		const int tail_i = before + ntiles <= tail_from ? 0 : (int)(before + ntiles - (tail_from > before ? tail_from : before));
+		dma::Args& a = ga.a[i];
+		a = dma::Args{(const bf16_t*)q.dY, (const bf16_t*)q.X, q.acc, nullptr, (bf16_t*)q.grad_bf16, q.lddy, q.ldx, q.N, 0, q.N, q.M, q.N, K, q.M / 256, q.N / dma::BN,
+		              tail_i ? splits : 1, tail_i, 0, nullptr, 0, 0, 0, tail_i ? tag : 0, scale, turn_base};
+		a.walk = ga.compact ? 2 : !((int64_t)q.M * K * 2 < big && (int64_t)q.N * K * 2 >= big);
+		turn_base += (uint32_t)tail_i;
+		ga.first[i] = ga.compact ? (int)before : next;
+		ga.count[i] = ntiles + tail_i * (splits - 1);
+		next += (ga.count[i] + 7) & ~7;
+		before += ntiles;
+	}
+	if (ga.compact) next = 8 * (int)((tiles - tail + 7) / 8 + (tail + 7) / 8 * splits);
+	{
+		ProfScope prof(PROF_GEMM, flops, stream);
+		using Sh = dma::Shape<8, 2>;
+		constexpr int ring = Sh::NST * Sh::STAGE_BYTES + (Sh::LOADS_A > Sh::LOADS_B ? Sh::LOADS_A : Sh::LOADS_B) * 1024, epi = 8 * 32 * 136 * 4;
+		constexpr int smem = ring > epi ? ring : epi;
+		static bool attr_set = false;
+		if (!attr_set) {
+			ELF_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dma::gemm_dw_group_kernel<EPI_F32_ACC>), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+			ELF_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dma::gemm_dw_group_kernel<EPI_F32_ACC_SCALE>), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+			attr_set = true;
+		}
+		if (scale != 0.f) ELF_LAUNCH(dma::gemm_dw_group_kernel<EPI_F32_ACC_SCALE>, dim3(next), dim3(512), smem, stream, ga);
+		else ELF_LAUNCH(dma::gemm_dw_group_kernel<EPI_F32_ACC>, dim3(next), dim3(512), smem, stream, ga);
+		ELF_CHECK_HIP(hipGetLastError());
+	}
+	// split tiles have no single epilogue that could scale them: a small kernel behind the launch does those
+	if (scale != 0.f)
+		for (int i = 0; i < n; i++)
+			if (ga.a[i].tail_tiles > 0) {
+				ELF_LAUNCH(dma::scale_tail_kernel, dim3(ga.a[i].tail_tiles), dim3(256), 0, stream, ga.a[i]);
+				ELF_CHECK_HIP(hipGetLastError());
+			}
+	return 0;
 }
 
 }  // namespace elf

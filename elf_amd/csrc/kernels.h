@@ -45,6 +45,24 @@ int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t 
 int gemm_dw_final(int M, int N, int K, const void* dY, int64_t lddy, const void* X, int64_t ldx, float* acc, void* grad_bf16, float scale,
                   hipStream_t stream);
 
+// The W pass of a stage in one launch: for each of n (at most 16) problems acc [M, N] (fp32, dense) += dY^T X with
+// dY [K, M] and X [K, N] over the same K tokens, on 256x256 tiles whose workgroups fill the chip together (one partly
+// filled round per launch instead of one per layer; when that round would leave half of the chip idle its tiles are
+// split along K and add in a fixed order).  scale != 0: every accumulator leaves multiplied by it, with its bf16 copy in
+// grad_bf16 (from the epilogue for whole tiles, by a small kernel behind the launch for split ones: same bits).  gemm_dw_groupable: a problem's
+// shape and operands fit (M, N multiples of 256, K of 64, 16-byte aligned, dense enough).
+struct DwProblem {
+	const void* dY;
+	int64_t lddy;
+	const void* X;
+	int64_t ldx;
+	float* acc;
+	void* grad_bf16;  // may be null when scale == 0
+	int M, N;
+};
+bool gemm_dw_groupable(int M, int N, int K, const void* dY, int64_t lddy, const void* X, int64_t ldx, const void* acc);
+int gemm_dw_group(int n, const DwProblem* problems, int K, float scale, hipStream_t stream);
+
 // The attention block's packed q | k | v projection with the rotary embedding of the q and k heads: C [M, N] =
 // A W^T rounded to bf16, then rope_apply's rotation on the first n_rot_heads heads of width D (cs: the table of
 // rope_table for sequence length S; row r is at position r mod S).  One kernel (rotation in the GEMM epilogue, the

@@ -510,8 +510,23 @@ static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool gra
 // copy written (PipelineBlock.scale_grads, elf/execution/block.py:518-527, folded into the pass that holds the tiles).
 static int run_backward_params(Stage* s, MbState& m, hipStream_t st, float scale = 0.f) {
 	const int T = s->T, d = s->d, F = s->F;
-	// dW[N_out, K_in] += dY[T, N_out]^T X[T, K_in]
+	// dW[N_out, K_in] += dY[T, N_out]^T X[T, K_in] for every linear layer of the stage: the layers whose shapes fit go
+	// into launches of up to 16 (their workgroups fill the chip together), in the stage's layer order; the others
+	// (a head whose vocabulary is not a multiple of 256) run one by one.  Which way a layer goes depends on its shape
+	// alone, so every stream that reaches this W pass accumulates its gradients in the same order of roundings.
+	DwProblem group[16];
+	int ng = 0;
+	static const bool no_group = getenv("ELF_NO_DW_GROUP") != nullptr;  // one launch per layer instead (for comparisons)
+	auto flush = [&]() -> int {
+		const int n = ng;
+		ng = 0;
+		return n ? gemm_dw_group(n, group, T, scale, st) : 0;
+	};
 	auto dw = [&](int M, int N, const void* dy, int64_t lddy, const void* x, int64_t ldx, float* acc, void* g16) -> int {
+		if (!no_group && gemm_dw_groupable(M, N, T, dy, lddy, x, ldx, acc) && (scale == 0.f || g16)) {
+			group[ng++] = DwProblem{dy, lddy, x, ldx, acc, g16, M, N};
+			return ng == 16 ? flush() : 0;
+		}
 		if (scale != 0.f) return gemm_dw_final(M, N, T, dy, lddy, x, ldx, acc, g16, scale, st);
 		return gemm_bf16(1, 1, M, N, T, dy, lddy, x, ldx, acc, N, EPI_F32_ACC, nullptr, 0, 0, 0, st);
 	};
@@ -525,6 +540,7 @@ static int run_backward_params(Stage* s, MbState& m, hipStream_t st, float scale
 		ELF_TRY(dw(s->nqkv, d, bs.b[B_DQKV].p, s->nqkv, bs.b[B_H1].p, d, p.g[P_WQKV], p.g16[P_WQKV]));
 	}
 	if (s->vocab_out) ELF_TRY(dw(s->vld, d, m.head.b[B_DQKV].p, s->vld, m.head.b[B_H1].p, d, s->xg[XP_HEAD], s->xg16[XP_HEAD]));
+	ELF_TRY(flush());
 	free_mask(s, m, WIN_MASK | WGRAD_MASK);
 	m.has_win = m.has_wgrad = false;
 	return 0;

@@ -4,6 +4,7 @@ torch is used for device memory and streams only; every op below is one call int
 libelf_stage.so on ``torch.cuda.current_stream()``.
 """
 
+import ctypes
 import math
 
 import torch
@@ -50,10 +51,39 @@ def gemm(a, b, *, a_t=False, b_t=False, out=None, epilogue=EPI_BF16, residual=No
 	return out
 
 
+class _DwProblem(ctypes.Structure):
+	"""``elf_dw_problem`` of include/elf_stage.h."""
+
+	_fields_ = [("dY", ctypes.c_void_p), ("lddy", ctypes.c_int64), ("X", ctypes.c_void_p), ("ldx", ctypes.c_int64), ("acc", ctypes.c_void_p),
+	            ("grad_bf16", ctypes.c_void_p), ("M", ctypes.c_int), ("N", ctypes.c_int)]
+
+
+def gemm_dw_group(problems, *, scale=0.0):
+	"""The weight gradients of several linear layers over the same tokens in one launch.  ``problems``: tuples
+	``(dy [K, M] bf16, x [K, N] bf16, acc [M, N] fp32)`` or ``(dy, x, acc, grad_bf16 [M, N] bf16)``: ``acc += dy.T @ x``;
+	with ``scale`` every ``acc`` is then multiplied by it and ``grad_bf16`` receives its bf16 rounding."""
+	arr = (_DwProblem * len(problems))()
+	K = problems[0][0].shape[0] if problems else 0
+	for q, pr in zip(arr, problems):
+		dy, x, acc = pr[0], pr[1], pr[2]
+		g16 = pr[3] if len(pr) > 3 else None
+		_need(dy, torch.bfloat16, "gemm_dw_group.dy")
+		_need(x, torch.bfloat16, "gemm_dw_group.x")
+		_need(acc, torch.float32, "gemm_dw_group.acc")
+		M, N = dy.shape[1], x.shape[1]
+		if dy.shape[0] != K or x.shape[0] != K:
+			raise _lib.ElfStageError(f"gemm_dw_group: every problem reduces over the same {K} rows")
+		if tuple(acc.shape) != (M, N) or not acc.is_contiguous() or (g16 is not None and (tuple(g16.shape) != (M, N) or not g16.is_contiguous())):
+			raise _lib.ElfStageError(f"gemm_dw_group: accumulators are dense [{M}, {N}]")
+		if g16 is not None:
+			_need(g16, torch.bfloat16, "gemm_dw_group.grad_bf16")
+		q.dY, q.lddy, q.X, q.ldx, q.acc, q.grad_bf16, q.M, q.N = _ptr(dy), dy.stride(0), _ptr(x), x.stride(0), _ptr(acc), _ptr(g16), M, N
+	rc = _lib.load().elf_gemm_dw_group(len(problems), ctypes.cast(arr, ctypes.c_void_p), K, float(scale), _stream())
+	_lib.check(rc, "elf_gemm_dw_group")
+
+
 def gemm_turn_giveups():
 	"""Waves of split-K GEMM launches on the current device that added out of turn since the library was loaded."""
-	import ctypes
-
 	n = ctypes.c_uint64()
 	_lib.check(_lib.load().elf_gemm_turn_giveups(ctypes.byref(n)), "elf_gemm_turn_giveups")
 	return n.value

@@ -53,6 +53,29 @@ int elf_gemm_bf16(int a_t, int b_t, int M, int N, int K, const void* A, int64_t 
  * reference (torch.mm's split-K is not reproducible either way). */
 int elf_gemm_turn_giveups(uint64_t* out);
 
+/* The weight gradients of several linear layers over the same K tokens in one launch: for problem i,
+ * acc[M, N] (fp32, dense) += dY^T X with dY [K, M] (leading dim lddy) and X [K, N] (leading dim ldx), i.e. what n calls of
+ * elf_gemm_bf16(1, 1, ..., epilogue 2) compute.  The workgroups of all problems fill the chip together: only the
+ * launch's last round of 256 tiles is partly filled, and when it would be at most half full its tiles (the last ones of
+ * the last problems) are split along K, up to 8 ways with at least 16 slices of 64 each; split tiles add in the order of
+ * their K ranges (see elf_gemm_turn_giveups), so the sums are bit-identical from run to run.  A tile's sum is rounded
+ * once per K range: the bits equal elf_gemm_bf16's when that call splits the tile the same way.
+ * scale != 0: every acc leaves multiplied by scale and grad_bf16[M, N] receives its bf16 rounding (the step's last W
+ * pass with PipelineBlock.scale_grads folded in, elf/execution/block.py:518-527); grad_bf16 may be NULL otherwise.
+ * n <= 16; M, N multiples of 256, K of 64; pointers 16-byte aligned.
+ * Replaces: the loop over LayerDW modules of PipelineBlock.backward_params (elf/execution/block.py:384-389), each
+ *           iteration torch.mm(go.t(), inp) + weight.grad.add_ of LinearDW.backward (elf/zb_utils.py:238-244). */
+typedef struct elf_dw_problem {
+	const void* dY;
+	int64_t lddy;
+	const void* X;
+	int64_t ldx;
+	float* acc;
+	void* grad_bf16;
+	int M, N;
+} elf_dw_problem;
+int elf_gemm_dw_group(int n, const elf_dw_problem* problems, int K, float scale, void* stream);
+
 /* The MLP's up-projection with its activation: pre = A W^T with A [M, K] and W [N, K], both k contiguous;
  * act 0 (GELU): N = F, out[M, F] = gelu(pre); act 1 (SwiGLU): N = 2F, W = [gate rows; up rows],
  * pre[M, 2F] = [g | u], out[M, F] = silu(g) * u.  pre is kept because the backward needs it.  SwiGLU is

@@ -442,6 +442,80 @@ def test_split_k_on_one_stream_never_gives_up_its_turn_and_wide_splits_are_refus
 		K.gemm(A, B, a_t=True, b_t=True, out=runs[0], epilogue=K.EPI_F32_ACC, k_splits=256, tile_cfg=7)
 
 
+def _dw_problems(shapes, Kd, seed):
+	"""(dy [Kd, M], x [Kd, N], acc [M, N] with what earlier micro-batches left in it) per (M, N)."""
+	out = []
+	for i, (M, N) in enumerate(shapes):
+		g = torch.Generator(device="cuda").manual_seed(seed + i)
+		out.append((_randn(Kd, M, seed=seed + 10 * i), _randn(Kd, N, seed=seed + 10 * i + 1, scale=0.05), torch.randn(M, N, generator=g, device="cuda")))
+	return out
+
+
+def test_grouped_weight_gradients_equal_the_single_launches(K):
+	"""Several layers' dW += dY^T X in one launch (the W pass of a stage) against one elf_gemm_bf16 call per layer that
+	splits K the same way: whole tiles (K too short to split); the GPT-2-small layers at K = 4096, whose 108 tiles are all
+	in the launch's only round and split two ways; and a large layer (256 whole tiles, one round) followed by two small
+	ones whose 36 tiles make up the last round and are split four ways.  Bit for bit, run after run, no turn given up; and
+	against fp32 torch."""
+	before = K.gemm_turn_giveups()
+	for shapes, Kd, splits in (
+		(((256, 512), (768, 256), (512, 768), (256, 256)), 512, (1, 1, 1, 1)),
+		(((768, 3072), (3072, 768), (768, 768), (2304, 768)), 4096, (2, 2, 2, 2)),
+		(((4096, 4096), (768, 768), (768, 2304)), 4096, (1, 4, 4)),
+	):
+		print(f"[case] gemm_dw_group {shapes} K={Kd}", flush=True)
+		problems = _dw_problems(shapes, Kd, seed=400)
+		start = [acc.clone() for _, _, acc in problems]
+		want = []
+		for (dy, x, _), acc0, ks in zip(problems, start, splits):
+			acc = acc0.clone()
+			K.gemm(dy, x, a_t=True, b_t=True, out=acc, epilogue=K.EPI_F32_ACC, tile_cfg=7, k_splits=ks)
+			want.append(acc)
+		runs = []
+		for _ in range(3):
+			accs = [a.clone() for a in start]
+			K.gemm_dw_group([(dy, x, acc) for (dy, x, _), acc in zip(problems, accs)])
+			runs.append(accs)
+		torch.cuda.synchronize()
+		for i, (dy, x, _) in enumerate(problems):
+			assert torch.equal(runs[0][i], want[i]), f"layer {i} {shapes[i]}: grouped launch differs from the single one"
+			assert torch.equal(runs[1][i], want[i]) and torch.equal(runs[2][i], want[i]), f"layer {i}: not reproducible"
+			ref = start[i].double() + dy.double().t() @ x.double()
+			assert ((want[i].double() - ref).abs().max() / ref.abs().max()).item() <= 1e-5
+	assert K.gemm_turn_giveups() == before
+
+
+def test_grouped_weight_gradients_with_the_gradient_scale(K):
+	"""scale != 0: the accumulators leave multiplied by the scale with their bf16 copies written, from the epilogue for
+	whole tiles and by a small kernel behind the launch for split ones (here: none split, all split, and a whole layer
+	followed by a split one): all equal the unscaled launch followed by elf_scale_grads bit for bit."""
+	for shapes, Kd in ((((256, 512), (768, 256)), 512), (((768, 3072), (768, 768)), 8192), (((4096, 4096), (768, 768)), 4096)):
+		problems = _dw_problems(shapes, Kd, seed=500)
+		plain = [acc.clone() for _, _, acc in problems]
+		K.gemm_dw_group([(dy, x, acc) for (dy, x, _), acc in zip(problems, plain)])
+		plain16 = [torch.empty_like(a, dtype=torch.bfloat16) for a in plain]
+		for a, h in zip(plain, plain16):
+			K.scale_grads_(a, h, 1 / 32)
+		folded = [acc.clone() for _, _, acc in problems]
+		folded16 = [torch.full_like(a, 7.0, dtype=torch.bfloat16) for a in folded]
+		K.gemm_dw_group([(dy, x, acc, h) for (dy, x, _), acc, h in zip(problems, folded, folded16)], scale=1 / 32)
+		torch.cuda.synchronize()
+		for i in range(len(problems)):
+			assert torch.equal(folded[i], plain[i]) and torch.equal(folded16[i], plain16[i]), f"layer {i} {shapes[i]} K={Kd}"
+
+
+def test_grouped_weight_gradients_refuse_what_the_tiles_cannot_hold(K):
+	from elf_amd import _lib
+
+	ok = _dw_problems(((256, 256),), 512, seed=600)
+	with pytest.raises(_lib.ElfStageError):
+		K.gemm_dw_group(ok * 17)
+	with pytest.raises(_lib.ElfStageError):
+		K.gemm_dw_group(_dw_problems(((256, 320),), 512, seed=601))
+	with pytest.raises(_lib.ElfStageError):
+		K.gemm_dw_group(ok, scale=0.5)  # a scaling pass needs somewhere to put the bf16 gradients
+
+
 def test_split_k_gemms_on_two_streams_stay_correct(K):
 	"""Weight-gradient GEMMs launched concurrently on two streams share the turn counters of their split tiles; whatever
 	the interleaving, every sum must be the right one to fp32 rounding (a workgroup that finds its counter taken by
