@@ -877,58 +877,68 @@ __global__ __launch_bounds__(256) void embedding_fwd_kernel(const int64_t* __res
 		store8(out + t * d + c, x);
 	}
 }
-// dtable[ids[t], :] += dx[t, :] in fp32.  One workgroup per token position.  The workgroup of a token's first
-// occurrence sums the rows of all its occurrences in ascending position and is the only writer of that table
-// row: no atomics, and the sums do not depend on the order in which workgroups run.  The other workgroups find an
-// earlier occurrence and leave (the ids are a few KiB and stay in cache).
+// dtable[ids[t], :] += dx[t, :] in fp32.  One workgroup of four waves per (token position, 512-column slice).  The
+// workgroups of a token's first occurrence sum the rows of all its occurrences, each over its own column slice, and are
+// the only writers of that table row: no atomics.  The positions behind the first occurrence are dealt to the four
+// waves in runs of 64 (run k to wave k % 4); a wave adds its occurrences in ascending position, 16 row loads in flight
+// at a time, and the four partial sums are folded in wave order: a fixed order of additions whatever the order in
+// which waves run (bit-reproducible), and a token that fills the whole batch (padding) is summed by d / 128 waves
+// instead of one.  The other workgroups find an earlier occurrence and leave (the ids are a few KiB and stay in cache).
 __global__ __launch_bounds__(256) void embedding_bwd_kernel(const int64_t* __restrict__ ids, const bf16_t* __restrict__ dx,
                                                             float* __restrict__ dtable, int T, int d, int V) {
-	__shared__ unsigned long long hit[4];
+	__shared__ float part[4][512];
 	const int t = blockIdx.x;
 	const int64_t id = ids[t];
 	if (id < 0 || id >= V) return;
 	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-	for (int base = 0; base < t; base += 256) {
-		const int u = base + threadIdx.x;
-		if (__syncthreads_or(u < t && ids[u] == id)) return;
+	{
+		// an earlier occurrence?  The first 256 positions with one barrier (a frequent token is found there), then each wave
+		// takes every fourth run of 128 positions without a barrier in between
+		if (__syncthreads_or((int)threadIdx.x < t && ids[threadIdx.x] == id)) return;
+		bool seen = false;
+		for (int base = 256 + wave * 128; base < t && !seen; base += 512) {
+			const int u = base + 2 * lane;
+			const int64_t a = u < t ? ids[u] : -1, b = u + 1 < t ? ids[u + 1] : -1;
+			seen = __ballot(a == id || b == id) != 0;
+		}
+		if (__syncthreads_or(seen)) return;
 	}
-	constexpr int MAXC = 4;  // d <= 8192: at most four 8-column chunks per lane
-	const int cpr = d / 8;
-	float acc[MAXC][8];
+	const int ch = blockIdx.y * 64 + lane;  // this lane's 8-column chunk
+	const bool mine = ch < d / 8;
+	float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+	for (int base = t + wave * 64; base < T; base += 256) {
+		const int u = base + lane;
+		unsigned long long bits = __ballot(u < T && ids[u] == id);
+		while (bits) {
+			constexpr int AHEAD = 16;
+			Chunk x[AHEAD];
+			int n = 0;
 #pragma unroll
-	for (int i = 0; i < MAXC; i++)
-#pragma unroll
-		for (int k = 0; k < 8; k++) acc[i][k] = 0.f;
-	for (int base = t; base < T; base += 256) {
-		const int u = base + threadIdx.x;
-		const unsigned long long b = __ballot(u < T && ids[u] == id);
-		if (lane == 0) hit[wave] = b;
-		__syncthreads();
-		for (int w = 0; w < 4; w++) {
-			unsigned long long bits = hit[w];
-			while (bits) {
-				const int64_t row = base + w * 64 + (__ffsll(bits) - 1);
-				bits &= bits - 1;
-#pragma unroll
-				for (int i = 0; i < MAXC; i++) {
-					const int ch = threadIdx.x + i * 256;
-					if (ch < cpr) {
-						const Chunk x = load8(dx + row * d + ch * 8);
-#pragma unroll
-						for (int k = 0; k < 8; k++) acc[i][k] += x.v[k];
-					}
+			for (int k = 0; k < AHEAD; k++) {
+				if (bits) {
+					const int64_t row = base + (__ffsll(bits) - 1);
+					bits &= bits - 1;
+					if (mine) x[k] = load8(dx + row * d + ch * 8);
+					n = k + 1;
 				}
 			}
+#pragma unroll
+			for (int k = 0; k < AHEAD; k++)
+				if (k < n && mine) {
+#pragma unroll
+					for (int j = 0; j < 8; j++) acc[j] += x[k].v[j];
+				}
 		}
-		__syncthreads();
 	}
 #pragma unroll
-	for (int i = 0; i < MAXC; i++) {
-		const int ch = threadIdx.x + i * 256;
-		if (ch < cpr) {
-			float* g = dtable + id * d + ch * 8;
+	for (int j = 0; j < 8; j++) part[wave][lane * 8 + j] = acc[j];
+	__syncthreads();
+	if (wave == 0 && mine) {
+		float* g = dtable + id * d + ch * 8;
 #pragma unroll
-			for (int k = 0; k < 8; k++) g[k] += acc[i][k];
+		for (int j = 0; j < 8; j++) {
+			const float sum = ((part[0][lane * 8 + j] + part[1][lane * 8 + j]) + part[2][lane * 8 + j]) + part[3][lane * 8 + j];
+			g[j] += sum;
 		}
 	}
 }
@@ -944,7 +954,7 @@ int embedding_bwd(const void* ids, const void* dx, void* dtable_f32, int64_t T, 
 	ELF_REQUIRE(ids && dx && dtable_f32 && T > 0 && V > 0 && d > 0 && d % 8 == 0 && d <= 8192 && T < (int64_t(1) << 31),
 	            "embedding_bwd: bad argument (d must be a multiple of 8 and at most 8192)");
 	ProfScope prof(PROF_EMBED, 10.0 * T * d, s);
-	ELF_LAUNCH(embedding_bwd_kernel, dim3((unsigned)T), dim3(256), 0, s, (const int64_t*)ids, (const bf16_t*)dx, (float*)dtable_f32, (int)T, d, V);
+	ELF_LAUNCH(embedding_bwd_kernel, dim3((unsigned)T, (unsigned)((d / 8 + 63) / 64)), dim3(256), 0, s, (const int64_t*)ids, (const bf16_t*)dx, (float*)dtable_f32, (int)T, d, V);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
 }

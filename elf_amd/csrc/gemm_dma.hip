@@ -1084,14 +1084,15 @@ static int launch_pers(const Args& a, hipStream_t stream) {
 
 // The split tiles of a launch with the scaling accumulate epilogue: their workgroups add partial sums and none of them
 // holds the finished tile, so the scale and the bf16 copy of those (few, at most 128) tiles are applied here, behind the
-// GEMM on the same stream.  One workgroup per tile; tile index and origin as in the GEMM.
+// GEMM on the same stream.  Eight workgroups per tile (32 rows each); tile index and origin as in the GEMM.
 __global__ __launch_bounds__(256) void scale_tail_kernel(Args g) {
 	const int ntiles = g.tiles_m * g.tiles_n;
-	const int pid = ntiles - g.tail_tiles + (int)blockIdx.x;
+	const int pid = ntiles - g.tail_tiles + (int)(blockIdx.x >> 3);
 	int m0, n0;
 	tile_origin<256>(g, pid, m0, n0);
+	m0 += (int)(blockIdx.x & 7) * 32;
 	float* C = reinterpret_cast<float*>(g.C);
-	for (int i = threadIdx.x; i < 256 * 64; i += 256) {
+	for (int i = threadIdx.x; i < 32 * 64; i += 256) {
 		const int row = i >> 6, c4 = (i & 63) * 4;
 		float* c = C + (int64_t)(m0 + row) * g.ldc + n0 + c4;
 		f32x4 v = *reinterpret_cast<const f32x4*>(c);
@@ -1204,7 +1205,7 @@ int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t 
 	if (a_t && b_t) {
 		if (int rc = dma::launch_epi<8, 2, true, true>(a, epi, stream)) return rc;
 		if (epi == EPI_F32_ACC_SCALE && a.tail_tiles > 0) {
-			ELF_LAUNCH(dma::scale_tail_kernel, dim3(a.tail_tiles), dim3(256), 0, stream, a);
+			ELF_LAUNCH(dma::scale_tail_kernel, dim3(a.tail_tiles * 8), dim3(256), 0, stream, a);
 			ELF_CHECK_HIP(hipGetLastError());
 		}
 		return 0;
@@ -1288,7 +1289,7 @@ int gemm_dw_group(int n, const DwProblem* pr, int K, float scale, hipStream_t st
 	if (scale != 0.f)
 		for (int i = 0; i < n; i++)
 			if (ga.a[i].tail_tiles > 0) {
-				ELF_LAUNCH(dma::scale_tail_kernel, dim3(ga.a[i].tail_tiles), dim3(256), 0, stream, ga.a[i]);
+				ELF_LAUNCH(dma::scale_tail_kernel, dim3(ga.a[i].tail_tiles * 8), dim3(256), 0, stream, ga.a[i]);
 				ELF_CHECK_HIP(hipGetLastError());
 			}
 	return 0;
