@@ -188,7 +188,7 @@ __device__ __forceinline__ void store_dk_dv(const f32x16 (&acc_dk)[D / 32], cons
 // a workgroup takes the tiles kt and nkt-1-kt one after the other: every workgroup then does
 // the same amount of work.
 template <int D, bool CAUSAL>
-__global__ __launch_bounds__(256) void attn_bwd_kernel(AttnBwdArgs a) {
+__global__ __launch_bounds__(256, D == 64 ? 2 : 1) void attn_bwd_kernel(AttnBwdArgs a) {
 	using TL = BwdTile<D>;
 	constexpr int BKV = 128, BQ = 32;
 	constexpr int NF = D / 16;  // fragments per operand tile
