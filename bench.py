@@ -578,7 +578,7 @@ def main():
 			"tokens_per_step": tokens, "ops_per_step": len(stream), "offload": bool(w.get("offload")), "hip_graph": bool(args.graph),
 		},
 		"roofline": {"bound": "mfma", "achieved": g["tflops"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": g["tflops"] / PEAK_BF16_TFLOPS, "traffic": gemm_traffic_bytes(args.workload),
-		             "kernel": "elf::dma::gemm_pers_kernel / elf::dma::gemm_dma_kernel / elf::gemm_kernel (bf16 MFMA GEMM, all layouts)", "launches": g["launches"], "avg_launch_ms": g["avg_ms"]},
+		             "kernel": "elf::dma::gemm_pers_kernel / elf::dma::gemm_dma_kernel / elf::dma::gemm_dw_group_kernel / elf::gemm_kernel (bf16 MFMA GEMM, all layouts)", "launches": g["launches"], "avg_launch_ms": g["avg_ms"]},
 		"stream_mfu": stream_flops(w) / (elapsed / args.steps) / (PEAK_BF16_TFLOPS * 1e12),
 		"kernels": per_kernel,
 		"peak_stage_memory_bytes": mem["peak_bytes"] + mem["workspace_bytes"] + torch.cuda.max_memory_allocated(),
