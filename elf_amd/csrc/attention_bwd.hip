@@ -812,10 +812,11 @@ __global__ __launch_bounds__(256) void dq_reduce_kernel(const bf16_t* __restrict
 		const int ns = causal ? q / 128 + 1 : nkt;
 		float lo[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, hi[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 		const bf16_t* pb = part + (int64_t)b * rows_b * cols + c;
-#pragma unroll 4
+#pragma unroll 8
 		for (int kt = 0; kt < ns; kt++) {
 			const bf16_t* pr_row = pb + (part_row0(kt, S, causal) + q - (causal ? 128 * kt : 0)) * cols;
-			const bf16x8 v = *reinterpret_cast<const bf16x8*>(pr_row), w = *reinterpret_cast<const bf16x8*>(pr_row + half);
+			// read once: no point in keeping the partials in the caches
+			const bf16x8 v = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(pr_row)), w = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(pr_row + half));
 #pragma unroll
 			for (int t = 0; t < 8; t++) {
 				lo[t] += (float)v[t];
