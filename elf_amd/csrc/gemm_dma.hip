@@ -547,8 +547,8 @@ __device__ __forceinline__ void gemm_dma_tile(const Args& g, const int pid, cons
 #pragma unroll
 			for (int it = 0; it < 8; it++) {
 				const bf16_t* r = g.R + (int64_t)(grow0 + it * 4 + (lane >> 4)) * g.ldr + gcol0 + (lane & 15) * 8;
-				gs[it] = *reinterpret_cast<const bf16x8*>(r);
-				us[it] = *reinterpret_cast<const bf16x8*>(r + F);
+				gs[it] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(r));  // the pre-activation is read this once in B
+				us[it] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(r + F));
 			}
 #pragma unroll
 			for (int it = 0; it < 8; it++) {
@@ -674,7 +674,7 @@ __device__ __forceinline__ void gemm_dma_tile(const Args& g, const int pid, cons
 			if constexpr (ACCUM) {
 #pragma unroll
 				for (int it = 0; it < 16; it++)
-					cv[it] = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(g.C) + (int64_t)(grow0 + it * 2 + (lane >> 5)) * g.ldc + gcol0 + (lane & 31) * 4);
+					cv[it] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(g.C) + (int64_t)(grow0 + it * 2 + (lane >> 5)) * g.ldc + gcol0 + (lane & 31) * 4));
 			}
 #pragma unroll
 			for (int it = 0; it < 16; it++) {
@@ -691,7 +691,8 @@ __device__ __forceinline__ void gemm_dma_tile(const Args& g, const int pid, cons
 					for (int t = 0; t < 4; t++) o[t] = (bf16_t)v[t];
 					*reinterpret_cast<bf16x4*>(g.C2 + (int64_t)(grow0 + row) * g.ldc2 + gcol0 + c4) = o;
 				}
-				*reinterpret_cast<f32x4*>(c) = v;
+				if constexpr (ACCUM) __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(c));  // next touched by the next W pass
+				else *reinterpret_cast<f32x4*>(c) = v;
 			}
 		}
 	}
