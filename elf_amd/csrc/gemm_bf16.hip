@@ -518,18 +518,24 @@ bool gemm_swiglu_bwd_fused(int M, int F, int K) {
 }
 
 int gemm_swiglu_bwd_bf16(int M, int F, int K, const void* dY, int64_t lddy, const void* W, int64_t ldw, const void* gu,
-                         int64_t ldgu, void* dgu, int64_t lddgu, void* scratch, hipStream_t stream) {
+                         int64_t ldgu, void* dgu, int64_t lddgu, void* scratch, hipStream_t stream, void* act, int64_t ldact) {
 	ELF_REQUIRE(M > 0 && F > 0 && K > 0 && dY && W && gu && dgu, "gemm_swiglu_bwd: empty problem or null operand");
 	if (gemm_swiglu_bwd_fused(M, F, K) && lddy >= K && ldw >= F && ldgu >= 2 * F && lddgu >= 2 * F && lddy % 8 == 0 && ldw % 8 == 0 && ldgu % 8 == 0 &&
 	    lddgu % 8 == 0 && ((uintptr_t)dY % 16) == 0 && ((uintptr_t)W % 16) == 0 && ((uintptr_t)gu % 16) == 0 && ((uintptr_t)dgu % 16) == 0) {
 		// the activation backward's arithmetic is not counted: the figure stays the GEMM's
 		ProfScope prof(PROF_GEMM, 2.0 * M * F * K, stream);
-		return gemm_bf16_dma(0, 1, M, F, K, dY, lddy, W, ldw, dgu, lddgu, EPI_BF16_SWIGLU_BWD, gu, ldgu, 1, 0, 256, stream, nullptr, 0);
+		ELF_REQUIRE(!act || (ldact >= F && ldact % 8 == 0 && ((uintptr_t)act % 16) == 0), "gemm_swiglu_bwd: bad activation output");
+		return gemm_bf16_dma(0, 1, M, F, K, dY, lddy, W, ldw, dgu, lddgu, EPI_BF16_SWIGLU_BWD, gu, ldgu, 1, 0, 256, stream, act, ldact);
 	}
 	ELF_REQUIRE(scratch, "gemm_swiglu_bwd: this shape needs a scratch buffer of M x F bf16");
 	ELF_REQUIRE(ldgu == 2 * F && lddgu == 2 * F, "gemm_swiglu_bwd: the unfused path needs dense [M, 2F] buffers");
 	if (int rc = gemm_bf16(0, 1, M, F, K, dY, lddy, W, ldw, scratch, F, EPI_BF16, nullptr, 0, 0, 0, stream)) return rc;
-	return swiglu_bwd(scratch, gu, dgu, M, F, stream);
+	if (int rc = swiglu_bwd(scratch, gu, dgu, M, F, stream)) return rc;
+	if (act) {
+		ELF_REQUIRE(ldact == F, "gemm_swiglu_bwd: the unfused path needs a dense activation output");
+		return swiglu_fwd(gu, act, M, F, stream);
+	}
+	return 0;
 }
 
 }  // namespace elf

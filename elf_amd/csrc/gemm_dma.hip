@@ -567,6 +567,14 @@ __device__ __forceinline__ void gemm_dma_tile(const Args& g, const int pid, cons
 				bf16_t* c = reinterpret_cast<bf16_t*>(g.C) + (int64_t)(grow0 + row) * g.ldc + gcol0 + c8;
 				*reinterpret_cast<bf16x8*>(c) = og;
 				*reinterpret_cast<bf16x8*>(c + F) = ou;
+				if (g.C2) {
+					// a stash that dropped the activation gets it back here, from the g and u this epilogue holds anyway (the
+					// forward's own arithmetic: the bits of swiglu_fwd)
+					bf16x8 oa;
+#pragma unroll
+					for (int t = 0; t < 8; t++) oa[t] = (bf16_t)swiglu_f((float)gs[it][t], (float)us[it][t]);
+					*reinterpret_cast<bf16x8*>(g.C2 + (int64_t)(grow0 + row) * g.ldc2 + gcol0 + c8) = oa;
+				}
 			}
 		} else if constexpr (EPI == EPI_BF16_ROPE) {
 			// A 128-column strip holds whole heads (rope_D = 64 or 128).  A lane takes, for one row, 8 columns of a

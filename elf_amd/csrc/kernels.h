@@ -94,9 +94,11 @@ int gemm_act_bf16(int act, int M, int F, int K, const void* A, int64_t lda, cons
 // gate/up product.  One kernel (activation backward in the GEMM epilogue, d never reaches memory) when the shape
 // fits the direct-to-LDS tiles; otherwise the GEMM writes d into `scratch` [M, F] and the activation backward
 // kernel follows.  Both ways give the same bits.  `scratch` may be null when gemm_swiglu_bwd_fused(M, F, K).
+// act non-null: the activation silu(g) * u [M, F] (leading dim ldact) is written as well, with the bits of swiglu_fwd
+// (a stash that dropped it after the forward gets it back from the g and u the epilogue reads anyway).
 bool gemm_swiglu_bwd_fused(int M, int F, int K);
 int gemm_swiglu_bwd_bf16(int M, int F, int K, const void* dY, int64_t lddy, const void* W, int64_t ldw, const void* gu,
-                         int64_t ldgu, void* dgu, int64_t lddgu, void* scratch, hipStream_t stream);
+                         int64_t ldgu, void* dgu, int64_t lddgu, void* scratch, hipStream_t stream, void* act = nullptr, int64_t ldact = 0);
 
 enum NormKind { NORM_RMS = 0, NORM_LAYER = 1 };
 

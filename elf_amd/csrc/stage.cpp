@@ -388,11 +388,11 @@ static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool gra
 		PoolTmp d_h(s->pool, (size_t)T * d * 2);
 		if (!d_h.p) return -3;
 		if (s->llama && !pre && gemm_swiglu_bwd_fused(T, F, d)) {
-			ELF_TRY(gemm_swiglu_bwd_bf16(T, F, d, dyin, d, p.w[P_W2], F, bs.b[B_GU].p, s->ffn_in, bs.b[B_DGU].p, s->ffn_in, nullptr, st));
-			if (reform && bs.b[B_A].dropped) {
-				ELF_TRY(buf_alloc(s, bs, B_A));
-				ELF_TRY(swiglu_fwd(bs.b[B_GU].p, bs.b[B_A].p, T, F, st));
-			}
+			// a dropped FFN activation (lean stash) is formed again by the same kernel, from the gate/up values its epilogue reads
+			const bool form_a = reform && bs.b[B_A].dropped;
+			if (form_a) ELF_TRY(buf_alloc(s, bs, B_A));
+			ELF_TRY(gemm_swiglu_bwd_bf16(T, F, d, dyin, d, p.w[P_W2], F, bs.b[B_GU].p, s->ffn_in, bs.b[B_DGU].p, s->ffn_in, nullptr, st,
+			                             form_a ? bs.b[B_A].p : nullptr, F));
 			ELF_TRY(gemm_bf16(0, 1, T, d, s->ffn_in, bs.b[B_DGU].p, s->ffn_in, p.w[P_W1], d, d_h.p, d, EPI_BF16, nullptr, 0, 0, 0, st));
 		} else {
 			PoolTmp d_a(s->pool, (size_t)T * F * 2);
