@@ -638,9 +638,11 @@ __global__ __launch_bounds__(256) void swiglu_fwd_kernel(const bf16_t* __restric
 		store8(h + row * F + c8, g);
 	}
 }
-// dgu[:, :F] = dh * u * (sig + g sig (1 - sig));  dgu[:, F:] = dh * g * sig
+// dgu[:, :F] = dh * u * (sig + g sig (1 - sig));  dgu[:, F:] = dh * g * sig.  ACT: the activation silu(g) * u goes to
+// `act` [T, F] as well (a stash that dropped it gets it back from the g and u read here anyway: the bits of swiglu_fwd).
+template <bool ACT>
 __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const bf16_t* __restrict__ dh, const bf16_t* __restrict__ gu,
-                                                         bf16_t* __restrict__ dgu, int64_t T, int F) {
+                                                         bf16_t* __restrict__ dgu, bf16_t* __restrict__ act, int64_t T, int F) {
 	const int cpr = F >> 3;
 	const int64_t n = T * cpr;
 	for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
@@ -652,6 +654,11 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const bf16_t* __restric
 		for (int j = 0; j < 8; j++) swiglu_bwd_f(d.v[j], g.v[j], u.v[j], dg.v[j], du.v[j]);
 		store8(dgu + row * 2 * F + c8, dg);
 		store8(dgu + row * 2 * F + F + c8, du);
+		if constexpr (ACT) {
+#pragma unroll
+			for (int j = 0; j < 8; j++) g.v[j] = swiglu_f(g.v[j], u.v[j]);
+			store8(act + row * F + c8, g);
+		}
 	}
 }
 
@@ -682,11 +689,11 @@ int swiglu_fwd(const void* gu, void* h, int64_t T, int F, hipStream_t s) {
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
 }
-int swiglu_bwd(const void* dh, const void* gu, void* dgu, int64_t T, int F, hipStream_t s) {
+int swiglu_bwd(const void* dh, const void* gu, void* dgu, int64_t T, int F, hipStream_t s, void* act) {
 	ELF_REQUIRE(T > 0 && F > 0 && F % 8 == 0 && gu && dh && dgu, "swiglu_bwd: F must be a positive multiple of 8");
-	ProfScope prof(PROF_ACT_BWD, 10.0 * T * F, s);
-	ELF_LAUNCH(swiglu_bwd_kernel, dim3(ew_grid(T * (F / 8))), dim3(256), 0, s, (const bf16_t*)dh,
-	                   (const bf16_t*)gu, (bf16_t*)dgu, T, F);
+	ProfScope prof(PROF_ACT_BWD, (act ? 12.0 : 10.0) * T * F, s);
+	if (act) ELF_LAUNCH(swiglu_bwd_kernel<true>, dim3(ew_grid(T * (F / 8))), dim3(256), 0, s, (const bf16_t*)dh, (const bf16_t*)gu, (bf16_t*)dgu, (bf16_t*)act, T, F);
+	else ELF_LAUNCH(swiglu_bwd_kernel<false>, dim3(ew_grid(T * (F / 8))), dim3(256), 0, s, (const bf16_t*)dh, (const bf16_t*)gu, (bf16_t*)dgu, (bf16_t*)nullptr, T, F);
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
 }

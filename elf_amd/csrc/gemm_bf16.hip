@@ -530,12 +530,8 @@ int gemm_swiglu_bwd_bf16(int M, int F, int K, const void* dY, int64_t lddy, cons
 	ELF_REQUIRE(scratch, "gemm_swiglu_bwd: this shape needs a scratch buffer of M x F bf16");
 	ELF_REQUIRE(ldgu == 2 * F && lddgu == 2 * F, "gemm_swiglu_bwd: the unfused path needs dense [M, 2F] buffers");
 	if (int rc = gemm_bf16(0, 1, M, F, K, dY, lddy, W, ldw, scratch, F, EPI_BF16, nullptr, 0, 0, 0, stream)) return rc;
-	if (int rc = swiglu_bwd(scratch, gu, dgu, M, F, stream)) return rc;
-	if (act) {
-		ELF_REQUIRE(ldact == F, "gemm_swiglu_bwd: the unfused path needs a dense activation output");
-		return swiglu_fwd(gu, act, M, F, stream);
-	}
-	return 0;
+	ELF_REQUIRE(!act || ldact == F, "gemm_swiglu_bwd: the unfused path needs a dense activation output");
+	return swiglu_bwd(scratch, gu, dgu, M, F, stream, act);
 }
 
 }  // namespace elf

@@ -117,7 +117,8 @@ int norm_bwd_noalloc(int kind, const void* dy, const void* x, const void* gamma,
 int gelu_fwd(const void* x, void* y, int64_t n, hipStream_t s);
 int gelu_bwd(const void* dy, const void* x, void* dx, int64_t n, hipStream_t s);
 int swiglu_fwd(const void* gu, void* h, int64_t T, int F, hipStream_t s);
-int swiglu_bwd(const void* dh, const void* gu, void* dgu, int64_t T, int F, hipStream_t s);
+// act non-null: silu(g) * u [T, F] is written as well (the bits of swiglu_fwd)
+int swiglu_bwd(const void* dh, const void* gu, void* dgu, int64_t T, int F, hipStream_t s, void* act = nullptr);
 int rope_table(void* cs, int S, int D, double theta, hipStream_t s);
 int rope_apply(void* buf, const void* cs, int64_t T, int S, int ld, int n_heads, int D, int backward, hipStream_t s);
 int scale_grads(void* acc_f32, void* out_bf16, int64_t n, float scale, hipStream_t s);

@@ -409,12 +409,12 @@ static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool gra
 				const bf16_t* gu_c = (const bf16_t*)bs.b[B_GU].p + (size_t)c * Tc * s->ffn_in;
 				bf16_t* dgu_c = (bf16_t*)bs.b[B_DGU].p + (size_t)c * Tc * s->ffn_in;
 				const bf16_t* da_c = (const bf16_t*)d_a.p + (size_t)c * Tc * F;
-				if (s->llama) ELF_TRY(swiglu_bwd(da_c, gu_c, dgu_c, Tc, F, st));
-				else ELF_TRY(gelu_bwd(da_c, gu_c, dgu_c, (int64_t)Tc * F, st));
-				if (form_a) {
-					bf16_t* a_c = (bf16_t*)bs.b[B_A].p + (size_t)c * Tc * F;
-					if (s->llama) ELF_TRY(swiglu_fwd(gu_c, a_c, Tc, F, st));
-					else ELF_TRY(gelu_fwd(gu_c, a_c, (int64_t)Tc * F, st));
+				bf16_t* a_c = form_a ? (bf16_t*)bs.b[B_A].p + (size_t)c * Tc * F : nullptr;
+				if (s->llama) {
+					ELF_TRY(swiglu_bwd(da_c, gu_c, dgu_c, Tc, F, st, a_c));  // the activation, when dropped, from the same pass over g and u
+				} else {
+					ELF_TRY(gelu_bwd(da_c, gu_c, dgu_c, (int64_t)Tc * F, st));
+					if (form_a) ELF_TRY(gelu_fwd(gu_c, a_c, (int64_t)Tc * F, st));
 				}
 				ELF_TRY(gemm_bf16(0, 1, Tc, d, s->ffn_in, dgu_c, s->ffn_in, p.w[P_W1], d, (bf16_t*)d_h.p + (size_t)c * Tc * d, d, EPI_BF16, nullptr, 0, 0, 0, st));
 			}
