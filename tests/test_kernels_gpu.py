@@ -485,6 +485,30 @@ def test_grouped_weight_gradients_equal_the_single_launches(K):
 	assert K.gemm_turn_giveups() == before
 
 
+@pytest.mark.parametrize("shapes", [((2048, 2048), (2048, 2048), (2048, 2048), (3072, 3072)), ((4608, 4608),), ((768, 768),)], ids=["small_layers", "one_large_layer", "one_small_layer"])
+def test_grouped_weight_gradients_with_the_split_boundary_inside_a_layer(K, shapes):
+	"""The launch's last round may begin in the middle of a layer: 3 x 64 + 144 tiles (80 of the last layer's tiles split
+	three ways; small layers, laid on the XCDs as contiguous runs), one layer of 324 tiles (68 split three ways; its own
+	tile walk), and a lone 9-tile layer (all split).  Against fp64 torch, twice with equal bits, with the scale folded in."""
+	Kd = 4096
+	problems = _dw_problems(shapes, Kd, seed=700)
+	before = K.gemm_turn_giveups()
+	runs = []
+	for _ in range(2):
+		accs = [acc.clone() for _, _, acc in problems]
+		g16 = [torch.empty_like(a, dtype=torch.bfloat16) for a in accs]
+		K.gemm_dw_group([(dy, x, acc, h) for (dy, x, _), acc, h in zip(problems, accs, g16)], scale=0.25)
+		runs.append((accs, g16))
+	torch.cuda.synchronize()
+	assert K.gemm_turn_giveups() == before
+	for i, (dy, x, start) in enumerate(problems):
+		ref = (start.double() + dy.double().t() @ x.double()) * 0.25
+		got = runs[0][0][i]
+		assert ((got.double() - ref).abs().max() / ref.abs().max()).item() <= 1e-5, f"layer {i} {shapes[i]}"
+		assert torch.equal(runs[0][1][i], got.to(torch.bfloat16)), f"layer {i}: bf16 copy"
+		assert torch.equal(runs[1][0][i], got) and torch.equal(runs[1][1][i], runs[0][1][i]), f"layer {i}: not reproducible"
+
+
 def test_grouped_weight_gradients_with_the_gradient_scale(K):
 	"""scale != 0: the accumulators leave multiplied by the scale with their bf16 copies written, from the epilogue for
 	whole tiles and by a small kernel behind the launch for split ones (here: none split, all split, and a whole layer
