@@ -41,6 +41,13 @@ __device__ __forceinline__ void store8(bf16_t* p, const Chunk& c) {
 //                LN :  y = (x - mean) * rsqrt(var + eps) * gamma + beta   (biased variance)
 // stats[row] = {mean (0 for RMS), rstd}.
 // WPR = waves per row: 1 (four rows per workgroup, d <= 2048) or 4 (one row per workgroup).
+// One output element of the norm from its row statistics: shared by the forward kernels and by the backward kernel that
+// forms a dropped output again, so that both give the same bits (LN: one fused multiply-add for gamma and beta).
+template <bool LN>
+__device__ __forceinline__ float norm_out(float x, float mean, float rstd, float g, float b) {
+	return LN ? __builtin_fmaf((x - mean) * rstd, g, b) : x * rstd * g;
+}
+
 template <int WPR>
 __device__ __forceinline__ float row_sum(float v, float* red) {
 	v = wave_sum(v);
@@ -105,15 +112,10 @@ __global__ __launch_bounds__(256) void norm_fwd_kernel(const bf16_t* __restrict_
 		const int ch = tr + i * TPR;
 		if (ch < nchunks) {
 			Chunk g = load8(gamma + ch * 8);
-			Chunk o;
-			if (LN) {
-				Chunk b = load8(beta + ch * 8);
+			Chunk o, b;
+			if (LN) b = load8(beta + ch * 8);
 #pragma unroll
-				for (int j = 0; j < 8; j++) o.v[j] = (c[i].v[j] - mean) * rstd * g.v[j] + b.v[j];
-			} else {
-#pragma unroll
-				for (int j = 0; j < 8; j++) o.v[j] = c[i].v[j] * rstd * g.v[j];
-			}
+			for (int j = 0; j < 8; j++) o.v[j] = norm_out<LN>(c[i].v[j], mean, rstd, g.v[j], LN ? b.v[j] : 0.f);
 			store8(yr + ch * 8, o);
 		}
 	}
@@ -124,13 +126,15 @@ __global__ __launch_bounds__(256) void norm_fwd_kernel(const bf16_t* __restrict_
 //   LN : dx = rstd * (g - mean(g) - xhat * mean(g * xhat))
 // dx (+)= dres when a residual gradient bypasses the norm.  Per-workgroup partial sums of
 // dgamma (= sum dy*xhat) and dbeta (= sum dy) go to part[blockIdx][2][d]; a second kernel
-// folds them into the fp32 gradient accumulators.
-template <int NCH, int WPR, bool LN>
+// folds them into the fp32 gradient accumulators.  YOUT: the norm's output y (a stash that dropped it after the forward)
+// is written again as well, from the row the kernel holds anyway: the forward's arithmetic, the forward's bits.
+template <int NCH, int WPR, bool LN, bool YOUT>
 __global__ __launch_bounds__(256) void norm_bwd_kernel(const bf16_t* __restrict__ dy, const bf16_t* __restrict__ x,
                                                        const bf16_t* __restrict__ gamma,
                                                        const float2* __restrict__ stats,
                                                        const bf16_t* __restrict__ dres, bf16_t* __restrict__ dx,
-                                                       float* __restrict__ part, int T, int d) {
+                                                       float* __restrict__ part, int T, int d,
+                                                       const bf16_t* __restrict__ beta, bf16_t* __restrict__ yout) {
 	__shared__ float red[4];
 	__shared__ float fold[WPR == 1 ? ROWS_PER_BLOCK : 1][WPR == 1 ? 64 * 8 : 1];
 	const int lane = threadIdx.x & 63;
@@ -208,6 +212,13 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(const bf16_t* __restrict_
 					if (dres) o.v[j] += (float)rres[i][j];
 				}
 				store8(dxr + ch * 8, o);
+				if constexpr (YOUT) {
+					Chunk y, b;
+					if (LN) b = load8(beta + ch * 8);
+#pragma unroll
+					for (int j = 0; j < 8; j++) y.v[j] = norm_out<LN>((float)rx[i][j], mean, rstd, g[i].v[j], LN ? b.v[j] : 0.f);
+					store8(yout + (int64_t)row * d + ch * 8, y);
+				}
 			}
 		}
 	}
@@ -348,7 +359,7 @@ __global__ __launch_bounds__(256) void norm_fwd_half_kernel(const bf16_t* __rest
 		for (int i = 0; i < NCH; i++) {
 			Chunk o;
 #pragma unroll
-			for (int j = 0; j < 8; j++) o.v[j] = LN ? (c[i][j] - mean) * rstd * g[i].v[j] + b[i].v[j] : c[i][j] * rstd * g[i].v[j];
+			for (int j = 0; j < 8; j++) o.v[j] = norm_out<LN>(c[i][j], mean, rstd, g[i].v[j], LN ? b[i].v[j] : 0.f);
 			store8(y + (int64_t)row * d + (l32 + 32 * i) * 8, o);
 		}
 	}
@@ -442,6 +453,8 @@ __global__ __launch_bounds__(256) void norm_bwd_half_kernel(const bf16_t* __rest
 // (at d = 1024 the backward's four chunks per lane of three tensors, current and next row, fill the register file and the
 // full-wave kernel is faster)
 static inline bool norm_half_rows(int d) { return d % 256 == 0 && d <= 768; }
+// the full-wave backward kernel can write the norm's output again (see norm_bwd_kernel); the narrow-row one does not
+bool norm_bwd_forms_output(int d) { return !norm_half_rows(d); }
 
 static inline int norm_bwd_blocks(int T, int d) {
 	if (norm_half_rows(d)) {
@@ -503,7 +516,7 @@ int64_t norm_bwd_workspace_floats(int T, int d) { return (int64_t)norm_bwd_block
 
 template <bool LN>
 static int norm_bwd_dispatch(const void* dy, const void* x, const void* gamma, const void* stats, const void* dres,
-                             void* dx, float* part, int T, int d, hipStream_t s) {
+                             void* dx, float* part, int T, int d, hipStream_t s, const void* beta, void* yout) {
 	const dim3 grid(norm_bwd_blocks(T, d)), block(256);
 	if (norm_half_rows(d)) {
 #define ELF_NORM_BWD_HALF(N) ELF_LAUNCH((norm_bwd_half_kernel<N, LN>), grid, block, 0, s, (const bf16_t*)dy, (const bf16_t*)x, (const bf16_t*)gamma, (const float2*)stats, (const bf16_t*)dres, (bf16_t*)dx, part, T)
@@ -516,27 +529,35 @@ static int norm_bwd_dispatch(const void* dy, const void* x, const void* gamma, c
 		ELF_CHECK_HIP(hipGetLastError());
 		return 0;
 	}
-#define ELF_NORM_BWD(N, W)                                                                                      \
-	ELF_LAUNCH((norm_bwd_kernel<N, W, LN>), grid, block, 0, s, (const bf16_t*)dy, (const bf16_t*)x,       \
-	                   (const bf16_t*)gamma, (const float2*)stats, (const bf16_t*)dres, (bf16_t*)dx, part, T, d)
+#define ELF_NORM_BWD_Y(N, W, Y)                                                                                  \
+	ELF_LAUNCH((norm_bwd_kernel<N, W, LN, Y>), grid, block, 0, s, (const bf16_t*)dy, (const bf16_t*)x,     \
+	                   (const bf16_t*)gamma, (const float2*)stats, (const bf16_t*)dres, (bf16_t*)dx, part, T, d, (const bf16_t*)beta, (bf16_t*)yout)
+#define ELF_NORM_BWD(N, W)              \
+	do {                                \
+		if (yout) ELF_NORM_BWD_Y(N, W, true); \
+		else ELF_NORM_BWD_Y(N, W, false);     \
+	} while (0)
 	if (d <= 512) ELF_NORM_BWD(1, 1);
 	else if (d <= 1024) ELF_NORM_BWD(2, 1);
 	else if (d <= 2048) ELF_NORM_BWD(4, 1);
 	else if (d <= 4096) ELF_NORM_BWD(2, 4);
 	else ELF_NORM_BWD(4, 4);
 #undef ELF_NORM_BWD
+#undef ELF_NORM_BWD_Y
 	ELF_CHECK_HIP(hipGetLastError());
 	return 0;
 }
 
 static int norm_bwd_launch(int kind, const void* dy, const void* x, const void* gamma, const void* stats, const void* dres,
-                           void* dx, float* dgamma, float* dbeta, float* workspace, int T, int d, hipStream_t s) {
+                           void* dx, float* dgamma, float* dbeta, float* workspace, int T, int d, hipStream_t s, const void* beta = nullptr,
+                           void* yout = nullptr) {
 	int rc;
+	ELF_REQUIRE(!yout || (norm_bwd_forms_output(d) && (kind != NORM_LAYER || beta)), "norm_bwd: the output cannot be formed again at this width (d=%d)", d);
 	if (kind == NORM_LAYER) {
 		ELF_REQUIRE(dbeta != nullptr, "norm_bwd: LayerNorm needs dbeta");
-		rc = norm_bwd_dispatch<true>(dy, x, gamma, stats, dres, dx, workspace, T, d, s);
+		rc = norm_bwd_dispatch<true>(dy, x, gamma, stats, dres, dx, workspace, T, d, s, beta, yout);
 	} else {
-		rc = norm_bwd_dispatch<false>(dy, x, gamma, stats, dres, dx, workspace, T, d, s);
+		rc = norm_bwd_dispatch<false>(dy, x, gamma, stats, dres, dx, workspace, T, d, s, beta, yout);
 	}
 	if (rc) return rc;
 	const int nparts = norm_bwd_blocks(T, d);
@@ -547,11 +568,11 @@ static int norm_bwd_launch(int kind, const void* dy, const void* x, const void* 
 }
 
 int norm_bwd(int kind, const void* dy, const void* x, const void* gamma, const void* stats, const void* dres,
-             void* dx, float* dgamma, float* dbeta, float* workspace, int T, int d, hipStream_t s) {
+             void* dx, float* dgamma, float* dbeta, float* workspace, int T, int d, hipStream_t s, const void* beta, void* y_out) {
 	ELF_REQUIRE(T > 0 && d > 0 && d % 8 == 0 && d <= 8192, "norm_bwd: d must be a multiple of 8 and <= 8192 (d=%d)", d);
 	ELF_REQUIRE(dy && x && gamma && stats && dx && dgamma && workspace, "norm_bwd: null pointer");
-	ProfScope prof(PROF_NORM_BWD, (dres ? 8.0 : 6.0) * T * d, s);
-	return norm_bwd_launch(kind, dy, x, gamma, stats, dres, dx, dgamma, dbeta, workspace, T, d, s);
+	ProfScope prof(PROF_NORM_BWD, (dres ? 8.0 : 6.0) * T * d + (y_out ? 2.0 * T * d : 0.0), s);
+	return norm_bwd_launch(kind, dy, x, gamma, stats, dres, dx, dgamma, dbeta, workspace, T, d, s, beta, y_out);
 }
 
 // Norm backward for callers that cannot allocate (code under HIP graph capture, tight serving loops): the

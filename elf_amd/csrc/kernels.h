@@ -106,8 +106,12 @@ enum NormKind { NORM_RMS = 0, NORM_LAYER = 1 };
 int norm_fwd(int kind, const void* x, const void* gamma, const void* beta, void* y, void* stats, int T, int d,
              float eps, hipStream_t s);
 int64_t norm_bwd_workspace_floats(int T, int d);
+// y_out non-null (norm_bwd_forms_output(d) only: rows wider than 768): the norm's output is written again as well, with
+// the forward's bits (a stash that dropped it gets it back from the row this pass reads anyway); LayerNorm then needs beta.
+bool norm_bwd_forms_output(int d);
 int norm_bwd(int kind, const void* dy, const void* x, const void* gamma, const void* stats, const void* dres,
-             void* dx, float* dgamma, float* dbeta, float* workspace, int T, int d, hipStream_t s);
+             void* dx, float* dgamma, float* dbeta, float* workspace, int T, int d, hipStream_t s, const void* beta = nullptr,
+             void* y_out = nullptr);
 // The same with the partial sums in an array of the library's device image instead of a workspace argument
 // (no allocation anywhere on the path); norm_bwd_scratch_prepare looks the array's address up for the
 // current device (done by the first call on a device otherwise).

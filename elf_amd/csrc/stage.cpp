@@ -423,8 +423,11 @@ static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool gra
 		if (pre) ELF_CHECK_HIP(hipStreamWaitEvent(st, bs.pre_ev, 0));  // the rest of the block's stash
 		// what the attention backward reads and the offload / lean stash / module checkpoints dropped, formed again with the
 		// forward's own calls: the first norm's output and statistics, the QKV projection, the attention output and log-sum-exp
+		// the first norm's output, when only W reads it (projection kept, statistics kept), comes out of that norm's backward
+		// at the end of the block (the recompute of a first block's W stash stops before that norm: forward again there)
+		const bool h1_from_bwd = reform && bs.b[B_H1].dropped && !bs.b[B_QKV].dropped && !bs.b[B_ST1].dropped && norm_bwd_forms_output(d) && !(grads_only && i == 0);
 		auto reform_attention_inputs = [&]() -> int {
-			if ((bs.b[B_H1].dropped && (reform || bs.b[B_QKV].dropped)) || bs.b[B_ST1].dropped) {
+			if (!h1_from_bwd && ((bs.b[B_H1].dropped && (reform || bs.b[B_QKV].dropped)) || bs.b[B_ST1].dropped)) {
 				ELF_TRY(buf_alloc(s, bs, B_H1));
 				ELF_TRY(buf_alloc(s, bs, B_ST1));
 				ELF_TRY(norm_fwd(norm_kind, bs.b[B_X].p, p.w[P_NORM1_G], p.w[P_NORM1_B], bs.b[B_H1].p, bs.b[B_ST1].p, T, d, s->cfg.eps, st));
@@ -452,13 +455,20 @@ static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool gra
 			ELF_TRY(buf_alloc(s, bs, B_X2));
 			ELF_TRY(gemm_bf16(0, 0, T, d, s->Hq * s->D, bs.b[B_O].p, s->Hq * s->D, p.w[P_WO], s->Hq * s->D, bs.b[B_X2].p, d, EPI_BF16_RESID, bs.b[B_X].p, d, 0, 0, st));
 		}
-		if ((reform && bs.b[B_H2].dropped) || bs.b[B_ST2].dropped) {  // dropped by the lean stash / offload, or a checkpointed norm
+		// A norm output that the lean stash / offload dropped is only read by W (the FFN's first linear layer): the norm's
+		// backward writes it again from the row it holds anyway.  A checkpointed norm has no statistics either: forward again.
+		void* h2_out = nullptr;
+		if (reform && bs.b[B_H2].dropped && !bs.b[B_ST2].dropped && norm_bwd_forms_output(d)) {
+			ELF_TRY(buf_alloc(s, bs, B_H2));
+			h2_out = bs.b[B_H2].p;
+		} else if ((reform && bs.b[B_H2].dropped) || bs.b[B_ST2].dropped) {
 			ELF_TRY(buf_alloc(s, bs, B_H2));
 			ELF_TRY(buf_alloc(s, bs, B_ST2));
 			ELF_TRY(norm_fwd(norm_kind, bs.b[B_X2].p, p.w[P_NORM2_G], p.w[P_NORM2_B], bs.b[B_H2].p, bs.b[B_ST2].p, T, d, s->cfg.eps, st));
 		}
 		ELF_TRY(norm_bwd(norm_kind, d_h.p, bs.b[B_X2].p, p.w[P_NORM2_G], bs.b[B_ST2].p, dyin, bs.b[B_DX2].p,
-		                 grads_only ? s->dummy_grad : p.g[P_NORM2_G], grads_only ? s->dummy_grad + d : p.g[P_NORM2_B], s->norm_ws, T, d, st));
+		                 grads_only ? s->dummy_grad : p.g[P_NORM2_G], grads_only ? s->dummy_grad + d : p.g[P_NORM2_B], s->norm_ws, T, d, st,
+		                 p.w[P_NORM2_B], h2_out));
 		// attention
 		PoolTmp d_o(s->pool, (size_t)T * s->Hq * s->D * 2);
 		if (!d_o.p) return -3;
@@ -489,8 +499,10 @@ static int run_backward(Stage* s, MbState& m, const void* dy, void* dx, bool gra
 				ELF_TRY(buf_alloc(s, pv, B_DY));
 				dxout = pv.b[B_DY].p;
 			}
+			if (h1_from_bwd) ELF_TRY(buf_alloc(s, bs, B_H1));
 			ELF_TRY(norm_bwd(norm_kind, d_h.p, bs.b[B_X].p, p.w[P_NORM1_G], bs.b[B_ST1].p, bs.b[B_DX2].p, dxout,
-			                 grads_only ? s->dummy_grad : p.g[P_NORM1_G], grads_only ? s->dummy_grad + d : p.g[P_NORM1_B], s->norm_ws, T, d, st));
+			                 grads_only ? s->dummy_grad : p.g[P_NORM1_G], grads_only ? s->dummy_grad + d : p.g[P_NORM1_B], s->norm_ws, T, d, st,
+			                 p.w[P_NORM1_B], h1_from_bwd ? bs.b[B_H1].p : nullptr));
 			if (i == 0 && s->vocab_in) {
 				// first stage: the embedding is not a split layer, its gradient accumulates inside B
 				if (!grads_only) ELF_TRY(embedding_bwd(m.ids, d_emb.p, s->xg[XP_EMBED], T, d, s->vocab_in, st));
