@@ -458,9 +458,10 @@ bool norm_bwd_forms_output(int d) { return !norm_half_rows(d); }
 
 static inline int norm_bwd_blocks(int T, int d) {
 	if (norm_half_rows(d)) {
-		// eight rows per workgroup at a time, at most two workgroups per compute unit: 512 partial rows for the fold
+		// eight rows per workgroup at a time, one workgroup per compute unit: 256 partial rows for the fold kernel (with 512
+		// the pair took 21 us at 8192 x 768, with 256 18 us, with 128 20 us)
 		const int want = (T + 7) / 8;
-		return want < 512 ? want : 512;
+		return want < 256 ? want : 256;
 	}
 	const int rows_per_block = d <= 2048 ? ROWS_PER_BLOCK : 1;
 	const int want = (T + rows_per_block - 1) / rows_per_block;
