@@ -317,9 +317,10 @@ int elf_stage_set_ends(elf_stage_t* s, int vocab_in, int vocab_out, int vocab_ou
 int elf_stage_set_mb_samples(elf_stage_t* s, int mb, int samples);
 /* Lean stash (no counterpart in the reference, where autograd decides what a forward keeps): with on != 0
  * a forward that keeps its activations drops the two norm outputs and the FFN activation of every block
- * (a third of the stash at the Llama shapes) and backward_inputs forms them again with the forward's
- * kernels from the buffers it holds anyway: same results bit for bit, 2 % of a block's B time.  For stages
- * that run under a memory budget; applies to forwards issued after the call. */
+ * (a third of the stash at the Llama shapes) and backward_inputs writes them again where W needs them, from
+ * passes that read their inputs anyway (the norms' backward kernels, the SwiGLU backward's epilogue) and with
+ * the forward's arithmetic: same results bit for bit, under 1 % of a block's B time.  For stages that run
+ * under a memory budget; applies to forwards issued after the call. */
 int elf_stage_set_lean_stash(elf_stage_t* s, int on);
 /* F: PipelineBlock.forward (block.py:210-279). x, y: bf16 [T, d_model]. */
 int elf_stage_forward(elf_stage_t* s, int mb, const void* x, void* y, uint32_t flags, void* stream);
