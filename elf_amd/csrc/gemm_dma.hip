@@ -982,59 +982,6 @@ __global__ __launch_bounds__(256) void gemm_pers_kernel(Args g) {
 					*reinterpret_cast<bf16x8*>(g.C2 + row * g.ldc2 + c) = oa;
 				}
 			}
-		} else if constexpr (EPI == EPI_BF16_ROPE) {
-			// heads of 128: the wave's strip is one head, its halves are the two half-steps (runs t and t + 2); heads of
-			// 64: each half-step is a head, its halves are runs t = 0 and 1 (2 and 3).  Rounded to bf16 before the rotation,
-			// as the RoPE kernel would read the projection from memory.
-			const int half = g.rope_D >> 1;
-			auto rope_rows = [&](auto widec) {
-				constexpr bool WIDE = decltype(widec)::value;
-				// pair p of a row: runs (lo, hi) = (p, p + 2) for heads of 128, (2 p, 2 p + 1) for heads of 64; the lane's 8
-				// columns within the head's first half start at c_in_head
-				const int c_in_head[2] = {g4 * 8, WIDE ? 32 + g4 * 8 : g4 * 8};
-				const bool rot[2] = {gcol0 + run_col(0) < g.rope_cols, gcol0 + run_col(WIDE ? 1 : 2) < g.rope_cols};
-				// (cos, sin) of row i's 2 x 8 column pairs: fetched two rows ahead of their use - a lone wave has nothing
-				// else to cover a trip to the cache with
-				f32x4 tab[3][2][4] = {};
-				auto fetch = [&](int i, int slot) {
-					const int pos = (int)((grow0 + i * 16) % g.rope_S);
-#pragma unroll
-					for (int p = 0; p < 2; p++)
-						if (rot[p]) {
-							const f32x4* tp = reinterpret_cast<const f32x4*>(g.rope_cs + (int64_t)pos * half + c_in_head[p]);
-#pragma unroll
-							for (int q = 0; q < 4; q++) tab[slot][p][q] = tp[q];
-						}
-				};
-				fetch(0, 0);
-				fetch(1, 1);
-				static_for<RF>([&](auto ic) {
-					constexpr int i = decltype(ic)::value;
-					__builtin_amdgcn_sched_barrier(0);  // one row group at a time, its table entries fetched two groups earlier
-					if constexpr (i + 2 < RF) fetch(i + 2, (i + 2) % 3);
-					bf16_t* cp = reinterpret_cast<bf16_t*>(g.C) + (int64_t)(grow0 + i * 16) * g.ldc + gcol0;
-#pragma unroll
-					for (int p = 0; p < 2; p++) {
-						const int tlo = WIDE ? p : 2 * p, thi = WIDE ? p + 2 : 2 * p + 1;
-						float a[8], b[8];
-						run(i, tlo, a);
-						run(i, thi, b);
-						bf16x8 olo, ohi;
-#pragma unroll
-						for (int e = 0; e < 8; e++) {
-							const float x = (float)(bf16_t)a[e], y = (float)(bf16_t)b[e];
-							float ra = x, rb = y;
-							if (rot[p]) rope_rot(x, y, tab[i % 3][p][e >> 1][(e & 1) * 2], tab[i % 3][p][e >> 1][(e & 1) * 2 + 1], ra, rb);
-							olo[e] = (bf16_t)ra;
-							ohi[e] = (bf16_t)rb;
-						}
-						*reinterpret_cast<bf16x8*>(cp + run_col(tlo)) = olo;
-						*reinterpret_cast<bf16x8*>(cp + run_col(thi)) = ohi;
-					}
-				});
-			};
-			if (g.rope_D == 128) rope_rows(std::true_type{});
-			else rope_rows(std::false_type{});
 		} else {
 			static_assert(EPI == EPI_BF16 || EPI == EPI_BF16_RESID, "epilogues of the persistent forward kernel");
 			// residual (or bias row, ldr = 0): every load of the wave's 128 x 128 share goes out before the first store (a lone
@@ -1201,12 +1148,12 @@ int gemm_bf16_dma(int a_t, int b_t, int M, int N, int K, const void* A, int64_t 
 	// waves with 64x128 wave tiles (with two transpose reads per fragment on both operands the lone wave wins on
 	// some shapes by 2-3 % and loses on most by 1-10 %)
 	if (!a_t && !b_t && (K / dma::BKS) % 2 == 0 && !getenv("ELF_NO_PERSISTENT_GEMM")) {
-		// forward shapes: persistent workgroups, register epilogue
+		// forward shapes: persistent workgroups, register epilogue (the QKV projection with its rotary epilogue stays on the
+		// one-tile kernel: with the table fetches in a lone wave's register epilogue the persistent form ran 3 % slower)
 		switch (epi) {
 			case EPI_BF16: return dma::launch_pers<EPI_BF16>(a, stream);
 			case EPI_BF16_RESID: return dma::launch_pers<EPI_BF16_RESID>(a, stream);
 			case EPI_BF16_SWIGLU: return dma::launch_pers<EPI_BF16_SWIGLU>(a, stream);
-			case EPI_BF16_ROPE: return dma::launch_pers<EPI_BF16_ROPE>(a, stream);
 		}
 	}
 	if (!a_t && !b_t) return dma::launch_epi<4, 4, false, false>(a, epi, stream);
