@@ -25,8 +25,9 @@ struct FwdTile {
 template <int D, bool CAUSAL>
 __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnArgs a) {
 	using TL = FwdTile<D>;
-	constexpr int BQ = 128, BKV = 64;
+	constexpr int BQ = 128, BKV = 64, KT = BKV / 32;
 	constexpr int KSTEPS = D / 16, DT = D / 32;
+	constexpr int NF = D == 128 ? 8 : 4;  // LDS fragments in flight ahead of the MFMA that uses them
 	constexpr int STAGE = 2 * TL::TILE_BYTES;
 	extern __shared__ __attribute__((aligned(1024))) unsigned char smem_raw[];
 
@@ -98,24 +99,34 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnArgs a) {
 		const unsigned char* sK = smem_raw + (j & 1) * STAGE;
 		const unsigned char* sV = sK + TL::TILE_BYTES;
 
-		// S^T[key][q] for the two 32-key halves
-		f32x16 s[2];
+		// S^T[key][q] for the two 32-key halves.  Fragment i = (k step i / KT, key half i % KT): the two accumulators
+		// alternate, and a fragment is read NF MFMAs before its use (left to itself the compiler reads each one
+		// right before its MFMA, into one register quad, and every MFMA waits out an LDS round trip).
+		f32x16 s[KT];
 #pragma unroll
-		for (int kt = 0; kt < 2; kt++) {
+		for (int kt = 0; kt < KT; kt++)
 #pragma unroll
 			for (int r = 0; r < 16; r++) s[kt][r] = 0.f;
-			const int row = kt * 32 + ql;
-			const unsigned char* rowp = sK + row * TL::ROW_BYTES;
+		{
+			auto kread = [&](int i) __attribute__((always_inline)) {
+				const int row = (i % KT) * 32 + ql, ks = i / KT;
+				return *reinterpret_cast<const bf16x8*>(sK + row * TL::ROW_BYTES + (((2 * ks + g) ^ TL::k_swz(row)) << 4));
+			};
+			bf16x8 kf[NF];
 #pragma unroll
-			for (int ks = 0; ks < KSTEPS; ks++) {
-				const bf16x8 kf = *reinterpret_cast<const bf16x8*>(rowp + (((2 * ks + g) ^ TL::k_swz(row)) << 4));
-				s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], s[kt], 0, 0, 0);
+			for (int i = 0; i < NF; i++) kf[i] = kread(i);
+			__builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+			for (int i = 0; i < KT * KSTEPS; i++) {
+				s[i % KT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i % NF], qf[i / KT], s[i % KT], 0, 0, 0);
+				if (i + NF < KT * KSTEPS) kf[i % NF] = kread(i + NF);
+				__builtin_amdgcn_sched_barrier(0);
 			}
 		}
 		// causal mask only where the tile crosses the diagonal of this wave's queries
 		if (CAUSAL && k0 + BKV - 1 > q0) {
 #pragma unroll
-			for (int kt = 0; kt < 2; kt++)
+			for (int kt = 0; kt < KT; kt++)
 #pragma unroll
 				for (int r = 0; r < 16; r++) {
 					const int key = k0 + kt * 32 + (r >> 2) * 8 + 4 * g + (r & 3);
@@ -124,23 +135,18 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnArgs a) {
 		}
 		float mx = s[0][0];
 #pragma unroll
-		for (int kt = 0; kt < 2; kt++)
+		for (int kt = 0; kt < KT; kt++)
 #pragma unroll
 			for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[kt][r]);
 		mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-		// every query sees key 0 in its first tile, so the running max is finite from then on
-		const float m_new = fmaxf(m_run, mx * sc);
-		float psum = 0.f;
-#pragma unroll
-		for (int kt = 0; kt < 2; kt++)
-#pragma unroll
-			for (int r = 0; r < 16; r++) {
-				const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][r], sc, -m_new));
-				s[kt][r] = p;
-				psum += p;
-			}
-		// rescale only when some query of the wave raised its maximum
-		if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {
+		// The reference point of the exponentials follows the running maximum lazily: it moves (and the sums and the
+		// output are rescaled) only when some query of the wave has a score more than 2^SLACK above its reference, so
+		// the weights stay below 2^SLACK: exact in fp32 and bf16 alike, and any reference point gives the same quotient.
+		// Every query sees key 0 in its first tile, so the reference is finite from then on.
+		constexpr float SLACK = 8.f;
+		mx *= sc;
+		if (__builtin_amdgcn_ballot_w64(mx > m_run + SLACK) != 0) {
+			const float m_new = fmaxf(m_run, mx);
 			const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
 			l_run *= alpha;
 #pragma unroll
@@ -149,30 +155,47 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnArgs a) {
 				for (int r = 0; r < 16; r++) acc_o[i][r] *= alpha;
 			m_run = m_new;
 		}
-		l_run += psum;
-		// O^T[d][q] += V^T[d][key] P^T[key][q]
+		float psum = 0.f;
 #pragma unroll
-		for (int kt = 0; kt < 2; kt++) {
+		for (int kt = 0; kt < KT; kt++)
 #pragma unroll
-			for (int u = 0; u < 2; u++) {
-				float pv[8];
-#pragma unroll
-				for (int t = 0; t < 8; t++) pv[t] = s[kt][u * 8 + t];
-				const bf16x8 pf = pack8(pv);
-				// keys {kk..kk+3} and {kk+8..kk+11}: the row order of the accumulator tile
-				const int j16 = lane & 15;
-				const int kk = kt * 32 + u * 16 + 4 * g + (j16 >> 2);
-#pragma unroll
-				for (int dt = 0; dt < DT; dt++) {
-					const int c = (dt * 32 + 16 * (ql >> 4) + 4 * (j16 & 3)) >> 3;
-					const unsigned char* p0 = sV + kk * TL::ROW_BYTES + ((c ^ TL::v_swz(kk)) << 4) + (j16 & 1) * 8;
-					const unsigned char* p1 = sV + (kk + 8) * TL::ROW_BYTES + ((c ^ TL::v_swz(kk + 8)) << 4) + (j16 & 1) * 8;
-					s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 ELF_LDS*)(p0));
-					s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 ELF_LDS*)(p1));
-					const bf16x8 vf = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-					acc_o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf, acc_o[dt], 0, 0, 0);
-				}
+			for (int r = 0; r < 16; r++) {
+				const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][r], sc, -m_run));
+				s[kt][r] = p;
+				psum += p;
 			}
+		l_run += psum;
+		// O^T[d][q] += V^T[d][key] P^T[key][q].  Fragment i = (16-key group i / DT, 32-wide d block i % DT), read NF MFMAs
+		// ahead like the K fragments above.
+		{
+			auto vread = [&](int i) __attribute__((always_inline)) {
+				// keys {kk..kk+3} and {kk+8..kk+11}: the row order of the accumulator tile
+				const int j16 = lane & 15, dt = i % DT;
+				const int kk = (i / DT) * 16 + 4 * g + (j16 >> 2);
+				const int c = (dt * 32 + 16 * (ql >> 4) + 4 * (j16 & 3)) >> 3;
+				const unsigned char* p0 = sV + kk * TL::ROW_BYTES + ((c ^ TL::v_swz(kk)) << 4) + (j16 & 1) * 8;
+				const unsigned char* p1 = sV + (kk + 8) * TL::ROW_BYTES + ((c ^ TL::v_swz(kk + 8)) << 4) + (j16 & 1) * 8;
+				s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 ELF_LDS*)(p0));
+				s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 ELF_LDS*)(p1));
+				return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+			};
+			bf16x8 vf[NF];
+#pragma unroll
+			for (int i = 0; i < NF; i++) vf[i] = vread(i);
+			bf16x8 pf;
+#pragma unroll
+			for (int i = 0; i < 2 * KT * DT; i++) {
+				if (i % DT == 0) {
+					float pv[8];
+#pragma unroll
+					for (int t = 0; t < 8; t++) pv[t] = s[i / DT / 2][(i / DT % 2) * 8 + t];
+					pf = pack8(pv);
+				}
+				__builtin_amdgcn_sched_barrier(0);
+				acc_o[i % DT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[i % NF], pf, acc_o[i % DT], 0, 0, 0);
+				if (i + NF < 2 * KT * DT) vf[i % NF] = vread(i + NF);
+			}
+			__builtin_amdgcn_sched_barrier(0);
 		}
 	}
 
