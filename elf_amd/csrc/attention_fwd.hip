@@ -133,19 +133,33 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnArgs a) {
 					if (key > qpos) s[kt][r] = -INFINITY;
 				}
 		}
-		float mx = s[0][0];
+		// The exponentials are taken against a reference point per query that follows the running maximum lazily: any
+		// reference gives the same quotient, and as long as the weights stay moderate they are as exact in fp32 and
+		// bf16 as those against the maximum.  A reference never lies above the running maximum, so nothing underflows
+		// that would not against the maximum.  Every query sees key 0 in its first tile, so the reference is finite
+		// from then on.
+		f32x16 pr[KT];
+		float psum = 0.f;
+		auto weights = [&]() __attribute__((always_inline)) {
+			psum = 0.f;
 #pragma unroll
-		for (int kt = 0; kt < KT; kt++)
+			for (int kt = 0; kt < KT; kt++)
 #pragma unroll
-			for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[kt][r]);
-		mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-		// The reference point of the exponentials follows the running maximum lazily: it moves (and the sums and the
-		// output are rescaled) only when some query of the wave has a score more than 2^SLACK above its reference, so
-		// the weights stay below 2^SLACK: exact in fp32 and bf16 alike, and any reference point gives the same quotient.
-		// Every query sees key 0 in its first tile, so the reference is finite from then on.
-		constexpr float SLACK = 8.f;
-		mx *= sc;
-		if (__builtin_amdgcn_ballot_w64(mx > m_run + SLACK) != 0) {
+				for (int r = 0; r < 16; r++) {
+					const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][r], sc, -m_run));
+					pr[kt][r] = p;
+					psum += p;
+				}
+		};
+		auto tile_max = [&]() __attribute__((always_inline)) {
+			float mx = s[0][0];
+#pragma unroll
+			for (int kt = 0; kt < KT; kt++)
+#pragma unroll
+				for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[kt][r]);
+			return fmaxf(mx, __shfl_xor(mx, 32, 64)) * sc;
+		};
+		auto move_reference = [&](float mx) __attribute__((always_inline)) {
 			const float m_new = fmaxf(m_run, mx);
 			const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
 			l_run *= alpha;
@@ -154,16 +168,25 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnArgs a) {
 #pragma unroll
 				for (int r = 0; r < 16; r++) acc_o[i][r] *= alpha;
 			m_run = m_new;
-		}
-		float psum = 0.f;
-#pragma unroll
-		for (int kt = 0; kt < KT; kt++)
-#pragma unroll
-			for (int r = 0; r < 16; r++) {
-				const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][r], sc, -m_run));
-				s[kt][r] = p;
-				psum += p;
+		};
+		if constexpr (D == 128) {
+			// The common tile computes no maximum at all: only when a lane's weights sum past LIMIT (or are not finite:
+			// the first tile, whose reference is -inf) does the wave move the references to the running maxima, rescale
+			// sums and output, and take the tile's exponentials again.
+			constexpr float LIMIT = 0x1p20f;
+			weights();
+			if (__builtin_amdgcn_ballot_w64(!(psum < LIMIT)) != 0) {
+				move_reference(tile_max());
+				weights();
 			}
+		} else {
+			// (with four waves on a SIMD there are no registers to keep the scores beside the weights) the reference
+			// moves when some query of the wave has a score more than 2^SLACK above it
+			constexpr float SLACK = 8.f;
+			const float mx = tile_max();
+			if (__builtin_amdgcn_ballot_w64(mx > m_run + SLACK) != 0) move_reference(mx);
+			weights();
+		}
 		l_run += psum;
 		// O^T[d][q] += V^T[d][key] P^T[key][q].  Fragment i = (16-key group i / DT, 32-wide d block i % DT), read NF MFMAs
 		// ahead like the K fragments above.
@@ -188,7 +211,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnArgs a) {
 				if (i % DT == 0) {
 					float pv[8];
 #pragma unroll
-					for (int t = 0; t < 8; t++) pv[t] = s[i / DT / 2][(i / DT % 2) * 8 + t];
+					for (int t = 0; t < 8; t++) pv[t] = pr[i / DT / 2][(i / DT % 2) * 8 + t];
 					pf = pack8(pv);
 				}
 				__builtin_amdgcn_sched_barrier(0);

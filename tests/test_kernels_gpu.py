@@ -403,6 +403,30 @@ def test_attention_fwd_bwd(K, cfg):
 	assert torch.equal(fused, K.rope_apply_(dqkv.clone(), cs, S, Hq + Hkv, D, backward=True))
 
 
+@pytest.mark.parametrize("D,causal,ramp,gain", [(128, True, 6.0, 1.0), (128, False, 6.0, 1.0), (64, True, 6.0, 1.0), (128, True, 0.0, 6.0),
+                                               (128, False, -6.0, 3.0), (64, False, 0.0, 6.0)])
+def test_attention_forward_with_scores_that_climb_along_the_keys(K, D, causal, ramp, gain):
+	"""The forward's softmax takes its exponentials against a reference point that follows the running maximum only
+	when it has to.  Here it has to, again and again: a component of k that grows (ramp > 0) or falls (ramp < 0) with the
+	key position against a constant component of q moves the row maxima by many powers of two from tile to tile, and
+	gain scales everything to scores of several hundred.  Output and log-sum-exp against the fp32 softmax."""
+	B, S, Hq, Hkv = 2, 1024, 4, 2
+	T = B * S
+	qkv = _randn(T, (Hq + 2 * Hkv) * D, seed=60).float() * gain
+	pos = (torch.arange(T, device="cuda") % S).float() / S  # 0 .. 1 along each sequence
+	for h in range(Hq):
+		qkv[:, h * D] = 4.0
+	for h in range(Hkv):
+		qkv[:, (Hq + h) * D] = ramp * pos * math.sqrt(D)  # adds ramp * 4 * pos to every score: up to 35 powers of two
+	qkv = qkv.to(torch.bfloat16)
+	o_ref, lse_ref, _ = _attn_ref(qkv, B, S, Hq, Hkv, D, causal)
+	o, lse = K.attn_fwd(qkv, B, S, Hq, Hkv, D, causal)
+	assert torch.isfinite(o.float()).all() and torch.isfinite(lse).all()
+	_close(o, o_ref, what=f"attn fwd, climbing scores D={D} causal={causal} ramp={ramp} gain={gain}")
+	_close(lse, lse_ref, rel_fro=1e-3, rel_max=1e-2, what="lse")
+	assert torch.equal(o, K.attn_fwd(qkv, B, S, Hq, Hkv, D, causal)[0])
+
+
 @pytest.mark.parametrize("T,N,ld", [(8192, 768, 768), (1000, 2304, 2304), (7, 64, 128), (4096, 8, 8), (333, 4104, 4104)])
 def test_colsum_is_exact_to_rounding_and_repeatable(K, T, N, ld):
 	"""The bias gradient of a split linear layer: column sums of a bf16 [T, N] view (row stride ld) added to an fp32
