@@ -90,13 +90,14 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnArgs a) {
 
 	const int n_kv = CAUSAL ? ((qt + 1) * BQ) / BKV : a.S / BKV;
 	issue(0);
-	for (int j = 0; j < n_kv; j++) {
+	// One tile, in the LDS stage at byte offset `stage`.
+	auto tile = [&](int j, int stage) __attribute__((always_inline)) {
 		wait_vmcnt<0>();
 		__syncthreads();  // tile j is in LDS for everyone; everyone is done with tile j-1
 		if (j + 1 < n_kv) issue(j + 1);
 		const int k0 = j * BKV;
-		if (CAUSAL && k0 > q0 + 31) continue;  // every key of the tile is in this wave's future
-		const unsigned char* sK = smem_raw + (j & 1) * STAGE;
+		if (CAUSAL && k0 > q0 + 31) return;  // every key of the tile is in this wave's future
+		const unsigned char* sK = smem_raw + stage;
 		const unsigned char* sV = sK + TL::TILE_BYTES;
 
 		// S^T[key][q] for the two 32-key halves.  Fragment i = (k step i / KT, key half i % KT): the two accumulators
@@ -220,6 +221,18 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnArgs a) {
 			}
 			__builtin_amdgcn_sched_barrier(0);
 		}
+	};
+	if constexpr (D == 128) {
+		// tiles in pairs (their number is even: 128 queries, sequences of a multiple of 128, 64-key tiles): the stage is a
+		// constant in each copy of the body and travels in the LDS instructions' offset fields instead of being added to
+		// every address
+		for (int j = 0; j < n_kv; j += 2) {
+			tile(j, 0);
+			tile(j + 1, STAGE);
+		}
+	} else {
+		// (the two copies cost the registers that keep four waves on a SIMD)
+		for (int j = 0; j < n_kv; j++) tile(j, (j & 1) * STAGE);
 	}
 
 	const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
