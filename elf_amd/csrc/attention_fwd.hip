@@ -181,11 +181,10 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnArgs a) {
 				weights();
 			}
 		} else {
-			// (with four waves on a SIMD there are no registers to keep the scores beside the weights) the reference
-			// moves when some query of the wave has a score more than 2^SLACK above it
-			constexpr float SLACK = 8.f;
+			// (with four waves on a SIMD there are no registers to keep the scores beside the weights) the reference is
+			// the running maximum itself; output and sums are rescaled when some query of the wave raised it
 			const float mx = tile_max();
-			if (__builtin_amdgcn_ballot_w64(mx > m_run + SLACK) != 0) move_reference(mx);
+			if (__builtin_amdgcn_ballot_w64(mx > m_run) != 0) move_reference(mx);
 			weights();
 		}
 		l_run += psum;

@@ -1,5 +1,6 @@
 """Shared helpers of the parity tests (oracle <-> product glue)."""
 
+import os
 import torch
 
 from oracle import stage_ref as R
@@ -70,6 +71,8 @@ def assert_close(got, ref, what, rel_max=2e-2, rel_fro=1e-2):
 	scale = ref.abs().max().item() + 1e-12
 	err = (got - ref).abs().max().item()
 	fro = ((got - ref).norm() / (ref.norm() + 1e-12)).item()
+	if os.environ.get("ELF_TEST_MARGINS"):  # how far inside the bounds each comparison lands (pytest -s)
+		print(f"[margin] {what}: max {err / scale:.4f} of {rel_max}, fro {fro:.4f} of {rel_fro}", flush=True)
 	assert err <= rel_max * scale, f"{what}: max abs err {err:.4g} > {rel_max} * {scale:.4g}"
 	assert fro <= rel_fro, f"{what}: relative Frobenius error {fro:.4g} > {rel_fro}"
 	return err / scale, fro
