@@ -86,6 +86,8 @@ def assert_close_dev(got, ref, what, rel_max=2e-2, rel_fro=1e-2):
 	scale = ref.abs().max().item() + 1e-12
 	err = diff.abs().max().item()
 	fro = (diff.double().norm() / (ref.double().norm() + 1e-12)).item()
+	if os.environ.get("ELF_TEST_MARGINS"):
+		print(f"[margin] {what}: max {err / scale:.4f} of {rel_max}, fro {fro:.4f} of {rel_fro}", flush=True)
 	assert err <= rel_max * scale, f"{what}: max abs err {err:.4g} > {rel_max} * {scale:.4g}"
 	assert fro <= rel_fro, f"{what}: relative Frobenius error {fro:.4g} > {rel_fro}"
 	return err / scale, fro
