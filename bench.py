@@ -468,6 +468,10 @@ def main():
 	ap.add_argument("--no-cpu-baseline", action="store_true")
 	ap.add_argument("--prefetching-time", type=int, default=None,
 	                help="offload workloads: how many compute ops before its B a micro-batch's PREFETCH_ACTIVATIONS is placed (reference default 1)")
+	ap.add_argument("--time-one-in", type=int, default=4, metavar="N",
+	                help="per-kernel figures (the roofline's among them) from HIP events carried by one launch in N of the timed steps, "
+	                     "picked pseudo-randomly, the same picks every run (default 4; 1 = every launch: an event pair costs the stream "
+	                     "about 2 us per launch, 0.5 %% of a Llama step and 8 %% of a GPT-2-small step)")
 	ap.add_argument("--graph", action="store_true",
 	                help="time replays of the step captured as one HIP graph (Engine.capture) instead of eager steps; the per-kernel figures "
 	                     "then come from one extra eager step after the timed region (a replay runs no host code that could bracket launches)")
@@ -541,7 +545,7 @@ def main():
 		step()
 		torch.cuda.synchronize()
 	else:
-		lib.elf_prof_enable(1)
+		lib.elf_prof_enable(args.time_one_in)
 	mem_before = block.mem_stats()
 	telemetry = Telemetry() if args.telemetry else contextlib.nullcontext()
 	with telemetry:
@@ -551,7 +555,7 @@ def main():
 		torch.cuda.synchronize()
 		elapsed = time.perf_counter() - t0
 	if args.graph:
-		lib.elf_prof_enable(1)
+		lib.elf_prof_enable(args.time_one_in)
 		eager_step()
 		torch.cuda.synchronize()
 	kinds = ["gemm", "attn_fwd", "attn_bwd", "norm_fwd", "norm_bwd", "act_fwd", "act_bwd", "rope", "grad_scale", "add", "embed", "loss"]
@@ -560,9 +564,14 @@ def main():
 		ms, work = ctypes.c_double(), ctypes.c_double()
 		n = lib.elf_prof_collect(i, ctypes.byref(ms), ctypes.byref(work))
 		if n > 0:
+			# the family's rate = work over duration of the launches that carried events; "launches" counts all launches and
+			# "avg_ms" is their mean duration at that rate (all launches' work / rate / launches: with every launch timed,
+			# the plain mean of the event durations)
 			rate = work.value / (ms.value * 1e-3)
-			per_kernel[name] = {"launches": n, "avg_ms": ms.value / n, "total_ms": ms.value,
-			                    ("tflops" if i < 3 else "gbs"): rate / (1e12 if i < 3 else 1e9)}
+			all_work = ctypes.c_double()
+			launches = lib.elf_prof_launches(i, ctypes.byref(all_work))
+			per_kernel[name] = {"launches": launches, "timed_launches": n, "avg_ms": all_work.value / rate / launches * 1e3,
+			                    "timed_ms": ms.value, ("tflops" if i < 3 else "gbs"): rate / (1e12 if i < 3 else 1e9)}
 	lib.elf_prof_enable(0)
 	mem = block.mem_stats()
 	tokens = w["mb"] * w["seq"] * w["n_mb"]

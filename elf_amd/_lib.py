@@ -48,6 +48,7 @@ _SIGNATURES = {
 	"elf_hbm_probe": (c_int, [c_int, _P, _P, c_int64, _P]),
 	"elf_prof_enable": (None, [c_int]),
 	"elf_prof_collect": (c_int, [c_int, POINTER(c_double), POINTER(c_double)]),
+	"elf_prof_launches": (c_int64, [c_int, POINTER(c_double)]),
 	"elf_attn_bwd": (c_int, [_P] * 10 + [c_int64] * 8 + [c_int] * 6 + [c_float, _P]),
 	"elf_attn_bwd_rope": (c_int, [_P] * 10 + [c_int64] * 8 + [c_int] * 6 + [c_float, _P, _P]),
 }

@@ -119,6 +119,7 @@ int elf_gemm_turn_giveups(uint64_t* out) {
 }
 
 void elf_prof_enable(int on) { elf::prof_enable(on); }
+int64_t elf_prof_launches(int kind, double* total_work) { return elf::prof_launches(kind, total_work); }
 int elf_prof_collect(int kind, double* total_ms, double* total_work) {
 	if (kind < 0 || kind >= elf::PROF_COUNT) return -1;
 	return elf::prof_collect(kind, total_ms, total_work);

@@ -159,7 +159,7 @@ enum ProfKind {
 	PROF_GEMM = 0, PROF_ATTN_FWD, PROF_ATTN_BWD, PROF_NORM_FWD, PROF_NORM_BWD, PROF_ACT_FWD, PROF_ACT_BWD, PROF_ROPE,
 	PROF_SCALE, PROF_ADD, PROF_EMBED, PROF_LOSS, PROF_COUNT
 };
-void prof_enable(int on);
+void prof_enable(int on);  // 0 off, 1 every launch carries events, n > 1 one launch in n (pseudo-random, the same picks every run)
 bool prof_on();
 struct ProfScope {
 	// record = false: an inert scope (launches inside it are not timed)
@@ -197,5 +197,7 @@ inline void launch_kernel(void (*kern)(P...), dim3 grid, dim3 block, unsigned sm
 #define ELF_LAUNCH(kern, grid, block, smem, stream, ...) elf::launch_kernel(kern, grid, block, smem, stream, __VA_ARGS__)
 // Waits for the recorded events; totals since the last prof_enable(1). Returns the launch count.
 int prof_collect(int kind, double* total_ms, double* total_work);
+// All launches of the kind since prof_enable, timed or not, and their summed work.
+int64_t prof_launches(int kind, double* total_work);
 
 }  // namespace elf

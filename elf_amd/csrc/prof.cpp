@@ -14,6 +14,10 @@ struct ProfRec {
 	bool started;  // a launch has taken the start event
 };
 static bool g_on = false;
+static int g_one_in = 1;          // a launch carries events with probability 1 / g_one_in
+static uint32_t g_pick = 1u;      // state of the generator that picks them (restarted by prof_enable: same picks every run)
+static int64_t g_launches[PROF_COUNT];
+static double g_work[PROF_COUNT];
 static std::vector<ProfRec> g_recs;
 static std::vector<hipEvent_t> g_free_events;
 static thread_local ProfScope* t_scope = nullptr;
@@ -38,11 +42,26 @@ void prof_enable(int on) {
 	}
 	g_recs.clear();
 	g_on = on != 0;
+	g_one_in = on > 1 ? on : 1;
+	g_pick = 1u;
+	for (int k = 0; k < PROF_COUNT; k++) {
+		g_launches[k] = 0;
+		g_work[k] = 0.0;
+	}
 }
 bool prof_on() { return g_on; }
 
 ProfScope::ProfScope(int kind, double work, hipStream_t s, bool record) : slot(-1), stream(s), outer(nullptr) {
 	if (!g_on || !record) return;
+	g_launches[kind]++;
+	g_work[kind] += work;
+	if (g_one_in > 1) {
+		// an in-dispatch event pair costs the stream about 2 us per launch (a completion signal and two timestamps
+		// for every dispatch instead of one signal per batch): timing a pseudo-random subset keeps the family
+		// averages and most of the stream's speed
+		g_pick = g_pick * 1664525u + 1013904223u;
+		if ((g_pick >> 16) % (uint32_t)g_one_in != 0) return;
+	}
 	ProfRec r{kind, work, get_event(), get_event(), false};
 	if (!r.e0 || !r.e1) return;
 	slot = (int)g_recs.size();
@@ -78,6 +97,12 @@ int prof_collect(int kind, double* total_ms, double* total_work) {
 	if (total_ms) *total_ms = ms;
 	if (total_work) *total_work = work;
 	return n;
+}
+
+int64_t prof_launches(int kind, double* total_work) {
+	if (kind < 0 || kind >= PROF_COUNT) return 0;
+	if (total_work) *total_work = g_work[kind];
+	return g_launches[kind];
 }
 
 // ---------------------------------------------------------------------------------------------

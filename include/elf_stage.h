@@ -383,8 +383,11 @@ int elf_pinned_pool_free_segment(elf_pinned_pool_t* p, int parent, int i, int64_
  * launch with a HIP event pair on the launch stream.  kind: 0 GEMM (work = 2MNK flops),
  * 1 attention fwd, 2 attention bwd (algorithmic flops), 3 norm fwd, 4 norm bwd, 5 activation fwd,
  * 6 activation bwd, 7 RoPE, 8 grad scale, 9 add (work = algorithmic bytes).
- * elf_prof_collect waits for the events and returns the number of launches of that kind since
- * elf_prof_enable(1), with their summed duration (ms) and summed work. */
+ * elf_prof_enable(0) switches the timing off, (1) on for every launch, (n > 1) on for one launch in n, picked
+ * pseudo-randomly (the same picks every run): an event pair carried in a dispatch costs the stream about 2 us.
+ * elf_prof_collect waits for the events and returns the number of TIMED launches of that kind since
+ * elf_prof_enable, with their summed duration (ms) and summed work; elf_prof_launches returns the number of
+ * ALL launches of the kind since then and their summed work. */
 /* Memory-system yardstick for the bandwidth-bound kernels (no counterpart in the reference): mode 0 reads `bytes`
  * bytes from src (dst receives at most 8192 * 256 * 16 bytes of per-lane sums), mode 1 copies them to dst, mode 2 writes
  * `bytes` bytes to dst, mode 3 reads three streams of `bytes` bytes each (src, src + bytes, src + 2 bytes: src holds
@@ -393,6 +396,7 @@ int elf_pinned_pool_free_segment(elf_pinned_pool_t* p, int parent, int i, int64_
 int elf_hbm_probe(int mode, const void* src, void* dst, int64_t bytes, void* stream);
 void elf_prof_enable(int on);
 int elf_prof_collect(int kind, double* total_ms, double* total_work);
+int64_t elf_prof_launches(int kind, double* total_work);
 
 #ifdef __cplusplus
 }

@@ -179,3 +179,45 @@ def test_capture_with_live_kernel_timing_switched_on():
 			assert torch.equal(out, ref)
 	finally:
 		lib.elf_prof_enable(0)
+
+
+def test_kernel_timing_on_a_sample_of_the_launches():
+	"""``elf_prof_enable(n)`` lets one launch in n carry events (the same pseudo-random picks every run);
+	``elf_prof_launches`` still counts every launch and its work, and the sample gives the rate of all of them."""
+	import ctypes
+
+	from elf_amd import _lib
+	from elf_amd import kernels as K
+
+	lib = _lib.load()
+	g = torch.Generator(device="cuda").manual_seed(12)
+	a = torch.randn(1024, 512, device="cuda", generator=g).bfloat16()
+	w = (torch.randn(1024, 512, device="cuda", generator=g) * 0.05).bfloat16()
+	out = torch.empty(1024, 1024, device="cuda", dtype=torch.bfloat16)
+	flops = 2.0 * 1024 * 1024 * 512
+
+	def run(one_in, n=400):
+		lib.elf_prof_enable(one_in)
+		try:
+			for _ in range(n):
+				K.gemm(a, w, out=out)
+			torch.cuda.synchronize()
+			ms, work, all_work = ctypes.c_double(), ctypes.c_double(), ctypes.c_double()
+			timed = lib.elf_prof_collect(0, ctypes.byref(ms), ctypes.byref(work))
+			launches = lib.elf_prof_launches(0, ctypes.byref(all_work))
+			return timed, launches, ms.value, work.value, all_work.value
+		finally:
+			lib.elf_prof_enable(0)
+
+	for _ in range(50):
+		K.gemm(a, w, out=out)  # warm
+	t1, l1, ms1, w1, aw1 = run(1)
+	assert t1 == l1 == 400 and w1 == aw1 == 400 * flops
+	t4, l4, ms4, w4, aw4 = run(4)
+	assert l4 == 400 and aw4 == 400 * flops and w4 == t4 * flops
+	assert 60 <= t4 <= 140  # a quarter of 400, give or take
+	assert run(4)[0] == t4  # the same picks every run
+	# same kernel, same rate: the sampled mean duration within 15 % or 3 us of the full one (a timed dispatch behind an
+	# untimed one stamps its start before the predecessor has drained: 1-2 us on an 8 us kernel)
+	assert abs(ms4 / t4 - ms1 / t1) <= max(0.15 * (ms1 / t1), 3e-3)
+	assert lib.elf_prof_launches(99, None) == 0
