@@ -195,7 +195,7 @@ inline void launch_kernel(void (*kern)(P...), dim3 grid, dim3 block, unsigned sm
 	else hipLaunchKernelGGL(kern, grid, block, smem, s, static_cast<P>(a)...);
 }
 #define ELF_LAUNCH(kern, grid, block, smem, stream, ...) elf::launch_kernel(kern, grid, block, smem, stream, __VA_ARGS__)
-// Waits for the recorded events; totals since the last prof_enable(1). Returns the launch count.
+// Waits for the recorded events; totals over the timed launches since the last prof_enable. Returns their count.
 int prof_collect(int kind, double* total_ms, double* total_work);
 // All launches of the kind since prof_enable, timed or not, and their summed work.
 int64_t prof_launches(int kind, double* total_work);
