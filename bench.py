@@ -118,10 +118,15 @@ def plan_stream(w, block):
 	if not w.get("memory_budget_mib"):
 		return op_stream(w), None
 	from elf_amd.registry import SCHEDULERS
-	from elf_amd.scheduling.ilp import RematScheduler, profile_stage, solve_remat
+	from elf_amd.scheduling.ilp import RematScheduler, profile_stage, solve_remat_best
 
 	placement = w.get("placement", PLACEMENT)
-	stats, _ = profile_stage(block, n_iter=3)
+	# as Pipeline does: the stage profiled at both lean stash levels, the ILP's makespan picks one
+	by_level = {}
+	for level in (1, 2):
+		block.set_lean_stash(level)
+		by_level[level] = profile_stage(block, n_iter=3)[0]
+	stats = by_level[1]
 	# The budget is for everything this process holds on the device.  The ILP's memory model covers weights,
 	# fp32 gradient accumulators, the stage's fixed scratch (2 x Mparams) and the activations; what is resident
 	# beyond that comes off the budget it is given: the boundary tensors of all micro-batches (inputs and
@@ -130,9 +135,13 @@ def plan_stream(w, block):
 	unmodelled_mib = max(0.0, torch.cuda.memory_allocated() / 2**20 + stats["Mworkspace"] - 2 * stats["Mparams"])
 	unmodelled_mib += w["n_mb"] * (stats["Minput"] + stats["Moutput"]) + sum(p.numel() * 2 for p in block._fused_w) / 2**20
 	t_ilp = time.perf_counter()
-	solution = solve_remat([stats] * len(placement), placement, SCHEDULERS[w["scheduler"]], w["n_mb"], w["memory_budget_mib"] - unmodelled_mib)
+	alternatives = [(f"lean stash level {level}", [by_level[level]] * len(placement), None) for level in (1, 2)]
+	k, solution = solve_remat_best(alternatives, placement, SCHEDULERS[w["scheduler"]], w["n_mb"], w["memory_budget_mib"] - unmodelled_mib)
 	t_ilp = time.perf_counter() - t_ilp
+	block.set_lean_stash(k + 1)
+	stats = by_level[k + 1]
 	remat = {
+		"lean_stash_level": k + 1,
 		"memory_budget_mib": w["memory_budget_mib"], "unmodelled_resident_mib": unmodelled_mib, "ilp_seconds": t_ilp, "ilp_makespan_ms": solution["objective"],
 		"ilp_peak_mib_rank": solution["peak_mems"][placement[BLOCK_ID]],
 		"decisions_block": {k: int(sum(solution[k][BLOCK_ID])) for k in ("full_fwd", "activations_bwd", "full_bwd")},

@@ -49,7 +49,8 @@ static const unsigned WIN_MASK = (1u << B_H1) | (1u << B_O) | (1u << B_H2) | (1u
 // link twice (a third of the stash bytes; the same kernels on the same inputs: bit-identical).  A stage with a
 // lean stash (elf_stage_set_lean_stash) does the same for every micro-batch, to hold less between F and B.
 static const unsigned REFORM_MASK = (1u << B_H1) | (1u << B_H2) | (1u << B_A);
-// An offloaded micro-batch also leaves out the outputs of the two projections that a GEMM over buffers it holds anyway
+// An offloaded micro-batch (and every micro-batch of a stage at lean level 2) also leaves out the outputs of the two
+// projections that a GEMM over buffers it holds anyway
 // gives back for a third of their link time: the QKV projection's output (one GEMM over the re-formed norm output, plus
 // RoPE: 1.0 ms against 2 x 3.4 ms of link time for its 168 MB at the 70B shape) and the attention residual x2 = x + o Wo^T
 // (0.8 ms against 2 x 2.7 ms for 134 MB; the forward's own GEMM call with its residual epilogue: bit-identical).
@@ -108,7 +109,7 @@ struct Stage {
 	// optional final norm + output head behind the last block (logits [T, vld], vld >= vocab_out)
 	int vocab_in = 0, vocab_out = 0, vld = 0;
 	bool final_norm = false;
-	bool lean = false;  // elf_stage_set_lean_stash: F keeps no REFORM_MASK buffer, B forms them again
+	int lean = 0;  // elf_stage_set_lean_stash: F keeps no REFORM_MASK (1) / OFFLOAD_REFORM_MASK (2) buffer, B forms them again
 	void* xw[XP_COUNT] = {};
 	float* xg[XP_COUNT] = {};
 	void* xg16[XP_COUNT] = {};
@@ -311,7 +312,7 @@ static int run_forward(Stage* s, MbState& m, const void* x, void* y, FwdMode mod
 		if (remat_drop) drop(bs, remat_drop);
 		// the block's stash starts its way to the host while the next block computes
 		if (offload && mode == SAVE_ALL) ELF_TRY(do_offload_block(s, bs, st));
-		else if (s->lean && mode == SAVE_ALL) drop(bs, REFORM_MASK);
+		else if (s->lean && mode == SAVE_ALL) drop(bs, s->lean >= 2 ? OFFLOAD_REFORM_MASK : REFORM_MASK);
 	}
 	if (s->vocab_out) {
 		// last stage: (final norm,) logits = h W_head^T   (benchmarks/models/simple.py:497, 508)
@@ -831,10 +832,11 @@ int elf_stage_set_ends(elf_stage_t* h, int vocab_in, int vocab_out, int vocab_ou
 	return 0;
 }
 
-int elf_stage_set_lean_stash(elf_stage_t* h, int on) {
+int elf_stage_set_lean_stash(elf_stage_t* h, int level) {
 	Stage* s = (Stage*)h;
 	ELF_REQUIRE(s, "elf_stage_set_lean_stash: null stage");
-	s->lean = on != 0;
+	ELF_REQUIRE(level >= 0 && level <= 2, "elf_stage_set_lean_stash: level must be 0, 1 or 2 (got %d)", level);
+	s->lean = level;
 	return 0;
 }
 

@@ -236,8 +236,11 @@ class HipStageBlock(StageBlockBase):
 	the W passes of a step; ``scale_grads`` divides by the batch size and writes the bf16
 	``param.grad`` the reference exposes.
 
-	``lean_stash=True``: forwards keep neither the norm outputs nor the FFN activation and B forms them
-	again (a third less held between F and B, same results); ``Pipeline`` sets it under a memory budget.
+	``lean_stash`` (False / 0, True / 1, 2): at level 1 forwards keep neither the norm outputs nor the FFN
+	activation and B forms them again (a third less held between F and B, same results); level 2 also leaves
+	out the QKV projection and the attention residual, which B forms again with two GEMMs (a quarter less
+	again, about 5 % of a block's time).  ``Pipeline`` picks the level under a memory budget
+	(``set_lean_stash``: between steps only).
 	"""
 
 	def __init__(self, model, id_, placement, signature, pp_group=None, dp_group=None, recv_pgs=None, send_pgs=None, *, mb_size, seq_len=None, lean_stash=False):
@@ -251,8 +254,14 @@ class HipStageBlock(StageBlockBase):
 		self._samples = {}  # mb -> sequences in it, where fewer than mb_size
 		self._kept = {}  # mb -> external tensors the library still points at (x until B/recompute, dy until W)
 		self._remat_cache = {}  # id(strategy) -> (strategy, forward flags)
-		self.lean_stash = bool(lean_stash)
+		self.lean_stash = int(lean_stash)
 		self._build(mb_size, seq_len)
+
+	def set_lean_stash(self, level):
+		"""What the forwards issued from now on keep (0, 1 or 2, see the class docstring).  Between steps only: a
+		micro-batch's B reads the stash its own F left."""
+		_lib.check(self.lib.elf_stage_set_lean_stash(self._handle, int(level)), "elf_stage_set_lean_stash")
+		self.lean_stash = int(level)
 
 	# ------------------------------------------------------------------ set-up
 	def _build(self, mb_size, seq_len):
@@ -283,7 +292,7 @@ class HipStageBlock(StageBlockBase):
 		_lib.check(self.lib.elf_stage_create(ctypes.byref(cfg), ctypes.byref(handle)), "elf_stage_create")
 		self._handle = handle
 		if self.lean_stash:
-			_lib.check(self.lib.elf_stage_set_lean_stash(self._handle, 1), "elf_stage_set_lean_stash")
+			_lib.check(self.lib.elf_stage_set_lean_stash(self._handle, self.lean_stash), "elf_stage_set_lean_stash")
 
 		def fuse(params, pad_rows=0):
 			"""Move `params` (row blocks of one matrix) into one bf16 buffer + one fp32 grad buffer

@@ -182,9 +182,21 @@ class Pipeline:
 		if self.cfg.memory_budget is not None:
 			if any(not isinstance(b, HipStageBlock) for b in self.blocks):
 				raise NotImplementedError("Pipeline: memory_budget profiles stages on the native executor; a stage that is not a chain of transformer blocks cannot be profiled")
-			own = {b.id: profile_stage(b)[0] for b in self.blocks}
-			assert len(own) == len(self.placement), "memory_budget needs the statistics of every stage of the placement"
-			self._remat_stats = [own[i] for i in range(len(self.placement))]
+			# the stages profiled at both lean stash levels: the ILP's makespan decides which one the step runs with (the
+			# leaner stash costs two GEMMs per block in B and saves whole recomputed forwards where memory is tight)
+			assert len(self.blocks) == len(self.placement), "memory_budget needs the statistics of every stage of the placement"
+
+			def at_level(level):
+				def apply():
+					for b in self.blocks:
+						b.set_lean_stash(level)
+				return apply
+
+			self._remat_stats = []
+			for level in (1, 2):
+				at_level(level)()
+				own = {b.id: profile_stage(b)[0] for b in self.blocks}
+				self._remat_stats.append((f"lean stash level {level}", [own[i] for i in range(len(self.placement))], at_level(level)))
 			if self.scheduler is SCHEDULERS.get("auto"):
 				self.scheduler = AutoScheduler(self._remat_stats, self.cfg.memory_budget, self.cfg.worker)
 			else:
@@ -323,7 +335,8 @@ class Pipeline:
 	def get_profiling_statistics(self):
 		if not self._remat_stats:
 			raise ValueError("Profiling statistics are not available before the first step() with a memory budget")
-		return self._remat_stats
+		# of the stash level the stages are at (the one the ILP chose, once a step has run)
+		return self._remat_stats[max(1, self.blocks[0].lean_stash) - 1][1]
 
 	# ------------------------------------------------------------------ helpers (same arithmetic as the reference)
 	def _get_mb_sizes(self, split_size, batch):

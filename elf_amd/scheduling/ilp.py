@@ -22,7 +22,7 @@ from .scheduling import Operation, OperationType, OpOptions
 
 logger = logging.getLogger("ilp")
 
-__all__ = ["build_ilp_params", "solve_remat", "evaluate_remat", "RematScheduler", "stagerematify", "AutoScheduler", "RematOption", "profile_stage"]
+__all__ = ["build_ilp_params", "solve_remat", "solve_remat_best", "evaluate_remat", "RematScheduler", "stagerematify", "AutoScheduler", "RematOption", "profile_stage"]
 
 _OPS = ("f", "b", "w")
 _KIND = {OperationType.FORWARD: "f", OperationType.BACKWARD_INPUTS: "b", OperationType.BACKWARD_PARAMS: "w"}
@@ -507,13 +507,46 @@ def _my_rank():
 	return dist.get_rank() if dist.is_available() and dist.is_initialized() else 0
 
 
+def _alternatives(stats):
+	"""``stats`` as the callers give it -> [(label, statistics per stage, callable that puts the stages into that
+	state or None)].  Plain per-stage statistics are one alternative; a list of ``(label, statistics, apply)``
+	triples (e.g. the stages profiled at two stash levels) is taken as it is."""
+	if stats and isinstance(stats[0], tuple):
+		return list(stats)
+	return [(None, stats, None)]
+
+
+def solve_remat_best(stats, placement, scheduler, n_micro_batches, memory_budget, **kw):
+	"""``solve_remat`` over every alternative of ``stats`` (see ``_alternatives``) -> (index of the alternative
+	with the smallest makespan, its solution).  An alternative the budget cannot hold is skipped; when none
+	fits, the last error is raised."""
+	best, err = (None, None), None
+	for k, (label, st, _) in enumerate(_alternatives(stats)):
+		try:
+			sol = solve_remat(st, placement, scheduler, n_micro_batches, memory_budget, **kw)
+		except RuntimeError as e:
+			err = e
+			continue
+		if label is not None:
+			logger.info(f"remat ILP, {label}: makespan {sol['objective']:.2f} ms")
+		if best[1] is None or sol["objective"] < best[1]["objective"]:
+			best = (k, sol)
+	if best[1] is None:
+		raise err
+	return best
+
+
 def stagerematify(scheduler, stats, budget, worker=0):
 	"""scheduler -> scheduler that solves the ILP on rank ``worker`` (lazily, per call), shares the
-	solution with the other ranks and applies it."""
+	solution with the other ranks and applies it.  ``stats``: the statistics of every stage, or alternatives
+	of them (``_alternatives``): the one with the best makespan is applied, stages included."""
 
 	def StageRemat(placement, nmb):
-		solution = solve_remat(stats, placement, scheduler, nmb, budget) if _my_rank() == worker else None
-		solution = _broadcast(solution, worker)
+		choice = solve_remat_best(stats, placement, scheduler, nmb, budget) if _my_rank() == worker else None
+		k, solution = _broadcast(choice, worker)
+		apply = _alternatives(stats)[k][2]
+		if apply is not None:
+			apply()
 		return RematScheduler(scheduler, solution)(placement, nmb)
 
 	return StageRemat
@@ -527,17 +560,20 @@ class AutoScheduler:
 		self.schedulers = [k for k in SCHEDULERS.available() if k not in ("auto", "fixed", "full_remat")]
 
 	def __call__(self, placement, nmb):
-		best = (float("inf"), None, None)
+		best = (float("inf"), None, None, 0)
 		if _my_rank() == self.worker:
 			for name in self.schedulers:
 				try:
-					sol = solve_remat(self.stats, placement, resolve(name, SCHEDULERS), nmb, self.budget)
+					k, sol = solve_remat_best(self.stats, placement, resolve(name, SCHEDULERS), nmb, self.budget)
 					if sol["objective"] < best[0]:
-						best = (sol["objective"], name, sol)
+						best = (sol["objective"], name, sol, k)
 				except Exception as e:  # e.g. a multi-wave scheduler on a single-wave placement
 					logger.info(f"Error solving ILP for {name} scheduler: {e}. Skipping.")
 			logger.info(f"Best scheduler: {best[1]} with {best[0]:.2f}ms makespan")
 		best = _broadcast(best, self.worker)
 		if best[1] is None:
 			raise RuntimeError("AutoScheduler: no base scheduler admits a feasible remat plan for this budget and placement")
+		apply = _alternatives(self.stats)[best[3]][2]
+		if apply is not None:
+			apply()
 		return RematScheduler(resolve(best[1], SCHEDULERS), best[2])(placement, nmb)

@@ -315,13 +315,16 @@ int elf_stage_set_ends(elf_stage_t* s, int vocab_in, int vocab_out, int vocab_ou
  * Every buffer of that micro-batch then has T = samples * seq rows.  Call before the micro-batch's F;
  * the value holds until it is set again or elf_stage_clear; unset micro-batches have cfg.mb. */
 int elf_stage_set_mb_samples(elf_stage_t* s, int mb, int samples);
-/* Lean stash (no counterpart in the reference, where autograd decides what a forward keeps): with on != 0
- * a forward that keeps its activations drops the two norm outputs and the FFN activation of every block
+/* Lean stash (no counterpart in the reference, where autograd decides what a forward keeps).  Level 1: a
+ * forward that keeps its activations drops the two norm outputs and the FFN activation of every block
  * (a third of the stash at the Llama shapes) and backward_inputs writes them again where W needs them, from
  * passes that read their inputs anyway (the norms' backward kernels, the SwiGLU backward's epilogue) and with
- * the forward's arithmetic: same results bit for bit, under 1 % of a block's B time.  For stages that run
- * under a memory budget; applies to forwards issued after the call. */
-int elf_stage_set_lean_stash(elf_stage_t* s, int on);
+ * the forward's arithmetic: same results bit for bit, under 1 % of a block's B time.  Level 2 also drops the
+ * QKV projection's output and the attention residual (a quarter of what level 1 keeps); backward_inputs forms
+ * them again with the forward's own two GEMM calls (bit for bit; about 5 % of a block's F + B + W time): worth it
+ * where the memory it frees saves whole recomputed forwards.  Level 0 keeps everything.  For stages that run under
+ * a memory budget; applies to forwards issued after the call. */
+int elf_stage_set_lean_stash(elf_stage_t* s, int level);
 /* F: PipelineBlock.forward (block.py:210-279). x, y: bf16 [T, d_model]. */
 int elf_stage_forward(elf_stage_t* s, int mb, const void* x, void* y, uint32_t flags, void* stream);
 /* B: PipelineBlock.backward_inputs (block.py:624-694, 281-306). dy, dx: bf16 [T, d_model]; x is the

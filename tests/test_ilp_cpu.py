@@ -124,3 +124,48 @@ def test_auto_scheduler_picks_the_best_base_scheduler_and_stagerematify_applies_
 	assert [(o.op, o.block_id, o.mb_id, o.rank) for o in s1] == [(o.op, o.block_id, o.mb_id, o.rank) for o in s2] and remat_ops(s1)
 	with pytest.raises(RuntimeError):
 		AutoScheduler(st, 1.0)(placement, nmb)  # no scheduler fits 1 MiB
+
+
+def test_alternatives_of_the_stage_statistics_compete_on_the_makespan():
+	"""``Pipeline(memory_budget=)`` profiles its stages at two lean stash levels and hands both to the ILP wrappers
+	(no counterpart in the reference, whose stages have one stash): a leaner stash costs backward time and frees
+	memory.  With a loose budget the faster alternative wins, with a tight one the leaner one (it needs fewer
+	recomputed forwards), an alternative the budget cannot hold at all is skipped, and the winner's ``apply`` is
+	the one that runs."""
+	from elf_amd.scheduling.ilp import AutoScheduler, RematScheduler, solve_remat_best, stagerematify
+
+	placement, nmb = [0, 1], 4
+	fast = [_stats(), _stats()]                                        # stash 100 per micro-batch
+	lean = [_stats(Tb=13.0, Mf=60.0, Pf=110.0), _stats(Tb=13.0, Mf=60.0, Pf=110.0)]  # 40 less, backward 1 ms slower
+	applied = []
+	alts = [("fast", fast, lambda: applied.append("fast")), ("lean", lean, lambda: applied.append("lean"))]
+
+	k, sol = solve_remat_best(alts, placement, SCHEDULERS["1f1b"], nmb, 10_000)
+	assert k == 0 and sol["objective"] == pytest.approx(solve_remat(fast, placement, SCHEDULERS["1f1b"], nmb, 10_000)["objective"])
+	# plain statistics are one alternative
+	k1, sol1 = solve_remat_best(fast, placement, SCHEDULERS["1f1b"], nmb, 10_000)
+	assert k1 == 0 and sol1["objective"] == pytest.approx(sol["objective"])
+
+	tight = 400  # below the fast stash's no-remat peak of 410; the lean stash fits without recomputing
+	o_fast = solve_remat(fast, placement, SCHEDULERS["1f1b"], nmb, tight)["objective"]
+	o_lean = solve_remat(lean, placement, SCHEDULERS["1f1b"], nmb, tight)["objective"]
+	assert o_lean < o_fast
+	k, sol = solve_remat_best(alts, placement, SCHEDULERS["1f1b"], nmb, tight)
+	assert k == 1 and sol["objective"] == pytest.approx(o_lean)
+
+	got = stagerematify(SCHEDULERS["1f1b"], alts, tight)(placement, nmb)
+	assert applied == ["lean"]
+	want = RematScheduler(SCHEDULERS["1f1b"], solve_remat(lean, placement, SCHEDULERS["1f1b"], nmb, tight))(placement, nmb)
+	assert [(o.op, o.block_id, o.mb_id, o.rank) for o in got] == [(o.op, o.block_id, o.mb_id, o.rank) for o in want]
+	stagerematify(SCHEDULERS["1f1b"], alts, 10_000)(placement, nmb)
+	assert applied == ["lean", "fast"]
+	AutoScheduler(alts, tight)(placement, nmb)
+	assert applied[-1] == "lean"
+
+	# the fast stash cannot fit 300 at all (its infeasibility is not an error while another alternative fits)
+	with pytest.raises(RuntimeError):
+		solve_remat(fast, placement, SCHEDULERS["1f1b"], nmb, 300)
+	k, _ = solve_remat_best(alts, placement, SCHEDULERS["1f1b"], nmb, 300)
+	assert k == 1
+	with pytest.raises(RuntimeError, match="infeasible"):
+		solve_remat_best(alts, placement, SCHEDULERS["1f1b"], nmb, 100)

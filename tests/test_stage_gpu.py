@@ -132,7 +132,7 @@ def test_short_micro_batches_share_a_stage(kind):
 
 
 @pytest.mark.parametrize("kind", ["gpt", "llama"])
-@pytest.mark.parametrize("lean", [False, True])
+@pytest.mark.parametrize("lean", [0, 1, 2])
 @pytest.mark.parametrize("variant", ["full_fwd", "activations_bwd", "full_bwd", "offload", "offload_no_prefetch", "lean_stash"])
 def test_remat_and_offload_variants_equal_plain(kind, variant, lean):
 	"""Every remat / offload variant must give the results of the plain F-B-W sequence bit for bit: the
@@ -141,8 +141,8 @@ def test_remat_and_offload_variants_equal_plain(kind, variant, lean):
 	folded by one writer per column)."""
 	from elf_amd.scheduling import OpOptions
 
-	if lean and variant == "lean_stash":
-		pytest.skip("the lean stash alone is the lean = False case of this variant")
+	if not lean and variant == "lean_stash":
+		pytest.skip("the lean stash alone needs a level")
 	mb = 16 if variant.startswith("offload") else 2  # only buffers above 1 MiB are offloaded
 	stage = _stage(kind)
 	R, cfg, _ = _oracle(stage, mb)
@@ -152,7 +152,7 @@ def test_remat_and_offload_variants_equal_plain(kind, variant, lean):
 	held_after_f = {}
 
 	def run(variant):
-		blk = _block(stage, mb, lean_stash=variant == "lean_stash" or (lean and variant != "plain"))
+		blk = _block(stage, mb, lean_stash=0 if variant == "plain" else lean)
 		blk.zero_grad()
 		blk.set_boundary(inputs=xs, grads=dys, keep_sent=True)
 		root = lambda name, module: name == ""
@@ -213,9 +213,19 @@ def test_remat_and_offload_variants_equal_plain(kind, variant, lean):
 	y0, dx0, g0 = run("plain")
 	y1, dx1, g1 = run(variant)
 	if variant == "lean_stash":
-		# two micro-batches after F: per block the two norm outputs and the FFN activation less
+		# two micro-batches after F: per block the two norm outputs and the FFN activation less; at level 2 the QKV
+		# projection's output and the attention residual as well
 		T = mb * cfg["seq"]
-		assert held_after_f["plain"] - held_after_f["lean_stash"] == 2 * cfg["n_blocks"] * (2 * T * cfg["d_model"] + T * cfg["ffn"]) * 2
+
+		def pooled(elements):  # what the device pool holds for a bf16 buffer: 512-byte granules, 2 MiB ones from 1 MiB on
+			b = 2 * elements
+			gran = 2 << 20 if b >= 1 << 20 else 512
+			return (b + gran - 1) // gran * gran
+
+		less = 2 * pooled(T * cfg["d_model"]) + pooled(T * cfg["ffn"])
+		if lean == 2:
+			less += pooled(T * (cfg["n_heads"] + 2 * cfg["n_kv_heads"]) * cfg["head_dim"]) + pooled(T * cfg["d_model"])
+		assert held_after_f["plain"] - held_after_f["lean_stash"] == 2 * cfg["n_blocks"] * less
 	for m in range(2):
 		assert torch.equal(y0[m], y1[m]), "forward outputs must be bit-identical"
 		assert torch.equal(dx1[m], dx0[m]), f"{variant} dx[{m}] must be bit-identical"
@@ -499,3 +509,16 @@ def test_preallocate_pool_reserves_the_pinned_arena_before_the_first_step(monkey
 	monkeypatch.setenv("ELF_PREALLOCATE_POOL", "q4:1")
 	with pytest.raises(KeyError):
 		Engine([blk])
+
+
+def test_lean_stash_levels_are_zero_one_or_two():
+	from elf_amd._lib import ElfStageError
+
+	blk = _block(_stage("llama"), 2)
+	for level in (0, 1, 2, 1, 0):
+		blk.set_lean_stash(level)
+		assert blk.lean_stash == level
+	for bad in (3, -1):
+		with pytest.raises(ElfStageError, match="level must be 0, 1 or 2"):
+			blk.set_lean_stash(bad)
+	assert blk.lean_stash == 0
