@@ -52,7 +52,7 @@ WORKLOADS = {
 	                       scheduler="1f1b", causal=True, rope_theta=5e5),
 	# small configuration: GPT-2-small-shaped stage, 1F1B
 	"gpt2s_1f1b": dict(arch="gpt", n_blocks=3, d=768, heads=12, kv_heads=12, head_dim=64, ffn=3072, seq=1024, mb=8, n_mb=8,
-	                   scheduler="1f1b", causal=False),
+	                   scheduler="1f1b", causal=False, time_one_in=16),
 	# offload configuration: Llama-3-70B-shaped stage, 1F1B with activation offload
 	"llama3_70b_offload": dict(arch="llama", n_blocks=2, d=8192, heads=64, kv_heads=8, head_dim=128, ffn=28672, seq=8192, mb=1, n_mb=8,
 	                           scheduler="1f1b", causal=True, rope_theta=5e5, offload=True),
@@ -477,10 +477,11 @@ def main():
 	ap.add_argument("--no-cpu-baseline", action="store_true")
 	ap.add_argument("--prefetching-time", type=int, default=None,
 	                help="offload workloads: how many compute ops before its B a micro-batch's PREFETCH_ACTIVATIONS is placed (reference default 1)")
-	ap.add_argument("--time-one-in", type=int, default=4, metavar="N",
+	ap.add_argument("--time-one-in", type=int, default=None, metavar="N",
 	                help="per-kernel figures (the roofline's among them) from HIP events carried by one launch in N of the timed steps, "
-	                     "picked pseudo-randomly, the same picks every run (default 4; 1 = every launch: an event pair costs the stream "
-	                     "about 2 us per launch, 0.5 %% of a Llama step and 8 %% of a GPT-2-small step)")
+	                     "picked pseudo-randomly, the same picks every run (default 4, 16 for the GPT-2-small stream of 25 us kernels; "
+	                     "1 = every launch: an event pair costs the stream about 2 us per launch, 0.5 %% of a Llama step and 8 %% of a "
+	                     "GPT-2-small step)")
 	ap.add_argument("--graph", action="store_true",
 	                help="time replays of the step captured as one HIP graph (Engine.capture) instead of eager steps; the per-kernel figures "
 	                     "then come from one extra eager step after the timed region (a replay runs no host code that could bracket launches)")
@@ -514,6 +515,8 @@ def main():
 		sys.exit(1)
 	lib = _lib.load()
 	w = dict(WORKLOADS[args.workload])
+	if args.time_one_in is None:
+		args.time_one_in = w.get("time_one_in", 4)
 	if args.prefetching_time is not None:
 		w["prefetching_time"] = args.prefetching_time
 	stage = build_stage(w)
