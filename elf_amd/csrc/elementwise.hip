@@ -465,9 +465,10 @@ static inline int norm_bwd_blocks(int T, int d) {
 	}
 	const int rows_per_block = d <= 2048 ? ROWS_PER_BLOCK : 1;
 	const int want = (T + rows_per_block - 1) / rows_per_block;
-	// fewer, longer workgroups for narrow rows and for the widest ones: the partial rows are overhead traffic that the fold
-	// kernel reads back (d = 8192: 3.8 -> 4.1 TB/s with 512 instead of 1024; d = 4096 is faster with 1024: 4.9 against 4.0)
-	const int cap = (d <= 1024 || d > 4096) ? 512 : 1024;
+	// fewer, longer workgroups for narrow rows and for the wide ones: the partial rows are overhead traffic that the fold
+	// kernel reads back (d = 8192: 3.8 -> 4.1 TB/s with 512 instead of 1024; d = 4096 inside a stage's stream: 5.28 TB/s
+	// with 512, 5.05 with 1024, 5.12 with 256, 4.7 with 384 or 2048 - two workgroups per compute unit, no ragged round)
+	const int cap = (d <= 1024 || d >= 4096) ? 512 : 1024;
 	return want < cap ? want : cap;
 }
 
