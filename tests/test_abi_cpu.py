@@ -55,7 +55,7 @@ def test_argument_errors_without_device(lib):
 	assert rc == -1
 	with pytest.raises(_lib.ElfStageError):
 		_lib.check(rc, "elf_norm_fwd")
-	assert lib.elf_norm_bwd_workspace_floats(8192, 4096) == 1024 * 2 * 4096
+	assert lib.elf_norm_bwd_workspace_floats(8192, 4096) == 512 * 2 * 4096
 	# bf16 dQ partials of the 32 key tiles (causal: tile kt only meets the queries from 128 kt on) + two floats per (token, head)
 	stats = 2 * (2 * 4096 * 32 * 4)
 	assert lib.elf_attn_bwd_workspace_bytes(2, 4096, 32, 128, 0) == 2 * (32 * 4096) * 32 * 128 * 2 + stats
