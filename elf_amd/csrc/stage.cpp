@@ -302,7 +302,8 @@ static int run_forward(Stage* s, MbState& m, const void* x, void* y, FwdMode mod
 			ELF_TRY(buf_alloc(s, nx, B_X));
 			yout = nx.b[B_X].p;
 		}
-		ELF_TRY(gemm_bf16(0, 0, T, d, F, bs.b[B_A].p, F, p.w[P_W2], F, yout, d, EPI_BF16_RESID, bs.b[B_X2].p, d, 0, 0, st));
+		// (a recompute passes no y: the stage's output went downstream the first time and no backward reads it)
+		if (yout) ELF_TRY(gemm_bf16(0, 0, T, d, F, bs.b[B_A].p, F, p.w[P_W2], F, yout, d, EPI_BF16_RESID, bs.b[B_X2].p, d, 0, 0, st));
 		// drop what this mode does not keep (the block input is needed until here)
 		if (mode != SAVE_ALL) {
 			const unsigned keep = mode == SAVE_WIN ? WIN_MASK : 0u;
@@ -322,7 +323,7 @@ static int run_forward(Stage* s, MbState& m, const void* x, void* y, FwdMode mod
 			ELF_TRY(buf_alloc(s, hd, B_H1));
 			ELF_TRY(norm_fwd(norm_kind, hd.b[B_X].p, s->xw[XP_FNORM_G], s->xw[XP_FNORM_B], hd.b[B_H1].p, hd.b[B_ST1].p, T, d, s->cfg.eps, st));
 		}
-		ELF_TRY(gemm_bf16(0, 0, T, s->vld, d, hd.b[B_H1].p, d, s->xw[XP_HEAD], d, y, s->vld, EPI_BF16, nullptr, 0, 0, 0, st));
+		if (y) ELF_TRY(gemm_bf16(0, 0, T, s->vld, d, hd.b[B_H1].p, d, s->xw[XP_HEAD], d, y, s->vld, EPI_BF16, nullptr, 0, 0, 0, st));
 		if (remat_drop) drop(hd, remat_drop & (1u << B_ST1));
 		if (mode != SAVE_ALL) {
 			const unsigned keep = mode == SAVE_WIN ? WIN_MASK : 0u;
@@ -880,11 +881,7 @@ int elf_stage_backward_inputs(elf_stage_t* h, int mb, const void* x, const void*
 	if (m.remat_root) {
 		// the forward kept only the stage input: re-run it, this time keeping the stash
 		ELF_REQUIRE(x != nullptr, "elf_stage_backward_inputs: micro-batch %d was checkpointed, the stage input is needed", mb);
-		void* ytmp = s->pool.alloc((size_t)s->T * (s->vocab_out ? s->vld : s->d) * 2);
-		if (!ytmp) return -3;
-		int rc = run_forward(s, m, x, ytmp, SAVE_ALL, st);
-		s->pool.free(ytmp);
-		if (rc) return rc;
+		ELF_TRY(run_forward(s, m, x, nullptr, SAVE_ALL, st));
 		m.remat_root = false;
 	}
 	ELF_REQUIRE(m.has_acts, "elf_stage_backward_inputs: micro-batch %d has no saved activations", mb);
@@ -954,11 +951,7 @@ int elf_stage_recompute_forward(elf_stage_t* h, int mb, const void* x, int save,
 	ELF_REQUIRE(!m.has_acts && !m.has_win, "elf_stage_recompute_forward: micro-batch %d still holds its activations", mb);
 	hipStream_t st = (hipStream_t)stream;
 	use_mb(s, mb);
-	void* ytmp = s->pool.alloc((size_t)s->T * (s->vocab_out ? s->vld : s->d) * 2);
-	if (!ytmp) return -3;
-	int rc = run_forward(s, m, x, ytmp, save ? SAVE_ALL : SAVE_WIN, st);
-	s->pool.free(ytmp);
-	return rc;
+	return run_forward(s, m, x, nullptr, save ? SAVE_ALL : SAVE_WIN, st);
 }
 
 int elf_stage_recompute_backward_inputs(elf_stage_t* h, int mb, const void* dy, void* stream) {
